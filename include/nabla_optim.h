@@ -1,0 +1,212 @@
+/*
+ * nabla_optim.h -- C ABI of the MI355X (gfx950) fused optimizer-step engine.
+ *
+ * This is the drop-in boundary for ONE path of fumishiki/nabla: the optimizer
+ * step of nabla-train (Sgd / Adam / AdamW step, GradScaler unscale + found-inf +
+ * dynamic scale, clip_grad_norm, zero_grad, exportable moments and master
+ * weights).  A Rust `impl Optimizer<T, B>` / `impl OptimState<T, B>` in
+ * nabla-train binds these symbols through `extern "C"`; nothing here needs a
+ * C++ or torch type.  Each declaration cites the reference item it replaces
+ * (paths relative to the reference checkout).
+ *
+ * Conventions
+ *   - Every function returns an nbo_status.  Nothing aborts or throws; the
+ *     language-level shim turns NBO_ERR_LEN_MISMATCH / NBO_ERR_COUNT_MISMATCH /
+ *     NBO_ERR_SHAPE into the reference's panics and the NBO_ERR_STATE_* /
+ *     NBO_ERR_KIND codes into its Err(String) values.  nbo_last_error() returns
+ *     the message of the calling thread's last failure.
+ *   - Tensors are dense row-major (rows, cols) matrices in device memory owned by
+ *     the caller (nabla-core/src/cpu/mod.rs:7-11,28-30 layout); only rows*cols
+ *     matters to the arithmetic.  The engine owns moments and master weights.
+ *   - All work is enqueued on one HIP stream (the null stream unless
+ *     nbo_set_stream is called), in call order; calls that return a value to the
+ *     host (ok flags, norms, state reads) synchronise that stream, the others do
+ *     not.  One caller at a time: the reference's Optimizer takes &mut self and
+ *     has no Send bound (optim/core.rs:9-44).
+ *   - Device 0, like the reference's HIP context (cuda_hip/hip/core.rs:331-355).
+ */
+#ifndef NABLA_OPTIM_H
+#define NABLA_OPTIM_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#pragma GCC visibility push(default)
+
+typedef enum nbo_status {
+    NBO_OK = 0,
+    NBO_ERR_LEN_MISMATCH = 1,   /* params.len() != grads.len()         alg.rs:110-114 */
+    NBO_ERR_COUNT_MISMATCH = 2, /* params.len() != optimizer's count   alg.rs:115-119 */
+    NBO_ERR_SHAPE = 3,          /* "shapes must match"                 tensor/ops.rs:638-646 */
+    NBO_ERR_STATE_KEY = 4,      /* "bad tensor key: {name}"            alg.rs:491-494 */
+    NBO_ERR_STATE_INDEX = 5,    /* "m index out of range: {i}"         alg.rs:495-497 */
+    NBO_ERR_KIND = 6,           /* "optim kind mismatch"               alg.rs:531-545 */
+    NBO_ERR_DTYPE = 7,          /* element types of the lists / optimizer do not fit */
+    NBO_ERR_ARG = 8,            /* null pointer, zero-sized list, bad enum value */
+    NBO_ERR_NO_MASTER = 9,      /* bf16 step before master weights were set */
+    NBO_ERR_TOO_LARGE = 10,     /* more than 2^32-1 chunks of 4096 elements */
+    NBO_ERR_NO_DEVICE = 11,     /* no gfx950 device / code object not loadable */
+    NBO_ERR_HIP = 1000          /* NBO_ERR_HIP + hipError_t */
+} nbo_status;
+
+/* Element type of caller tensors. */
+typedef enum nbo_dtype { NBO_DT_F32 = 0, NBO_DT_BF16 = 1, NBO_DT_F64 = 2 } nbo_dtype;
+
+/* OptimKind, in the reference's order (optim/core.rs:46-51). */
+typedef enum nbo_kind { NBO_KIND_ADAMW = 0, NBO_KIND_ADAM = 1, NBO_KIND_SGD = 2 } nbo_kind;
+
+/* OptimMeta (optim/core.rs:53-62).  Hyper-parameters cross the boundary as f64 and
+ * are narrowed to the arithmetic type inside, exactly as alg.rs:122-135 does. */
+typedef struct nbo_meta {
+    int32_t kind;
+    int32_t reserved;
+    double lr, beta1, beta2, eps, weight_decay, momentum;
+    uint64_t step_count;
+} nbo_meta;
+
+/* GradScalerState (optim/core.rs:326-332). */
+typedef struct nbo_scaler_state {
+    double scale, growth_factor, backoff_factor;
+    uint64_t growth_interval, consecutive_ok;
+} nbo_scaler_state;
+
+/* What one fused step decided; also one entry of the step trace. */
+typedef struct nbo_step_info {
+    double scale;        /* scaler scale after this step's update (0 without scaler) */
+    double norm;         /* pre-clip global norm; 0 if skipped or clipping disabled */
+    uint64_t step_count; /* optimizer step_count after the step */
+    uint32_t found_inf;  /* 1: a gradient was inf/NaN, the step was skipped */
+    uint32_t clipped;    /* 1: norm > max_norm, gradients were rescaled */
+} nbo_step_info;
+
+typedef struct nbo_list nbo_list;     /* a list of same-dtype device tensors */
+typedef struct nbo_optim nbo_optim;   /* Sgd / Adam / AdamW + its state */
+typedef struct nbo_scaler nbo_scaler; /* GradScaler */
+
+/* ---- runtime -------------------------------------------------------------------- */
+
+/* Load the precompiled gfx950 code object on device 0 and create the runtime
+ * (the reference does this lazily in cuda_hip/hip/core.rs:331-355; every other
+ * entry point calls it implicitly). */
+int nbo_init(void);
+/* Use `hip_stream` (a hipStream_t) for all subsequent work; NULL = the null stream,
+ * which is what the reference's HIP backend launches on (hip/backend.rs:337). */
+int nbo_set_stream(void *hip_stream);
+/* B::sync (common/backend/mod.rs:82-216): wait for all enqueued work. */
+int nbo_sync(void);
+const char *nbo_last_error(void);
+const char *nbo_status_string(int status);
+/* "major.minor.patch" of this library. */
+const char *nbo_version(void);
+
+/* ---- tensor lists: the &[&Tensor<T,B>] / &mut [&mut Tensor<T,B>] arguments ----- */
+
+/* `dev_ptrs[i]` is the device address of tensor i (RtcStorage buffer of the HIP
+ * backend, common/rtc.rs:34-37), rows[i] x cols[i] elements of `dtype`.  The
+ * packed descriptor is built and uploaded once; nbo_list_set_ptrs re-uploads the
+ * addresses when the caller's tensors have moved. */
+int nbo_list_create(uint64_t n_tensors, const uint64_t *rows, const uint64_t *cols, int dtype,
+                    const void *const *dev_ptrs, nbo_list **out);
+int nbo_list_set_ptrs(nbo_list *list, const void *const *dev_ptrs);
+int nbo_list_destroy(nbo_list *list);
+
+/* ---- optimizer: Sgd / Adam / AdamW (optim/alg.rs) -------------------------------- */
+
+/* Sgd::new / Adam::new / AdamW::new (alg.rs:319-330, 181-199, 20-39) + the builder
+ * setters, all at once through `meta` (meta->kind selects the algorithm;
+ * meta->step_count seeds step_count).  Moments are created zero-filled.
+ * state_dtype: NBO_DT_F32 or NBO_DT_F64 -- the arithmetic type T.
+ * keep_master != 0: additionally hold f32 master weights so that the caller's
+ * parameters and gradients may be bf16 (T = f32). */
+int nbo_optim_create(const nbo_meta *meta, uint64_t n_tensors, const uint64_t *rows,
+                     const uint64_t *cols, int state_dtype, int keep_master, nbo_optim **out);
+int nbo_optim_destroy(nbo_optim *opt);
+
+/* Optimizer::step (optim/core.rs:10; alg.rs:109-150, 254-291, 382-416).  Gradients
+ * are used as they are.  Asynchronous. */
+int nbo_optim_step(nbo_optim *opt, nbo_list *params, nbo_list *grads);
+/* Optimizer::reset (alg.rs:152-162, 293-303, 418-423). */
+int nbo_optim_reset(nbo_optim *opt);
+/* Optimizer::set_lr (alg.rs:164-166, 305-307, 425-427). */
+int nbo_optim_set_lr(nbo_optim *opt, double lr);
+/* OptimState::meta / load_meta (alg.rs:518-545, 595-615, 650-670).  load_meta
+ * returns NBO_ERR_KIND when meta->kind differs from the optimizer's. */
+int nbo_optim_get_meta(nbo_optim *opt, nbo_meta *out);
+int nbo_optim_load_meta(nbo_optim *opt, const nbo_meta *meta);
+
+/* OptimState::state_tensors / load_state_tensors (alg.rs:476-516, 553-593, 623-648),
+ * one tensor at a time.  `name` is "m{i}" / "v{i}" (Adam, AdamW), "v{i}" (Sgd
+ * velocity), or "w{i}" for the f32 master weights (no counterpart in the reference,
+ * which has no mixed-precision optimizer).  `n_elems` must equal rows*cols of
+ * tensor i; elements have the optimizer's state dtype.  `on_device` says whether
+ * `buf` is a device or a host address. */
+int nbo_optim_state_read(nbo_optim *opt, const char *name, void *buf, uint64_t n_elems,
+                         int on_device);
+int nbo_optim_state_write(nbo_optim *opt, const char *name, const void *buf, uint64_t n_elems,
+                          int on_device);
+/* master = f32(params) for bf16 parameter lists (Tensor::cast, tensor/shape.rs:489-493),
+ * and the converse params = bf16(master). */
+int nbo_optim_master_from_params(nbo_optim *opt, nbo_list *params_bf16);
+int nbo_optim_params_from_master(nbo_optim *opt, nbo_list *params_bf16);
+
+/* ---- GradScaler (optim/core.rs:254-260, 334-413) ---------------------------------- */
+
+/* GradScaler::new + load_state; state == NULL gives the defaults of core.rs:336-344. */
+int nbo_scaler_create(const nbo_scaler_state *state, nbo_scaler **out);
+int nbo_scaler_destroy(nbo_scaler *s);
+int nbo_scaler_state_get(nbo_scaler *s, nbo_scaler_state *out); /* GradScaler::state */
+int nbo_scaler_load_state(nbo_scaler *s, const nbo_scaler_state *state);
+/* GradScaler::unscale_and_update (core.rs:351-388) on f32 / f64 gradients, in place.
+ * *ok = 1 if all gradients were finite (they are now unscaled), 0 otherwise (they
+ * are now zeros, scale was backed off).  Synchronous. */
+int nbo_scaler_unscale_and_update(nbo_scaler *s, nbo_list *grads, int *ok);
+
+/* ---- gradient utilities ------------------------------------------------------------ */
+
+/* clip_grad_norm (nabla-train/src/trainer.rs:500-523), in place on f32 / f64
+ * gradients; *norm receives the pre-clip norm (0 when max_norm <= 0).  Synchronous. */
+int nbo_clip_grad_norm(nbo_list *grads, double max_norm, double *norm);
+/* zero_grad (nabla-ml/src/autograd/ops.rs:1668-1673; trainer.rs:285-290). */
+int nbo_zero_grad(nbo_list *grads);
+/* scale_grad (autograd/ops.rs:1675-1680), f32 / f64 gradients. */
+int nbo_scale_grad(nbo_list *grads, double factor);
+
+/* ---- the fused Trainer tail ---------------------------------------------------------- */
+
+#define NBO_STEP_ZERO_GRADS 1u     /* trainer.rs:285-290 folded into the update */
+#define NBO_STEP_SKIP_NONFINITE 2u /* GradNanPolicy::Skip (trainer.rs:239-245) without a scaler */
+
+/* One Trainer iteration after backward (trainer.rs:230-291) in three launches:
+ *   scaler.unscale_and_update(grads)  -> found_inf, skip, scale update
+ *   clip_grad_norm(grads, max_norm)   -> only when max_norm > 0
+ *   optimizer.step(params, grads)     -> unscale and clip factors applied on the fly
+ *   params = bf16(master)             -> for bf16 lists
+ *   zero grads                        -> with NBO_STEP_ZERO_GRADS
+ * `scaler` may be NULL.  Gradients are not modified (except for the optional
+ * zeroing): the two factors are applied inside the update, element by element,
+ * with the same roundings as the reference's in-place passes.  The skip decision
+ * is taken on the device; nothing is read back.  Asynchronous. */
+int nbo_fused_step(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, nbo_list *grads,
+                   double max_norm, uint32_t flags);
+/* Outcome of the optimizer's most recent fused step.  Synchronous. */
+int nbo_optim_last_step(nbo_optim *opt, nbo_step_info *out);
+/* The last `max_entries` (at most 1024) fused-step outcomes, oldest first; *n_out
+ * receives how many were written, *total how many fused steps ran in all. */
+int nbo_optim_trace_read(nbo_optim *opt, nbo_step_info *out, uint64_t max_entries,
+                         uint64_t *n_out, uint64_t *total);
+
+/* ---- measurement helpers --------------------------------------------------------------- */
+
+/* Device-to-device streaming copy of `bytes` (multiple of 16) with the engine's own
+ * copy kernel; used to calibrate HBM byte counters against a known transfer. */
+int nbo_copy_bytes(const void *src_dev, void *dst_dev, uint64_t bytes);
+
+#pragma GCC visibility pop
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,749 @@
+// extern "C" entry points of include/nabla_optim.h.
+#include <cstdlib>
+#include <cstring>
+#include <new>
+
+#include "nbo_host.hpp"
+
+using namespace nbo;
+
+namespace {
+
+// Runs `body`, mapping internal errors to status codes; nothing escapes the C ABI.
+template <typename F> int guarded(F &&body)
+{
+    try {
+        body();
+        return NBO_OK;
+    } catch (const Error &e) {
+        set_last_error(e.msg);
+        return e.status;
+    } catch (const std::bad_alloc &) {
+        set_last_error("host allocation failed");
+        return NBO_ERR_ARG;
+    } catch (...) {
+        set_last_error("unexpected internal error");
+        return NBO_ERR_ARG;
+    }
+}
+
+void require(bool cond, int status, const char *msg)
+{
+    if (!cond) fail(status, msg);
+}
+
+const char *kind_name(int kind)
+{
+    return kind == NBO_KIND_ADAMW ? "AdamW" : kind == NBO_KIND_ADAM ? "Adam" : "SGD";
+}
+
+NboHyper hyper_of(const nbo_optim *o)
+{
+    NboHyper h;
+    h.lr = o->meta.lr;
+    h.beta1 = o->meta.beta1;
+    h.beta2 = o->meta.beta2;
+    h.eps = o->meta.eps;
+    h.weight_decay = o->meta.weight_decay;
+    h.momentum = o->meta.momentum;
+    h.kind = (uint32_t)o->meta.kind;
+    h.pad = 0;
+    return h;
+}
+
+// The reference's two length asserts (alg.rs:110-119 and siblings), then the shape
+// assert of axpy_inplace (tensor/ops.rs:638-646), then what only this engine can get
+// wrong: element types.
+void check_step_args(const nbo_optim *opt, const nbo_list *params, const nbo_list *grads)
+{
+    require(opt && params && grads, NBO_ERR_ARG, "null optimizer or tensor list");
+    const char *k = kind_name(opt->meta.kind);
+    if (params->layout.nt() != grads->layout.nt())
+        fail(NBO_ERR_LEN_MISMATCH, std::string("nabla-train: ") + k + " params/grads length mismatch");
+    if (params->layout.nt() != opt->layout.nt())
+        fail(NBO_ERR_COUNT_MISMATCH, std::string("nabla-train: ") + k + " params count mismatch");
+    for (uint64_t t = 0; t < opt->layout.nt(); t++) {
+        const bool same = params->layout.rows[t] == grads->layout.rows[t] &&
+                          params->layout.cols[t] == grads->layout.cols[t] &&
+                          params->layout.rows[t] == opt->layout.rows[t] &&
+                          params->layout.cols[t] == opt->layout.cols[t];
+        if (!same)
+            fail(NBO_ERR_SHAPE,
+                 "nabla: axpy_inplace (" + std::to_string(opt->layout.rows[t]) + "x" +
+                     std::to_string(opt->layout.cols[t]) + ") vs (" +
+                     std::to_string(grads->layout.rows[t]) + "x" +
+                     std::to_string(grads->layout.cols[t]) + ") -- shapes must match (tensor " +
+                     std::to_string(t) + ")");
+    }
+    require(params->dtype == grads->dtype, NBO_ERR_DTYPE, "params and grads differ in element type");
+    if (params->dtype == NBO_DT_BF16) {
+        require(opt->state_dtype == NBO_DT_F32 && opt->keep_master, NBO_ERR_DTYPE,
+                "bf16 tensors need an optimizer created with f32 state and keep_master");
+        require(opt->master_valid, NBO_ERR_NO_MASTER,
+                "bf16 step before the master weights were set (nbo_optim_master_from_params or "
+                "nbo_optim_state_write \"w{i}\")");
+    } else {
+        require(params->dtype == opt->state_dtype, NBO_ERR_DTYPE,
+                "tensor element type differs from the optimizer's state type");
+    }
+}
+
+NboUpdateArgs update_args(nbo_optim *opt, nbo_list *params, nbo_list *grads, bool with_gf,
+                          bool zero_grads)
+{
+    NboUpdateArgs a = {};
+    a.L = opt->layout.dev;
+    a.p_ptrs = params->ptrs_dev;
+    a.g_ptrs = grads->ptrs_dev;
+    a.master = params->dtype == NBO_DT_BF16 ? opt->master : nullptr;
+    a.m = opt->m;
+    a.v = opt->v;
+    a.opt = opt->dev;
+    a.gf = with_gf ? opt->gf : nullptr;
+    a.zero_grads = zero_grads ? 1u : 0u;
+    return a;
+}
+
+int update_kernel(const nbo_optim *opt, const nbo_list *params)
+{
+    return K_UPDATE_BASE + params->dtype * 3 + opt->meta.kind;
+}
+
+uint32_t norm_grid(const Layout &L)
+{
+    return L.nchunks < NBO_NORM_GRID_MAX ? L.nchunks : NBO_NORM_GRID_MAX;
+}
+
+// First stage of the norm / found_inf pass over `grads`; partials land in the
+// runtime's scratch.  Returns the grid used (0 for an empty list).
+uint32_t launch_norm(nbo_list *grads, const NboScalerDev *scaler)
+{
+    Runtime &rt = Runtime::get();
+    NboNormArgs a = {};
+    a.L = grads->layout.dev;
+    a.g_ptrs = grads->ptrs_dev;
+    a.scaler = scaler;
+    a.partial_sumsq = rt.partial_sumsq();
+    a.partial_flag = rt.partial_flag();
+    a.grid = norm_grid(grads->layout);
+    rt.launch(K_NORM_BASE + grads->dtype, a.grid, NBO_BLOCK, a);
+    return a.grid;
+}
+
+void launch_scale(nbo_list *grads, const NboGradFactors *gf, double factor, uint32_t mode)
+{
+    NboScaleArgs a = {};
+    a.L = grads->layout.dev;
+    a.g_ptrs = grads->ptrs_dev;
+    a.gf = gf;
+    a.factor = factor;
+    a.mode = mode;
+    Runtime::get().launch(K_SCALE_BASE + grads->dtype, grads->layout.nchunks, NBO_BLOCK, a);
+}
+
+// "m12" -> ('m', 12) with the reference's parsing rules (alg.rs:491-507): the prefix
+// letter, then what Rust's str::parse::<usize> accepts.
+void parse_state_name(const nbo_optim *opt, const char *name, char *which, uint64_t *index)
+{
+    require(name != nullptr, NBO_ERR_ARG, "null state name");
+    const char c = name[0];
+    const bool adam_like = opt->meta.kind != NBO_KIND_SGD;
+    const bool known = c == 'v' || (c == 'm' && adam_like) || (c == 'w' && opt->keep_master);
+    if (!known) fail(NBO_ERR_STATE_KEY, std::string("bad tensor key: ") + name);
+    const char *p = name + 1;
+    if (*p == '+') p++;
+    if (*p == '\0') fail(NBO_ERR_STATE_KEY, std::string("bad tensor key: ") + name);
+    uint64_t v = 0;
+    for (; *p; p++) {
+        if (*p < '0' || *p > '9') fail(NBO_ERR_STATE_KEY, std::string("bad tensor key: ") + name);
+        if (v > (UINT64_MAX - (uint64_t)(*p - '0')) / 10)
+            fail(NBO_ERR_STATE_KEY, std::string("bad tensor key: ") + name);
+        v = v * 10 + (uint64_t)(*p - '0');
+    }
+    if (v >= opt->layout.nt())
+        fail(NBO_ERR_STATE_INDEX, std::string(1, c) + " index out of range: " + std::to_string(v));
+    *which = c;
+    *index = v;
+}
+
+char *state_base(nbo_optim *opt, char which)
+{
+    if (which == 'w') return (char *)opt->master;
+    if (opt->meta.kind == NBO_KIND_SGD) return (char *)opt->m; // velocity
+    return which == 'm' ? (char *)opt->m : (char *)opt->v;
+}
+
+void state_copy(nbo_optim *opt, const char *name, void *buf, uint64_t n_elems, int on_device,
+                bool to_engine)
+{
+    require(opt != nullptr, NBO_ERR_ARG, "null optimizer");
+    require(buf != nullptr || n_elems == 0, NBO_ERR_ARG, "null buffer");
+    char which;
+    uint64_t i;
+    parse_state_name(opt, name, &which, &i);
+    if (n_elems != opt->layout.n[i])
+        fail(NBO_ERR_SHAPE, std::string("state tensor ") + name + " has " +
+                                std::to_string(opt->layout.n[i]) + " elements, buffer has " +
+                                std::to_string(n_elems));
+    Runtime &rt = Runtime::get();
+    const size_t eb = which == 'w' ? 4 : opt->elem_bytes();
+    char *dev = state_base(opt, which) + opt->layout.soff[i] * eb;
+    const size_t bytes = (size_t)n_elems * eb;
+    if (bytes == 0) return;
+    if (on_device) {
+        hip_check(hipMemcpyAsync(to_engine ? (void *)dev : buf, to_engine ? buf : (void *)dev, bytes,
+                                 hipMemcpyDeviceToDevice, rt.stream()),
+                  "hipMemcpyAsync D2D");
+    } else if (to_engine) {
+        rt.upload(dev, buf, bytes);
+    } else {
+        rt.read_back(buf, dev, bytes);
+    }
+    if (to_engine && which == 'w') {
+        // the master weights count as set once every tensor has been written; the
+        // caller writes them all before stepping, as a checkpoint load does
+        opt->master_valid = true;
+    }
+}
+
+void fill_info(const NboTraceEntry &e, nbo_step_info *out)
+{
+    out->scale = e.scale;
+    out->norm = e.norm;
+    out->step_count = e.step_count;
+    out->found_inf = e.found_inf;
+    out->clipped = e.clipped;
+}
+
+} // namespace
+
+extern "C" {
+
+int nbo_init(void)
+{
+    return guarded([] { Runtime::get(); });
+}
+
+int nbo_set_stream(void *hip_stream)
+{
+    return guarded([&] { Runtime::get().set_stream((hipStream_t)hip_stream); });
+}
+
+int nbo_sync(void)
+{
+    return guarded([] { Runtime::get().sync(); });
+}
+
+const char *nbo_last_error(void) { return get_last_error(); }
+
+const char *nbo_status_string(int status)
+{
+    switch (status) {
+    case NBO_OK: return "ok";
+    case NBO_ERR_LEN_MISMATCH: return "params/grads length mismatch";
+    case NBO_ERR_COUNT_MISMATCH: return "params count mismatch";
+    case NBO_ERR_SHAPE: return "shapes must match";
+    case NBO_ERR_STATE_KEY: return "bad tensor key";
+    case NBO_ERR_STATE_INDEX: return "index out of range";
+    case NBO_ERR_KIND: return "optim kind mismatch";
+    case NBO_ERR_DTYPE: return "element type mismatch";
+    case NBO_ERR_ARG: return "invalid argument";
+    case NBO_ERR_NO_MASTER: return "master weights not set";
+    case NBO_ERR_TOO_LARGE: return "tensor list too large";
+    case NBO_ERR_NO_DEVICE: return "no usable gfx950 device";
+    default: return status >= NBO_ERR_HIP ? "HIP runtime error" : "unknown status";
+    }
+}
+
+const char *nbo_version(void) { return "0.1.0"; }
+
+// ---- tensor lists -----------------------------------------------------------------
+
+static void list_upload_ptrs(nbo_list *list, const void *const *dev_ptrs)
+{
+    const uint64_t nt = list->layout.nt();
+    require(nt == 0 || dev_ptrs != nullptr, NBO_ERR_ARG, "null pointer array");
+    std::vector<uint64_t> ptrs(nt);
+    for (uint64_t t = 0; t < nt; t++) {
+        require(dev_ptrs[t] != nullptr || list->layout.n[t] == 0, NBO_ERR_ARG,
+                "null device address for a non-empty tensor");
+        ptrs[t] = (uint64_t)(uintptr_t)dev_ptrs[t];
+    }
+    if (nt) Runtime::get().upload(list->ptrs_dev, ptrs.data(), nt * 8);
+    list->ptrs.swap(ptrs);
+}
+
+int nbo_list_create(uint64_t n_tensors, const uint64_t *rows, const uint64_t *cols, int dtype,
+                    const void *const *dev_ptrs, nbo_list **out)
+{
+    return guarded([&] {
+        require(out != nullptr, NBO_ERR_ARG, "null output pointer");
+        *out = nullptr;
+        require(n_tensors == 0 || (rows && cols && dev_ptrs), NBO_ERR_ARG, "null shape or pointer array");
+        require(dtype == NBO_DT_F32 || dtype == NBO_DT_BF16 || dtype == NBO_DT_F64, NBO_ERR_ARG,
+                "unknown dtype");
+        require(n_tensors < (1ull << 31), NBO_ERR_TOO_LARGE, "too many tensors");
+        Runtime &rt = Runtime::get();
+        nbo_list *l = new nbo_list();
+        try {
+            l->dtype = dtype;
+            l->layout.build(n_tensors, rows, cols, false);
+            l->ptrs_dev = (uint64_t *)rt.dmalloc(n_tensors * 8);
+            list_upload_ptrs(l, dev_ptrs);
+            *out = l;
+        } catch (...) {
+            l->layout.release();
+            rt.dfree(l->ptrs_dev);
+            delete l;
+            throw;
+        }
+    });
+}
+
+int nbo_list_set_ptrs(nbo_list *list, const void *const *dev_ptrs)
+{
+    return guarded([&] {
+        require(list != nullptr, NBO_ERR_ARG, "null list");
+        list_upload_ptrs(list, dev_ptrs);
+    });
+}
+
+int nbo_list_destroy(nbo_list *list)
+{
+    return guarded([&] {
+        if (!list) return;
+        Runtime &rt = Runtime::get();
+        rt.sync();
+        list->layout.release();
+        rt.dfree(list->ptrs_dev);
+        delete list;
+    });
+}
+
+// ---- optimizer ----------------------------------------------------------------------
+
+int nbo_optim_create(const nbo_meta *meta, uint64_t n_tensors, const uint64_t *rows,
+                     const uint64_t *cols, int state_dtype, int keep_master, nbo_optim **out)
+{
+    return guarded([&] {
+        require(out != nullptr, NBO_ERR_ARG, "null output pointer");
+        *out = nullptr;
+        require(meta != nullptr, NBO_ERR_ARG, "null meta");
+        require(n_tensors == 0 || (rows && cols), NBO_ERR_ARG, "null shape array");
+        require(meta->kind >= NBO_KIND_ADAMW && meta->kind <= NBO_KIND_SGD, NBO_ERR_ARG,
+                "unknown optimizer kind");
+        require(state_dtype == NBO_DT_F32 || state_dtype == NBO_DT_F64, NBO_ERR_DTYPE,
+                "optimizer state is f32 or f64");
+        require(!keep_master || state_dtype == NBO_DT_F32, NBO_ERR_DTYPE,
+                "master weights are f32: keep_master needs f32 state");
+        require(n_tensors < (1ull << 31), NBO_ERR_TOO_LARGE, "too many tensors");
+        Runtime &rt = Runtime::get();
+        nbo_optim *o = new nbo_optim();
+        try {
+            o->meta = *meta;
+            o->state_dtype = state_dtype;
+            o->keep_master = keep_master != 0;
+            o->layout.build(n_tensors, rows, cols, true);
+            const size_t bytes = (size_t)o->layout.arena_elems * o->elem_bytes();
+            o->m = rt.dmalloc(bytes);
+            rt.dzero(o->m, bytes);
+            if (meta->kind != NBO_KIND_SGD) {
+                o->v = rt.dmalloc(bytes);
+                rt.dzero(o->v, bytes);
+            }
+            if (o->keep_master) {
+                o->master = rt.dmalloc((size_t)o->layout.arena_elems * 4);
+                rt.dzero(o->master, (size_t)o->layout.arena_elems * 4);
+            }
+            o->dev = (NboOptimDev *)rt.dmalloc(sizeof(NboOptimDev));
+            o->gf = (NboGradFactors *)rt.dmalloc(sizeof(NboGradFactors));
+            o->trace = (NboTraceDev *)rt.dmalloc(sizeof(NboTraceDev));
+            rt.dzero(o->gf, sizeof(NboGradFactors));
+            rt.dzero(o->trace, sizeof(NboTraceDev));
+            NboOptimDev d = {};
+            d.lr = meta->lr;
+            d.beta1 = meta->beta1;
+            d.beta2 = meta->beta2;
+            d.eps = meta->eps;
+            d.weight_decay = meta->weight_decay;
+            d.momentum = meta->momentum;
+            d.step_count = meta->kind == NBO_KIND_SGD ? 0 : meta->step_count;
+            d.kind = (uint32_t)meta->kind;
+            rt.upload(o->dev, &d, sizeof(d));
+            *out = o;
+        } catch (...) {
+            o->layout.release();
+            rt.dfree(o->m);
+            rt.dfree(o->v);
+            rt.dfree(o->master);
+            rt.dfree(o->dev);
+            rt.dfree(o->gf);
+            rt.dfree(o->trace);
+            delete o;
+            throw;
+        }
+    });
+}
+
+int nbo_optim_destroy(nbo_optim *opt)
+{
+    return guarded([&] {
+        if (!opt) return;
+        Runtime &rt = Runtime::get();
+        rt.sync();
+        opt->layout.release();
+        rt.dfree(opt->m);
+        rt.dfree(opt->v);
+        rt.dfree(opt->master);
+        rt.dfree(opt->dev);
+        rt.dfree(opt->gf);
+        rt.dfree(opt->trace);
+        delete opt;
+    });
+}
+
+int nbo_optim_step(nbo_optim *opt, nbo_list *params, nbo_list *grads)
+{
+    return guarded([&] {
+        check_step_args(opt, params, grads);
+        Runtime &rt = Runtime::get();
+        NboPrepArgs p = {};
+        p.opt = opt->dev;
+        p.gf = nullptr;
+        p.hyper = hyper_of(opt);
+        rt.launch(K_PREP, 1, 64, p);
+        const NboUpdateArgs a = update_args(opt, params, grads, false, false);
+        rt.launch(update_kernel(opt, params), opt->layout.nchunks, NBO_BLOCK, a);
+    });
+}
+
+int nbo_optim_reset(nbo_optim *opt)
+{
+    return guarded([&] {
+        require(opt != nullptr, NBO_ERR_ARG, "null optimizer");
+        Runtime &rt = Runtime::get();
+        const size_t bytes = (size_t)opt->layout.arena_elems * opt->elem_bytes();
+        rt.dzero(opt->m, bytes);
+        if (opt->v) rt.dzero(opt->v, bytes);
+        // step_count = 0 (Adam / AdamW); Sgd has none
+        rt.dzero(&opt->dev->step_count, sizeof(uint64_t));
+    });
+}
+
+int nbo_optim_set_lr(nbo_optim *opt, double lr)
+{
+    return guarded([&] {
+        require(opt != nullptr, NBO_ERR_ARG, "null optimizer");
+        opt->meta.lr = lr; // reaches the device with the next step's argument block
+    });
+}
+
+int nbo_optim_get_meta(nbo_optim *opt, nbo_meta *out)
+{
+    return guarded([&] {
+        require(opt && out, NBO_ERR_ARG, "null optimizer or output");
+        *out = opt->meta;
+        out->reserved = 0;
+        if (opt->meta.kind == NBO_KIND_SGD) {
+            // Sgd::meta reports zeros for what it does not have (alg.rs:650-661)
+            out->beta1 = out->beta2 = out->eps = 0.0;
+            out->step_count = 0;
+        } else {
+            uint64_t sc = 0;
+            Runtime::get().read_back(&sc, &opt->dev->step_count, sizeof(sc));
+            out->step_count = sc;
+            out->momentum = 0.0;
+            if (opt->meta.kind == NBO_KIND_ADAM) out->weight_decay = 0.0;
+        }
+    });
+}
+
+int nbo_optim_load_meta(nbo_optim *opt, const nbo_meta *meta)
+{
+    return guarded([&] {
+        require(opt && meta, NBO_ERR_ARG, "null optimizer or meta");
+        if (meta->kind != opt->meta.kind) fail(NBO_ERR_KIND, "optim kind mismatch");
+        // set_state of each kind copies exactly these fields (alg.rs:90-105, 244-250, 374-378)
+        opt->meta.lr = meta->lr;
+        if (opt->meta.kind == NBO_KIND_SGD) {
+            opt->meta.momentum = meta->momentum;
+            opt->meta.weight_decay = meta->weight_decay;
+            return;
+        }
+        opt->meta.beta1 = meta->beta1;
+        opt->meta.beta2 = meta->beta2;
+        opt->meta.eps = meta->eps;
+        if (opt->meta.kind == NBO_KIND_ADAMW) opt->meta.weight_decay = meta->weight_decay;
+        const uint64_t sc = meta->step_count;
+        Runtime::get().upload(&opt->dev->step_count, &sc, sizeof(sc));
+    });
+}
+
+int nbo_optim_state_read(nbo_optim *opt, const char *name, void *buf, uint64_t n_elems,
+                         int on_device)
+{
+    return guarded([&] { state_copy(opt, name, buf, n_elems, on_device, false); });
+}
+
+int nbo_optim_state_write(nbo_optim *opt, const char *name, const void *buf, uint64_t n_elems,
+                          int on_device)
+{
+    return guarded([&] { state_copy(opt, name, const_cast<void *>(buf), n_elems, on_device, true); });
+}
+
+static void cast_master(nbo_optim *opt, nbo_list *params, uint32_t mode)
+{
+    require(opt && params, NBO_ERR_ARG, "null optimizer or list");
+    require(opt->keep_master, NBO_ERR_DTYPE, "optimizer was created without master weights");
+    require(params->dtype == NBO_DT_BF16, NBO_ERR_DTYPE, "master casts take a bf16 list");
+    if (params->layout.nt() != opt->layout.nt())
+        fail(NBO_ERR_COUNT_MISMATCH, "params count mismatch");
+    for (uint64_t t = 0; t < opt->layout.nt(); t++)
+        if (params->layout.rows[t] != opt->layout.rows[t] || params->layout.cols[t] != opt->layout.cols[t])
+            fail(NBO_ERR_SHAPE, "shapes must match (tensor " + std::to_string(t) + ")");
+    NboCastArgs a = {};
+    a.L = opt->layout.dev;
+    a.src_ptrs = params->ptrs_dev;
+    a.dst_ptrs = params->ptrs_dev;
+    a.arena = opt->master;
+    a.mode = mode;
+    Runtime::get().launch(K_CAST_MASTER, opt->layout.nchunks, NBO_BLOCK, a);
+}
+
+int nbo_optim_master_from_params(nbo_optim *opt, nbo_list *params_bf16)
+{
+    return guarded([&] {
+        cast_master(opt, params_bf16, 0);
+        opt->master_valid = true;
+    });
+}
+
+int nbo_optim_params_from_master(nbo_optim *opt, nbo_list *params_bf16)
+{
+    return guarded([&] {
+        require(opt && opt->master_valid, NBO_ERR_NO_MASTER, "master weights not set");
+        cast_master(opt, params_bf16, 1);
+    });
+}
+
+// ---- GradScaler ------------------------------------------------------------------------
+
+int nbo_scaler_create(const nbo_scaler_state *state, nbo_scaler **out)
+{
+    return guarded([&] {
+        require(out != nullptr, NBO_ERR_ARG, "null output pointer");
+        *out = nullptr;
+        Runtime &rt = Runtime::get();
+        NboScalerDev d;
+        if (state) {
+            d.scale = state->scale;
+            d.growth_factor = state->growth_factor;
+            d.backoff_factor = state->backoff_factor;
+            d.growth_interval = state->growth_interval;
+            d.consecutive_ok = state->consecutive_ok;
+        } else { // GradScaler::new (core.rs:336-344)
+            d.scale = 65536.0;
+            d.growth_factor = 2.0;
+            d.backoff_factor = 0.5;
+            d.growth_interval = 2000;
+            d.consecutive_ok = 0;
+        }
+        nbo_scaler *s = new nbo_scaler();
+        try {
+            s->dev = (NboScalerDev *)rt.dmalloc(sizeof(NboScalerDev));
+            rt.upload(s->dev, &d, sizeof(d));
+            *out = s;
+        } catch (...) {
+            rt.dfree(s->dev);
+            delete s;
+            throw;
+        }
+    });
+}
+
+int nbo_scaler_destroy(nbo_scaler *s)
+{
+    return guarded([&] {
+        if (!s) return;
+        Runtime &rt = Runtime::get();
+        rt.sync();
+        rt.dfree(s->dev);
+        delete s;
+    });
+}
+
+int nbo_scaler_state_get(nbo_scaler *s, nbo_scaler_state *out)
+{
+    return guarded([&] {
+        require(s && out, NBO_ERR_ARG, "null scaler or output");
+        NboScalerDev d;
+        Runtime::get().read_back(&d, s->dev, sizeof(d));
+        out->scale = d.scale;
+        out->growth_factor = d.growth_factor;
+        out->backoff_factor = d.backoff_factor;
+        out->growth_interval = d.growth_interval;
+        out->consecutive_ok = d.consecutive_ok;
+    });
+}
+
+int nbo_scaler_load_state(nbo_scaler *s, const nbo_scaler_state *state)
+{
+    return guarded([&] {
+        require(s && state, NBO_ERR_ARG, "null scaler or state");
+        NboScalerDev d;
+        d.scale = state->scale;
+        d.growth_factor = state->growth_factor;
+        d.backoff_factor = state->backoff_factor;
+        d.growth_interval = state->growth_interval;
+        d.consecutive_ok = state->consecutive_ok;
+        Runtime::get().upload(s->dev, &d, sizeof(d));
+    });
+}
+
+int nbo_scaler_unscale_and_update(nbo_scaler *s, nbo_list *grads, int *ok)
+{
+    return guarded([&] {
+        require(s && grads && ok, NBO_ERR_ARG, "null scaler, list or output");
+        require(grads->dtype != NBO_DT_BF16, NBO_ERR_DTYPE,
+                "in-place unscale takes f32 / f64 gradients; bf16 gradients go through nbo_fused_step");
+        Runtime &rt = Runtime::get();
+        NboFinalizeArgs f = {};
+        f.partial_sumsq = rt.partial_sumsq();
+        f.partial_flag = rt.partial_flag();
+        f.grid = launch_norm(grads, s->dev);
+        f.check_finite = 1;
+        f.scaler = s->dev;
+        f.gf = rt.gf_scratch();
+        f.opt = nullptr;
+        f.trace = nullptr;
+        f.max_norm = 0.0;
+        rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
+        launch_scale(grads, rt.gf_scratch(), 1.0, 0);
+        NboGradFactors g;
+        rt.read_back(&g, rt.gf_scratch(), sizeof(g));
+        *ok = g.found_inf ? 0 : 1;
+    });
+}
+
+// ---- gradient utilities -------------------------------------------------------------------
+
+int nbo_clip_grad_norm(nbo_list *grads, double max_norm, double *norm)
+{
+    return guarded([&] {
+        require(grads && norm, NBO_ERR_ARG, "null list or output");
+        require(grads->dtype != NBO_DT_BF16, NBO_ERR_DTYPE,
+                "in-place clip takes f32 / f64 gradients; bf16 gradients go through nbo_fused_step");
+        *norm = 0.0;
+        if (max_norm <= 0.0) return; // trainer.rs:501-503
+        Runtime &rt = Runtime::get();
+        NboFinalizeArgs f = {};
+        f.partial_sumsq = rt.partial_sumsq();
+        f.partial_flag = rt.partial_flag();
+        f.grid = launch_norm(grads, nullptr);
+        f.check_finite = 0;
+        f.scaler = nullptr;
+        f.gf = rt.gf_scratch();
+        f.max_norm = max_norm;
+        rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
+        launch_scale(grads, rt.gf_scratch(), 1.0, 1);
+        NboGradFactors g;
+        rt.read_back(&g, rt.gf_scratch(), sizeof(g));
+        *norm = g.norm;
+    });
+}
+
+int nbo_zero_grad(nbo_list *grads)
+{
+    return guarded([&] {
+        require(grads != nullptr, NBO_ERR_ARG, "null list");
+        launch_scale(grads, nullptr, 0.0, 3);
+    });
+}
+
+int nbo_scale_grad(nbo_list *grads, double factor)
+{
+    return guarded([&] {
+        require(grads != nullptr, NBO_ERR_ARG, "null list");
+        require(grads->dtype != NBO_DT_BF16, NBO_ERR_DTYPE, "scale_grad takes f32 / f64 gradients");
+        launch_scale(grads, nullptr, factor, 2);
+    });
+}
+
+// ---- fused Trainer tail ---------------------------------------------------------------------
+
+int nbo_fused_step(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, nbo_list *grads,
+                   double max_norm, uint32_t flags)
+{
+    return guarded([&] {
+        check_step_args(opt, params, grads);
+        Runtime &rt = Runtime::get();
+        NboFinalizeArgs f = {};
+        f.partial_sumsq = rt.partial_sumsq();
+        f.partial_flag = rt.partial_flag();
+        // without scaler, clipping and nan policy the pass has nothing to decide, but
+        // it still runs so that the trace records every step
+        f.grid = launch_norm(grads, scaler ? scaler->dev : nullptr);
+        f.check_finite = (scaler || (flags & NBO_STEP_SKIP_NONFINITE)) ? 1u : 0u;
+        f.scaler = scaler ? scaler->dev : nullptr;
+        f.gf = opt->gf;
+        f.opt = opt->dev;
+        f.trace = opt->trace;
+        f.max_norm = max_norm;
+        f.hyper = hyper_of(opt);
+        rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
+        const NboUpdateArgs a =
+            update_args(opt, params, grads, true, (flags & NBO_STEP_ZERO_GRADS) != 0);
+        rt.launch(update_kernel(opt, params), opt->layout.nchunks, NBO_BLOCK, a);
+    });
+}
+
+int nbo_optim_last_step(nbo_optim *opt, nbo_step_info *out)
+{
+    return guarded([&] {
+        require(opt && out, NBO_ERR_ARG, "null optimizer or output");
+        std::memset(out, 0, sizeof(*out));
+        Runtime &rt = Runtime::get();
+        uint64_t count = 0;
+        rt.read_back(&count, &opt->trace->count, sizeof(count));
+        if (count == 0) return;
+        NboTraceEntry e;
+        rt.read_back(&e, &opt->trace->e[(count - 1) % NBO_TRACE_LEN], sizeof(e));
+        fill_info(e, out);
+    });
+}
+
+int nbo_optim_trace_read(nbo_optim *opt, nbo_step_info *out, uint64_t max_entries, uint64_t *n_out,
+                         uint64_t *total)
+{
+    return guarded([&] {
+        require(opt && n_out, NBO_ERR_ARG, "null optimizer or output");
+        require(out || max_entries == 0, NBO_ERR_ARG, "null entry buffer");
+        NboTraceDev *t = (NboTraceDev *)std::malloc(sizeof(NboTraceDev));
+        require(t != nullptr, NBO_ERR_ARG, "host allocation failed");
+        try {
+            Runtime::get().read_back(t, opt->trace, sizeof(NboTraceDev));
+        } catch (...) {
+            std::free(t);
+            throw;
+        }
+        uint64_t have = t->count < NBO_TRACE_LEN ? t->count : NBO_TRACE_LEN;
+        if (have > max_entries) have = max_entries;
+        for (uint64_t k = 0; k < have; k++)
+            fill_info(t->e[(t->count - have + k) % NBO_TRACE_LEN], &out[k]);
+        *n_out = have;
+        if (total) *total = t->count;
+        std::free(t);
+    });
+}
+
+int nbo_copy_bytes(const void *src_dev, void *dst_dev, uint64_t bytes)
+{
+    return guarded([&] {
+        require(src_dev && dst_dev, NBO_ERR_ARG, "null address");
+        require(bytes % 16 == 0 && ((uintptr_t)src_dev % 16) == 0 && ((uintptr_t)dst_dev % 16) == 0,
+                NBO_ERR_ARG, "copy needs 16-byte aligned addresses and size");
+        Runtime::get().launch_copy(src_dev, dst_dev, bytes / 16);
+    });
+}
+
+} // extern "C"

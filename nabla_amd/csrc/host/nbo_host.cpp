@@ -1,0 +1,214 @@
+// Runtime, module loading, launches and descriptor building for the fused
+// optimizer-step engine.
+#include "nbo_host.hpp"
+
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+
+// The gfx950 code object, embedded by nbo_code_object.S.
+extern "C" const unsigned char nbo_code_object[];
+extern "C" const unsigned char nbo_code_object_end[];
+
+namespace nbo {
+
+static thread_local std::string g_last_error;
+
+void set_last_error(const std::string &msg) { g_last_error = msg; }
+const char *get_last_error() { return g_last_error.c_str(); }
+
+void fail(int status, const std::string &msg) { throw Error{status, msg}; }
+
+void hip_check(hipError_t e, const char *what)
+{
+    if (e == hipSuccess) return;
+    std::string msg = std::string("HIP ") + what + " failed: " + hipGetErrorString(e);
+    // Leave no sticky error behind for the caller's own HIP calls to trip over.
+    (void)hipGetLastError();
+    fail(NBO_ERR_HIP + (int)e, msg);
+}
+
+static const char *const kKernelNames[K_COUNT] = {
+    "nbo_update_f32_adamw",  "nbo_update_f32_adam",  "nbo_update_f32_sgd",
+    "nbo_update_bf16_adamw", "nbo_update_bf16_adam", "nbo_update_bf16_sgd",
+    "nbo_update_f64_adamw",  "nbo_update_f64_adam",  "nbo_update_f64_sgd",
+    "nbo_norm_f32",          "nbo_norm_bf16",        "nbo_norm_f64",
+    "nbo_scale_f32",         "nbo_scale_bf16",       "nbo_scale_f64",
+    "nbo_prep",              "nbo_finalize",         "nbo_cast_master",
+    "nbo_copy_f32x4",
+};
+
+Runtime &Runtime::get()
+{
+    static std::mutex mu;
+    static Runtime *inst = nullptr;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!inst) inst = new Runtime(); // throws Error; retried on the next call
+    return *inst;
+}
+
+Runtime::Runtime()
+{
+    int ndev = 0;
+    hipError_t e = hipGetDeviceCount(&ndev);
+    if (e != hipSuccess || ndev < 1) {
+        (void)hipGetLastError();
+        fail(NBO_ERR_NO_DEVICE, "no HIP device is visible; this library runs on gfx950 only");
+    }
+    hip_check(hipSetDevice(0), "hipSetDevice(0)");
+    hipDeviceProp_t prop;
+    hip_check(hipGetDeviceProperties(&prop, 0), "hipGetDeviceProperties");
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        fail(NBO_ERR_NO_DEVICE, std::string("device 0 is ") + prop.gcnArchName +
+                                    "; the embedded code object is built for gfx950 only");
+    e = hipModuleLoadData(&module_, nbo_code_object);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        fail(NBO_ERR_NO_DEVICE,
+             std::string("hipModuleLoadData of the embedded gfx950 code object failed: ") +
+                 hipGetErrorString(e));
+    }
+    for (int k = 0; k < K_COUNT; k++)
+        hip_check(hipModuleGetFunction(&fn_[k], module_, kKernelNames[k]), kKernelNames[k]);
+    pinned_bytes_ = 1 << 20;
+    hip_check(hipHostMalloc(&pinned_, pinned_bytes_, hipHostMallocDefault), "hipHostMalloc");
+    partial_sumsq_ = (double *)dmalloc(NBO_NORM_GRID_MAX * sizeof(double));
+    partial_flag_ = (uint32_t *)dmalloc(NBO_NORM_GRID_MAX * sizeof(uint32_t));
+    gf_scratch_ = (NboGradFactors *)dmalloc(sizeof(NboGradFactors));
+}
+
+void Runtime::sync() { hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize"); }
+
+void Runtime::launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct)
+{
+    if (grid == 0) return;
+    void *args[1] = {arg_struct};
+    hip_check(hipModuleLaunchKernel(fn_[kernel], grid, 1, 1, block, 1, 1, 0, stream_, args, nullptr),
+              kKernelNames[kernel]);
+}
+
+void Runtime::launch_copy(const void *src, void *dst, uint64_t nvec)
+{
+    if (nvec == 0) return;
+    uint64_t blocks = (nvec + NBO_BLOCK - 1) / NBO_BLOCK;
+    // four 128-bit vectors per thread in flight keeps the loop short without
+    // starving the memory system
+    uint64_t grid = (blocks + 3) / 4;
+    if (grid > 0x7FFFFFFFull) grid = 0x7FFFFFFFull;
+    void *args[3] = {(void *)&src, (void *)&dst, (void *)&nvec};
+    hip_check(hipModuleLaunchKernel(fn_[K_COPY], (uint32_t)grid, 1, 1, NBO_BLOCK, 1, 1, 0, stream_,
+                                    args, nullptr),
+              kKernelNames[K_COPY]);
+}
+
+void Runtime::read_back(void *host_dst, const void *dev_src, size_t bytes)
+{
+    char *out = (char *)host_dst;
+    const char *src = (const char *)dev_src;
+    while (bytes) {
+        size_t chunk = bytes < pinned_bytes_ ? bytes : pinned_bytes_;
+        hip_check(hipMemcpyAsync(pinned_, src, chunk, hipMemcpyDeviceToHost, stream_),
+                  "hipMemcpyAsync D2H");
+        sync();
+        std::memcpy(out, pinned_, chunk);
+        out += chunk;
+        src += chunk;
+        bytes -= chunk;
+    }
+}
+
+void Runtime::upload(void *dev_dst, const void *host_src, size_t bytes)
+{
+    char *dst = (char *)dev_dst;
+    const char *src = (const char *)host_src;
+    while (bytes) {
+        size_t chunk = bytes < pinned_bytes_ ? bytes : pinned_bytes_;
+        std::memcpy(pinned_, src, chunk);
+        hip_check(hipMemcpyAsync(dst, pinned_, chunk, hipMemcpyHostToDevice, stream_),
+                  "hipMemcpyAsync H2D");
+        sync(); // the staging buffer is reused
+        dst += chunk;
+        src += chunk;
+        bytes -= chunk;
+    }
+}
+
+void *Runtime::dmalloc(size_t bytes)
+{
+    void *p = nullptr;
+    hip_check(hipMalloc(&p, bytes ? bytes : 16), "hipMalloc");
+    return p;
+}
+
+void Runtime::dfree(void *p)
+{
+    if (p) (void)hipFree(p);
+}
+
+void Runtime::dzero(void *p, size_t bytes)
+{
+    if (bytes) hip_check(hipMemsetAsync(p, 0, bytes, stream_), "hipMemsetAsync");
+}
+
+// ---------------------------------------------------------------------------------
+
+static uint64_t align_up(uint64_t x, uint64_t a) { return (x + a - 1) / a * a; }
+
+void Layout::build(uint64_t nt, const uint64_t *r, const uint64_t *c, bool with_arena)
+{
+    rows.assign(r, r + nt);
+    cols.assign(c, c + nt);
+    n.resize(nt);
+    soff.assign(nt, 0);
+    std::vector<uint32_t> chunk_begin(nt + 1, 0);
+    uint64_t chunks = 0, off = 0;
+    for (uint64_t t = 0; t < nt; t++) {
+        if (cols[t] != 0 && rows[t] > UINT64_MAX / cols[t])
+            fail(NBO_ERR_TOO_LARGE, "tensor element count overflows 64 bits");
+        n[t] = rows[t] * cols[t];
+        chunk_begin[t] = (uint32_t)chunks;
+        chunks += (n[t] + NBO_CHUNK - 1) / NBO_CHUNK;
+        if (chunks > 0xFFFFFFFFull)
+            fail(NBO_ERR_TOO_LARGE, "tensor list has more than 2^32-1 chunks of 4096 elements");
+        // every tensor starts on a 512-byte boundary of the arena, so state vectors
+        // are 16-byte aligned whatever the element type
+        soff[t] = off;
+        off += align_up(n[t], 128);
+    }
+    chunk_begin[nt] = (uint32_t)chunks;
+    nchunks = (uint32_t)chunks;
+    arena_elems = off;
+    std::vector<uint32_t> chunk_tensor(nchunks);
+    for (uint64_t t = 0; t < nt; t++)
+        for (uint32_t ch = chunk_begin[t]; ch < chunk_begin[t + 1]; ch++) chunk_tensor[ch] = (uint32_t)t;
+
+    // one blob: n | soff | chunk_begin | chunk_tensor, each 16-byte aligned
+    const size_t o_n = 0;
+    const size_t o_soff = align_up(o_n + nt * 8, 16);
+    const size_t o_cb = align_up(o_soff + nt * 8, 16);
+    const size_t o_ct = align_up(o_cb + (nt + 1) * 4, 16);
+    const size_t total = align_up(o_ct + (size_t)nchunks * 4, 16);
+    std::vector<unsigned char> host(total, 0);
+    std::memcpy(host.data() + o_n, n.data(), nt * 8);
+    std::memcpy(host.data() + o_soff, soff.data(), nt * 8);
+    std::memcpy(host.data() + o_cb, chunk_begin.data(), (nt + 1) * 4);
+    std::memcpy(host.data() + o_ct, chunk_tensor.data(), (size_t)nchunks * 4);
+    Runtime &rt = Runtime::get();
+    blob = rt.dmalloc(total);
+    rt.upload(blob, host.data(), total);
+    char *b = (char *)blob;
+    dev.n = (const uint64_t *)(b + o_n);
+    dev.soff = with_arena ? (const uint64_t *)(b + o_soff) : nullptr;
+    dev.chunk_begin = (const uint32_t *)(b + o_cb);
+    dev.chunk_tensor = (const uint32_t *)(b + o_ct);
+    dev.nt = (uint32_t)nt;
+    dev.nchunks = nchunks;
+}
+
+void Layout::release()
+{
+    if (blob) Runtime::get().dfree(blob);
+    blob = nullptr;
+}
+
+} // namespace nbo

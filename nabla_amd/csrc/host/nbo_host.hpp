@@ -1,0 +1,121 @@
+// Host runtime of the fused optimizer-step engine: internal classes behind the C ABI
+// of include/nabla_optim.h.  Device work goes through hipModuleLaunchKernel on
+// kernels of the embedded gfx950 code object and hipMemcpyAsync / hipMemsetAsync;
+// nothing here computes optimizer arithmetic on the host.
+#ifndef NBO_HOST_HPP
+#define NBO_HOST_HPP
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "../../../include/nabla_optim.h"
+#include "../nbo_device_types.h"
+
+namespace nbo {
+
+// Thrown internally, converted to a status code at the C boundary.
+struct Error {
+    int status;
+    std::string msg;
+};
+
+[[noreturn]] void fail(int status, const std::string &msg);
+void hip_check(hipError_t e, const char *what);
+void set_last_error(const std::string &msg);
+const char *get_last_error();
+
+enum KernelId {
+    K_UPDATE_BASE = 0, // + st * 3 + kind
+    K_NORM_BASE = 9,   // + st
+    K_SCALE_BASE = 12, // + st
+    K_PREP = 15,
+    K_FINALIZE = 16,
+    K_CAST_MASTER = 17,
+    K_COPY = 18,
+    K_COUNT = 19
+};
+
+// Process-wide runtime: device 0, the loaded module, the stream, scratch buffers.
+class Runtime {
+public:
+    static Runtime &get(); // creates on first use; throws Error on failure
+    hipStream_t stream() const { return stream_; }
+    void set_stream(hipStream_t s) { stream_ = s; }
+    void sync();
+
+    template <typename Args> void launch(int kernel, uint32_t grid, uint32_t block, const Args &args)
+    {
+        launch_raw(kernel, grid, block, const_cast<Args *>(&args));
+    }
+    void launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct);
+    void launch_copy(const void *src, void *dst, uint64_t nvec);
+
+    // synchronous small transfers through a pinned staging buffer
+    void read_back(void *host_dst, const void *dev_src, size_t bytes);
+    void upload(void *dev_dst, const void *host_src, size_t bytes);
+
+    void *dmalloc(size_t bytes);
+    void dfree(void *p);
+    void dzero(void *p, size_t bytes); // asynchronous on the stream
+
+    double *partial_sumsq() const { return partial_sumsq_; }
+    uint32_t *partial_flag() const { return partial_flag_; }
+    NboGradFactors *gf_scratch() const { return gf_scratch_; }
+
+private:
+    Runtime();
+    hipModule_t module_ = nullptr;
+    hipFunction_t fn_[K_COUNT] = {};
+    hipStream_t stream_ = nullptr;
+    void *pinned_ = nullptr;
+    size_t pinned_bytes_ = 0;
+    double *partial_sumsq_ = nullptr;
+    uint32_t *partial_flag_ = nullptr;
+    NboGradFactors *gf_scratch_ = nullptr;
+};
+
+// Host + device copy of the packed tensor-list descriptor.
+struct Layout {
+    std::vector<uint64_t> rows, cols, n, soff;
+    uint64_t arena_elems = 0; // elements an arena needs (with per-tensor alignment)
+    uint32_t nchunks = 0;
+    void *blob = nullptr; // one device allocation holding all tables
+    NboLayoutDev dev = {};
+
+    void build(uint64_t nt, const uint64_t *rows, const uint64_t *cols, bool with_arena);
+    void release();
+    uint64_t nt() const { return n.size(); }
+};
+
+} // namespace nbo
+
+struct nbo_list {
+    nbo::Layout layout;
+    int dtype = NBO_DT_F32;
+    std::vector<uint64_t> ptrs;
+    uint64_t *ptrs_dev = nullptr;
+};
+
+struct nbo_scaler {
+    NboScalerDev *dev = nullptr;
+};
+
+struct nbo_optim {
+    nbo::Layout layout;
+    nbo_meta meta = {};    // hyper-parameters: host copy is authoritative
+    int state_dtype = NBO_DT_F32;
+    bool keep_master = false;
+    bool master_valid = false;
+    void *m = nullptr;      // first moment / SGD velocity
+    void *v = nullptr;      // second moment (null for SGD)
+    void *master = nullptr; // f32 master weights (mixed precision)
+    NboOptimDev *dev = nullptr; // step_count lives here: the device decides skips
+    NboGradFactors *gf = nullptr;
+    NboTraceDev *trace = nullptr;
+    size_t elem_bytes() const { return state_dtype == NBO_DT_F64 ? 8 : 4; }
+};
+
+#endif

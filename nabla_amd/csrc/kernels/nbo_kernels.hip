@@ -1,0 +1,681 @@
+// gfx950 (CDNA4) device code for the fused optimizer-step engine.
+//
+// Built device-only into a code object that the host runtime loads with
+// hipModuleLoadData and launches with hipModuleLaunchKernel; every kernel takes
+// one by-value argument block from nbo_device_types.h.
+//
+// What is computed (reference = fumishiki/nabla, CPU backend):
+//   nbo_update_*    Sgd::step / Adam::step / AdamW::step   nabla-train/src/optim/alg.rs:382-416, 254-291, 109-150
+//   nbo_norm_*      finite scan of GradScaler::unscale_and_update (optim/core.rs:357-368)
+//                   + sum of squares of clip_grad_norm (trainer.rs:504-513), first stage
+//   nbo_finalize    second stage, scaler update (core.rs:369-385), clip decision
+//                   (trainer.rs:514-517) and the per-step scalars (alg.rs:120-135)
+//   nbo_scale_*     the in-place gradient rescale / zero of core.rs:372-380,
+//                   trainer.rs:518-520, autograd/ops.rs:1668-1680
+//   nbo_cast_*      bf16 <-> f32 casts (common/scalar/mod.rs:338-344)
+//
+// Numerics contract: every arithmetic operation of the reference is one IEEE
+// round-to-nearest operation here, in the same order, never contracted into an
+// FMA (the file is compiled with -ffp-contract=off and carries the pragma
+// below); division and square root are the correctly rounded ones.  The one
+// deliberate difference is denom: the reference calls powf(x, 0.5), this code
+// takes sqrt(x), which is within 1 ulp of any faithful powf.
+//
+// Memory access: the path is HBM-bound (about 0.5 flop per byte), so the
+// kernels are organised around 128-bit per-lane accesses that are contiguous
+// across the 64 lanes of a wavefront (1 KiB per wave per instruction), all
+// loads of a chunk issued before the first use, and streaming (non-temporal)
+// hints on data that is not touched again until the next step.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../nbo_device_types.h"
+
+#pragma clang fp contract(off)
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+#define DEV static __device__ __forceinline__
+// Caller tensor addresses arrive as integers; telling the compiler that they are
+// global memory turns flat_* accesses into global_* ones.
+#define GLOBAL_PTR(type, p) ((__attribute__((address_space(1))) type *)(uintptr_t)(p))
+
+// ---------------------------------------------------------------------------------
+// bf16 <-> f32, bit for bit what half::bf16 does (from_f32: NaN keeps its payload and
+// gets the quiet bit, everything else rounds to nearest even).
+DEV float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+DEV uint32_t f32_to_bf16_bits(float f)
+{
+    uint32_t x = __float_as_uint(f);
+    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (x >> 16) | 0x0040u;
+    return (x + 0x7FFFu + ((x >> 16) & 1u)) >> 16;
+}
+
+DEV bool nonfinite_f32(float f) { return (__float_as_uint(f) & 0x7F800000u) == 0x7F800000u; }
+DEV bool nonfinite_f64(double d)
+{
+    return ((uint32_t)(__double_as_longlong(d) >> 32) & 0x7FF00000u) == 0x7FF00000u;
+}
+
+// f64::powi as compiler-rt's __powidf2 (alg.rs:122-123).
+DEV double powi_f64(double a, int n)
+{
+    bool recip = n < 0;
+    uint32_t b = recip ? 0u - (uint32_t)n : (uint32_t)n;
+    double r = 1.0;
+    for (;;) {
+        if (b & 1u) r *= a;
+        b >>= 1;
+        if (b == 0) break;
+        a *= a;
+    }
+    return recip ? 1.0 / r : r;
+}
+
+// ---------------------------------------------------------------------------------
+// Storage access.  ST is the caller-tensor element type (NBO_F32 / NBO_BF16 /
+// NBO_F64); the arithmetic type T is float for the first two and double for the
+// last.  One "vector" is VEC consecutive elements = 16 bytes of T.
+template <int ST> struct Traits;
+template <> struct Traits<NBO_F32> {
+    typedef float T;
+    enum { VEC = 4, SBYTES = 4 };
+};
+template <> struct Traits<NBO_BF16> {
+    typedef float T;
+    enum { VEC = 4, SBYTES = 2 };
+};
+template <> struct Traits<NBO_F64> {
+    typedef double T;
+    enum { VEC = 2, SBYTES = 8 };
+};
+
+// arena (engine-owned, always 16-byte aligned) vectors of T
+DEV void ld_state(const float *p, float (&x)[4])
+{
+    f32x4 v = __builtin_nontemporal_load(GLOBAL_PTR(const f32x4, p));
+    x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+}
+DEV void ld_state(const double *p, double (&x)[2])
+{
+    f64x2 v = __builtin_nontemporal_load(GLOBAL_PTR(const f64x2, p));
+    x[0] = v.x; x[1] = v.y;
+}
+DEV void st_state(float *p, const float (&x)[4])
+{
+    f32x4 v = {x[0], x[1], x[2], x[3]};
+    __builtin_nontemporal_store(v, GLOBAL_PTR(f32x4, p));
+}
+DEV void st_state(double *p, const double (&x)[2])
+{
+    f64x2 v = {x[0], x[1]};
+    __builtin_nontemporal_store(v, GLOBAL_PTR(f64x2, p));
+}
+
+// caller tensors: vector of VEC storage elements at byte address p
+template <int ST> struct IO;
+template <> struct IO<NBO_F32> {
+    DEV void ldv(const char *p, float (&x)[4]) { ld_state((const float *)p, x); }
+    DEV void stv(char *p, const float (&x)[4]) { st_state((float *)p, x); }
+    DEV float ld1(const char *p) { return *GLOBAL_PTR(const float, p); }
+    DEV void st1(char *p, float x) { *GLOBAL_PTR(float, p) = x; }
+};
+template <> struct IO<NBO_F64> {
+    DEV void ldv(const char *p, double (&x)[2]) { ld_state((const double *)p, x); }
+    DEV void stv(char *p, const double (&x)[2]) { st_state((double *)p, x); }
+    DEV double ld1(const char *p) { return *GLOBAL_PTR(const double, p); }
+    DEV void st1(char *p, double x) { *GLOBAL_PTR(double, p) = x; }
+};
+template <> struct IO<NBO_BF16> {
+    DEV void ldv(const char *p, float (&x)[4])
+    {
+        u32x2 v = __builtin_nontemporal_load(GLOBAL_PTR(const u32x2, p));
+        x[0] = __uint_as_float(v.x << 16);
+        x[1] = __uint_as_float(v.x & 0xFFFF0000u);
+        x[2] = __uint_as_float(v.y << 16);
+        x[3] = __uint_as_float(v.y & 0xFFFF0000u);
+    }
+    DEV void stv(char *p, const float (&x)[4])
+    {
+        u32x2 v;
+        v.x = f32_to_bf16_bits(x[0]) | (f32_to_bf16_bits(x[1]) << 16);
+        v.y = f32_to_bf16_bits(x[2]) | (f32_to_bf16_bits(x[3]) << 16);
+        __builtin_nontemporal_store(v, GLOBAL_PTR(u32x2, p));
+    }
+    DEV float ld1(const char *p) { return bf16_bits_to_f32(*GLOBAL_PTR(const uint16_t, p)); }
+    DEV void st1(char *p, float x) { *GLOBAL_PTR(uint16_t, p) = (uint16_t)f32_to_bf16_bits(x); }
+};
+
+// ---------------------------------------------------------------------------------
+// Per-step scalars in the arithmetic type T.
+template <typename T> struct Scal;
+template <> struct Scal<float> {
+    float b1, omb1, b2, omb2, eps, ss, ibc2, omw, neg_lr, mom, wd, inv, clip;
+    bool use_mom, use_wd;
+    __device__ Scal(const NboOptimDev *o, const NboGradFactors *f)
+        : b1(o->b1), omb1(o->omb1), b2(o->b2), omb2(o->omb2), eps(o->eps_t), ss(o->ss),
+          ibc2(o->ibc2), omw(o->omw), neg_lr(o->neg_lr), mom(o->momentum_t), wd(o->wd_t),
+          inv(f ? f->inv_scale32 : 1.0f), clip(f ? f->clip32 : 1.0f),
+          use_mom(o->momentum != 0.0), use_wd(o->weight_decay != 0.0)
+    {
+    }
+};
+template <> struct Scal<double> {
+    double b1, omb1, b2, omb2, eps, ss, ibc2, omw, neg_lr, mom, wd, inv, clip;
+    bool use_mom, use_wd;
+    __device__ Scal(const NboOptimDev *o, const NboGradFactors *f)
+        : b1(o->d_b1), omb1(o->d_omb1), b2(o->d_b2), omb2(o->d_omb2), eps(o->d_eps),
+          ss(o->d_ss), ibc2(o->d_ibc2), omw(o->d_omw), neg_lr(o->d_neg_lr), mom(o->d_momentum),
+          wd(o->d_wd), inv(f ? f->inv_scale64 : 1.0), clip(f ? f->clip64 : 1.0),
+          use_mom(o->momentum != 0.0), use_wd(o->weight_decay != 0.0)
+    {
+    }
+};
+
+DEV float sqrt_rn(float x) { return __builtin_sqrtf(x); }
+DEV double sqrt_rn(double x) { return __builtin_sqrt(x); }
+
+// One element of the update.  KIND: NBO_ADAMW, NBO_ADAM, NBO_SGD.
+// Each statement is one rounding, in the order of the reference's pass chain.
+template <typename T, int KIND> DEV void step_elem(T &p, T g, T &m, T &v, const Scal<T> &s)
+{
+    g = g * s.inv;  // core.rs:379   g.map(|x| x * inv_scale); exact identity when inv == 1
+    g = g * s.clip; // trainer.rs:519 g.map(|x| x * scale_t);   exact identity when clip == 1
+    if (KIND == NBO_SGD) {
+        // alg.rs:399-414
+        T ge = g;
+        if (s.use_wd) {
+            T pw = p * s.wd;
+            ge = g + pw;
+        }
+        if (s.use_mom) {
+            T vm = m * s.mom;
+            m = vm + ge;
+            ge = m;
+        }
+        T t = s.neg_lr * ge;
+        p = p + t;
+    } else {
+        // alg.rs:138-148 / 281-289
+        T m1 = m * s.b1;
+        T t1 = s.omb1 * g;
+        m = m1 + t1;
+        T v1 = v * s.b2;
+        T q = g * g;
+        T t2 = s.omb2 * q;
+        v = v1 + t2;
+        T sc = v * s.ibc2;
+        T r = sqrt_rn(sc); // reference: powf(sc, 0.5)
+        T d = r + s.eps;
+        T nn = m * s.ss;
+        T u = nn / d;
+        if (KIND == NBO_ADAMW) p = p * s.omw;
+        T nu = (T)(-1) * u;
+        p = p + nu;
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// Chunk addressing shared by all multi-tensor kernels.
+struct ChunkRef {
+    uint32_t t;    // tensor index
+    uint32_t cnt;  // elements of the chunk that exist (1..NBO_CHUNK)
+    uint64_t base; // first element of the chunk within its tensor
+    uint64_t soff; // tensor's element offset in the state arena
+};
+
+DEV ChunkRef chunk_ref(const NboLayoutDev &L, uint32_t c)
+{
+    ChunkRef r;
+    r.t = L.chunk_tensor[c];
+    r.base = (uint64_t)(c - L.chunk_begin[r.t]) * NBO_CHUNK;
+    uint64_t rem = L.n[r.t] - r.base;
+    r.cnt = rem < (uint64_t)NBO_CHUNK ? (uint32_t)rem : NBO_CHUNK;
+    r.soff = L.soff ? L.soff[r.t] : 0;
+    return r;
+}
+
+// ---------------------------------------------------------------------------------
+// Optimizer update: one workgroup per chunk.
+template <int ST, int KIND> DEV void update_body(const NboUpdateArgs &a)
+{
+    typedef typename Traits<ST>::T T;
+    enum { VEC = Traits<ST>::VEC, SB = Traits<ST>::SBYTES, ROW = NBO_BLOCK * VEC, U = NBO_CHUNK / ROW };
+    const bool mixed = ST == NBO_BF16; // f32 master lives in the arena
+    const bool has_v = KIND != NBO_SGD;
+    const uint32_t tid = threadIdx.x;
+    const ChunkRef c = chunk_ref(a.L, blockIdx.x);
+
+    char *pp = (char *)a.p_ptrs[c.t] + c.base * SB;
+    char *pg = (char *)a.g_ptrs[c.t] + c.base * SB;
+    T *am = (T *)a.m + c.soff + c.base;
+    T *av = has_v ? (T *)a.v + c.soff + c.base : nullptr;
+    T *aw = mixed ? (T *)a.master + c.soff + c.base : nullptr;
+    const bool zero_g = a.zero_grads != 0;
+    const uint32_t vbytes = VEC * SB;
+    const bool vec_ok = ((((uintptr_t)pp) | ((uintptr_t)pg)) & (vbytes - 1)) == 0;
+
+    if (a.opt->skip) {
+        // found_inf: parameters, moments and step_count stay untouched
+        // (trainer.rs:230-236); the gradients become zeros (core.rs:372-375).
+        if (zero_g)
+            for (uint32_t i = tid; i < c.cnt; i += NBO_BLOCK) IO<ST>::st1(pg + (uint64_t)i * SB, (T)0);
+        return;
+    }
+    const Scal<T> s(a.opt, a.gf);
+    const bool use_m = KIND != NBO_SGD || s.use_mom;
+
+    if (c.cnt == NBO_CHUNK && vec_ok) {
+        T g[U][VEC], p[U][VEC], m[U][VEC] = {}, v[U][VEC] = {};
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t e = u * ROW + tid * VEC;
+            IO<ST>::ldv(pg + (uint64_t)e * SB, g[u]);
+            if (mixed) ld_state(aw + e, p[u]);
+            else IO<ST>::ldv(pp + (uint64_t)e * SB, p[u]);
+            if (use_m) ld_state(am + e, m[u]);
+            if (has_v) ld_state(av + e, v[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t e = u * ROW + tid * VEC;
+#pragma unroll
+            for (int k = 0; k < VEC; k++) step_elem<T, KIND>(p[u][k], g[u][k], m[u][k], v[u][k], s);
+            if (mixed) st_state(aw + e, p[u]);
+            IO<ST>::stv(pp + (uint64_t)e * SB, p[u]);
+            if (use_m) st_state(am + e, m[u]);
+            if (has_v) st_state(av + e, v[u]);
+            if (zero_g) {
+                T z[VEC] = {};
+                IO<ST>::stv(pg + (uint64_t)e * SB, z);
+            }
+        }
+        return;
+    }
+
+    // ragged chunk: whole vectors while they last (if the caller's pointers allow),
+    // then single elements
+    const uint32_t nvec = vec_ok ? c.cnt / VEC : 0;
+    for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
+        const uint32_t e = q * VEC;
+        T g[VEC], p[VEC], m[VEC] = {}, v[VEC] = {};
+        IO<ST>::ldv(pg + (uint64_t)e * SB, g);
+        if (mixed) ld_state(aw + e, p);
+        else IO<ST>::ldv(pp + (uint64_t)e * SB, p);
+        if (use_m) ld_state(am + e, m);
+        if (has_v) ld_state(av + e, v);
+#pragma unroll
+        for (int k = 0; k < VEC; k++) step_elem<T, KIND>(p[k], g[k], m[k], v[k], s);
+        if (mixed) st_state(aw + e, p);
+        IO<ST>::stv(pp + (uint64_t)e * SB, p);
+        if (use_m) st_state(am + e, m);
+        if (has_v) st_state(av + e, v);
+        if (zero_g) {
+            T z[VEC] = {};
+            IO<ST>::stv(pg + (uint64_t)e * SB, z);
+        }
+    }
+    for (uint32_t e = nvec * VEC + tid; e < c.cnt; e += NBO_BLOCK) {
+        T g = IO<ST>::ld1(pg + (uint64_t)e * SB);
+        T p = mixed ? aw[e] : IO<ST>::ld1(pp + (uint64_t)e * SB);
+        T m = use_m ? am[e] : (T)0;
+        T v = has_v ? av[e] : (T)0;
+        step_elem<T, KIND>(p, g, m, v, s);
+        if (mixed) aw[e] = p;
+        IO<ST>::st1(pp + (uint64_t)e * SB, p);
+        if (use_m) am[e] = m;
+        if (has_v) av[e] = v;
+        if (zero_g) IO<ST>::st1(pg + (uint64_t)e * SB, (T)0);
+    }
+}
+
+#define NBO_UPDATE_KERNEL(name, ST, KIND)                                                   \
+    extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboUpdateArgs a)     \
+    {                                                                                       \
+        update_body<ST, KIND>(a);                                                           \
+    }
+
+NBO_UPDATE_KERNEL(nbo_update_f32_adamw, NBO_F32, NBO_ADAMW)
+NBO_UPDATE_KERNEL(nbo_update_f32_adam, NBO_F32, NBO_ADAM)
+NBO_UPDATE_KERNEL(nbo_update_f32_sgd, NBO_F32, NBO_SGD)
+NBO_UPDATE_KERNEL(nbo_update_bf16_adamw, NBO_BF16, NBO_ADAMW)
+NBO_UPDATE_KERNEL(nbo_update_bf16_adam, NBO_BF16, NBO_ADAM)
+NBO_UPDATE_KERNEL(nbo_update_bf16_sgd, NBO_BF16, NBO_SGD)
+NBO_UPDATE_KERNEL(nbo_update_f64_adamw, NBO_F64, NBO_ADAMW)
+NBO_UPDATE_KERNEL(nbo_update_f64_adam, NBO_F64, NBO_ADAM)
+NBO_UPDATE_KERNEL(nbo_update_f64_sgd, NBO_F64, NBO_SGD)
+
+// ---------------------------------------------------------------------------------
+// Deterministic block reduction: xor-butterfly inside each 64-lane wavefront, then
+// the four wave results are added in wave order by thread 0.
+DEV double block_sum(double x, double *lds)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) x = x + __shfl_xor(x, off, 64);
+    const uint32_t wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63u) == 0) lds[wave] = x;
+    __syncthreads();
+    double r = 0.0;
+    if (threadIdx.x == 0) {
+        r = lds[0];
+        for (uint32_t w = 1; w < NBO_BLOCK / 64; w++) r = r + lds[w];
+    }
+    __syncthreads();
+    return r; // valid in thread 0
+}
+
+DEV uint32_t block_or(uint32_t x, uint32_t *lds)
+{
+    x = __any(x != 0) ? 1u : 0u; // wave-wide
+    const uint32_t wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63u) == 0) lds[wave] = x;
+    __syncthreads();
+    uint32_t r = 0;
+    if (threadIdx.x == 0)
+        for (uint32_t w = 0; w < NBO_BLOCK / 64; w++) r |= lds[w];
+    __syncthreads();
+    return r;
+}
+
+// First stage of the norm / found_inf pass.  A fixed grid walks the chunks with
+// stride grid, so each block's partial sum depends only on the tensor list.
+//   u = g * inv_scale rounded to T (the unscaled gradient the reference stores),
+//   sumsq += (f64)u * (f64)u   (trainer.rs:509-510)
+// For f32/bf16 inputs the f64 product is exact, so fma(d, d, acc) rounds exactly
+// like the reference's separate multiply and add; for f64 inputs it would not, so
+// that case keeps the two roundings.
+template <int ST> DEV double sq_acc(double acc, typename Traits<ST>::T u)
+{
+    const double d = (double)u;
+    if (ST == NBO_F64) {
+        const double q = d * d;
+        return acc + q;
+    }
+    return __builtin_fma(d, d, acc);
+}
+
+template <int ST> DEV bool nonfinite(typename Traits<ST>::T x);
+template <> __device__ __forceinline__ bool nonfinite<NBO_F32>(float x) { return nonfinite_f32(x); }
+template <> __device__ __forceinline__ bool nonfinite<NBO_BF16>(float x) { return nonfinite_f32(x); }
+template <> __device__ __forceinline__ bool nonfinite<NBO_F64>(double x) { return nonfinite_f64(x); }
+
+template <int ST> DEV void norm_body(const NboNormArgs &a)
+{
+    typedef typename Traits<ST>::T T;
+    enum { SB = Traits<ST>::SBYTES, VEC = Traits<ST>::VEC };
+    __shared__ double lds_d[NBO_BLOCK / 64];
+    __shared__ uint32_t lds_u[NBO_BLOCK / 64];
+    const uint32_t tid = threadIdx.x;
+    const T inv = a.scaler ? (T)(1.0 / a.scaler->scale) : (T)1; // core.rs:355
+    double acc = 0.0;
+    uint32_t bad = 0;
+
+    for (uint32_t ci = blockIdx.x; ci < a.L.nchunks; ci += a.grid) {
+        const ChunkRef c = chunk_ref(a.L, ci);
+        const char *pg = (const char *)a.g_ptrs[c.t] + c.base * SB;
+        uint32_t done = 0;
+        if (ST == NBO_BF16) {
+            // 8 bf16 per 128-bit load
+            if ((((uintptr_t)pg) & 15u) == 0) {
+                const uint32_t nvec = c.cnt / 8;
+                for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
+                    const u32x4 w = __builtin_nontemporal_load(GLOBAL_PTR(const u32x4, pg) + q);
+                    const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        const float lo = __uint_as_float(ww[k] << 16);
+                        const float hi = __uint_as_float(ww[k] & 0xFFFF0000u);
+                        bad |= (uint32_t)nonfinite_f32(lo) | (uint32_t)nonfinite_f32(hi);
+                        acc = sq_acc<ST>(acc, (T)(lo * inv));
+                        acc = sq_acc<ST>(acc, (T)(hi * inv));
+                    }
+                }
+                done = nvec * 8;
+            }
+        } else {
+            if ((((uintptr_t)pg) & 15u) == 0) {
+                const uint32_t nvec = c.cnt / VEC;
+                for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
+                    T x[VEC];
+                    IO<ST>::ldv(pg + (uint64_t)q * VEC * SB, x);
+#pragma unroll
+                    for (int k = 0; k < VEC; k++) {
+                        bad |= (uint32_t)nonfinite<ST>(x[k]);
+                        acc = sq_acc<ST>(acc, x[k] * inv);
+                    }
+                }
+                done = nvec * VEC;
+            }
+        }
+        for (uint32_t e = done + tid; e < c.cnt; e += NBO_BLOCK) {
+            const T x = IO<ST>::ld1(pg + (uint64_t)e * SB);
+            bad |= (uint32_t)nonfinite<ST>(x);
+            acc = sq_acc<ST>(acc, x * inv);
+        }
+    }
+    const double bs = block_sum(acc, lds_d);
+    const uint32_t bo = block_or(bad, lds_u);
+    if (tid == 0) {
+        a.partial_sumsq[blockIdx.x] = bs;
+        a.partial_flag[blockIdx.x] = bo;
+    }
+}
+
+#define NBO_NORM_KERNEL(name, ST)                                                           \
+    extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboNormArgs a)       \
+    {                                                                                       \
+        norm_body<ST>(a);                                                                   \
+    }
+NBO_NORM_KERNEL(nbo_norm_f32, NBO_F32)
+NBO_NORM_KERNEL(nbo_norm_bf16, NBO_BF16)
+NBO_NORM_KERNEL(nbo_norm_f64, NBO_F64)
+
+// ---------------------------------------------------------------------------------
+// Per-step scalars (alg.rs:120-135 AdamW, 265-277 Adam, 393-395 Sgd).  A skipped
+// step leaves step_count alone, because the reference never calls step() then.
+DEV void prep_step(NboOptimDev *o, const NboHyper &h, const NboGradFactors *f)
+{
+    o->lr = h.lr;
+    o->beta1 = h.beta1;
+    o->beta2 = h.beta2;
+    o->eps = h.eps;
+    o->weight_decay = h.weight_decay;
+    o->momentum = h.momentum;
+    o->kind = h.kind;
+    if (f && f->found_inf) {
+        o->skip = 1;
+        return;
+    }
+    o->skip = 0;
+    if (o->kind == NBO_SGD) {
+        const float lr_t = (float)o->lr;
+        o->neg_lr = -lr_t;
+        o->momentum_t = (float)o->momentum;
+        o->wd_t = (float)o->weight_decay;
+        o->d_neg_lr = -o->lr;
+        o->d_momentum = o->momentum;
+        o->d_wd = o->weight_decay;
+        return;
+    }
+    o->step_count += 1;
+    const int step = (int)o->step_count;
+    const double bc1 = 1.0 - powi_f64(o->beta1, step);
+    const double bc2 = 1.0 - powi_f64(o->beta2, step);
+    const double step_size = o->lr / bc1;
+    const double omb1 = 1.0 - o->beta1;
+    const double omb2 = 1.0 - o->beta2;
+    const double wd_lr = o->weight_decay * o->lr;
+    const double ibc2 = 1.0 / bc2;
+    o->b1 = (float)o->beta1;
+    o->omb1 = (float)omb1;
+    o->b2 = (float)o->beta2;
+    o->omb2 = (float)omb2;
+    o->eps_t = (float)o->eps;
+    o->ss = (float)step_size;
+    o->ibc2 = (float)ibc2;
+    const float wd_lr_t = (float)wd_lr;
+    o->omw = 1.0f - wd_lr_t; // T::one() - wd_lr, in T (alg.rs:135)
+    o->d_b1 = o->beta1;
+    o->d_omb1 = omb1;
+    o->d_b2 = o->beta2;
+    o->d_omb2 = omb2;
+    o->d_eps = o->eps;
+    o->d_ss = step_size;
+    o->d_ibc2 = ibc2;
+    o->d_omw = 1.0 - wd_lr;
+}
+
+extern "C" __global__ __launch_bounds__(64) void nbo_prep(const NboPrepArgs a)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) prep_step(a.opt, a.hyper, a.gf);
+}
+
+// Second stage: reduce the per-block partials in a fixed order, then the scalar
+// logic of GradScaler::unscale_and_update (core.rs:369-385) and clip_grad_norm
+// (trainer.rs:501-517).  Single workgroup.
+extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_finalize(const NboFinalizeArgs a)
+{
+    __shared__ double lds_d[NBO_BLOCK / 64];
+    __shared__ uint32_t lds_u[NBO_BLOCK / 64];
+    const uint32_t tid = threadIdx.x;
+    double acc = 0.0;
+    uint32_t bad = 0;
+    for (uint32_t i = tid; i < a.grid; i += NBO_BLOCK) {
+        acc = acc + a.partial_sumsq[i];
+        bad |= a.partial_flag[i];
+    }
+    const double sumsq = block_sum(acc, lds_d);
+    const uint32_t any_bad = block_or(bad, lds_u);
+    if (tid != 0) return;
+
+    NboGradFactors f;
+    f.sumsq = sumsq;
+    const bool found = a.check_finite && any_bad;
+    double inv = 1.0;
+    double scale_after = 0.0;
+    if (a.scaler) {
+        NboScalerDev s = *a.scaler;
+        inv = 1.0 / s.scale; // core.rs:355, from the scale before its update
+        if (found) {
+            s.scale = s.scale * s.backoff_factor;
+            s.consecutive_ok = 0;
+        } else {
+            s.consecutive_ok += 1;
+            if (s.consecutive_ok >= s.growth_interval) {
+                s.scale = s.scale * s.growth_factor;
+                s.consecutive_ok = 0;
+            }
+        }
+        *a.scaler = s;
+        scale_after = s.scale;
+    }
+    f.inv_scale64 = inv;
+    f.inv_scale32 = (float)inv;
+    f.found_inf = found ? 1u : 0u;
+    f.norm = 0.0;
+    f.clip64 = 1.0;
+    f.clip32 = 1.0f;
+    f.clipped = 0;
+    if (!found && a.max_norm > 0.0) {
+        const double norm = __builtin_sqrt(sumsq);
+        f.norm = norm;
+        if (norm > a.max_norm && norm > 0.0) {
+            const double c = a.max_norm / norm;
+            f.clip64 = c;
+            f.clip32 = (float)c;
+            f.clipped = 1;
+        }
+    }
+    *a.gf = f;
+    if (a.opt) prep_step(a.opt, a.hyper, &f);
+    if (a.trace) {
+        const uint64_t i = a.trace->count;
+        NboTraceEntry e;
+        e.scale = scale_after;
+        e.norm = f.norm;
+        e.step_count = a.opt ? a.opt->step_count : 0;
+        e.found_inf = f.found_inf;
+        e.clipped = f.clipped;
+        a.trace->e[i % NBO_TRACE_LEN] = e;
+        a.trace->count = i + 1;
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// In-place gradient passes of the unfused API: multiply by a factor, or zero.
+template <int ST> DEV void scale_body(const NboScaleArgs &a)
+{
+    typedef typename Traits<ST>::T T;
+    enum { SB = Traits<ST>::SBYTES, VEC = Traits<ST>::VEC };
+    const uint32_t tid = threadIdx.x;
+    const ChunkRef c = chunk_ref(a.L, blockIdx.x);
+    char *pg = (char *)a.g_ptrs[c.t] + c.base * SB;
+    bool zero = a.mode == 3;
+    T f = (T)a.factor;
+    if (a.gf) {
+        if (a.mode == 0) {
+            if (a.gf->found_inf) zero = true;
+            f = sizeof(T) == 4 ? (T)a.gf->inv_scale32 : (T)a.gf->inv_scale64;
+        } else if (a.mode == 1) {
+            if (!a.gf->clipped) return; // trainer.rs:515: untouched when norm <= max_norm
+            f = sizeof(T) == 4 ? (T)a.gf->clip32 : (T)a.gf->clip64;
+        }
+    }
+    const bool vec_ok = (((uintptr_t)pg) & (VEC * SB - 1)) == 0;
+    const uint32_t nvec = vec_ok ? c.cnt / VEC : 0;
+    for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
+        T x[VEC] = {};
+        char *p = pg + (uint64_t)q * VEC * SB;
+        if (!zero) {
+            IO<ST>::ldv(p, x);
+#pragma unroll
+            for (int k = 0; k < VEC; k++) x[k] = x[k] * f;
+        }
+        IO<ST>::stv(p, x);
+    }
+    for (uint32_t e = nvec * VEC + tid; e < c.cnt; e += NBO_BLOCK) {
+        char *p = pg + (uint64_t)e * SB;
+        const T x = zero ? (T)0 : IO<ST>::ld1(p) * f;
+        IO<ST>::st1(p, x);
+    }
+}
+
+#define NBO_SCALE_KERNEL(name, ST)                                                          \
+    extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboScaleArgs a)      \
+    {                                                                                       \
+        scale_body<ST>(a);                                                                  \
+    }
+NBO_SCALE_KERNEL(nbo_scale_f32, NBO_F32)
+NBO_SCALE_KERNEL(nbo_scale_bf16, NBO_BF16)
+NBO_SCALE_KERNEL(nbo_scale_f64, NBO_F64)
+
+// ---------------------------------------------------------------------------------
+// Master-weight casts: arena f32 <- bf16 tensors (exact widening) and
+// bf16 tensors <- arena f32 (round to nearest even).
+extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_cast_master(const NboCastArgs a)
+{
+    const ChunkRef c = chunk_ref(a.L, blockIdx.x);
+    float *aw = (float *)a.arena + c.soff + c.base;
+    if (a.mode == 0) {
+        const uint16_t *src = (const uint16_t *)a.src_ptrs[c.t] + c.base;
+        for (uint32_t e = threadIdx.x; e < c.cnt; e += NBO_BLOCK) aw[e] = bf16_bits_to_f32(src[e]);
+    } else {
+        uint16_t *dst = (uint16_t *)a.dst_ptrs[c.t] + c.base;
+        for (uint32_t e = threadIdx.x; e < c.cnt; e += NBO_BLOCK)
+            dst[e] = (uint16_t)f32_to_bf16_bits(aw[e]);
+    }
+}
+
+// Plain streaming copy used only to calibrate the HBM byte counters of a profile
+// against a transfer of known size.
+extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_copy_f32x4(const f32x4 *src, f32x4 *dst,
+                                                                      uint64_t nvec)
+{
+    const uint64_t stride = (uint64_t)gridDim.x * NBO_BLOCK;
+    for (uint64_t i = (uint64_t)blockIdx.x * NBO_BLOCK + threadIdx.x; i < nvec; i += stride)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}

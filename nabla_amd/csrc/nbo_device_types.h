@@ -1,0 +1,157 @@
+// Plain-old-data layouts shared by the gfx950 kernels and the host runtime.
+// Everything here is passed either by value as the single kernel argument or
+// lives in device memory; no pointers to host memory appear in any of them.
+#ifndef NBO_DEVICE_TYPES_H
+#define NBO_DEVICE_TYPES_H
+
+#include <stdint.h>
+
+// One work unit ("chunk") is this many consecutive elements of one tensor.  A
+// 256-thread workgroup handles a chunk in CHUNK / (256 * vec) unrolled rows.
+#define NBO_CHUNK 4096u
+#define NBO_BLOCK 256u
+// The norm pass runs a fixed grid so that its per-block partial sums, and hence
+// the reduced norm, do not depend on anything but the tensor list itself.
+#define NBO_NORM_GRID_MAX 2048u
+// Per-step trace ring kept on the device (found_inf / skipped / scale / step_count).
+#define NBO_TRACE_LEN 1024u
+
+// Element storage types of caller tensors.
+enum { NBO_F32 = 0, NBO_BF16 = 1, NBO_F64 = 2 };
+// OptimKind order of the reference (nabla-train/src/optim/core.rs:46-51).
+enum { NBO_ADAMW = 0, NBO_ADAM = 1, NBO_SGD = 2 };
+
+// Packed tensor-list descriptor, resident in device memory.
+//   n[t]             element count of tensor t
+//   chunk_begin[t]   index of tensor t's first chunk (chunk_begin[nt] = nchunks)
+//   chunk_tensor[c]  tensor that chunk c belongs to
+// Element offsets into the optimizer's state arena are in soff[t].
+struct NboLayoutDev {
+    const uint64_t *n;
+    const uint64_t *soff;
+    const uint32_t *chunk_begin;
+    const uint32_t *chunk_tensor;
+    uint32_t nt;
+    uint32_t nchunks;
+};
+
+// GradScalerState (optim/core.rs:326-332), device resident.
+struct NboScalerDev {
+    double scale, growth_factor, backoff_factor;
+    uint64_t growth_interval, consecutive_ok;
+};
+
+// Result of the norm / found_inf pass after its deterministic second stage.
+// inv_scale and clip are the two factors the reference multiplies every gradient
+// element by (core.rs:379, trainer.rs:519); 1.0 when the respective stage is off.
+struct NboGradFactors {
+    double sumsq;       // sum of squares of the unscaled gradients
+    double norm;        // sqrt(sumsq); what clip_grad_norm returns
+    double inv_scale64; // T::from_f64(1/scale) for T = f64
+    double clip64;      // T::from_f64(max_norm/norm) for T = f64
+    float inv_scale32;  // same, narrowed for T = f32
+    float clip32;
+    uint32_t found_inf; // 1: a gradient was inf/NaN, step is skipped
+    uint32_t clipped;   // 1: norm > max_norm, gradients are rescaled
+};
+
+// OptimMeta (optim/core.rs:53-62) plus the per-step scalars derived from it
+// (alg.rs:120-135, 266-277, 393-395), device resident.
+struct NboOptimDev {
+    double lr, beta1, beta2, eps, weight_decay, momentum;
+    uint64_t step_count;
+    uint32_t kind;
+    uint32_t skip; // this step is skipped (found_inf)
+    // scalars narrowed to T exactly as the reference narrows them
+    float b1, omb1, b2, omb2, eps_t, ss, ibc2, omw;
+    float neg_lr, momentum_t, wd_t, pad0;
+    double d_b1, d_omb1, d_b2, d_omb2, d_eps, d_ss, d_ibc2, d_omw;
+    double d_neg_lr, d_momentum, d_wd;
+};
+
+// Hyper-parameters as the host holds them; handed to the device with every step so
+// that set_lr and friends need no copy of their own.
+struct NboHyper {
+    double lr, beta1, beta2, eps, weight_decay, momentum;
+    uint32_t kind;
+    uint32_t pad;
+};
+
+// One entry of the device-side step trace.
+struct NboTraceEntry {
+    double scale;        // scaler scale after the step's update
+    double norm;         // pre-clip norm (0 if skipped)
+    uint64_t step_count; // optimizer step_count after the step
+    uint32_t found_inf;
+    uint32_t clipped;
+};
+
+struct NboTraceDev {
+    uint64_t count; // total entries ever written; entry i lives at i % NBO_TRACE_LEN
+    NboTraceEntry e[NBO_TRACE_LEN];
+};
+
+// ---- kernel argument blocks (each kernel takes exactly one, by value) ----------
+
+struct NboUpdateArgs {
+    NboLayoutDev L;
+    const uint64_t *p_ptrs; // caller parameter tensors (device addresses)
+    const uint64_t *g_ptrs; // caller gradient tensors
+    void *master;           // f32 master weights (mixed precision) or null
+    void *m;                // first moment / SGD velocity arena
+    void *v;                // second moment arena
+    const NboOptimDev *opt;
+    const NboGradFactors *gf; // null: gradients are used as they are
+    uint32_t zero_grads;      // write zeros over the gradients after reading them
+    uint32_t pad;
+};
+
+struct NboNormArgs {
+    NboLayoutDev L;
+    const uint64_t *g_ptrs;
+    const NboScalerDev *scaler; // null: no unscale, inv_scale = 1
+    double *partial_sumsq;      // [grid]
+    uint32_t *partial_flag;     // [grid]
+    uint32_t grid;
+    uint32_t pad;
+};
+
+struct NboFinalizeArgs {
+    const double *partial_sumsq;
+    const uint32_t *partial_flag;
+    uint32_t grid;
+    uint32_t check_finite; // GradScaler semantics (found_inf => skip); 0 for plain clip
+    NboScalerDev *scaler;  // may be null
+    NboGradFactors *gf;    // out
+    NboOptimDev *opt;      // may be null: if set, also advance step_count + scalars
+    NboTraceDev *trace;    // may be null
+    double max_norm;       // <= 0 disables clipping (trainer.rs:501-503)
+    NboHyper hyper;        // copied into *opt before the scalars are derived
+};
+
+struct NboPrepArgs {
+    NboOptimDev *opt;
+    const NboGradFactors *gf; // may be null
+    NboHyper hyper;
+};
+
+struct NboScaleArgs {
+    NboLayoutDev L;
+    const uint64_t *g_ptrs;
+    const NboGradFactors *gf; // if set: multiply by inv_scale (mode 0) or clip (mode 1);
+                              // on found_inf (mode 0) write zeros instead
+    double factor;            // used when gf is null
+    uint32_t mode;            // 0 unscale, 1 clip, 2 plain factor, 3 zero fill
+    uint32_t pad;
+};
+
+struct NboCastArgs {
+    NboLayoutDev L;
+    const uint64_t *src_ptrs;
+    const uint64_t *dst_ptrs;
+    void *arena; // master arena when one side is the optimizer's own state
+    uint32_t mode; // 0: arena(f32) <- src(bf16) widen; 1: dst(bf16) <- arena(f32) narrow
+    uint32_t pad;
+};
+
+#endif
