@@ -1,0 +1,271 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused optimizer step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama3-8b]
+
+One "step" is one Trainer tail over the whole synthetic parameter set, with
+gradients already resident in HBM: unscale + found-inf check, global-norm clip to
+1.0, mixed-precision AdamW update (bf16 params/grads, f32 master/m/v).  Prints one
+JSON line: whole-step algorithmic HBM throughput (30 B/param/step), the roofline
+figure of the dominant kernel measured with HIP events on its launch stream, and the
+CPU restatement of the reference timed on this host's cores on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
+BYTES_UPDATE = 28       # per param: R g2 + master4 + m4 + v4, W master4 + m4 + v4 + p2
+BYTES_NORM = 2          # per param: R g2
+ROOT = os.path.dirname(os.path.abspath(__file__))
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="llama3-8b",
+                    choices=["llama3-8b", "llama-1.1b", "gpt2-small-f32", "mlp-sgd-f32", "ragged-4096"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0,
+                    help="rough budget for the CPU baseline sample")
+    return ap.parse_args()
+
+
+def workload(name):
+    from nabla_amd import workloads as W
+
+    if name == "llama3-8b":
+        return dict(shapes=W.llama_8b_shapes(), mixed=True, kind="adamw", lr=2e-4, wd=0.1,
+                    betas=(0.9, 0.95), scaler=True, clip=1.0, p_sigma=0.02, g_sigma=1e-3)
+    if name == "llama-1.1b":
+        return dict(shapes=W.llama_1b_shapes(), mixed=True, kind="adamw", lr=2e-4, wd=0.1,
+                    betas=(0.9, 0.95), scaler=True, clip=1.0, p_sigma=0.02, g_sigma=1e-3)
+    if name == "ragged-4096":
+        return dict(shapes=[(1, n) for n in W.ragged_sizes()], mixed=True, kind="adamw", lr=2e-4,
+                    wd=0.1, betas=(0.9, 0.95), scaler=True, clip=1.0, p_sigma=0.02, g_sigma=1e-3)
+    if name == "gpt2-small-f32":
+        return dict(shapes=W.gpt2_small_shapes(), mixed=False, kind="adam", lr=3e-4, wd=0.0,
+                    betas=(0.9, 0.999), scaler=False, clip=0.0, p_sigma=0.02, g_sigma=1e-3)
+    return dict(shapes=W.MLP_SHAPES, mixed=False, kind="sgd", lr=0.01, wd=0.0, betas=(0.0, 0.0),
+                scaler=False, clip=0.0, p_sigma=0.05, g_sigma=1e-2)
+
+
+def bytes_per_param(cfg):
+    if cfg["kind"] == "sgd":
+        return 12, 0
+    if cfg["mixed"]:
+        return BYTES_UPDATE, BYTES_NORM
+    return 28, 0
+
+
+def cpu_baseline(cfg, budget_s):
+    """The oracle ("port" of the reference's CPU backend) on this host: every Backend
+    primitive a separate pass with a fresh output, element-parallel passes on all
+    cores, the reference's serial passes serial.  Timed on a sample of the workload's
+    own tensors sized to roughly `budget_s` seconds."""
+    import numpy as np
+
+    import oracle as O
+
+    cores = len(os.sched_getaffinity(0))
+    O.set_threads(cores)
+    shapes = cfg["shapes"]
+    # take tensors in list order until the sample holds ~24 M params (one pass chain
+    # over that takes seconds), but at least one tensor
+    sample, n = [], 0
+    for s in shapes:
+        if n and n + s[0] * s[1] > 64_000_000:
+            continue
+        sample.append(s)
+        n += s[0] * s[1]
+        if n >= 24_000_000:
+            break
+    rng = np.random.default_rng(0)
+    f32 = np.float32
+    master = [(rng.standard_normal(r * c, dtype=f32) * f32(cfg["p_sigma"])) for r, c in sample]
+    m = [np.zeros_like(a) for a in master]
+    v = [np.zeros_like(a) for a in master]
+    scale = 65536.0 if cfg["scaler"] else 1.0
+    g32 = [(rng.standard_normal(r * c, dtype=f32) * f32(cfg["g_sigma"] * scale)) for r, c in sample]
+    if cfg["kind"] == "sgd":
+        meta = O.sgd_meta(cfg["lr"])
+    elif cfg["kind"] == "adam":
+        meta = O.adam_meta(cfg["lr"], *cfg["betas"])
+    else:
+        meta = O.adamw_meta(cfg["lr"], *cfg["betas"], weight_decay=cfg["wd"])
+    scaler = O.default_scaler() if cfg["scaler"] else None
+    if cfg["mixed"]:
+        g = [O.bf16_from_f32(a) for a in g32]
+        p = [O.bf16_from_f32(a) for a in master]
+        run = lambda: O.mixed_step(meta, scaler, cfg["clip"], p, g, master, m, v)  # noqa: E731
+    else:
+        def run():
+            gg = [a.copy() for a in g32]
+            return O.f32_step(meta, scaler, cfg["clip"], master, gg, m, v)
+    run()  # warm (page faults, thread pool)
+    steps, t0 = 0, time.perf_counter()
+    while True:
+        run()
+        steps += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s or steps >= 50:
+            break
+    upd, nrm = bytes_per_param(cfg)
+    pps = n * steps / el
+    return {
+        "value": round(pps * (upd + nrm) / 1e9, 3),
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "params_per_s": round(pps, 1),
+        "ms_per_step_sample": round(el / steps * 1e3, 2),
+        "sample": f"first {len(sample)} tensors of the workload ({n} params), {steps} steps; "
+                  "reference-faithful pass chain (12 passes/tensor for AdamW, fresh output each), "
+                  f"rayon-parallel passes on {cores} threads, map/scan/clip passes serial",
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "
+              "the optimizer step has no multi-GPU path here", file=sys.stderr)
+        sys.exit(2)
+    sys.path.insert(0, ROOT)
+    import ctypes as C
+
+    import torch
+
+    from nabla_amd import _lib
+    from nabla_amd import optim as nb
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the engine has no CPU path", file=sys.stderr)
+        sys.exit(3)
+    _lib.init()
+    L = _lib.load()
+    cfg = workload(args.workload)
+    shapes = cfg["shapes"]
+    n = sum(r * c for r, c in shapes)
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+
+    pdt = torch.bfloat16 if cfg["mixed"] else torch.float32
+    params = [torch.empty(s, dtype=pdt, device=dev) for s in shapes]
+    grads = [torch.empty(s, dtype=pdt, device=dev) for s in shapes]
+    if cfg["kind"] == "sgd":
+        opt = nb.Sgd.new(cfg["lr"], shapes)
+    elif cfg["kind"] == "adam":
+        opt = nb.Adam.new(cfg["lr"], shapes).beta1(cfg["betas"][0]).beta2(cfg["betas"][1])
+    else:
+        opt = nb.AdamW.new(cfg["lr"], shapes, master=cfg["mixed"]).beta1(cfg["betas"][0]) \
+            .beta2(cfg["betas"][1]).weight_decay(cfg["wd"])
+    scale = 65536.0 if cfg["scaler"] else 1.0
+    for i, s in enumerate(shapes):  # synthetic, random-init
+        w = torch.randn(s, dtype=torch.float32, device=dev) * cfg["p_sigma"]
+        if cfg["mixed"]:
+            opt.write_state(f"w{i}", w)
+        else:
+            params[i].copy_(w)
+        grads[i].copy_((torch.randn(s, dtype=torch.float32, device=dev) * (cfg["g_sigma"] * scale)).to(pdt))
+        del w
+    plist, glist = nb.TensorList(params), nb.TensorList(grads)
+    if cfg["mixed"]:
+        opt.params_from_master(plist)
+    scaler = nb.GradScaler.new() if cfg["scaler"] else None
+    torch.cuda.empty_cache()
+
+    fused = cfg["scaler"] or cfg["clip"] > 0
+
+    def step():
+        if fused:
+            opt.fused_step(plist, glist, scaler=scaler, max_norm=cfg["clip"])
+        else:
+            opt.step(plist, glist)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.check(L.nbo_sync())
+    _lib.check(L.nbo_profile_enable(1))
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    _lib.check(L.nbo_sync())
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+
+    upd_b, nrm_b = bytes_per_param(cfg)
+    kern = {"sgd": "sgd", "adam": "adam", "adamw": "adamw"}[cfg["kind"]]
+    dom = f"nbo_update_{'bf16' if cfg['mixed'] else 'f32'}_{kern}"
+    per_kernel = {}
+    names = [dom] + ([f"nbo_norm_{'bf16' if cfg['mixed'] else 'f32'}", "nbo_finalize"] if fused else ["nbo_prep"])
+    for name in names:
+        cnt, ms = C.c_uint64(0), C.c_double(0.0)
+        _lib.check(L.nbo_profile_read(name.encode(), C.byref(cnt), C.byref(ms)))
+        per_kernel[name] = (cnt.value, ms.value)
+    _lib.check(L.nbo_profile_enable(0))
+
+    ms_step = (t1 - t0) / args.steps * 1e3
+    gbps = n * (upd_b + nrm_b) / (ms_step * 1e-3) / 1e9
+    dom_ms = per_kernel[dom][1] / max(per_kernel[dom][0], 1)
+    dom_gbps = n * upd_b / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
+    info = opt.last_step() if fused else None
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get(f"{args.workload}:{dom}")
+
+    out = {
+        "metric": "AdamW step HBM GB/s (bf16-mixed, whole step: unscale+found_inf+clip+update)"
+        if cfg["kind"] == "adamw" else f"{cfg['kind']} step HBM GB/s",
+        "value": round(gbps, 1),
+        "unit": "GB/s",
+        "pct_of_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "params_per_s": round(n / (ms_step * 1e-3), 1),
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16 params/grads, f32 master/m/v" if cfg["mixed"] else "f32",
+        "data": "synthetic (random-init parameters and gradients of the named shapes, resident in HBM)",
+        "config": {"workload": args.workload, "tensors": len(shapes), "params": n,
+                   "bytes_per_param_step": upd_b + nrm_b, "optimizer": cfg["kind"],
+                   "loss_scale": scale if cfg["scaler"] else None, "clip_max_norm": cfg["clip"] or None},
+        "roofline": {
+            "kernel": dom,
+            "bound": "hbm",
+            "achieved": round(dom_gbps, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(dom_gbps / HBM_PEAK_GBPS, 4),
+            "traffic": traffic,
+            "algorithmic_bytes_per_launch": n * upd_b,
+            "avg_launch_ms": round(dom_ms, 4),
+            "launches": per_kernel[dom][0],
+        },
+        "kernels_ms": {k: round(v[1] / max(v[0], 1), 4) for k, v in per_kernel.items()},
+    }
+    if info is not None:
+        out["last_step"] = {"found_inf": info.found_inf, "clipped": info.clipped,
+                            "norm": info.norm, "scale": info.scale, "step_count": info.step_count}
+    if not args.no_cpu_baseline:
+        del params, grads, plist, glist
+        out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_seconds)
+        out["cpu_baseline"]["gpu_over_cpu"] = round(out["value"] / max(out["cpu_baseline"]["value"], 1e-9), 1)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

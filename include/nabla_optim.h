@@ -203,6 +203,13 @@ int nbo_optim_trace_read(nbo_optim *opt, nbo_step_info *out, uint64_t max_entrie
 /* Device-to-device streaming copy of `bytes` (multiple of 16) with the engine's own
  * copy kernel; used to calibrate HBM byte counters against a known transfer. */
 int nbo_copy_bytes(const void *src_dev, void *dst_dev, uint64_t bytes);
+/* Per-kernel timing: while enabled, every kernel launch is bracketed by HIP events on
+ * the launch stream.  nbo_profile_read synchronises and returns the number of
+ * launches of `kernel_name` (e.g. "nbo_update_bf16_adamw") since profiling was
+ * enabled and the sum of their durations.  (The reference times its steps with host
+ * timers around a stream sync, nabla-train/src/profiler.rs:176-197.) */
+int nbo_profile_enable(int on);
+int nbo_profile_read(const char *kernel_name, uint64_t *launches, double *total_ms);
 
 #pragma GCC visibility pop
 

@@ -106,6 +106,8 @@ SYMBOLS = {
     "nbo_optim_last_step": (C.c_int, [_P, C.POINTER(StepInfo)]),
     "nbo_optim_trace_read": (C.c_int, [_P, C.POINTER(StepInfo), C.c_uint64, _U64P, _U64P]),
     "nbo_copy_bytes": (C.c_int, [_P, _P, C.c_uint64]),
+    "nbo_profile_enable": (C.c_int, [C.c_int]),
+    "nbo_profile_read": (C.c_int, [C.c_char_p, _U64P, C.POINTER(C.c_double)]),
 }
 
 

@@ -746,4 +746,17 @@ int nbo_copy_bytes(const void *src_dev, void *dst_dev, uint64_t bytes)
     });
 }
 
+int nbo_profile_enable(int on)
+{
+    return guarded([&] { Runtime::get().profile_enable(on != 0); });
+}
+
+int nbo_profile_read(const char *kernel_name, uint64_t *launches, double *total_ms)
+{
+    return guarded([&] {
+        require(kernel_name && launches && total_ms, NBO_ERR_ARG, "null argument");
+        Runtime::get().profile_read(kernel_name, launches, total_ms);
+    });
+}
+
 } // extern "C"

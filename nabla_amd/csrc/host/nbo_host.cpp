@@ -83,8 +83,48 @@ void Runtime::launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_st
 {
     if (grid == 0) return;
     void *args[1] = {arg_struct};
+    ProfRec rec = {kernel, nullptr, nullptr};
+    if (profiling_) {
+        hip_check(hipEventCreate(&rec.begin), "hipEventCreate");
+        hip_check(hipEventCreate(&rec.end), "hipEventCreate");
+        hip_check(hipEventRecord(rec.begin, stream_), "hipEventRecord");
+    }
     hip_check(hipModuleLaunchKernel(fn_[kernel], grid, 1, 1, block, 1, 1, 0, stream_, args, nullptr),
               kKernelNames[kernel]);
+    if (profiling_) {
+        hip_check(hipEventRecord(rec.end, stream_), "hipEventRecord");
+        prof_.push_back(rec);
+    }
+}
+
+void Runtime::profile_enable(bool on)
+{
+    for (ProfRec &r : prof_) {
+        (void)hipEventDestroy(r.begin);
+        (void)hipEventDestroy(r.end);
+    }
+    prof_.clear();
+    profiling_ = on;
+}
+
+void Runtime::profile_read(const char *kernel_name, uint64_t *launches, double *total_ms)
+{
+    int id = -1;
+    for (int k = 0; k < K_COUNT; k++)
+        if (std::strcmp(kernel_name, kKernelNames[k]) == 0) id = k;
+    if (id < 0) fail(NBO_ERR_ARG, std::string("unknown kernel name: ") + kernel_name);
+    sync();
+    uint64_t n = 0;
+    double ms = 0.0;
+    for (const ProfRec &r : prof_) {
+        if (r.kernel != id) continue;
+        float t = 0.0f;
+        hip_check(hipEventElapsedTime(&t, r.begin, r.end), "hipEventElapsedTime");
+        ms += t;
+        n++;
+    }
+    *launches = n;
+    *total_ms = ms;
 }
 
 void Runtime::launch_copy(const void *src, void *dst, uint64_t nvec)

@@ -61,6 +61,11 @@ public:
     void dfree(void *p);
     void dzero(void *p, size_t bytes); // asynchronous on the stream
 
+    // Per-kernel timing with HIP events recorded on the launch stream, for the
+    // benchmark's roofline figure.  Off by default.
+    void profile_enable(bool on);
+    void profile_read(const char *kernel_name, uint64_t *launches, double *total_ms);
+
     double *partial_sumsq() const { return partial_sumsq_; }
     uint32_t *partial_flag() const { return partial_flag_; }
     NboGradFactors *gf_scratch() const { return gf_scratch_; }
@@ -75,6 +80,12 @@ private:
     double *partial_sumsq_ = nullptr;
     uint32_t *partial_flag_ = nullptr;
     NboGradFactors *gf_scratch_ = nullptr;
+    struct ProfRec {
+        int kernel;
+        hipEvent_t begin, end;
+    };
+    bool profiling_ = false;
+    std::vector<ProfRec> prof_;
 };
 
 // Host + device copy of the packed tensor-list descriptor.
