@@ -32,6 +32,10 @@ def parse_args():
     ap.add_argument("--workload", default="llama3-8b",
                     choices=["llama3-8b", "llama-1.1b", "gpt2-small-f32", "mlp-sgd-f32", "ragged-4096"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", type=float, default=0.0, metavar="GiB",
+                    help="instead of the benchmark, run the library's plain copy kernel over "
+                         "this many GiB (--steps times); a transfer of known size against which "
+                         "rocprofv3's FETCH_SIZE / WRITE_SIZE counters are scaled")
     ap.add_argument("--cpu-seconds", type=float, default=20.0,
                     help="rough budget for the CPU baseline sample")
     return ap.parse_args()
@@ -150,11 +154,25 @@ def main():
         sys.exit(3)
     _lib.init()
     L = _lib.load()
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    if args.calibrate_copy > 0:
+        nbytes = int(args.calibrate_copy * (1 << 30)) // 16 * 16
+        src = torch.ones(nbytes // 4, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        _lib.check(L.nbo_profile_enable(1))
+        for _ in range(args.steps):
+            _lib.check(L.nbo_copy_bytes(src.data_ptr(), dst.data_ptr(), nbytes))
+        cnt, ms = C.c_uint64(0), C.c_double(0.0)
+        _lib.check(L.nbo_profile_read(b"nbo_copy_f32x4", C.byref(cnt), C.byref(ms)))
+        print(json.dumps({"calibrate": "nbo_copy_f32x4", "bytes_read": nbytes, "bytes_written": nbytes,
+                          "launches": cnt.value, "avg_launch_ms": round(ms.value / max(cnt.value, 1), 4),
+                          "GBps": round(2 * nbytes / (ms.value / max(cnt.value, 1)) / 1e6, 1)}))
+        return
     cfg = workload(args.workload)
     shapes = cfg["shapes"]
     n = sum(r * c for r, c in shapes)
-    dev = torch.device("cuda:0")
-    torch.manual_seed(0)
 
     pdt = torch.bfloat16 if cfg["mixed"] else torch.float32
     params = [torch.empty(s, dtype=pdt, device=dev) for s in shapes]

@@ -95,9 +95,7 @@ NboUpdateArgs update_args(nbo_optim *opt, nbo_list *params, nbo_list *grads, boo
     a.L = opt->layout.dev;
     a.p_ptrs = params->ptrs_dev;
     a.g_ptrs = grads->ptrs_dev;
-    a.master = params->dtype == NBO_DT_BF16 ? opt->master : nullptr;
-    a.m = opt->m;
-    a.v = opt->v;
+    a.arena = opt->arena;
     a.opt = opt->dev;
     a.gf = with_gf ? opt->gf : nullptr;
     a.zero_grads = zero_grads ? 1u : 0u;
@@ -166,11 +164,32 @@ void parse_state_name(const nbo_optim *opt, const char *name, char *which, uint6
     *index = v;
 }
 
-char *state_base(nbo_optim *opt, char which)
+// Index of the arena part a state-name prefix refers to.
+uint32_t state_part_index(const nbo_optim *opt, char which)
 {
-    if (which == 'w') return (char *)opt->master;
-    if (opt->meta.kind == NBO_KIND_SGD) return (char *)opt->m; // velocity
-    return which == 'm' ? (char *)opt->m : (char *)opt->v;
+    if (which == 'w') return opt->arena.part_w;
+    if (opt->meta.kind == NBO_KIND_SGD) return 0; // velocity
+    return which == 'm' ? 0 : opt->arena.part_v;
+}
+
+// Copies the n elements of tensor i's part `part` between the arena and a dense
+// buffer.
+void part_copy(nbo_optim *opt, uint64_t i, uint32_t part, void *buf, bool on_device, bool to_engine)
+{
+    Runtime &rt = Runtime::get();
+    const size_t eb = opt->elem_bytes();
+    const size_t bytes = (size_t)opt->layout.n[i] * eb;
+    if (bytes == 0) return;
+    char *dev = (char *)opt->arena.base +
+                ((size_t)part * opt->arena.part_stride + opt->layout.soff[i]) * eb;
+    if (on_device)
+        hip_check(hipMemcpyAsync(to_engine ? (void *)dev : buf, to_engine ? buf : (void *)dev, bytes,
+                                 hipMemcpyDeviceToDevice, rt.stream()),
+                  "hipMemcpyAsync D2D");
+    else if (to_engine)
+        rt.upload(dev, buf, bytes);
+    else
+        rt.read_back(buf, dev, bytes);
 }
 
 void state_copy(nbo_optim *opt, const char *name, void *buf, uint64_t n_elems, int on_device,
@@ -185,25 +204,20 @@ void state_copy(nbo_optim *opt, const char *name, void *buf, uint64_t n_elems, i
         fail(NBO_ERR_SHAPE, std::string("state tensor ") + name + " has " +
                                 std::to_string(opt->layout.n[i]) + " elements, buffer has " +
                                 std::to_string(n_elems));
-    Runtime &rt = Runtime::get();
-    const size_t eb = which == 'w' ? 4 : opt->elem_bytes();
-    char *dev = state_base(opt, which) + opt->layout.soff[i] * eb;
-    const size_t bytes = (size_t)n_elems * eb;
-    if (bytes == 0) return;
-    if (on_device) {
-        hip_check(hipMemcpyAsync(to_engine ? (void *)dev : buf, to_engine ? buf : (void *)dev, bytes,
-                                 hipMemcpyDeviceToDevice, rt.stream()),
-                  "hipMemcpyAsync D2D");
-    } else if (to_engine) {
-        rt.upload(dev, buf, bytes);
-    } else {
-        rt.read_back(buf, dev, bytes);
-    }
+    part_copy(opt, i, state_part_index(opt, which), buf, on_device != 0, to_engine);
     if (to_engine && which == 'w') {
-        // the master weights count as set once every tensor has been written; the
-        // caller writes them all before stepping, as a checkpoint load does
+        // the master weights count as set once a tensor has been written; the caller
+        // writes them all before stepping, as a checkpoint load does
         opt->master_valid = true;
     }
+}
+
+// Zero-fills one part of the whole arena (asynchronous).
+void part_zero(nbo_optim *opt, uint32_t part)
+{
+    const size_t eb = opt->elem_bytes();
+    Runtime::get().dzero((char *)opt->arena.base + (size_t)part * opt->arena.part_stride * eb,
+                         (size_t)opt->layout.arena_elems * eb);
 }
 
 void fill_info(const NboTraceEntry &e, nbo_step_info *out)
@@ -344,17 +358,16 @@ int nbo_optim_create(const nbo_meta *meta, uint64_t n_tensors, const uint64_t *r
             o->state_dtype = state_dtype;
             o->keep_master = keep_master != 0;
             o->layout.build(n_tensors, rows, cols, true);
-            const size_t bytes = (size_t)o->layout.arena_elems * o->elem_bytes();
-            o->m = rt.dmalloc(bytes);
-            rt.dzero(o->m, bytes);
-            if (meta->kind != NBO_KIND_SGD) {
-                o->v = rt.dmalloc(bytes);
-                rt.dzero(o->v, bytes);
-            }
-            if (o->keep_master) {
-                o->master = rt.dmalloc((size_t)o->layout.arena_elems * 4);
-                rt.dzero(o->master, (size_t)o->layout.arena_elems * 4);
-            }
+            // one device arena holding every state part (see NboArenaDev)
+            const bool adam_like = meta->kind != NBO_KIND_SGD;
+            o->arena.nparts = 1u + (adam_like ? 1u : 0u) + (o->keep_master ? 1u : 0u);
+            o->arena.part_v = 1;
+            o->arena.part_w = adam_like ? 2 : 1;
+            o->arena.part_stride = o->layout.arena_elems;
+            const size_t bytes = ((size_t)o->arena.part_stride * (o->arena.nparts - 1) +
+                                  (size_t)o->layout.arena_elems) * o->elem_bytes();
+            o->arena.base = rt.dmalloc(bytes);
+            rt.dzero(o->arena.base, bytes);
             o->dev = (NboOptimDev *)rt.dmalloc(sizeof(NboOptimDev));
             o->gf = (NboGradFactors *)rt.dmalloc(sizeof(NboGradFactors));
             o->trace = (NboTraceDev *)rt.dmalloc(sizeof(NboTraceDev));
@@ -373,9 +386,7 @@ int nbo_optim_create(const nbo_meta *meta, uint64_t n_tensors, const uint64_t *r
             *out = o;
         } catch (...) {
             o->layout.release();
-            rt.dfree(o->m);
-            rt.dfree(o->v);
-            rt.dfree(o->master);
+            rt.dfree(o->arena.base);
             rt.dfree(o->dev);
             rt.dfree(o->gf);
             rt.dfree(o->trace);
@@ -392,9 +403,7 @@ int nbo_optim_destroy(nbo_optim *opt)
         Runtime &rt = Runtime::get();
         rt.sync();
         opt->layout.release();
-        rt.dfree(opt->m);
-        rt.dfree(opt->v);
-        rt.dfree(opt->master);
+        rt.dfree(opt->arena.base);
         rt.dfree(opt->dev);
         rt.dfree(opt->gf);
         rt.dfree(opt->trace);
@@ -422,9 +431,8 @@ int nbo_optim_reset(nbo_optim *opt)
     return guarded([&] {
         require(opt != nullptr, NBO_ERR_ARG, "null optimizer");
         Runtime &rt = Runtime::get();
-        const size_t bytes = (size_t)opt->layout.arena_elems * opt->elem_bytes();
-        rt.dzero(opt->m, bytes);
-        if (opt->v) rt.dzero(opt->v, bytes);
+        part_zero(opt, 0);
+        if (opt->meta.kind != NBO_KIND_SGD) part_zero(opt, opt->arena.part_v);
         // step_count = 0 (Adam / AdamW); Sgd has none
         rt.dzero(&opt->dev->step_count, sizeof(uint64_t));
     });
@@ -505,7 +513,7 @@ static void cast_master(nbo_optim *opt, nbo_list *params, uint32_t mode)
     a.L = opt->layout.dev;
     a.src_ptrs = params->ptrs_dev;
     a.dst_ptrs = params->ptrs_dev;
-    a.arena = opt->master;
+    a.arena = opt->arena;
     a.mode = mode;
     Runtime::get().launch(K_CAST_MASTER, opt->layout.nchunks, NBO_BLOCK, a);
 }

@@ -136,9 +136,19 @@ void Runtime::launch_copy(const void *src, void *dst, uint64_t nvec)
     uint64_t grid = (blocks + 3) / 4;
     if (grid > 0x7FFFFFFFull) grid = 0x7FFFFFFFull;
     void *args[3] = {(void *)&src, (void *)&dst, (void *)&nvec};
+    ProfRec rec = {K_COPY, nullptr, nullptr};
+    if (profiling_) {
+        hip_check(hipEventCreate(&rec.begin), "hipEventCreate");
+        hip_check(hipEventCreate(&rec.end), "hipEventCreate");
+        hip_check(hipEventRecord(rec.begin, stream_), "hipEventRecord");
+    }
     hip_check(hipModuleLaunchKernel(fn_[K_COPY], (uint32_t)grid, 1, 1, NBO_BLOCK, 1, 1, 0, stream_,
                                     args, nullptr),
               kKernelNames[K_COPY]);
+    if (profiling_) {
+        hip_check(hipEventRecord(rec.end, stream_), "hipEventRecord");
+        prof_.push_back(rec);
+    }
 }
 
 void Runtime::read_back(void *host_dst, const void *dev_src, size_t bytes)
@@ -209,11 +219,11 @@ void Layout::build(uint64_t nt, const uint64_t *r, const uint64_t *c, bool with_
         chunk_begin[t] = (uint32_t)chunks;
         chunks += (n[t] + NBO_CHUNK - 1) / NBO_CHUNK;
         if (chunks > 0xFFFFFFFFull)
-            fail(NBO_ERR_TOO_LARGE, "tensor list has more than 2^32-1 chunks of 4096 elements");
-        // every tensor starts on a 512-byte boundary of the arena, so state vectors
-        // are 16-byte aligned whatever the element type
+            fail(NBO_ERR_TOO_LARGE, "tensor list has more than 2^32-1 work chunks");
+        // every tensor is padded to whole chunks, so a chunk never straddles two
+        // state tiles
         soff[t] = off;
-        off += align_up(n[t], 128);
+        off += align_up(n[t], NBO_CHUNK);
     }
     chunk_begin[nt] = (uint32_t)chunks;
     nchunks = (uint32_t)chunks;

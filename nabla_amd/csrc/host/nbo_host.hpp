@@ -120,9 +120,7 @@ struct nbo_optim {
     int state_dtype = NBO_DT_F32;
     bool keep_master = false;
     bool master_valid = false;
-    void *m = nullptr;      // first moment / SGD velocity
-    void *v = nullptr;      // second moment (null for SGD)
-    void *master = nullptr; // f32 master weights (mixed precision)
+    NboArenaDev arena = {}; // the one device allocation m, v and master live in
     NboOptimDev *dev = nullptr; // step_count lives here: the device decides skips
     NboGradFactors *gf = nullptr;
     NboTraceDev *trace = nullptr;

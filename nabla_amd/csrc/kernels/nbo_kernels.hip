@@ -39,6 +39,28 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 #define DEV static __device__ __forceinline__
+
+// Tuning knobs (the defaults are the measured best on MI355X).
+#ifndef NBO_UNROLL
+#define NBO_UNROLL 8 // 128-bit rows per thread whose loads are issued back to back (f32;
+                     // half as many for f64, whose vectors hold half the elements)
+#endif
+#ifndef NBO_NT_LOADS
+#define NBO_NT_LOADS 1
+#endif
+#ifndef NBO_NT_STORES
+#define NBO_NT_STORES 1
+#endif
+#if NBO_NT_LOADS
+#define NBO_LOAD(p) __builtin_nontemporal_load(p)
+#else
+#define NBO_LOAD(p) (*(p))
+#endif
+#if NBO_NT_STORES
+#define NBO_STORE(v, p) __builtin_nontemporal_store(v, p)
+#else
+#define NBO_STORE(v, p) (*(p) = (v))
+#endif
 // Caller tensor addresses arrive as integers; telling the compiler that they are
 // global memory turns flat_* accesses into global_* ones.
 #define GLOBAL_PTR(type, p) ((__attribute__((address_space(1))) type *)(uintptr_t)(p))
@@ -97,23 +119,23 @@ template <> struct Traits<NBO_F64> {
 // arena (engine-owned, always 16-byte aligned) vectors of T
 DEV void ld_state(const float *p, float (&x)[4])
 {
-    f32x4 v = __builtin_nontemporal_load(GLOBAL_PTR(const f32x4, p));
+    f32x4 v = NBO_LOAD(GLOBAL_PTR(const f32x4, p));
     x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
 }
 DEV void ld_state(const double *p, double (&x)[2])
 {
-    f64x2 v = __builtin_nontemporal_load(GLOBAL_PTR(const f64x2, p));
+    f64x2 v = NBO_LOAD(GLOBAL_PTR(const f64x2, p));
     x[0] = v.x; x[1] = v.y;
 }
 DEV void st_state(float *p, const float (&x)[4])
 {
     f32x4 v = {x[0], x[1], x[2], x[3]};
-    __builtin_nontemporal_store(v, GLOBAL_PTR(f32x4, p));
+    NBO_STORE(v, GLOBAL_PTR(f32x4, p));
 }
 DEV void st_state(double *p, const double (&x)[2])
 {
     f64x2 v = {x[0], x[1]};
-    __builtin_nontemporal_store(v, GLOBAL_PTR(f64x2, p));
+    NBO_STORE(v, GLOBAL_PTR(f64x2, p));
 }
 
 // caller tensors: vector of VEC storage elements at byte address p
@@ -133,7 +155,7 @@ template <> struct IO<NBO_F64> {
 template <> struct IO<NBO_BF16> {
     DEV void ldv(const char *p, float (&x)[4])
     {
-        u32x2 v = __builtin_nontemporal_load(GLOBAL_PTR(const u32x2, p));
+        u32x2 v = NBO_LOAD(GLOBAL_PTR(const u32x2, p));
         x[0] = __uint_as_float(v.x << 16);
         x[1] = __uint_as_float(v.x & 0xFFFF0000u);
         x[2] = __uint_as_float(v.y << 16);
@@ -144,7 +166,7 @@ template <> struct IO<NBO_BF16> {
         u32x2 v;
         v.x = f32_to_bf16_bits(x[0]) | (f32_to_bf16_bits(x[1]) << 16);
         v.y = f32_to_bf16_bits(x[2]) | (f32_to_bf16_bits(x[3]) << 16);
-        __builtin_nontemporal_store(v, GLOBAL_PTR(u32x2, p));
+        NBO_STORE(v, GLOBAL_PTR(u32x2, p));
     }
     DEV float ld1(const char *p) { return bf16_bits_to_f32(*GLOBAL_PTR(const uint16_t, p)); }
     DEV void st1(char *p, float x) { *GLOBAL_PTR(uint16_t, p) = (uint16_t)f32_to_bf16_bits(x); }
@@ -239,12 +261,27 @@ DEV ChunkRef chunk_ref(const NboLayoutDev &L, uint32_t c)
     return r;
 }
 
+// Address of chunk c within state part `part` of the arena.
+template <typename T> DEV T *state_part(const NboArenaDev &A, const ChunkRef &c, uint32_t part)
+{
+    return (T *)A.base + part * A.part_stride + c.soff + c.base;
+}
+
 // ---------------------------------------------------------------------------------
 // Optimizer update: one workgroup per chunk.
 template <int ST, int KIND> DEV void update_body(const NboUpdateArgs &a)
 {
     typedef typename Traits<ST>::T T;
-    enum { VEC = Traits<ST>::VEC, SB = Traits<ST>::SBYTES, ROW = NBO_BLOCK * VEC, U = NBO_CHUNK / ROW };
+    enum {
+        VEC = Traits<ST>::VEC,
+        SB = Traits<ST>::SBYTES,
+        ROW = NBO_BLOCK * VEC,
+        ROWS = NBO_CHUNK / ROW,
+        UMAX = sizeof(T) == 8 ? NBO_UNROLL / 2 : NBO_UNROLL,
+        U = ROWS < UMAX ? ROWS : UMAX,
+        ITERS = ROWS / U
+    };
+    static_assert(ROWS % U == 0 && ROWS * ROW == NBO_CHUNK, "chunk must be a whole number of unrolled rows");
     const bool mixed = ST == NBO_BF16; // f32 master lives in the arena
     const bool has_v = KIND != NBO_SGD;
     const uint32_t tid = threadIdx.x;
@@ -252,9 +289,9 @@ template <int ST, int KIND> DEV void update_body(const NboUpdateArgs &a)
 
     char *pp = (char *)a.p_ptrs[c.t] + c.base * SB;
     char *pg = (char *)a.g_ptrs[c.t] + c.base * SB;
-    T *am = (T *)a.m + c.soff + c.base;
-    T *av = has_v ? (T *)a.v + c.soff + c.base : nullptr;
-    T *aw = mixed ? (T *)a.master + c.soff + c.base : nullptr;
+    T *am = state_part<T>(a.arena, c, 0);
+    T *av = has_v ? state_part<T>(a.arena, c, a.arena.part_v) : nullptr;
+    T *aw = mixed ? state_part<T>(a.arena, c, a.arena.part_w) : nullptr;
     const bool zero_g = a.zero_grads != 0;
     const uint32_t vbytes = VEC * SB;
     const bool vec_ok = ((((uintptr_t)pp) | ((uintptr_t)pg)) & (vbytes - 1)) == 0;
@@ -270,28 +307,31 @@ template <int ST, int KIND> DEV void update_body(const NboUpdateArgs &a)
     const bool use_m = KIND != NBO_SGD || s.use_mom;
 
     if (c.cnt == NBO_CHUNK && vec_ok) {
-        T g[U][VEC], p[U][VEC], m[U][VEC] = {}, v[U][VEC] = {};
+        for (int it = 0; it < ITERS; it++) {
+            const uint32_t e0 = it * (U * ROW) + tid * VEC;
+            T g[U][VEC], p[U][VEC], m[U][VEC] = {}, v[U][VEC] = {};
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const uint32_t e = u * ROW + tid * VEC;
-            IO<ST>::ldv(pg + (uint64_t)e * SB, g[u]);
-            if (mixed) ld_state(aw + e, p[u]);
-            else IO<ST>::ldv(pp + (uint64_t)e * SB, p[u]);
-            if (use_m) ld_state(am + e, m[u]);
-            if (has_v) ld_state(av + e, v[u]);
-        }
+            for (int u = 0; u < U; u++) {
+                const uint32_t e = e0 + u * ROW;
+                IO<ST>::ldv(pg + (uint64_t)e * SB, g[u]);
+                if (mixed) ld_state(aw + e, p[u]);
+                else IO<ST>::ldv(pp + (uint64_t)e * SB, p[u]);
+                if (use_m) ld_state(am + e, m[u]);
+                if (has_v) ld_state(av + e, v[u]);
+            }
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const uint32_t e = u * ROW + tid * VEC;
+            for (int u = 0; u < U; u++) {
+                const uint32_t e = e0 + u * ROW;
 #pragma unroll
-            for (int k = 0; k < VEC; k++) step_elem<T, KIND>(p[u][k], g[u][k], m[u][k], v[u][k], s);
-            if (mixed) st_state(aw + e, p[u]);
-            IO<ST>::stv(pp + (uint64_t)e * SB, p[u]);
-            if (use_m) st_state(am + e, m[u]);
-            if (has_v) st_state(av + e, v[u]);
-            if (zero_g) {
-                T z[VEC] = {};
-                IO<ST>::stv(pg + (uint64_t)e * SB, z);
+                for (int k = 0; k < VEC; k++) step_elem<T, KIND>(p[u][k], g[u][k], m[u][k], v[u][k], s);
+                if (mixed) st_state(aw + e, p[u]);
+                IO<ST>::stv(pp + (uint64_t)e * SB, p[u]);
+                if (use_m) st_state(am + e, m[u]);
+                if (has_v) st_state(av + e, v[u]);
+                if (zero_g) {
+                    T z[VEC] = {};
+                    IO<ST>::stv(pg + (uint64_t)e * SB, z);
+                }
             }
         }
         return;
@@ -659,7 +699,7 @@ NBO_SCALE_KERNEL(nbo_scale_f64, NBO_F64)
 extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_cast_master(const NboCastArgs a)
 {
     const ChunkRef c = chunk_ref(a.L, blockIdx.x);
-    float *aw = (float *)a.arena + c.soff + c.base;
+    float *aw = state_part<float>(a.arena, c, a.arena.part_w);
     if (a.mode == 0) {
         const uint16_t *src = (const uint16_t *)a.src_ptrs[c.t] + c.base;
         for (uint32_t e = threadIdx.x; e < c.cnt; e += NBO_BLOCK) aw[e] = bf16_bits_to_f32(src[e]);

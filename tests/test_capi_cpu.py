@@ -1,0 +1,150 @@
+"""CPU-side checks of the C-ABI library and the host mirror: the shared object loads,
+exports every symbol include/nabla_optim.h declares, and fails loudly (never
+computes) without a gfx950 device.  No kernel is launched here."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from nabla_amd import _lib
+from nabla_amd import optim as nb
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "nabla_optim.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(nbo_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    declared = _declared_symbols()
+    assert len(declared) >= 30
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in nabla_optim.h but not exported"
+    assert sorted(_lib.SYMBOLS) == declared, "ctypes table and header disagree"
+
+
+def test_struct_layouts_match_the_header():
+    assert C.sizeof(_lib.Meta) == 8 + 6 * 8 + 8
+    assert C.sizeof(_lib.ScalerState) == 5 * 8
+    assert C.sizeof(_lib.StepInfo) == 3 * 8 + 2 * 4
+
+
+def test_version_and_status_strings():
+    lib = _lib.load()
+    assert lib.nbo_version().decode() == "0.1.0"
+    assert lib.nbo_status_string(0) == b"ok"
+    assert b"length mismatch" in lib.nbo_status_string(_lib.ERR_LEN_MISMATCH)
+    assert b"kind mismatch" in lib.nbo_status_string(_lib.ERR_KIND)
+    assert b"HIP" in lib.nbo_status_string(_lib.ERR_HIP + 2)
+
+
+def _no_gpu():
+    try:
+        import torch
+
+        return not torch.cuda.is_available()
+    except Exception:
+        return True
+
+
+@pytest.mark.skipif(not _no_gpu(), reason="checks the behaviour without a GPU")
+def test_no_device_is_an_error_not_a_fallback():
+    lib = _lib.load()
+    assert lib.nbo_init() == _lib.ERR_NO_DEVICE
+    assert b"gfx950" in lib.nbo_last_error()
+    with pytest.raises(_lib.NablaOptimError):
+        _lib.init()
+    # every object constructor needs the runtime and therefore fails the same way
+    h = C.c_void_p()
+    rows = (C.c_uint64 * 1)(1)
+    meta = _lib.Meta(_lib.KIND_SGD, 0, 0.1, 0, 0, 0, 0, 0, 0)
+    assert lib.nbo_optim_create(C.byref(meta), 1, rows, rows, _lib.DT_F32, 0, C.byref(h)) == \
+        _lib.ERR_NO_DEVICE
+    assert not h.value
+    assert lib.nbo_scaler_create(None, C.byref(h)) == _lib.ERR_NO_DEVICE
+
+
+def test_argument_errors_are_reported_before_any_device_work():
+    lib = _lib.load()
+    assert lib.nbo_optim_create(None, 0, None, None, _lib.DT_F32, 0, None) == _lib.ERR_ARG
+    assert lib.nbo_optim_step(None, None, None) == _lib.ERR_ARG
+    assert lib.nbo_zero_grad(None) == _lib.ERR_ARG
+    out = C.c_double()
+    assert lib.nbo_clip_grad_norm(None, 1.0, C.byref(out)) == _lib.ERR_ARG
+    assert lib.nbo_list_destroy(None) in (_lib.OK, _lib.ERR_NO_DEVICE)
+
+
+# ---- host mirror: the parts of OptimState that are plain string / key logic -----------------
+
+def test_rust_f64_display():
+    """Rust's Display for f64 (used by optim_meta_pairs, core.rs:263-277): shortest
+    round-trip digits, no exponent, integers without a fraction."""
+    f = nb.rust_f64_str
+    assert f(1e-8) == "0.00000001"
+    assert f(0.1) == "0.1" and f(0.9) == "0.9" and f(0.999) == "0.999"
+    assert f(65536.0) == "65536" and f(0.0) == "0" and f(2.0) == "2"
+    assert f(3e-4) == "0.0003" and f(2e-4) == "0.0002"
+    assert f(1e21) == "1000000000000000000000"
+    assert f(-1.5e-7) == "-0.00000015"
+    assert f(float("inf")) == "inf" and f(float("nan")) == "NaN"
+    for x in (1e-8, 3e-4, 0.95, 123456.789, 1e-300, 1.7976931348623157e308):
+        assert float(f(x)) == x
+
+
+def test_meta_pairs_round_trip_and_errors():
+    meta = nb.OptimMeta("adamw", 2e-4, 0.9, 0.95, 1e-8, 0.1, 0.0, 48)
+    pairs = nb.optim_meta_pairs(meta)
+    assert pairs[0] == ("optim.kind", "adamw") and pairs[4] == ("optim.eps", "0.00000001")
+    assert pairs[-1] == ("optim.step_count", "48")
+    assert nb.parse_optim_meta(dict(pairs)) == meta
+    m = dict(pairs)
+    del m["optim.beta2"]
+    with pytest.raises(nb.OptimStateError, match="missing optim.beta2"):
+        nb.parse_optim_meta(m)
+    m = dict(pairs, **{"optim.kind": "lion"})
+    with pytest.raises(nb.OptimStateError, match="bad optim.kind: lion"):
+        nb.parse_optim_meta(m)
+    m = dict(pairs, **{"optim.step_count": "-3"})
+    with pytest.raises(nb.OptimStateError, match="bad optim.step_count: -3"):
+        nb.parse_optim_meta(m)
+    m = dict(pairs, **{"optim.lr": "fast"})
+    with pytest.raises(nb.OptimStateError, match="bad optim.lr: fast"):
+        nb.parse_optim_meta(m)
+
+
+def test_load_state_tensors_key_errors_follow_the_reference():
+    """alg.rs:487-516: checks run before anything is written, so no device is needed."""
+    opt = nb.AdamW.new(1e-3, [(1, 1), (2, 2)])
+    with pytest.raises(nb.OptimStateError, match="bad tensor key: mx"):
+        opt.load_state_tensors([("mx", None)])
+    with pytest.raises(nb.OptimStateError, match="m index out of range: 2"):
+        opt.load_state_tensors([("m2", None)])
+    with pytest.raises(nb.OptimStateError, match="missing m0"):
+        opt.load_state_tensors([("m1", None), ("v0", None), ("v1", None), ("other", None)])
+    with pytest.raises(nb.OptimStateError, match="missing v1"):
+        opt.load_state_tensors([("m0", None), ("m1", None), ("v0", None)])
+    sgd = nb.Sgd.new(0.1, [(1, 1)])
+    with pytest.raises(nb.OptimStateError, match="missing v0"):
+        sgd.load_state_tensors([("m0", None)])  # Sgd ignores every prefix but 'v'
+    with pytest.raises(nb.OptimStateError, match="optim kind mismatch"):
+        sgd.load_meta(nb.OptimMeta("adam", 0.1, 0.9, 0.999, 1e-8, 0.0, 0.0, 0))
+
+
+def test_meta_before_first_use_reports_constructor_defaults():
+    """alg.rs:29-38, 190-198, 324-329 and the zeros each kind's meta() reports."""
+    a = nb.AdamW.new(2e-4, [(1, 1)]).beta2(0.95).weight_decay(0.1).meta()
+    assert (a.kind, a.lr, a.beta1, a.beta2, a.eps, a.weight_decay, a.momentum, a.step_count) == \
+        ("adamw", 2e-4, 0.9, 0.95, 1e-8, 0.1, 0.0, 0)
+    d = nb.Adam.new(3e-4, [(1, 1)]).meta()
+    assert (d.kind, d.beta2, d.weight_decay) == ("adam", 0.999, 0.0)
+    s = nb.Sgd.new(0.01, [(1, 1)]).momentum(0.9).meta()
+    assert (s.kind, s.beta1, s.eps, s.momentum, s.step_count) == ("sgd", 0.0, 0.0, 0.9, 0)
+    g = nb.GradScaler.new().state()
+    assert (g.scale, g.growth_factor, g.backoff_factor, g.growth_interval, g.consecutive_ok) == \
+        (65536.0, 2.0, 0.5, 2000, 0)

@@ -20,8 +20,10 @@ from tests import helpers as H
 
 pytestmark = pytest.mark.gpu
 
-RAGGED = [(1, 1), (1, 3), (3, 5), (1, 4095), (1, 4096), (1, 4097), (64, 130), (7, 1171), (1, 8192),
-          (1, 12289), (0, 5), (33, 1000)]
+# sizes around the engine's work-chunk (8192 elements) and vector (4 / 8 elements)
+# boundaries, an empty tensor, and a few ordinary ones
+RAGGED = [(1, 1), (1, 3), (3, 5), (1, 4095), (1, 4097), (64, 130), (7, 1171), (1, 8191), (1, 8192),
+          (1, 8193), (1, 16385), (0, 5), (33, 1000)]
 
 
 def _param_close(p_dev, p_ref, lr, steps, what):

@@ -1,0 +1,494 @@
+"""Pins the CPU oracle (oracle/nabla_cpu_oracle.c) before anything is checked against it.
+
+Three kinds of evidence, none of which re-uses the oracle's own formulas in floating
+point:
+  1. the known answers the reference's own tests hold for this path
+     (nabla-train/tests/optim.rs, nabla-train/tests/trainer.rs);
+  2. exact rational arithmetic (fractions.Fraction) with an explicit
+     round-to-nearest-even after every operation of the reference's pass chain --
+     a dropped term, a fused multiply-add, a swapped operand or a wrong order of
+     operations changes bits here;
+  3. closed forms, invariants and library cross-checks (torch.optim, torch's bf16
+     cast, the published first output of xorshift64).
+"""
+import math
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+import oracle as O
+
+
+# ---- exact arithmetic helpers -------------------------------------------------------
+
+def rne(q: Fraction, mant_bits: int, emin: int) -> Fraction:
+    """Round an exact rational to the nearest binary float (ties to even) with
+    `mant_bits` significand bits and minimum exponent `emin` of the last place."""
+    if q == 0:
+        return Fraction(0)
+    sign = -1 if q < 0 else 1
+    q = abs(q)
+    e = q.numerator.bit_length() - q.denominator.bit_length() - mant_bits
+    while q / Fraction(2) ** e >= 2 ** mant_bits:
+        e += 1
+    while q / Fraction(2) ** e < 2 ** (mant_bits - 1):
+        e -= 1
+    e = max(e, emin)
+    scaled = q / Fraction(2) ** e
+    fl = scaled.numerator // scaled.denominator
+    rem = scaled - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+        fl += 1
+    return sign * fl * Fraction(2) ** e
+
+
+def r32(q):  # IEEE binary32
+    return rne(Fraction(q), 24, -149)
+
+
+def r64(q):  # IEEE binary64
+    return rne(Fraction(q), 53, -1074)
+
+
+def sqrt_r32(q: Fraction) -> Fraction:
+    """Correctly rounded f32 square root of an exact non-negative rational."""
+    if q == 0:
+        return Fraction(0)
+    # sqrt(q) to 80 extra bits, then round; the truncation cannot flip an f32 rounding
+    # for the inputs used here because the 24-bit midpoint squared is never hit exactly
+    # unless q is a perfect square of a midpoint, which binary32 inputs cannot be.
+    shift = 200
+    num = (q.numerator << (2 * shift)) // q.denominator
+    root = math.isqrt(num)
+    approx = Fraction(root, 1 << shift)
+    if root * root != num:
+        approx += Fraction(1, 1 << (shift + 2))  # strictly between root and root+1 ulp
+    return r32(approx)
+
+
+def f32_exact(x) -> Fraction:
+    return Fraction(float(np.float32(x)))
+
+
+def as_f32(q: Fraction) -> np.float32:
+    return np.float32(float(q))
+
+
+# ---- 1. the reference's own known answers ---------------------------------------------
+
+def test_kat_sgd_step_updates_param():
+    """tests/optim.rs:47-57: 1.0 - 0.1 * 1.0 = 0.9 (f64, 1x1)."""
+    p, g, v = [np.array([1.0])], [np.array([1.0])], [np.zeros(1)]
+    O.sgd_step(O.sgd_meta(0.1), p, g, v)
+    assert abs(p[0][0] - 0.9) < 1e-10
+
+
+def test_kat_adam_adamw_decrease_param():
+    """tests/optim.rs:59-81: after one step from p=1, g=1 the parameter is < 1;
+    closed form: step 1 from m=v=0 is p - lr*g/(|g|+eps) (+ decay for AdamW)."""
+    for meta, expect in ((O.adam_meta(0.1), 0.9), (O.adamw_meta(0.1), 0.899)):
+        p, g = [np.array([1.0])], [np.array([1.0])]
+        m, v = [np.zeros(1)], [np.zeros(1)]
+        O.adam_step(meta, p, g, m, v)
+        assert p[0][0] < 1.0
+        assert p[0][0] == pytest.approx(expect, abs=1e-8)
+        assert meta.step_count == 1
+        assert m[0][0] == pytest.approx(0.1) and v[0][0] == pytest.approx(0.001)
+
+
+def test_kat_group_weight_decay_exclusion():
+    """tests/optim.rs:140-165: SGD lr=1, wd=0.1, g=0: weight 2.0 -> 1.8; wd=0: bias 3.0 -> 3.0."""
+    w, b, z = [np.array([2.0])], [np.array([3.0])], [np.zeros(1)]
+    O.sgd_step(O.sgd_meta(1.0, 0.0, 0.1), w, z, [np.zeros(1)])
+    O.sgd_step(O.sgd_meta(1.0, 0.0, 0.0), b, z, [np.zeros(1)])
+    assert abs(w[0][0] - 1.8) < 1e-10 and abs(b[0][0] - 3.0) < 1e-10
+
+
+def test_kat_grad_scaler_unscale_and_detect_inf():
+    """tests/optim.rs:120-138 with the defaults of core.rs:336-344."""
+    s = O.default_scaler()
+    assert (s.scale, s.growth_factor, s.backoff_factor, s.growth_interval, s.consecutive_ok) == \
+        (65536.0, 2.0, 0.5, 2000, 0)
+    g = [np.array([2.0])]
+    assert O.scaler_unscale_and_update(s, g) is True
+    assert g[0][0] == 2.0 / 65536.0 and g[0][0] < 2.0
+    assert s.consecutive_ok == 1 and s.scale == 65536.0
+    g = [np.array([np.inf])]
+    assert O.scaler_unscale_and_update(s, g) is False
+    assert abs(g[0][0]) < 1e-12
+    assert s.scale == 32768.0 and s.consecutive_ok == 0
+
+
+def test_kat_clip_grad_norm_scales():
+    """tests/trainer.rs:171-203: grads (3), (4): reported norm 5, norm after clip 2.5."""
+    g = [np.array([3.0]), np.array([4.0])]
+    reported = O.clip_grad_norm(g, 2.5)
+    after = math.sqrt(sum(float((x * x).sum()) for x in g))
+    assert abs(reported - 5.0) < 1e-10 and abs(after - 2.5) < 1e-10
+    # trainer.rs:501-503 and :515
+    g = [np.array([3.0]), np.array([4.0])]
+    assert O.clip_grad_norm(g, 0.0) == 0.0 and O.clip_grad_norm(g, -1.0) == 0.0
+    assert O.clip_grad_norm(g, 5.0) == 5.0 and g[0][0] == 3.0 and g[1][0] == 4.0
+
+
+def test_kat_lr_schedules():
+    """tests/optim.rs:83-118."""
+    lin = O.Schedule(1, 0, 10, 0.0, 0.0)
+    assert abs(O.lr_at_step(lin, 1.0, 0) - 1.0) < 1e-10 and O.lr_at_step(lin, 1.0, 10) <= 1e-10
+    stp = O.Schedule(3, 2, 0, 0.1, 0.0)
+    assert abs(O.lr_at_step(stp, 1.0, 0) - 1.0) < 1e-10
+    assert abs(O.lr_at_step(stp, 1.0, 2) - 0.1) < 1e-10
+    assert abs(O.lr_at_step(stp, 1.0, 4) - 0.01) < 1e-10
+    one = O.Schedule(2, 0, 10, 1.0, 0.5)
+    assert O.lr_at_step(one, 0.1, 3) > 0.1
+    # closed forms: cosine mid-point and end, warm-up ramp
+    cos = O.Schedule(0, 10, 110, 0.1, 0.0)
+    assert O.lr_at_step(cos, 1.0, 5) == pytest.approx(0.5)
+    assert O.lr_at_step(cos, 1.0, 60) == pytest.approx(0.55)
+    assert O.lr_at_step(cos, 1.0, 110) == pytest.approx(0.1)
+
+
+# ---- 2. exact-rational evaluation of every rounding ----------------------------------------
+
+def _rand_f32(rng, n, lo=-8, hi=2):
+    return (rng.standard_normal(n) * 10.0 ** rng.uniform(lo, hi, n)).astype(np.float32)
+
+
+def test_primitives_round_once_per_operation():
+    rng = np.random.default_rng(0)
+    a, b = _rand_f32(rng, 64), _rand_f32(rng, 64)
+    s = np.float32(0.899999976158142)
+    out = O.scale(a, s)
+    for i in range(a.size):
+        assert f32_exact(out[i]) == r32(f32_exact(a[i]) * f32_exact(s))
+    out = O.emul(a, b)
+    for i in range(a.size):
+        assert f32_exact(out[i]) == r32(f32_exact(a[i]) * f32_exact(b[i]))
+    out = O.ediv(a, b)
+    for i in range(a.size):
+        assert f32_exact(out[i]) == r32(f32_exact(a[i]) / f32_exact(b[i]))
+    out = O.add(a, b)
+    for i in range(a.size):
+        assert f32_exact(out[i]) == r32(f32_exact(a[i]) + f32_exact(b[i]))
+
+
+def test_axpy_is_multiply_then_add_not_fma():
+    """cpu/mod.rs:221: *yi = *yi + alpha * xi -- two roundings.  The sample must contain
+    elements where a fused multiply-add would give different bits, or the check could
+    not tell the two apart."""
+    rng = np.random.default_rng(1)
+    y, x = _rand_f32(rng, 512, -2, 0), _rand_f32(rng, 512, -2, 0)
+    alpha = np.float32(0.1)
+    y0 = y.copy()
+    O.axpy_inplace(y, alpha, x)
+    fused_differs = 0
+    for i in range(y.size):
+        prod = f32_exact(alpha) * f32_exact(x[i])
+        two = r32(f32_exact(y0[i]) + r32(prod))
+        one = r32(f32_exact(y0[i]) + prod)
+        assert f32_exact(y[i]) == two
+        fused_differs += two != one
+    assert fused_differs > 10
+
+
+def _exact_adam(kind, lr, b1, b2, eps, wd, steps, p0, grads):
+    """Adam / AdamW on f32 in exact arithmetic with RNE after each operation of
+    alg.rs:120-148, taking the correctly rounded sqrt for powf(x, 0.5)."""
+    p = [f32_exact(x) for x in p0]
+    m = [Fraction(0)] * len(p)
+    v = [Fraction(0)] * len(p)
+    B1, B2, LR, EPS, WD = (Fraction(x) for x in (b1, b2, lr, eps, wd))
+    for t in range(1, steps + 1):
+        # f64 scalars: powi by repeated squaring as __powidf2 does, each multiply rounded
+        def powi(a, n):
+            r, a = Fraction(1), Fraction(a)
+            while True:
+                if n & 1:
+                    r = r64(r * a)
+                n >>= 1
+                if n == 0:
+                    return r
+                a = r64(a * a)
+        bc1 = r64(1 - powi(B1, t))
+        bc2 = r64(1 - powi(B2, t))
+        ss = r32(r64(LR / bc1))
+        ibc2 = r32(r64(1 / bc2))
+        fb1, fomb1 = r32(B1), r32(r64(1 - B1))
+        fb2, fomb2 = r32(B2), r32(r64(1 - B2))
+        feps = r32(EPS)
+        omw = r32(1 - r32(r64(WD * LR)))
+        g = [f32_exact(x) for x in grads[t - 1]]
+        for i in range(len(p)):
+            m[i] = r32(r32(m[i] * fb1) + r32(fomb1 * g[i]))
+            v[i] = r32(r32(v[i] * fb2) + r32(fomb2 * r32(g[i] * g[i])))
+            denom = r32(sqrt_r32(r32(v[i] * ibc2)) + feps)
+            upd = r32(r32(m[i] * ss) / denom)
+            if kind == "adamw":
+                p[i] = r32(p[i] * omw)
+            p[i] = r32(p[i] + (-upd))
+    return p, m, v
+
+
+@pytest.mark.parametrize("kind", ["adam", "adamw"])
+def test_adam_chain_bit_exact_against_exact_arithmetic(kind):
+    rng = np.random.default_rng(2)
+    n, steps = 8, 3
+    lr, b1, b2, eps, wd = 3e-4, 0.9, 0.95, 1e-8, 0.1
+    p0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    grads = [(rng.standard_normal(n) * 1e-3).astype(np.float32) for _ in range(steps)]
+    pe, me, ve = _exact_adam(kind, lr, b1, b2, eps, wd, steps, p0, grads)
+    p, m, v = [p0.copy()], [np.zeros(n, np.float32)], [np.zeros(n, np.float32)]
+    meta = O.adam_meta(lr, b1, b2, eps) if kind == "adam" else O.adamw_meta(lr, b1, b2, eps, wd)
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        for t in range(steps):
+            O.adam_step(meta, p, [grads[t]], m, v)
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+    for i in range(n):
+        assert f32_exact(m[0][i]) == me[i], f"m[{i}]"
+        assert f32_exact(v[0][i]) == ve[i], f"v[{i}]"
+        assert f32_exact(p[0][i]) == pe[i], f"p[{i}]"
+    # the libm-powf variant: moments identical, params within 2 ulp
+    p2, m2, v2 = [p0.copy()], [np.zeros(n, np.float32)], [np.zeros(n, np.float32)]
+    meta2 = O.adam_meta(lr, b1, b2, eps) if kind == "adam" else O.adamw_meta(lr, b1, b2, eps, wd)
+    for t in range(steps):
+        O.adam_step(meta2, p2, [grads[t]], m2, v2)
+    assert np.array_equal(m2[0].view(np.uint32), m[0].view(np.uint32))
+    assert np.array_equal(v2[0].view(np.uint32), v[0].view(np.uint32))
+    assert O.ulp_distance_f32(p2[0], p[0]).max() <= 2
+
+
+def test_adamw_step_single_equals_adamw_step():
+    """adamw_step (alg.rs:431-469) is AdamW::step's body for one tensor."""
+    rng = np.random.default_rng(3)
+    p0 = (rng.standard_normal(100) * 0.02).astype(np.float32)
+    g = (rng.standard_normal(100) * 1e-3).astype(np.float32)
+    pa, ma, va = [p0.copy()], [np.zeros_like(p0)], [np.zeros_like(p0)]
+    meta = O.adamw_meta(1e-3, 0.9, 0.999, 1e-8, 0.01, step_count=4)
+    O.adam_step(meta, pa, [g], ma, va)
+    pb, mb, vb = p0.copy(), np.zeros_like(p0), np.zeros_like(p0)
+    O.adamw_step_single(pb, g, mb, vb, 1e-3, 0.9, 0.999, 1e-8, 0.01, 5)
+    assert np.array_equal(pa[0], pb) and np.array_equal(ma[0], mb) and np.array_equal(va[0], vb)
+
+
+def test_sgd_momentum_weight_decay_exact():
+    """alg.rs:404-413 in exact arithmetic."""
+    rng = np.random.default_rng(4)
+    n = 16
+    p0, g = _rand_f32(rng, n, -2, 0), _rand_f32(rng, n, -3, -1)
+    lr, mu, wd = 0.05, 0.9, 0.01
+    p, vel = [p0.copy()], [np.zeros(n, np.float32)]
+    meta = O.sgd_meta(lr, mu, wd)
+    pe = [f32_exact(x) for x in p0]
+    ve = [Fraction(0)] * n
+    for _ in range(3):
+        O.sgd_step(meta, p, [g], vel)
+        for i in range(n):
+            ge = r32(f32_exact(g[i]) + r32(pe[i] * r32(wd)))
+            ve[i] = r32(r32(ve[i] * r32(mu)) + ge)
+            pe[i] = r32(pe[i] + r32(-r32(lr) * ve[i]))
+    for i in range(n):
+        assert f32_exact(p[0][i]) == pe[i] and f32_exact(vel[0][i]) == ve[i]
+
+
+def test_clip_sum_is_serial_f64_and_scale_is_narrowed_once():
+    """trainer.rs:504-521: sum += v*v in f64 in list order; scale_t = T(max_norm / norm)."""
+    rng = np.random.default_rng(5)
+    g = [_rand_f32(rng, 37, -3, 0), _rand_f32(rng, 5, -3, 0)]
+    g0 = [x.copy() for x in g]
+    s = Fraction(0)
+    for t in g0:
+        for x in t:
+            s = r64(s + r64(f32_exact(x) * f32_exact(x)))
+    norm = O.clip_grad_norm(g, 1e-3)
+    assert Fraction(norm) ** 2 == pytest.approx(float(s), rel=1e-15)
+    assert norm == math.sqrt(float(s))
+    c = r32(r64(Fraction(1e-3) / Fraction(norm)))
+    for t, t0 in zip(g, g0):
+        for x, x0 in zip(t, t0):
+            assert f32_exact(x) == r32(f32_exact(x0) * c)
+
+
+def test_unscale_multiplies_by_narrowed_reciprocal():
+    """core.rs:355,379: inv_scale = T(1/scale); g = g * inv_scale (not g / scale)."""
+    s = O.ScalerState(3.0, 2.0, 0.5, 2000, 0)  # 1/3 is inexact: g*T(1/3) != g/3 in general
+    rng = np.random.default_rng(6)
+    g0 = _rand_f32(rng, 256, -2, 2)
+    g = [g0.copy()]
+    assert O.scaler_unscale_and_update(s, g)
+    inv = r32(r64(Fraction(1) / 3))
+    differs_from_division = 0
+    for x, x0 in zip(g[0], g0):
+        assert f32_exact(x) == r32(f32_exact(x0) * inv)
+        differs_from_division += r32(f32_exact(x0) * inv) != r32(f32_exact(x0) / 3)
+    assert differs_from_division > 0
+
+
+# ---- 3. closed forms, invariants, library cross-checks -------------------------------------
+
+def test_powi_matches_exact_powers():
+    assert O.powi(0.5, 10) == 2.0 ** -10 and O.powi(2.0, 30) == 2.0 ** 30
+    assert O.powi(0.9, 0) == 1.0 and O.powi(0.9, 1) == 0.9 and O.powi(2.0, -2) == 0.25
+    for a, n in ((0.9, 7), (0.95, 100), (0.999, 2000), (0.1, 5)):
+        exact = Fraction(a) ** n
+        got = Fraction(O.powi(a, n))
+        # each of the ~2*log2(n) multiplies rounds once; errors scale with the exponent
+        assert abs(got - exact) / exact < Fraction(n, 2 ** 52)
+
+
+def test_zero_gradient_is_pure_decay_and_moments_stay_zero():
+    p0 = np.float32([1.0, -2.0, 0.5])
+    p, m, v = [p0.copy()], [np.zeros(3, np.float32)], [np.zeros(3, np.float32)]
+    meta = O.adamw_meta(0.1, weight_decay=0.1)
+    g = [np.zeros(3, np.float32)]
+    for _ in range(5):
+        O.adam_step(meta, p, g, m, v)
+    assert not m[0].any() and not v[0].any()
+    omw = np.float32(1.0) - np.float32(0.1 * 0.1)
+    expect = p0.copy()
+    for _ in range(5):
+        expect = expect * omw
+    assert np.array_equal(p[0], expect)
+
+
+def test_constant_gradient_gives_geometric_moments():
+    g = [np.full(4, 0.25, np.float32)]
+    p, m, v = [np.ones(4, np.float32)], [np.zeros(4, np.float32)], [np.zeros(4, np.float32)]
+    meta = O.adam_meta(1e-3)
+    for t in range(1, 21):
+        O.adam_step(meta, p, g, m, v)
+        assert m[0][0] == pytest.approx(0.25 * (1 - 0.9 ** t), rel=1e-5)
+        assert v[0][0] == pytest.approx(0.0625 * (1 - 0.999 ** t), rel=1e-5)
+    # bias-corrected update is lr * sign(g) for a constant gradient
+    assert p[0][0] == pytest.approx(1.0 - 20 * 1e-3, rel=1e-5)
+
+
+def test_moments_do_not_depend_on_params():
+    rng = np.random.default_rng(7)
+    g = [(rng.standard_normal(50) * 1e-3).astype(np.float32)]
+    res = []
+    for scale in (1.0, 100.0):
+        p = [(rng.standard_normal(50) * scale).astype(np.float32)]
+        m, v = [np.zeros(50, np.float32)], [np.zeros(50, np.float32)]
+        meta = O.adamw_meta(1e-3)
+        for _ in range(3):
+            O.adam_step(meta, p, g, m, v)
+        res.append((m[0].copy(), v[0].copy()))
+    assert np.array_equal(res[0][0], res[1][0]) and np.array_equal(res[0][1], res[1][1])
+
+
+def test_matches_torch_optim_within_a_few_ulp():
+    """Same mathematics, different rounding order (torch: sqrt(v)/sqrt(bc2) + eps, addcdiv)."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(8)
+    p0 = (rng.standard_normal(1000) * 0.02).astype(np.float32)
+    grads = [(rng.standard_normal(1000) * 1e-3).astype(np.float32) for _ in range(10)]
+    for kind in ("adam", "adamw", "sgd"):
+        tp = torch.nn.Parameter(torch.from_numpy(p0.copy()))
+        if kind == "adam":
+            topt = torch.optim.Adam([tp], lr=3e-4, betas=(0.9, 0.999), eps=1e-8)
+            meta = O.adam_meta(3e-4)
+        elif kind == "adamw":
+            topt = torch.optim.AdamW([tp], lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+            meta = O.adamw_meta(3e-4, 0.9, 0.95, 1e-8, 0.1)
+        else:
+            topt = torch.optim.SGD([tp], lr=0.01, momentum=0.9, weight_decay=0.01)
+            meta = O.sgd_meta(0.01, 0.9, 0.01)
+        p, m, v = [p0.copy()], [np.zeros_like(p0)], [np.zeros_like(p0)]
+        for g in grads:
+            tp.grad = torch.from_numpy(g.copy())
+            topt.step()
+            if kind == "sgd":
+                O.sgd_step(meta, p, [g], m)
+            else:
+                O.adam_step(meta, p, [g], m, v)
+        np.testing.assert_allclose(p[0], tp.detach().numpy(), rtol=2e-5, atol=2e-9)
+
+
+def test_bf16_cast_matches_torch_for_all_exponents_and_is_rne():
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(9)
+    bits = rng.integers(0, 2 ** 32, size=1 << 22, dtype=np.uint64).astype(np.uint32)
+    # every exponent with tie / just-above-tie / just-below-tie / max mantissas
+    exps = np.arange(256, dtype=np.uint32) << 23
+    tails = np.array([0x0000, 0x7FFF, 0x8000, 0x8001, 0x18000, 0x17FFF, 0x7F7FFF, 0x7F8000,
+                      0x7FFFFF], dtype=np.uint32)
+    edge = (exps[:, None] | tails[None, :]).reshape(-1)
+    bits = np.concatenate([bits, edge, edge | np.uint32(0x80000000)])
+    f = bits.view(np.float32)
+    finite_or_inf = ~np.isnan(f)
+    got = O.bf16_from_f32(f)
+    ref = torch.from_numpy(f.copy()).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(got[finite_or_inf], ref[finite_or_inf])
+    # NaN: stays NaN, quiet bit set, sign and top payload kept (crate half's rule)
+    nan = np.uint32([0x7F800001, 0xFFC12345, 0x7FBFFFFF]).view(np.float32)
+    out = O.bf16_from_f32(nan)
+    assert list(out) == [0x7FC0, 0xFFC1, 0x7FFF]
+    # widening is exact
+    h = np.arange(0, 65536, dtype=np.uint32).astype(np.uint16)
+    w = O.bf16_to_f32(h)
+    assert np.array_equal(w.view(np.uint32), h.astype(np.uint32) << 16)
+
+
+def test_randn_stream_anchors():
+    """xorshift64 with shifts (13, 7, 17): state 1 -> 1082269761 is the published first
+    output; the Box-Muller pair built from the first two outputs must reproduce."""
+    s = 1
+    outs = []
+    for _ in range(2):
+        s ^= (s << 13) & 0xFFFFFFFFFFFFFFFF
+        s ^= s >> 7
+        s ^= (s << 17) & 0xFFFFFFFFFFFFFFFF
+        outs.append(s)
+    assert outs[0] == 1082269761
+    u1, u2 = outs[0] / 2.0 ** 64, outs[1] / 2.0 ** 64
+    r, th = math.sqrt(-2.0 * math.log(u1)), 2.0 * math.pi * u2
+    z = O.randn_f64(3, 1)
+    assert z[0] == pytest.approx(r * math.cos(th), rel=1e-15)
+    assert z[1] == pytest.approx(r * math.sin(th), rel=1e-15)
+    # seed 0 is replaced by 0x123456789ABCDEF0 (constructors.rs:20-24)
+    assert np.array_equal(O.randn_f64(8, 0), O.randn_f64(8, 0x123456789ABCDEF0))
+    big = O.randn_f64(200_000, 42)
+    assert abs(big.mean()) < 0.01 and abs(big.std() - 1.0) < 0.01
+
+
+def test_scaler_trace_closed_form():
+    """growth_interval 4, inf injected every 4th step: only 3 clean steps fit between
+    injections, so the scale only halves; every 5th step: it grows once, then halves."""
+    for period, steps in ((4, 64), (5, 60)):
+        s = O.ScalerState(65536.0, 2.0, 0.5, 4, 0)
+        trace = []
+        for step in range(steps):
+            g = [np.ones(3, np.float32)]
+            if step % period == period - 1:
+                g[0][1] = np.nan
+            ok = O.scaler_unscale_and_update(s, g)
+            trace.append((ok, s.scale, s.consecutive_ok))
+        skipped = sum(1 for t in trace if not t[0])
+        assert skipped == steps // period
+        if period == 4:
+            assert s.scale == 65536.0 * 0.5 ** 16 == 1.0
+            assert max(t[2] for t in trace) == 3
+        else:
+            assert s.scale == 65536.0
+            assert [t[1] for t in trace[:5]] == [65536.0, 65536.0, 65536.0, 131072.0, 65536.0]
+
+
+def test_found_inf_leaves_everything_but_the_scaler_untouched():
+    rng = np.random.default_rng(10)
+    shapes = [(3, 5), (1, 9)]
+    master = [(rng.standard_normal(r * c) * 0.02).astype(np.float32) for r, c in shapes]
+    m = [np.full_like(a, 0.5) for a in master]
+    v = [np.full_like(a, 0.25) for a in master]
+    p = [O.bf16_from_f32(a) for a in master]
+    g = [O.bf16_from_f32(np.ones_like(a)) for a in master]
+    g[1][4] = 0x7F80  # +inf
+    before = [x.copy() for x in master + m + v + p]
+    meta, s = O.adamw_meta(1e-3, step_count=7), O.default_scaler()
+    ran, norm = O.mixed_step(meta, s, 1.0, p, g, master, m, v)
+    assert not ran and norm == 0.0 and meta.step_count == 7
+    assert s.scale == 32768.0 and s.consecutive_ok == 0
+    for a, b in zip(before, master + m + v + p):
+        assert np.array_equal(a, b)
