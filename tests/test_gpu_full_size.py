@@ -1,0 +1,204 @@
+"""The benchmark configurations at their full sizes.
+
+The oracle cannot chew through 8 G parameters, so at full size the device results are
+checked (a) through what does not depend on size -- the decision trace, the global
+norm against an independent f64 reduction, step counts -- and (b) element for element
+on slices of every tensor (head, a chunk boundary in the middle, tail): every
+operation of the step is element-wise once the two global scalars (found_inf, norm)
+are known, so the oracle run on a slice must reproduce that slice bit for bit.
+Synthetic inputs come from torch's generator on the device; oracle and device consume
+the same bytes.
+"""
+import numpy as np
+import pytest
+
+import oracle as O
+from nabla_amd import optim as nb
+from nabla_amd import workloads as W
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+SL = 4096  # elements per slice
+
+
+def _slices(n):
+    """Index ranges checked inside a tensor of n elements."""
+    if n <= 3 * SL:
+        return [(0, n)]
+    mid = (n // 2) // 8192 * 8192  # straddles a work-chunk boundary
+    mid = max(SL, min(mid, n - 2 * SL))
+    return [(0, SL), (mid - SL // 2, mid + SL // 2), (n - SL, n)]
+
+
+def _take(t, n):
+    """Host copy of the checked slices of device tensor t, concatenated."""
+    flat = t.reshape(-1)
+    import torch
+
+    return H.to_host(torch.cat([flat[a:b] for a, b in _slices(n)]))
+
+
+def _take_list(tensors, shapes):
+    return [_take(t, r * c) for t, (r, c) in zip(tensors, shapes)]
+
+
+def test_gpt2_small_adam_f32_10_steps(gpu):
+    """Config 2: Adam f32, 148 tensors, 124,439,808 params, fresh grads each step."""
+    import torch
+
+    shapes = W.gpt2_small_shapes()
+    assert len(shapes) == 148 and W.n_params(shapes) == 124_439_808
+    torch.manual_seed(2)
+    p = [torch.randn(s, device=gpu) * 0.02 for s in shapes]
+    ref_p = _take_list(p, shapes)
+    ref_m, ref_v = H.zeros_like_list(ref_p), H.zeros_like_list(ref_p)
+    opt = nb.Adam.new(3e-4, shapes)
+    meta = O.adam_meta(3e-4)
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        for step in range(10):
+            g = [torch.randn(s, device=gpu) * 1e-3 for s in shapes]
+            opt.step(p, g)
+            O.adam_step(meta, ref_p, _take_list(g, shapes), ref_m, ref_v)
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+    assert opt.step_count() == 10
+    m, v = opt.moments()
+    H.assert_bits_equal(_take_list(m, shapes), ref_m, "m slices")
+    H.assert_bits_equal(_take_list(v, shapes), ref_v, "v slices")
+    H.assert_bits_equal(_take_list(p, shapes), ref_p, "param slices")
+
+
+def _mixed_full(gpu, shapes, steps, seed):
+    """Configs 3 / 5: AdamW, bf16 params/grads, f32 master/m/v, scale 65536, clip 1.0."""
+    import torch
+
+    lr, wd = 2e-4, 0.1
+    torch.manual_seed(seed)
+    n_t = len(shapes)
+    opt = nb.AdamW.new(lr, shapes, master=True).beta2(0.95).weight_decay(wd)
+    params = [torch.empty(s, dtype=torch.bfloat16, device=gpu) for s in shapes]
+    ref_w = []
+    for i, s in enumerate(shapes):
+        w = torch.randn(s, device=gpu) * 0.02
+        opt.write_state(f"w{i}", w)
+        ref_w.append(_take(w, s[0] * s[1]))
+        del w
+    opt.params_from_master(params)
+    ref_m, ref_v = H.zeros_like_list(ref_w), H.zeros_like_list(ref_w)
+    scaler = nb.GradScaler.new()
+    meta = O.adamw_meta(lr, 0.9, 0.95, 1e-8, wd)
+    inv = np.float32(1.0 / 65536.0)
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        for step in range(steps):
+            grads, sumsq = [], torch.zeros((), dtype=torch.float64, device=gpu)
+            for s in shapes:
+                g = (torch.randn(s, device=gpu) * (1e-3 * 65536.0)).to(torch.bfloat16)
+                u = g.float() * float(inv)
+                sumsq += (u.double() ** 2).sum()
+                grads.append(g)
+                del u
+            opt.fused_step(params, grads, scaler=scaler, max_norm=1.0)
+            info = opt.last_step()
+            # size-independent: decisions and the global norm
+            assert (info.found_inf, info.scale, info.step_count) == (0, 65536.0, step + 1)
+            norm_ref = float(torch.sqrt(sumsq))
+            assert info.norm == pytest.approx(norm_ref, rel=1e-9)
+            assert info.clipped == 1 and norm_ref > 1.0
+            # slices: the reference's chain with the device's (verified) norm
+            c = np.float32(1.0 / info.norm)
+            g32 = [(O.bf16_to_f32(_take(g, s[0] * s[1])) * inv) * c for g, s in zip(grads, shapes)]
+            O.adam_step(meta, ref_w, g32, ref_m, ref_v)
+            del grads
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+    m, v = opt.moments()
+    H.assert_bits_equal(_take_list(m, shapes), ref_m, "m slices")
+    H.assert_bits_equal(_take_list(v, shapes), ref_v, "v slices")
+    del m, v
+    w = [opt.read_state(f"w{i}") for i in range(n_t)]
+    H.assert_bits_equal(_take_list(w, shapes), ref_w, "master slices")
+    del w
+    H.assert_bits_equal(_take_list(params, shapes), [O.bf16_from_f32(a) for a in ref_w],
+                        "bf16 param slices")
+    # idempotence of the narrowing: params == bf16(master) everywhere, checked on the device
+    for i in range(0, n_t, 37):
+        wi = opt.read_state(f"w{i}")
+        assert torch.equal(wi.to(torch.bfloat16), params[i])
+        del wi
+
+
+def test_llama_1b_mixed_adamw_10_steps(gpu):
+    shapes = W.llama_1b_shapes()
+    assert len(shapes) == 200 and W.n_params(shapes) == 1_100_046_336
+    _mixed_full(gpu, shapes, 10, seed=3)
+
+
+def test_llama3_8b_mixed_adamw_2_steps(gpu):
+    shapes = W.llama_8b_shapes()
+    assert len(shapes) == 290 and W.n_params(shapes) == 8_030_257_152
+    _mixed_full(gpu, shapes, 2, seed=5)
+
+
+def test_ragged_4096_dynamic_scale_64_steps(gpu):
+    """Config 4 in full: 4096 tensors, sizes log-uniform in [1, 65536], packed back to
+    back (so most tensor addresses are only 2-byte aligned), growth interval 4, inf/NaN
+    injected every 4th step at a seeded 1e-6 of the positions; 64 steps.  Everything is
+    compared with the oracle run on the whole set."""
+    import torch
+
+    sizes = W.ragged_sizes()
+    shapes = [(1, n) for n in sizes]
+    total = sum(sizes)
+    offs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+    lr, wd = 2e-4, 0.1
+    rng = np.random.default_rng(4)
+    w0 = (rng.standard_normal(total) * 0.02).astype(np.float32)
+    flat_p = H.to_dev(O.bf16_from_f32(w0))
+    flat_g = torch.empty(total, dtype=torch.bfloat16, device=gpu)
+    views_p = [flat_p[offs[i]:offs[i + 1]] for i in range(len(sizes))]
+    views_g = [flat_g[offs[i]:offs[i + 1]] for i in range(len(sizes))]
+    assert any(v.data_ptr() % 16 for v in views_p), "the packed layout is meant to be unaligned"
+    opt = nb.AdamW.new(lr, shapes, master=True).beta2(0.95).weight_decay(wd)
+    opt.master_from_params(views_p)  # master = f32(bf16 params)
+    plist, glist = nb.TensorList(views_p), nb.TensorList(views_g)
+    scaler = nb.GradScaler.new()
+    scaler.load_state(nb.GradScalerState(65536.0, 2.0, 0.5, 4, 0))
+
+    ref_w_flat = O.bf16_to_f32(O.bf16_from_f32(w0))
+    ref_p_flat = O.bf16_from_f32(w0)
+    ref_m_flat, ref_v_flat = np.zeros(total, np.float32), np.zeros(total, np.float32)
+    split = lambda a: [a[offs[i]:offs[i + 1]] for i in range(len(sizes))]  # noqa: E731
+    ref_w, ref_p, ref_m, ref_v = split(ref_w_flat), split(ref_p_flat), split(ref_m_flat), split(ref_v_flat)
+    meta, s = O.adamw_meta(lr, 0.9, 0.95, 1e-8, wd), O.ScalerState(65536.0, 2.0, 0.5, 4, 0)
+    O.set_threads(8)
+    O.set_pow_mode(O.POW_SQRT)
+    ref_trace = []
+    try:
+        for step in range(64):
+            g_bits = O.bf16_from_f32((rng.standard_normal(total) * (1e-3 * s.scale)).astype(np.float32))
+            if step % 4 == 3:
+                for pos in rng.integers(0, total, size=max(1, int(total * 1e-6))):
+                    g_bits[pos] = (0x7F80, 0xFF80, 0x7FC0)[int(rng.integers(3))]
+            flat_g.copy_(H.to_dev(g_bits))
+            opt.fused_step(plist, glist, scaler=scaler, max_norm=1.0)
+            ran, norm = O.mixed_step(meta, s, 1.0, ref_p, split(g_bits), ref_w, ref_m, ref_v)
+            ref_trace.append((0 if ran else 1, s.scale, meta.step_count, norm))
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+        O.set_threads(1)
+    tr = opt.trace()
+    assert [(t.found_inf, t.scale, t.step_count) for t in tr] == [t[:3] for t in ref_trace]
+    for t, r in zip(tr, ref_trace):
+        assert t.norm == pytest.approx(r[3], rel=1e-12)
+    # closed form of the schedule: 16 skips, scale halves 16 times, 48 optimizer steps
+    assert sum(t.found_inf for t in tr) == 16 and tr[-1].scale == 1.0 and tr[-1].step_count == 48
+    st = scaler.state()
+    assert (st.scale, st.consecutive_ok) == (s.scale, s.consecutive_ok)
+    m, v = opt.moments()
+    H.assert_bits_equal(H.host_list(m), ref_m, "m")
+    H.assert_bits_equal(H.host_list(v), ref_v, "v")
+    H.assert_bits_equal(H.host_list([opt.read_state(f"w{i}") for i in range(len(sizes))]), ref_w, "master")
+    H.assert_bits_equal([H.to_host(flat_p)], [ref_p_flat], "bf16 params")
