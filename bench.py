@@ -260,7 +260,8 @@ def main():
         "data": "synthetic (random-init parameters and gradients of the named shapes, resident in HBM)",
         "config": {"workload": args.workload, "tensors": len(shapes), "params": n,
                    "bytes_per_param_step": upd_b + nrm_b, "optimizer": cfg["kind"],
-                   "loss_scale": scale if cfg["scaler"] else None, "clip_max_norm": cfg["clip"] or None},
+                   "loss_scale": scale if cfg["scaler"] else None, "clip_max_norm": cfg["clip"] or None,
+                   "state_hbm_regions": opt.state_regions()},
         "roofline": {
             "kernel": dom,
             "bound": "hbm",

@@ -152,6 +152,11 @@ int nbo_optim_state_write(nbo_optim *opt, const char *name, const void *buf, uin
 int nbo_optim_master_from_params(nbo_optim *opt, nbo_list *params_bf16);
 int nbo_optim_params_from_master(nbo_optim *opt, nbo_list *params_bf16);
 
+/* How the optimizer's state arrays were placed in HBM: *regions = 0 for plain
+ * allocations, otherwise the number of 96 GiB HBM regions their chunks were spread
+ * over (no counterpart in the reference; see nbo_placement.hpp). */
+int nbo_optim_state_regions(nbo_optim *opt, int *regions);
+
 /* ---- GradScaler (optim/core.rs:254-260, 334-413) ---------------------------------- */
 
 /* GradScaler::new + load_state; state == NULL gives the defaults of core.rs:336-344. */

@@ -94,6 +94,7 @@ SYMBOLS = {
     "nbo_optim_state_write": (C.c_int, [_P, C.c_char_p, _P, C.c_uint64, C.c_int]),
     "nbo_optim_master_from_params": (C.c_int, [_P, _P]),
     "nbo_optim_params_from_master": (C.c_int, [_P, _P]),
+    "nbo_optim_state_regions": (C.c_int, [_P, C.POINTER(C.c_int)]),
     "nbo_scaler_create": (C.c_int, [C.POINTER(ScalerState), C.POINTER(_P)]),
     "nbo_scaler_destroy": (C.c_int, [_P]),
     "nbo_scaler_state_get": (C.c_int, [_P, C.POINTER(ScalerState)]),

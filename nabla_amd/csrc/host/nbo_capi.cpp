@@ -180,8 +180,7 @@ void part_copy(nbo_optim *opt, uint64_t i, uint32_t part, void *buf, bool on_dev
     const size_t eb = opt->elem_bytes();
     const size_t bytes = (size_t)opt->layout.n[i] * eb;
     if (bytes == 0) return;
-    char *dev = (char *)opt->arena.base +
-                ((size_t)part * opt->arena.part_stride + opt->layout.soff[i]) * eb;
+    char *dev = (char *)opt->arena.part[part] + (size_t)opt->layout.soff[i] * eb;
     if (on_device)
         hip_check(hipMemcpyAsync(to_engine ? (void *)dev : buf, to_engine ? buf : (void *)dev, bytes,
                                  hipMemcpyDeviceToDevice, rt.stream()),
@@ -216,8 +215,15 @@ void state_copy(nbo_optim *opt, const char *name, void *buf, uint64_t n_elems, i
 void part_zero(nbo_optim *opt, uint32_t part)
 {
     const size_t eb = opt->elem_bytes();
-    Runtime::get().dzero((char *)opt->arena.base + (size_t)part * opt->arena.part_stride * eb,
-                         (size_t)opt->layout.arena_elems * eb);
+    Runtime::get().dzero(opt->arena.part[part], (size_t)opt->layout.arena_elems * eb);
+}
+
+// Allocates the state parts (region-aware, see nbo_placement.hpp), zero-filled.
+void alloc_state_parts(nbo_optim *o)
+{
+    const size_t bytes = (size_t)o->layout.arena_elems * o->elem_bytes();
+    o->placement.allocate(o->arena.nparts, bytes, o->arena.part);
+    for (uint32_t k = 0; k < o->arena.nparts; k++) Runtime::get().dzero(o->arena.part[k], bytes);
 }
 
 void fill_info(const NboTraceEntry &e, nbo_step_info *out)
@@ -358,16 +364,11 @@ int nbo_optim_create(const nbo_meta *meta, uint64_t n_tensors, const uint64_t *r
             o->state_dtype = state_dtype;
             o->keep_master = keep_master != 0;
             o->layout.build(n_tensors, rows, cols, true);
-            // one device arena holding every state part (see NboArenaDev)
             const bool adam_like = meta->kind != NBO_KIND_SGD;
             o->arena.nparts = 1u + (adam_like ? 1u : 0u) + (o->keep_master ? 1u : 0u);
             o->arena.part_v = 1;
             o->arena.part_w = adam_like ? 2 : 1;
-            o->arena.part_stride = o->layout.arena_elems;
-            const size_t bytes = ((size_t)o->arena.part_stride * (o->arena.nparts - 1) +
-                                  (size_t)o->layout.arena_elems) * o->elem_bytes();
-            o->arena.base = rt.dmalloc(bytes);
-            rt.dzero(o->arena.base, bytes);
+            alloc_state_parts(o);
             o->dev = (NboOptimDev *)rt.dmalloc(sizeof(NboOptimDev));
             o->gf = (NboGradFactors *)rt.dmalloc(sizeof(NboGradFactors));
             o->trace = (NboTraceDev *)rt.dmalloc(sizeof(NboTraceDev));
@@ -386,7 +387,7 @@ int nbo_optim_create(const nbo_meta *meta, uint64_t n_tensors, const uint64_t *r
             *out = o;
         } catch (...) {
             o->layout.release();
-            rt.dfree(o->arena.base);
+            o->placement.release();
             rt.dfree(o->dev);
             rt.dfree(o->gf);
             rt.dfree(o->trace);
@@ -403,7 +404,7 @@ int nbo_optim_destroy(nbo_optim *opt)
         Runtime &rt = Runtime::get();
         rt.sync();
         opt->layout.release();
-        rt.dfree(opt->arena.base);
+        opt->placement.release();
         rt.dfree(opt->dev);
         rt.dfree(opt->gf);
         rt.dfree(opt->trace);
@@ -531,6 +532,14 @@ int nbo_optim_params_from_master(nbo_optim *opt, nbo_list *params_bf16)
     return guarded([&] {
         require(opt && opt->master_valid, NBO_ERR_NO_MASTER, "master weights not set");
         cast_master(opt, params_bf16, 1);
+    });
+}
+
+int nbo_optim_state_regions(nbo_optim *opt, int *regions)
+{
+    return guarded([&] {
+        require(opt && regions, NBO_ERR_ARG, "null optimizer or output");
+        *regions = opt->placement.regions_used();
     });
 }
 

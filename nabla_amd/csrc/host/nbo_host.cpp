@@ -35,7 +35,7 @@ static const char *const kKernelNames[K_COUNT] = {
     "nbo_norm_f32",          "nbo_norm_bf16",        "nbo_norm_f64",
     "nbo_scale_f32",         "nbo_scale_bf16",       "nbo_scale_f64",
     "nbo_prep",              "nbo_finalize",         "nbo_cast_master",
-    "nbo_copy_f32x4",
+    "nbo_copy_f32x4",        "nbo_probe_rmw2",
 };
 
 Runtime &Runtime::get()
@@ -149,6 +149,31 @@ void Runtime::launch_copy(const void *src, void *dst, uint64_t nvec)
         hip_check(hipEventRecord(rec.end, stream_), "hipEventRecord");
         prof_.push_back(rec);
     }
+}
+
+double Runtime::probe_pair_gbps(void *a, void *b, size_t bytes)
+{
+    const uint64_t nvec = bytes / 16;
+    const uint32_t grid = (uint32_t)(nvec / 2048); // 8 rows of 256 vectors per workgroup
+    if (grid == 0) return 0.0;
+    void *args[2] = {(void *)&a, (void *)&b};
+    hipEvent_t e0, e1;
+    hip_check(hipEventCreate(&e0), "hipEventCreate");
+    hip_check(hipEventCreate(&e1), "hipEventCreate");
+    float best = 0.0f;
+    for (int rep = 0; rep < 4; rep++) {
+        hip_check(hipEventRecord(e0, stream_), "hipEventRecord");
+        hip_check(hipModuleLaunchKernel(fn_[K_PROBE], grid, 1, 1, NBO_BLOCK, 1, 1, 0, stream_, args, nullptr),
+                  kKernelNames[K_PROBE]);
+        hip_check(hipEventRecord(e1, stream_), "hipEventRecord");
+        hip_check(hipEventSynchronize(e1), "hipEventSynchronize");
+        float ms = 0.0f;
+        hip_check(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime");
+        if (rep > 0 && (best == 0.0f || ms < best)) best = ms; // first run warms up
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return best > 0.0f ? 4.0 * (double)grid * 2048 * 16 / best / 1e6 : 0.0;
 }
 
 void Runtime::read_back(void *host_dst, const void *dev_src, size_t bytes)

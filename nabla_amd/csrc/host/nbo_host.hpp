@@ -13,6 +13,7 @@
 
 #include "../../../include/nabla_optim.h"
 #include "../nbo_device_types.h"
+#include "nbo_placement.hpp"
 
 namespace nbo {
 
@@ -35,7 +36,8 @@ enum KernelId {
     K_FINALIZE = 16,
     K_CAST_MASTER = 17,
     K_COPY = 18,
-    K_COUNT = 19
+    K_PROBE = 19,
+    K_COUNT = 20
 };
 
 // Process-wide runtime: device 0, the loaded module, the stream, scratch buffers.
@@ -52,6 +54,9 @@ public:
     }
     void launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct);
     void launch_copy(const void *src, void *dst, uint64_t nvec);
+    // Bandwidth (GB/s, best of three) of reading and rewriting `bytes` bytes at a and at
+    // b together: the probe StatePlacement classifies HBM regions with.  Synchronous.
+    double probe_pair_gbps(void *a, void *b, size_t bytes);
 
     // synchronous small transfers through a pinned staging buffer
     void read_back(void *host_dst, const void *dev_src, size_t bytes);
@@ -120,7 +125,8 @@ struct nbo_optim {
     int state_dtype = NBO_DT_F32;
     bool keep_master = false;
     bool master_valid = false;
-    NboArenaDev arena = {}; // the one device allocation m, v and master live in
+    nbo::StatePlacement placement; // owns the memory behind arena.part[]
+    NboArenaDev arena = {};        // m, v and master
     NboOptimDev *dev = nullptr; // step_count lives here: the device decides skips
     NboGradFactors *gf = nullptr;
     NboTraceDev *trace = nullptr;

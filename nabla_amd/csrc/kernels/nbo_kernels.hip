@@ -264,7 +264,7 @@ DEV ChunkRef chunk_ref(const NboLayoutDev &L, uint32_t c)
 // Address of chunk c within state part `part` of the arena.
 template <typename T> DEV T *state_part(const NboArenaDev &A, const ChunkRef &c, uint32_t part)
 {
-    return (T *)A.base + part * A.part_stride + c.soff + c.base;
+    return (T *)A.part[part] + c.soff + c.base;
 }
 
 // ---------------------------------------------------------------------------------
@@ -718,4 +718,26 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_copy_f32x4(const f32
     const uint64_t stride = (uint64_t)gridDim.x * NBO_BLOCK;
     for (uint64_t i = (uint64_t)blockIdx.x * NBO_BLOCK + threadIdx.x; i < nvec; i += stride)
         __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
+// Placement probe: reads and rewrites the same 2048 vectors per workgroup of two
+// buffers together.  Two buffers in the same region of HBM run measurably slower than
+// two in different regions; the host times this to classify freshly created chunks
+// (their contents do not matter yet).
+extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_probe_rmw2(f32x4 *a, f32x4 *b)
+{
+    const uint64_t c0 = (uint64_t)blockIdx.x * 2048;
+    f32x4 va[8], vb[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+        const uint64_t i = c0 + u * 256 + threadIdx.x;
+        va[u] = __builtin_nontemporal_load(a + i);
+        vb[u] = __builtin_nontemporal_load(b + i);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+        const uint64_t i = c0 + u * 256 + threadIdx.x;
+        __builtin_nontemporal_store(va[u] + 1.0f, a + i);
+        __builtin_nontemporal_store(vb[u] + 1.0f, b + i);
+    }
 }

@@ -100,15 +100,15 @@ struct NboTraceDev {
 
 // ---- kernel argument blocks (each kernel takes exactly one, by value) ----------
 
-// The optimizer's state arena: one device allocation holding one planar array per
-// state "part", part_stride elements apart.  Part 0 is the first moment (SGD:
-// velocity), part 1 the second moment (Adam / AdamW), the last part the f32 master
-// weights when kept.  Within a part, tensor t starts at element soff[t] (a multiple
-// of NBO_CHUNK: every tensor is padded to whole chunks).  (A tiled variant that puts
-// the parts of each chunk back to back measured 1-2 % slower on MI355X.)
+// The optimizer's state: one planar device array per state "part".  Part 0 is the
+// first moment (SGD: velocity), part 1 the second moment (Adam / AdamW), the last
+// part the f32 master weights when kept.  Within a part, tensor t starts at element
+// soff[t] (a multiple of NBO_CHUNK: every tensor is padded to whole chunks).  The
+// parts are separate allocations so that the host can place them in different
+// regions of HBM.  (A tiled variant that puts the parts of each chunk back to back
+// measured 1-2 % slower on MI355X.)
 struct NboArenaDev {
-    void *base;
-    uint64_t part_stride; // elements between consecutive parts
+    void *part[3];
     uint32_t nparts;
     uint32_t part_v; // index of the second-moment part (unused for SGD)
     uint32_t part_w; // index of the master part (unused without master)

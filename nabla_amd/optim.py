@@ -330,6 +330,12 @@ class _Optimizer:
                                                C.byref(total)))
         return [buf[i] for i in range(n.value)]
 
+    def state_regions(self) -> int:
+        """0: state arrays are plain allocations; n: spread over n HBM regions."""
+        n = C.c_int(0)
+        _call(_lib.load().nbo_optim_state_regions(self._handle(), C.byref(n)))
+        return n.value
+
     # -- master weights (mixed precision) -----------------------------------------------
     def master_from_params(self, params) -> None:
         p = self._cache.get("p", params)
