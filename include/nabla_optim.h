@@ -196,6 +196,16 @@ int nbo_scale_grad(nbo_list *grads, double factor);
  * is taken on the device; nothing is read back.  Asynchronous. */
 int nbo_fused_step(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, nbo_list *grads,
                    double max_norm, uint32_t flags);
+/* The same tail for GroupOptimizer (optim/groups.rs:269-293): one unscale / found-inf /
+ * clip decision over `all_grads` (every gradient, in the module's order), then each
+ * group's update with its own hyper-parameters.  params[g] / grads[g] are the lists of
+ * group g's tensors; together the groups must cover all_grads.  Asynchronous. */
+int nbo_fused_step_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,
+                          nbo_list *const *grads, nbo_scaler *scaler, nbo_list *all_grads,
+                          double max_norm, uint32_t flags);
+/* Gradient accumulation of the Trainer, buf[i] = &buf[i] + g (trainer.rs:262-266),
+ * optionally zeroing the gradients in the same pass.  Asynchronous. */
+int nbo_accumulate(nbo_list *accum, nbo_list *grads, int zero_grads);
 /* Outcome of the optimizer's most recent fused step.  Synchronous. */
 int nbo_optim_last_step(nbo_optim *opt, nbo_step_info *out);
 /* The last `max_entries` (at most 1024) fused-step outcomes, oldest first; *n_out

@@ -89,7 +89,7 @@ void check_step_args(const nbo_optim *opt, const nbo_list *params, const nbo_lis
 }
 
 NboUpdateArgs update_args(nbo_optim *opt, nbo_list *params, nbo_list *grads, bool with_gf,
-                          bool zero_grads)
+                          bool zero_grads, const NboGradFactors *shared_gf = nullptr)
 {
     NboUpdateArgs a = {};
     a.L = opt->layout.dev;
@@ -97,7 +97,7 @@ NboUpdateArgs update_args(nbo_optim *opt, nbo_list *params, nbo_list *grads, boo
     a.g_ptrs = grads->ptrs_dev;
     a.arena = opt->arena;
     a.opt = opt->dev;
-    a.gf = with_gf ? opt->gf : nullptr;
+    a.gf = shared_gf ? shared_gf : with_gf ? opt->gf : nullptr;
     a.zero_grads = zero_grads ? 1u : 0u;
     return a;
 }
@@ -711,6 +711,69 @@ int nbo_fused_step(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, nbo_lis
         const NboUpdateArgs a =
             update_args(opt, params, grads, true, (flags & NBO_STEP_ZERO_GRADS) != 0);
         rt.launch(update_kernel(opt, params), opt->layout.nchunks, NBO_BLOCK, a);
+    });
+}
+
+int nbo_fused_step_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,
+                          nbo_list *const *grads, nbo_scaler *scaler, nbo_list *all_grads,
+                          double max_norm, uint32_t flags)
+{
+    return guarded([&] {
+        require(n_groups == 0 || (opts && params && grads), NBO_ERR_ARG, "null group arrays");
+        require(all_grads != nullptr, NBO_ERR_ARG, "null gradient list");
+        uint64_t covered = 0;
+        for (uint64_t g = 0; g < n_groups; g++) {
+            check_step_args(opts[g], params[g], grads[g]);
+            require(grads[g]->dtype == all_grads->dtype, NBO_ERR_DTYPE,
+                    "group gradients differ in element type from the whole list");
+            covered += grads[g]->layout.nt();
+        }
+        if (covered != all_grads->layout.nt())
+            fail(NBO_ERR_COUNT_MISMATCH, "nabla-train: GroupOptimizer param count mismatch");
+        Runtime &rt = Runtime::get();
+        // one decision for all groups: the reference unscales and clips the whole
+        // gradient list before any group's step (trainer.rs:230-283)
+        NboFinalizeArgs f = {};
+        f.partial_sumsq = rt.partial_sumsq();
+        f.partial_flag = rt.partial_flag();
+        f.grid = launch_norm(all_grads, scaler ? scaler->dev : nullptr);
+        f.check_finite = (scaler || (flags & NBO_STEP_SKIP_NONFINITE)) ? 1u : 0u;
+        f.scaler = scaler ? scaler->dev : nullptr;
+        f.gf = rt.gf_scratch();
+        f.max_norm = max_norm;
+        rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
+        for (uint64_t g = 0; g < n_groups; g++) {
+            NboPrepArgs p = {};
+            p.opt = opts[g]->dev;
+            p.gf = rt.gf_scratch();
+            p.scaler = scaler ? scaler->dev : nullptr;
+            p.trace = opts[g]->trace;
+            p.hyper = hyper_of(opts[g]);
+            rt.launch(K_PREP, 1, 64, p);
+            const NboUpdateArgs a = update_args(opts[g], params[g], grads[g], true,
+                                                (flags & NBO_STEP_ZERO_GRADS) != 0, rt.gf_scratch());
+            rt.launch(update_kernel(opts[g], params[g]), opts[g]->layout.nchunks, NBO_BLOCK, a);
+        }
+    });
+}
+
+int nbo_accumulate(nbo_list *accum, nbo_list *grads, int zero_grads)
+{
+    return guarded([&] {
+        require(accum && grads, NBO_ERR_ARG, "null list");
+        if (accum->layout.nt() != grads->layout.nt())
+            fail(NBO_ERR_LEN_MISMATCH, "nabla-train: accumulation buffers / grads length mismatch");
+        for (uint64_t t = 0; t < accum->layout.nt(); t++)
+            if (accum->layout.rows[t] != grads->layout.rows[t] || accum->layout.cols[t] != grads->layout.cols[t])
+                fail(NBO_ERR_SHAPE, "nabla: add -- shapes are not broadcast-compatible (tensor " +
+                                        std::to_string(t) + ")");
+        require(accum->dtype == grads->dtype, NBO_ERR_DTYPE, "lists differ in element type");
+        NboAccumArgs a = {};
+        a.L = accum->layout.dev;
+        a.a_ptrs = accum->ptrs_dev;
+        a.b_ptrs = grads->ptrs_dev;
+        a.zero_b = zero_grads ? 1u : 0u;
+        Runtime::get().launch(K_ACCUM_BASE + accum->dtype, accum->layout.nchunks, NBO_BLOCK, a);
     });
 }
 

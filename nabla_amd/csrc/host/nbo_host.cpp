@@ -35,7 +35,8 @@ static const char *const kKernelNames[K_COUNT] = {
     "nbo_norm_f32",          "nbo_norm_bf16",        "nbo_norm_f64",
     "nbo_scale_f32",         "nbo_scale_bf16",       "nbo_scale_f64",
     "nbo_prep",              "nbo_finalize",         "nbo_cast_master",
-    "nbo_copy_f32x4",        "nbo_probe_rmw2",
+    "nbo_copy_f32x4",        "nbo_probe_rmw2",       "nbo_accum_f32",
+    "nbo_accum_bf16",        "nbo_accum_f64",
 };
 
 Runtime &Runtime::get()

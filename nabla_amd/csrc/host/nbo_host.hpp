@@ -37,7 +37,8 @@ enum KernelId {
     K_CAST_MASTER = 17,
     K_COPY = 18,
     K_PROBE = 19,
-    K_COUNT = 20
+    K_ACCUM_BASE = 20, // + st
+    K_COUNT = 23
 };
 
 // Process-wide runtime: device 0, the loaded module, the stream, scratch buffers.

@@ -569,9 +569,24 @@ DEV void prep_step(NboOptimDev *o, const NboHyper &h, const NboGradFactors *f)
     o->d_omw = 1.0 - wd_lr;
 }
 
+DEV void trace_step(NboTraceDev *t, const NboGradFactors *f, const NboOptimDev *o, double scale)
+{
+    const uint64_t i = t->count;
+    NboTraceEntry e;
+    e.scale = scale;
+    e.norm = f ? f->norm : 0.0;
+    e.step_count = o ? o->step_count : 0;
+    e.found_inf = f ? f->found_inf : 0u;
+    e.clipped = f ? f->clipped : 0u;
+    t->e[i % NBO_TRACE_LEN] = e;
+    t->count = i + 1;
+}
+
 extern "C" __global__ __launch_bounds__(64) void nbo_prep(const NboPrepArgs a)
 {
-    if (threadIdx.x == 0 && blockIdx.x == 0) prep_step(a.opt, a.hyper, a.gf);
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    prep_step(a.opt, a.hyper, a.gf);
+    if (a.trace) trace_step(a.trace, a.gf, a.opt, a.scaler ? a.scaler->scale : 0.0);
 }
 
 // Second stage: reduce the per-block partials in a fixed order, then the scalar
@@ -632,17 +647,7 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_finalize(const NboFi
     }
     *a.gf = f;
     if (a.opt) prep_step(a.opt, a.hyper, &f);
-    if (a.trace) {
-        const uint64_t i = a.trace->count;
-        NboTraceEntry e;
-        e.scale = scale_after;
-        e.norm = f.norm;
-        e.step_count = a.opt ? a.opt->step_count : 0;
-        e.found_inf = f.found_inf;
-        e.clipped = f.clipped;
-        a.trace->e[i % NBO_TRACE_LEN] = e;
-        a.trace->count = i + 1;
-    }
+    if (a.trace) trace_step(a.trace, &f, a.opt, scale_after);
 }
 
 // ---------------------------------------------------------------------------------
@@ -692,6 +697,47 @@ template <int ST> DEV void scale_body(const NboScaleArgs &a)
 NBO_SCALE_KERNEL(nbo_scale_f32, NBO_F32)
 NBO_SCALE_KERNEL(nbo_scale_bf16, NBO_BF16)
 NBO_SCALE_KERNEL(nbo_scale_f64, NBO_F64)
+
+// Gradient accumulation of the Trainer: buf[i] = &buf[i] + g (trainer.rs:262-266 ->
+// B::add, cpu/mod.rs:181: one rounding in T; for bf16 the f32 sum is rounded to bf16,
+// scalar/mod.rs:253-351), optionally clearing g afterwards.
+template <int ST> DEV void accum_body(const NboAccumArgs &a)
+{
+    typedef typename Traits<ST>::T T;
+    enum { SB = Traits<ST>::SBYTES, VEC = Traits<ST>::VEC };
+    const uint32_t tid = threadIdx.x;
+    const ChunkRef c = chunk_ref(a.L, blockIdx.x);
+    char *pa = (char *)a.a_ptrs[c.t] + c.base * SB;
+    char *pb = (char *)a.b_ptrs[c.t] + c.base * SB;
+    const bool vec_ok = ((((uintptr_t)pa) | ((uintptr_t)pb)) & (VEC * SB - 1)) == 0;
+    const uint32_t nvec = vec_ok ? c.cnt / VEC : 0;
+    for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
+        T x[VEC], y[VEC];
+        IO<ST>::ldv(pa + (uint64_t)q * VEC * SB, x);
+        IO<ST>::ldv(pb + (uint64_t)q * VEC * SB, y);
+#pragma unroll
+        for (int k = 0; k < VEC; k++) x[k] = x[k] + y[k];
+        IO<ST>::stv(pa + (uint64_t)q * VEC * SB, x);
+        if (a.zero_b) {
+            T z[VEC] = {};
+            IO<ST>::stv(pb + (uint64_t)q * VEC * SB, z);
+        }
+    }
+    for (uint32_t e = nvec * VEC + tid; e < c.cnt; e += NBO_BLOCK) {
+        const T x = IO<ST>::ld1(pa + (uint64_t)e * SB) + IO<ST>::ld1(pb + (uint64_t)e * SB);
+        IO<ST>::st1(pa + (uint64_t)e * SB, x);
+        if (a.zero_b) IO<ST>::st1(pb + (uint64_t)e * SB, (T)0);
+    }
+}
+
+#define NBO_ACCUM_KERNEL(name, ST)                                                          \
+    extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboAccumArgs a)      \
+    {                                                                                       \
+        accum_body<ST>(a);                                                                  \
+    }
+NBO_ACCUM_KERNEL(nbo_accum_f32, NBO_F32)
+NBO_ACCUM_KERNEL(nbo_accum_bf16, NBO_BF16)
+NBO_ACCUM_KERNEL(nbo_accum_f64, NBO_F64)
 
 // ---------------------------------------------------------------------------------
 // Master-weight casts: arena f32 <- bf16 tensors (exact widening) and

@@ -151,8 +151,19 @@ struct NboFinalizeArgs {
 
 struct NboPrepArgs {
     NboOptimDev *opt;
-    const NboGradFactors *gf; // may be null
+    const NboGradFactors *gf;   // may be null
+    const NboScalerDev *scaler; // may be null; only read, for the trace entry
+    NboTraceDev *trace;         // may be null
     NboHyper hyper;
+};
+
+// a[i] = a[i] + b[i] over two lists of the same shapes (gradient accumulation).
+struct NboAccumArgs {
+    NboLayoutDev L;
+    const uint64_t *a_ptrs;
+    const uint64_t *b_ptrs;
+    uint32_t zero_b; // also clear b after it has been added
+    uint32_t pad;
 };
 
 struct NboScaleArgs {

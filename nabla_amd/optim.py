@@ -424,7 +424,8 @@ class _Optimizer:
             raise OptimStateError("optim kind mismatch")
         m = _lib.Meta(_KIND_CODE[meta.kind], 0, meta.lr, meta.beta1, meta.beta2, meta.eps,
                       meta.weight_decay, meta.momentum, int(meta.step_count))
-        _call(_lib.load().nbo_optim_load_meta(self._handle(), C.byref(m)))
+        if self._h is not None:  # otherwise the engine is created from the updated meta
+            _call(_lib.load().nbo_optim_load_meta(self._h, C.byref(m)))
         self._meta.lr = meta.lr
         if self.KIND == KIND_SGD:
             self._meta.momentum, self._meta.weight_decay = meta.momentum, meta.weight_decay
@@ -600,6 +601,13 @@ def scale_grad(grads, factor: float) -> None:
     """nabla-ml/src/autograd/ops.rs:1675-1680."""
     g = _free_cache.get("scale", grads)
     _call(_lib.load().nbo_scale_grad(g._h, float(factor)))
+
+
+def accumulate(accum, grads, zero_grads: bool = False) -> None:
+    """buf[i] = &buf[i] + g (nabla-train/src/trainer.rs:262-266), optionally clearing g."""
+    a = _free_cache.get("accum_a", accum)
+    g = _free_cache.get("accum_g", grads)
+    _call(_lib.load().nbo_accumulate(a._h, g._h, int(zero_grads)))
 
 
 def sync() -> None:

@@ -1,0 +1,283 @@
+"""The callers and data formats either side of the step: LR schedules, parameter groups,
+gradient accumulation, NBLA / meta.txt checkpoints.
+
+CPU tests cover the host logic (schedules against the pinned oracle and the
+reference's own test points; group assignment; the checkpoint byte layout against a
+hand-assembled file).  GPU tests run the grouped fused step and the checkpoint round
+trip through the C ABI against the oracle."""
+import os
+import struct
+
+import numpy as np
+import pytest
+
+import oracle as O
+from nabla_amd import checkpoint as ck
+from nabla_amd import groups as G
+from nabla_amd import optim as nb
+from nabla_amd import schedule as S
+
+
+# ---- LrSchedule (optim/core.rs:81-252) -------------------------------------------------------
+
+def test_lr_schedules_match_oracle_bit_for_bit():
+    cases = [
+        (S.Cosine(10, 110, 0.1), O.Schedule(0, 10, 110, 0.1, 0.0), 1.0),
+        (S.Cosine(0, 1000, 1e-5), O.Schedule(0, 0, 1000, 1e-5, 0.0), 3e-4),
+        (S.Linear(5, 50), O.Schedule(1, 5, 50, 0.0, 0.0), 2e-4),
+        (S.OneCycle(1.0, 10, 0.5), O.Schedule(2, 0, 10, 1.0, 0.5), 0.1),
+        (S.OneCycle(3e-3, 1000, 0.3), O.Schedule(2, 0, 1000, 3e-3, 0.3), 3e-4),
+        (S.Step(2, 0.1), O.Schedule(3, 2, 0, 0.1, 0.0), 1.0),
+        (S.Step(0, 0.5), O.Schedule(3, 0, 0, 0.5, 0.0), 1.0),
+    ]
+    for sched, osched, base in cases:
+        total = getattr(sched, "total_steps", 40)
+        for step in list(range(0, min(total, 60) + 1)) + [total]:
+            a, b = S.lr_at_step(sched, base, step), O.lr_at_step(osched, base, step)
+            assert np.float64(a).tobytes() == np.float64(b).tobytes(), (sched, step, a, b)
+
+
+def test_lr_schedule_reference_points():
+    """nabla-train/tests/optim.rs:83-118."""
+    lin = S.Linear(0, 10)
+    assert abs(S.lr_at_step(lin, 1.0, 0) - 1.0) < 1e-10 and S.lr_at_step(lin, 1.0, 10) <= 1e-10
+    st = S.Step(2, 0.1)
+    assert [round(S.lr_at_step(st, 1.0, k), 12) for k in (0, 2, 4)] == [1.0, 0.1, 0.01]
+    assert S.lr_at_step(S.OneCycle(1.0, 10, 0.5), 0.1, 3) > 0.1
+
+
+def test_schedule_pairs_round_trip():
+    for sched in (S.Cosine(10, 100, 1e-5), S.Linear(0, 10), S.OneCycle(1e-3, 500, 0.25), S.Step(1, 0.9)):
+        st = S.ScheduleState(0.1, sched)
+        pairs = S.schedule_pairs(st)
+        assert pairs[0] == ("schedule.enabled", "1") and pairs[1] == ("schedule.base_lr", "0.1")
+        assert S.parse_schedule_state(dict(pairs)) == st
+    assert S.parse_schedule_state({}) is None and S.parse_schedule_state({"schedule.enabled": "0"}) is None
+    with pytest.raises(nb.OptimStateError, match="bad schedule.kind: exp"):
+        S.parse_schedule_state({"schedule.enabled": "1", "schedule.base_lr": "0.1", "schedule.kind": "exp"})
+    with pytest.raises(nb.OptimStateError, match="missing schedule.gamma"):
+        S.parse_schedule_state({"schedule.enabled": "1", "schedule.base_lr": "0.1", "schedule.kind": "step",
+                                "schedule.step_size": "1"})
+
+
+# ---- parameter groups (optim/groups.rs) --------------------------------------------------------
+
+class _Named:
+    """Stands in for a tensor where only the shape matters."""
+
+    def __init__(self, shape):
+        self.shape = shape
+
+
+def test_group_assignment_first_match_wins_then_default():
+    named = [("embed.weight", _Named((10, 4))), ("layer.0.weight", _Named((4, 4))),
+             ("layer.0.bias", _Named((1, 4))), ("ln.gamma", _Named((1, 4))), ("head.weight", _Named((4, 10)))]
+    bias = G.ParamGroupConfig.sgd("no_decay", G.ParamSelector.Any([G.Suffix("bias"), G.Contains("ln")]), 1.0, 0.0, 0.0)
+    emb = G.ParamGroupConfig.adam("emb", G.ParamSelector.Any([G.Prefix("embed")]), 1e-3)
+    decay = G.ParamGroupConfig.adamw("decay", G.ParamSelector.All(), 2e-4, 0.1)
+    opt = G.GroupOptimizer.from_named_params(named, [bias, emb], decay)
+    assert opt.groups() == 3 and opt.group_indices() == [[2, 3], [0], [1, 4]]
+    assert [o.kind() for o in opt.group_optimizers()] == ["sgd", "adam", "adamw"]
+    with pytest.raises(nb.OptimStateError, match="group assignment incomplete"):
+        G.GroupOptimizer.from_named_params(named, [bias], None)
+    # empty groups are dropped (groups.rs:203-206)
+    none = G.ParamGroupConfig.adam("none", G.ParamSelector.Any([G.Equals("nope")]), 1e-3)
+    assert G.GroupOptimizer.from_named_params(named, [none], decay).groups() == 1
+    pre = G.GroupOptimizer.adamw_with_decay_presets(named, 2e-4, 0.1, ["bias", "norm", "embedding"])
+    assert pre.group_indices() == [[0, 2, 3], [1, 4]]  # "ln" and "embed" match by Contains
+    pairs = dict(opt.meta_pairs())
+    assert pairs["optim.group.count"] == "3" and pairs["optim.group.0.name"] == "no_decay"
+    assert pairs["optim.group.2.kind"] == "adamw" and pairs["optim.group.2.weight_decay"] == "0.1"
+    with pytest.raises(nb.NablaPanic, match="GroupOptimizer params/grads length mismatch"):
+        opt.step([1, 2], [1])
+    with pytest.raises(nb.NablaPanic, match="GroupOptimizer param count mismatch"):
+        opt.step([1, 2], [1, 2])
+    with pytest.raises(nb.OptimStateError, match="bad group tensor key: m0"):
+        opt.load_state_tensors([("m0", None)])
+    with pytest.raises(nb.OptimStateError, match="group index out of range: 7"):
+        opt.load_state_tensors([("g7.m0", None)])
+    with pytest.raises(nb.OptimStateError, match="optim.group.count mismatch"):
+        opt.load_meta_pairs({"optim.group.count": "2"})
+
+
+def test_group_set_lr_scales_every_group():
+    named = [("w", _Named((1, 1))), ("b", _Named((1, 1)))]
+    a = G.ParamGroupConfig.sgd("a", G.ParamSelector.Any([G.Equals("b")]), 0.5, 0.0, 0.0)
+    d = G.ParamGroupConfig.sgd("d", G.ParamSelector.All(), 0.1, 0.0, 0.1)
+    opt = G.GroupOptimizer.from_named_params(named, [a], d)
+    opt.set_lr(1.0)  # base_lr = first group's 0.5 -> scale 2 (groups.rs:301-312)
+    assert [o.lr() for o in opt.group_optimizers()] == [1.0, 0.2]
+
+
+# ---- NBLA / meta.txt ------------------------------------------------------------------------------
+
+def test_nbla_byte_layout(tmp_path):
+    path = os.path.join(tmp_path, "t.nbla")
+    ck.save_tensors([("w", np.float32([[1.5, -2.0], [0.25, 3.0]])), ("bias", np.float64([4.0, 5.0]))], path)
+    expect = b"NBLA" + struct.pack("<I", 2)
+    expect += struct.pack("<I", 1) + b"w" + struct.pack("<II", 2, 2) + struct.pack("<4d", 1.5, -2.0, 0.25, 3.0)
+    expect += struct.pack("<I", 4) + b"bias" + struct.pack("<II", 1, 2) + struct.pack("<2d", 4.0, 5.0)
+    assert open(path, "rb").read() == expect
+    back = ck.load_tensors(path)
+    assert [n for n, _ in back] == ["w", "bias"] and back[0][1].shape == (2, 2)
+    assert np.array_equal(back[0][1], [[1.5, -2.0], [0.25, 3.0]]) and np.array_equal(back[1][1], [[4.0, 5.0]])
+    open(path, "wb").write(b"NOPE")
+    with pytest.raises(ck.CheckpointError, match="not a nabla tensor file"):
+        ck.load_tensors(path)
+
+
+def test_meta_txt_layout_and_round_trip(tmp_path):
+    """checkpoint.rs:107-150 line order; tests/trainer.rs:249-305 restores epoch 2, step 3,
+    rng 42 and the schedule."""
+    path = os.path.join(tmp_path, "meta.txt")
+    opt = nb.Sgd.new(0.1, [(1, 1), (1, 1)])
+    sched = S.ScheduleState(0.1, S.Step(1, 0.9))
+    ck.write_meta(path, opt, nb.GradScaler.new(), sched, ck.TrainState(2, 3, 1, 42))
+    assert open(path).read().splitlines() == [
+        "version=1", "epoch=2", "step=3", "grad_accum=1", "rng.state=42",
+        "optim.kind=sgd", "optim.lr=0.1", "optim.beta1=0", "optim.beta2=0", "optim.eps=0",
+        "optim.weight_decay=0", "optim.momentum=0", "optim.step_count=0",
+        "schedule.enabled=1", "schedule.base_lr=0.1", "schedule.kind=step", "schedule.step_size=1",
+        "schedule.gamma=0.9",
+        "scaler.enabled=1", "scaler.scale=65536", "scaler.growth_factor=2", "scaler.backoff_factor=0.5",
+        "scaler.growth_interval=2000", "scaler.consecutive_ok=0"]
+    opt2 = nb.Sgd.new(0.5, [(1, 1), (1, 1)])
+    scaler_state, st, sched2 = ck.read_meta(path, opt2)
+    assert (st.epoch, st.step, st.grad_accum, st.rng_state) == (2, 3, 1, 42)
+    assert sched2 == sched and scaler_state.scale == 65536.0 and scaler_state.growth_interval == 2000
+    with pytest.raises(ck.CheckpointError, match="optim kind mismatch"):
+        ck.read_meta(path, nb.Adam.new(0.1, [(1, 1)]))
+    open(path, "a").write("garbage line\n")
+    with pytest.raises(ck.CheckpointError, match="garbage line"):
+        ck.read_meta(path, opt2)
+
+
+# ---- GPU ------------------------------------------------------------------------------------------------
+
+@pytest.mark.gpu
+def test_reference_group_weight_decay_exclusion_on_device(gpu):
+    """nabla-train/tests/optim.rs:140-165, f64 1x1: lr 1, wd 0.1, zero grads: weight 2.0 -> 1.8,
+    bias 3.0 -> 3.0."""
+    import torch
+
+    w = torch.tensor([[2.0]], dtype=torch.float64, device=gpu)
+    b = torch.tensor([[3.0]], dtype=torch.float64, device=gpu)
+    named = [("weight", w), ("bias", b)]
+    bias_group = G.ParamGroupConfig.sgd("no_decay", G.ParamSelector.Any([G.Suffix("bias")]), 1.0, 0.0, 0.0)
+    decay_group = G.ParamGroupConfig.sgd("decay", G.ParamSelector.All(), 1.0, 0.0, 0.1)
+    opt = G.GroupOptimizer.from_named_params(named, [bias_group], decay_group, dtype="f64")
+    grads = [torch.zeros(1, 1, dtype=torch.float64, device=gpu) for _ in range(2)]
+    opt.step([w, b], grads)
+    assert abs(w.item() - 1.8) < 1e-10 and abs(b.item() - 3.0) < 1e-10
+
+
+@pytest.mark.gpu
+def test_grouped_fused_step_matches_oracle(gpu):
+    """No-decay group for norms / biases, decay group for the rest; one scaler and one
+    clip over all gradients, then per-group AdamW -- against the reference's order:
+    unscale(all) -> clip(all) -> each group's step."""
+    from tests import helpers as H
+
+    names = ["embed", "l0.w", "l0.bias", "l0.norm", "l1.w", "l1.bias", "head"]
+    shapes = [(50, 16), (16, 16), (1, 16), (1, 16), (16, 9000), (1, 9000), (16, 50)]
+    w0 = H.randn_list(shapes, 60, 0.02)
+    p_dev = H.dev_list([O.bf16_from_f32(a) for a in w0], shapes)
+    named = list(zip(names, p_dev))
+    opt = G.GroupOptimizer.adamw_with_decay_exclusions(named, 2e-4, 0.1, ["bias", "norm"], master=True)
+    idx = opt.group_indices()
+    assert idx == [[2, 3, 5], [0, 1, 4, 6]]
+    for gi, o in zip(idx, opt.group_optimizers()):
+        for k, i in enumerate(gi):
+            o.write_state(f"w{k}", H.to_dev(w0[i], shapes[i]))
+    scaler = nb.GradScaler.new()
+    ref = dict(w=H.copy_list(w0), m=H.zeros_like_list(w0), v=H.zeros_like_list(w0))
+    metas = [O.adamw_meta(2e-4, weight_decay=0.0), O.adamw_meta(2e-4, weight_decay=0.1)]
+    s = O.default_scaler()
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        for step in range(4):
+            g32 = H.randn_list(shapes, 700 + 11 * step, 1e-3 * 65536.0)
+            g_bits = [O.bf16_from_f32(a) for a in g32]
+            if step == 2:
+                g_bits[4][123] = 0x7F80
+            opt.fused_step(p_dev, H.dev_list(g_bits, shapes), scaler=scaler, max_norm=1.0)
+            gf = [O.bf16_to_f32(b) for b in g_bits]
+            if not O.scaler_unscale_and_update(s, gf):
+                continue
+            O.clip_grad_norm(gf, 1.0)
+            for gi, meta in zip(idx, metas):
+                O.adam_step(meta, [ref["w"][i] for i in gi], [gf[i] for i in gi],
+                            [ref["m"][i] for i in gi], [ref["v"][i] for i in gi])
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+    assert [o.step_count() for o in opt.group_optimizers()] == [3, 3] == [m.step_count for m in metas]
+    assert scaler.state().scale == s.scale == 32768.0
+    H.assert_bits_equal(H.host_list(p_dev), [O.bf16_from_f32(a) for a in ref["w"]], "bf16 params")
+    state = dict(opt.state_tensors())
+    for g, gi in enumerate(idx):
+        for k, i in enumerate(gi):
+            H.assert_bits_equal([H.to_host(state[f"g{g}.m{k}"])], [ref["m"][i]], f"g{g}.m{k}")
+            H.assert_bits_equal([H.to_host(state[f"g{g}.v{k}"])], [ref["v"][i]], f"g{g}.v{k}")
+    tr = opt.group_optimizers()[1].trace()
+    assert [t.found_inf for t in tr] == [0, 0, 1, 0] and [t.step_count for t in tr] == [1, 2, 2, 3]
+
+
+@pytest.mark.gpu
+def test_accumulate_matches_add(gpu):
+    from tests import helpers as H
+
+    shapes = [(1, 5), (3, 2741), (1, 8193)]
+    a = H.randn_list(shapes, 5, 1.0)
+    b = H.randn_list(shapes, 9, 1e-3)
+    a_dev, b_dev = H.dev_list(a, shapes), H.dev_list(b, shapes)
+    nb.accumulate(a_dev, b_dev, zero_grads=True)
+    H.assert_bits_equal(H.host_list(a_dev), [O.add(x, y) for x, y in zip(a, b)], "buf + g")
+    for t in H.host_list(b_dev):
+        assert not t.any()
+    with pytest.raises(nb.NablaPanic):
+        nb.accumulate(a_dev, b_dev[:2])
+
+
+@pytest.mark.gpu
+def test_checkpoint_round_trip_restores_bit_identical_training(gpu, tmp_path):
+    """Train 3 steps, save, restore into fresh objects, train 2 more on both: identical bits."""
+    from tests import helpers as H
+
+    shapes = [(4, 7), (1, 9000), (1, 3)]
+
+    def fresh():
+        o = nb.AdamW.new(2e-4, shapes, master=True).beta2(0.95).weight_decay(0.1)
+        s = nb.GradScaler.new()
+        s.load_state(nb.GradScalerState(65536.0, 2.0, 0.5, 2, 0))
+        return o, s
+
+    w0 = H.randn_list(shapes, 80, 0.02)
+    p1 = H.dev_list([O.bf16_from_f32(a) for a in w0], shapes)
+    o1, s1 = fresh()
+    for i, a in enumerate(w0):
+        o1.write_state(f"w{i}", H.to_dev(a, shapes[i]))
+    grads = [H.dev_list([O.bf16_from_f32(a) for a in H.randn_list(shapes, 900 + k, 65.5)], shapes) for k in range(5)]
+    for k in range(3):
+        o1.fused_step(p1, grads[k], scaler=s1, max_norm=1.0)
+    sched = S.ScheduleState(2e-4, S.Cosine(2, 10, 1e-5))
+    master = [(f"p{i}", o1.read_state(f"w{i}")) for i in range(len(shapes))]
+    ck.save_checkpoint(str(tmp_path), master, o1, s1, sched, ck.TrainState(1, 3, 1, 7))
+    assert sorted(os.listdir(tmp_path)) == ["meta.txt", "optim.nbla", "params.nbla"]
+    names = [n for n, _ in ck.load_tensors(os.path.join(tmp_path, "optim.nbla"))]
+    assert names == ["m0", "m1", "m2", "v0", "v1", "v2"]
+
+    o2, s2 = fresh()
+    params, st, sched2 = ck.load_checkpoint(str(tmp_path), o2, s2)
+    assert (st.epoch, st.step, st.rng_state) == (1, 3, 7) and sched2 == sched
+    assert o2.step_count() == 3 and o2.meta() == o1.meta()
+    assert vars(s2.state()) == vars(s1.state())
+    p2 = H.dev_list([O.bf16_from_f32(a.astype(np.float32).reshape(-1)) for _, a in params], shapes)
+    for i, (_, a) in enumerate(params):
+        o2.write_state(f"w{i}", H.to_dev(a.astype(np.float32).reshape(-1), shapes[i]))
+    for k in range(3, 5):
+        o1.fused_step(p1, grads[k], scaler=s1, max_norm=1.0)
+        o2.fused_step(p2, grads[k], scaler=s2, max_norm=1.0)
+    H.assert_bits_equal(H.host_list(p2), H.host_list(p1), "params after resume")
+    H.assert_bits_equal(H.host_list(o2.moments()[0]), H.host_list(o1.moments()[0]), "m after resume")
+    H.assert_bits_equal(H.host_list(o2.moments()[1]), H.host_list(o1.moments()[1]), "v after resume")
+    assert o2.step_count() == o1.step_count() == 5
