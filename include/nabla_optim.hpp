@@ -1,0 +1,322 @@
+// nabla_optim.hpp -- C++ mirror of nabla-train's optimizer interface over the C ABI of
+// nabla_optim.h.  Header-only; link libnabla_optim.so.
+//
+// The reference's host language is Rust; this is the same surface for a C++ host:
+// the names, the argument meaning and the error behaviour of
+// nabla-train/src/optim/{core,alg}.rs and nabla-train/src/trainer.rs:500-523.
+//   trait Optimizer   (core.rs:9-44)    -> nabla::optim::Optimizer  {step, reset, set_lr}
+//   Sgd / Adam / AdamW (alg.rs)         -> same names, same builder setters
+//   trait OptimState  (core.rs:64-79)   -> kind, state_read / state_write, meta, load_meta
+//   GradScaler        (core.rs:334-413) -> same methods
+//   clip_grad_norm, zero_grad, scale_grad -> free functions
+// Where the reference panics (assert_eq! on list lengths, shape asserts) this throws
+// nabla::optim::Panic with the reference's message; where it returns Err(String) this
+// throws nabla::optim::StateError.
+#ifndef NABLA_OPTIM_HPP
+#define NABLA_OPTIM_HPP
+
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "nabla_optim.h"
+
+namespace nabla {
+namespace optim {
+
+struct Panic : std::logic_error {
+    using std::logic_error::logic_error;
+};
+struct StateError : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+struct RuntimeError : std::runtime_error {
+    int status;
+    RuntimeError(int s, const std::string &m) : std::runtime_error(m), status(s) {}
+};
+
+inline void check(int status)
+{
+    if (status == NBO_OK) return;
+    const std::string msg = nbo_last_error();
+    if (status == NBO_ERR_LEN_MISMATCH || status == NBO_ERR_COUNT_MISMATCH || status == NBO_ERR_SHAPE)
+        throw Panic(msg);
+    if (status == NBO_ERR_STATE_KEY || status == NBO_ERR_STATE_INDEX || status == NBO_ERR_KIND)
+        throw StateError(msg);
+    throw RuntimeError(status, msg);
+}
+
+// A dense row-major (rows x cols) matrix in device memory: what `&Tensor<T, B>` is to
+// the reference's optimizers.
+struct Tensor {
+    void *data = nullptr;
+    uint64_t rows = 0, cols = 0;
+    nbo_dtype dtype = NBO_DT_F32;
+    std::pair<uint64_t, uint64_t> shape() const { return {rows, cols}; }
+};
+
+// `&[&Tensor]`: described to the device once, reusable across steps.
+class TensorList {
+public:
+    TensorList() = default;
+    explicit TensorList(const std::vector<Tensor> &tensors) { assign(tensors); }
+    TensorList(const TensorList &) = delete;
+    TensorList &operator=(const TensorList &) = delete;
+    TensorList(TensorList &&o) noexcept : h_(o.h_), n_(o.n_) { o.h_ = nullptr; }
+    ~TensorList() { reset(); }
+
+    void assign(const std::vector<Tensor> &tensors)
+    {
+        reset();
+        std::vector<uint64_t> rows, cols;
+        std::vector<const void *> ptrs;
+        const nbo_dtype dt = tensors.empty() ? NBO_DT_F32 : tensors[0].dtype;
+        for (const Tensor &t : tensors) {
+            if (t.dtype != dt) throw RuntimeError(NBO_ERR_DTYPE, "all tensors of a list share one dtype");
+            rows.push_back(t.rows);
+            cols.push_back(t.cols);
+            ptrs.push_back(t.data);
+        }
+        n_ = tensors.size();
+        check(nbo_list_create(n_, rows.data(), cols.data(), dt, ptrs.data(), &h_));
+    }
+    nbo_list *handle() const { return h_; }
+    size_t size() const { return n_; }
+
+private:
+    void reset()
+    {
+        if (h_) nbo_list_destroy(h_);
+        h_ = nullptr;
+    }
+    nbo_list *h_ = nullptr;
+    size_t n_ = 0;
+};
+
+enum class OptimKind { AdamW = NBO_KIND_ADAMW, Adam = NBO_KIND_ADAM, Sgd = NBO_KIND_SGD };
+
+// optim/core.rs:53-62
+struct OptimMeta {
+    OptimKind kind;
+    double lr, beta1, beta2, eps, weight_decay, momentum;
+    uint64_t step_count;
+};
+
+// optim/core.rs:326-332; defaults of core.rs:336-344
+struct GradScalerState {
+    double scale = 65536.0, growth_factor = 2.0, backoff_factor = 0.5;
+    uint64_t growth_interval = 2000, consecutive_ok = 0;
+};
+
+class GradScaler {
+public:
+    GradScaler() = default;
+    GradScaler(const GradScaler &) = delete;
+    GradScaler &operator=(const GradScaler &) = delete;
+    ~GradScaler()
+    {
+        if (h_) nbo_scaler_destroy(h_);
+    }
+    // core.rs:351-388: true if every gradient was finite (they are now unscaled), false
+    // otherwise (they are now zeros and the scale has been backed off).
+    bool unscale_and_update(TensorList &grads)
+    {
+        int ok = 0;
+        check(nbo_scaler_unscale_and_update(handle(), grads.handle(), &ok));
+        return ok != 0;
+    }
+    double scale_factor() { return state().scale; }
+    GradScalerState state()
+    {
+        if (!h_) return init_;
+        nbo_scaler_state s;
+        check(nbo_scaler_state_get(h_, &s));
+        return {s.scale, s.growth_factor, s.backoff_factor, s.growth_interval, s.consecutive_ok};
+    }
+    void load_state(const GradScalerState &st)
+    {
+        init_ = st;
+        if (h_) {
+            const nbo_scaler_state s = {st.scale, st.growth_factor, st.backoff_factor, st.growth_interval,
+                                        st.consecutive_ok};
+            check(nbo_scaler_load_state(h_, &s));
+        }
+    }
+    nbo_scaler *handle()
+    {
+        if (!h_) {
+            const nbo_scaler_state s = {init_.scale, init_.growth_factor, init_.backoff_factor,
+                                        init_.growth_interval, init_.consecutive_ok};
+            check(nbo_scaler_create(&s, &h_));
+        }
+        return h_;
+    }
+
+private:
+    nbo_scaler *h_ = nullptr;
+    GradScalerState init_;
+};
+
+// trait Optimizer + trait OptimState.  T is float or double (the arithmetic type);
+// with `master` the caller's tensors may be bf16 while the state stays f32.
+class Optimizer {
+public:
+    Optimizer(const Optimizer &) = delete;
+    Optimizer &operator=(const Optimizer &) = delete;
+    virtual ~Optimizer()
+    {
+        if (h_) nbo_optim_destroy(h_);
+    }
+
+    // optim/core.rs:10: panics (throws Panic) on length or shape mismatch
+    void step(TensorList &params, TensorList &grads) { check(nbo_optim_step(handle(), params.handle(), grads.handle())); }
+    void step(const std::vector<Tensor> &params, const std::vector<Tensor> &grads)
+    {
+        TensorList p(params), g(grads);
+        step(p, g);
+    }
+    void reset() { check(nbo_optim_reset(handle())); }
+    void set_lr(double lr)
+    {
+        meta_.lr = lr;
+        if (h_) check(nbo_optim_set_lr(h_, lr));
+    }
+    double lr() const { return meta_.lr; }
+    uint64_t step_count() { return meta().step_count; }
+
+    // the Trainer tail (trainer.rs:230-291) in one asynchronous call
+    void fused_step(TensorList &params, TensorList &grads, GradScaler *scaler, double max_norm,
+                    bool zero_grads = false)
+    {
+        check(nbo_fused_step(handle(), scaler ? scaler->handle() : nullptr, params.handle(), grads.handle(),
+                             max_norm, zero_grads ? NBO_STEP_ZERO_GRADS : 0u));
+    }
+    nbo_step_info last_step()
+    {
+        nbo_step_info info;
+        check(nbo_optim_last_step(handle(), &info));
+        return info;
+    }
+
+    OptimKind kind() const { return (OptimKind)meta_.kind; }
+    OptimMeta meta()
+    {
+        nbo_meta m = meta_;
+        if (h_) check(nbo_optim_get_meta(h_, &m));
+        else if (meta_.kind == NBO_KIND_SGD) m.beta1 = m.beta2 = m.eps = 0.0, m.step_count = 0;
+        return {(OptimKind)m.kind, m.lr, m.beta1, m.beta2, m.eps, m.weight_decay, m.momentum, m.step_count};
+    }
+    // alg.rs:531-545: Err("optim kind mismatch") -> StateError
+    void load_meta(const OptimMeta &m)
+    {
+        const nbo_meta c = {(int32_t)m.kind, 0, m.lr, m.beta1, m.beta2, m.eps, m.weight_decay, m.momentum,
+                            m.step_count};
+        check(nbo_optim_load_meta(handle(), &c));
+        meta_.lr = m.lr;
+    }
+    // one state tensor ("m3", "v3", "w3"); buffers hold rows*cols elements of the state type
+    void state_read(const std::string &name, void *buf, uint64_t n, bool on_device)
+    {
+        check(nbo_optim_state_read(handle(), name.c_str(), buf, n, on_device ? 1 : 0));
+    }
+    void state_write(const std::string &name, const void *buf, uint64_t n, bool on_device)
+    {
+        check(nbo_optim_state_write(handle(), name.c_str(), buf, n, on_device ? 1 : 0));
+    }
+    void master_from_params(TensorList &params_bf16) { check(nbo_optim_master_from_params(handle(), params_bf16.handle())); }
+
+    nbo_optim *handle()
+    {
+        if (!h_) {
+            std::vector<uint64_t> rows, cols;
+            for (const auto &s : shapes_) {
+                rows.push_back(s.first);
+                cols.push_back(s.second);
+            }
+            check(nbo_optim_create(&meta_, shapes_.size(), rows.data(), cols.data(), state_dtype_,
+                                   master_ ? 1 : 0, &h_));
+        }
+        return h_;
+    }
+
+protected:
+    Optimizer(nbo_kind kind, double lr, std::vector<std::pair<uint64_t, uint64_t>> shapes, nbo_dtype state_dtype,
+              bool master)
+        : shapes_(std::move(shapes)), state_dtype_(state_dtype), master_(master)
+    {
+        meta_ = nbo_meta{(int32_t)kind, 0, lr, 0.0, 0.0, 0.0, 0.0, 0.0, 0};
+    }
+    void builder_guard() const
+    {
+        if (h_) throw RuntimeError(NBO_ERR_ARG, "builder setters apply before the first use");
+    }
+    nbo_meta meta_;
+
+private:
+    std::vector<std::pair<uint64_t, uint64_t>> shapes_;
+    nbo_dtype state_dtype_;
+    bool master_;
+    nbo_optim *h_ = nullptr;
+};
+
+using Shapes = std::vector<std::pair<uint64_t, uint64_t>>;
+
+// alg.rs:310-428
+class Sgd : public Optimizer {
+public:
+    Sgd(double lr, Shapes shapes, nbo_dtype state_dtype = NBO_DT_F32, bool master = false)
+        : Optimizer(NBO_KIND_SGD, lr, std::move(shapes), state_dtype, master)
+    {
+    }
+    Sgd &momentum(double m) { builder_guard(); meta_.momentum = m; return *this; }
+    Sgd &weight_decay(double wd) { builder_guard(); meta_.weight_decay = wd; return *this; }
+    double momentum_value() const { return meta_.momentum; }
+    double weight_decay_value() const { return meta_.weight_decay; }
+};
+
+// alg.rs:169-308
+class Adam : public Optimizer {
+public:
+    Adam(double lr, Shapes shapes, nbo_dtype state_dtype = NBO_DT_F32, bool master = false)
+        : Optimizer(NBO_KIND_ADAM, lr, std::move(shapes), state_dtype, master)
+    {
+        meta_.beta1 = 0.9, meta_.beta2 = 0.999, meta_.eps = 1e-8;
+    }
+    Adam &beta1(double b) { builder_guard(); meta_.beta1 = b; return *this; }
+    Adam &beta2(double b) { builder_guard(); meta_.beta2 = b; return *this; }
+    Adam &eps(double e) { builder_guard(); meta_.eps = e; return *this; }
+};
+
+// alg.rs:7-167
+class AdamW : public Optimizer {
+public:
+    AdamW(double lr, Shapes shapes, nbo_dtype state_dtype = NBO_DT_F32, bool master = false)
+        : Optimizer(NBO_KIND_ADAMW, lr, std::move(shapes), state_dtype, master)
+    {
+        meta_.beta1 = 0.9, meta_.beta2 = 0.999, meta_.eps = 1e-8, meta_.weight_decay = 0.01;
+    }
+    AdamW &beta1(double b) { builder_guard(); meta_.beta1 = b; return *this; }
+    AdamW &beta2(double b) { builder_guard(); meta_.beta2 = b; return *this; }
+    AdamW &eps(double e) { builder_guard(); meta_.eps = e; return *this; }
+    AdamW &weight_decay(double wd) { builder_guard(); meta_.weight_decay = wd; return *this; }
+};
+
+// nabla-train/src/trainer.rs:500-523; returns the pre-clip norm
+inline double clip_grad_norm(TensorList &grads, double max_norm)
+{
+    double norm = 0.0;
+    check(nbo_clip_grad_norm(grads.handle(), max_norm, &norm));
+    return norm;
+}
+// nabla-ml/src/autograd/ops.rs:1668-1680
+inline void zero_grad(TensorList &grads) { check(nbo_zero_grad(grads.handle())); }
+inline void scale_grad(TensorList &grads, double factor) { check(nbo_scale_grad(grads.handle(), factor)); }
+inline void sync() { check(nbo_sync()); }
+
+} // namespace optim
+} // namespace nabla
+
+#endif

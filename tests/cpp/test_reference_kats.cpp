@@ -1,0 +1,193 @@
+// The reference's own tests for the optimizer step (nabla-train/tests/optim.rs:47-138,
+// nabla-train/tests/trainer.rs:171-203), replayed through the C++ mirror of its
+// interface (include/nabla_optim.hpp) on the device: f64, 1x1 tensors, the same
+// values and the same assertions.  Exit code 0 = all passed.
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <limits>
+#include <string>
+#include <vector>
+
+#include "../../include/nabla_optim.hpp"
+
+using namespace nabla::optim;
+
+static int failures = 0;
+#define EXPECT(cond)                                                                   \
+    do {                                                                               \
+        if (!(cond)) {                                                                 \
+            std::printf("  FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);            \
+            failures++;                                                                \
+        }                                                                              \
+    } while (0)
+
+// mat![[v]] on the device
+struct Mat {
+    double *d = nullptr;
+    uint64_t n;
+    explicit Mat(std::vector<double> v) : n(v.size())
+    {
+        if (hipMalloc((void **)&d, n * sizeof(double)) != hipSuccess) std::abort();
+        if (hipMemcpy(d, v.data(), n * sizeof(double), hipMemcpyHostToDevice) != hipSuccess) std::abort();
+    }
+    ~Mat() { (void)hipFree(d); }
+    Tensor tensor() const { return Tensor{d, 1, n, NBO_DT_F64}; }
+    double get(uint64_t i = 0) const
+    {
+        sync();
+        double x;
+        if (hipMemcpy(&x, d + i, sizeof(double), hipMemcpyDeviceToHost) != hipSuccess) std::abort();
+        return x;
+    }
+};
+
+static void sgd_step_updates_param()  // optim.rs:47-57
+{
+    Mat param({1.0}), grad({1.0});
+    Sgd opt(0.1, {{1, 1}}, NBO_DT_F64);
+    opt.step({param.tensor()}, {grad.tensor()});
+    EXPECT(std::fabs(param.get() - 0.9) < 1e-10);
+}
+
+static void adam_step_updates_param()  // optim.rs:59-69
+{
+    Mat param({1.0}), grad({1.0});
+    Adam opt(0.1, {{1, 1}}, NBO_DT_F64);
+    opt.step({param.tensor()}, {grad.tensor()});
+    EXPECT(param.get() < 1.0);
+    EXPECT(std::fabs(param.get() - 0.9) < 1e-7);  // step 1 from m = v = 0 is sign-SGD
+    EXPECT(opt.step_count() == 1);
+}
+
+static void adamw_step_updates_param()  // optim.rs:71-81
+{
+    Mat param({1.0}), grad({1.0});
+    AdamW opt(0.1, {{1, 1}}, NBO_DT_F64);
+    opt.step({param.tensor()}, {grad.tensor()});
+    EXPECT(param.get() < 1.0);
+    EXPECT(std::fabs(param.get() - 0.899) < 1e-7);  // default weight_decay 0.01
+}
+
+static void grad_scaler_unscale()  // optim.rs:120-128
+{
+    GradScaler scaler;
+    Mat g({2.0});
+    TensorList grads({g.tensor()});
+    EXPECT(scaler.unscale_and_update(grads));
+    EXPECT(g.get() < 2.0);
+    EXPECT(g.get() == 2.0 / 65536.0);
+}
+
+static void grad_scaler_detects_inf()  // optim.rs:130-138
+{
+    GradScaler scaler;
+    Mat g({std::numeric_limits<double>::infinity()});
+    TensorList grads({g.tensor()});
+    EXPECT(!scaler.unscale_and_update(grads));
+    EXPECT(std::fabs(g.get()) < 1e-12);
+    EXPECT(scaler.scale_factor() == 32768.0);
+    EXPECT(scaler.state().consecutive_ok == 0);
+}
+
+static void clip_grad_norm_scales()  // trainer.rs:171-203
+{
+    Mat a({3.0}), b({4.0});
+    TensorList grads({a.tensor(), b.tensor()});
+    const double reported = clip_grad_norm(grads, 2.5);
+    const double after = std::sqrt(a.get() * a.get() + b.get() * b.get());
+    EXPECT(std::fabs(reported - 5.0) < 1e-10);
+    EXPECT(std::fabs(after - 2.5) < 1e-10);
+    EXPECT(clip_grad_norm(grads, 0.0) == 0.0);  // trainer.rs:501-503
+}
+
+static void weight_decay_exclusion()  // optim.rs:140-165, the two groups as two optimizers
+{
+    Mat weight({2.0}), bias({3.0}), zero({0.0});
+    Sgd decay(1.0, {{1, 1}}, NBO_DT_F64), no_decay(1.0, {{1, 1}}, NBO_DT_F64);
+    decay.weight_decay(0.1);
+    decay.step({weight.tensor()}, {zero.tensor()});
+    no_decay.step({bias.tensor()}, {zero.tensor()});
+    EXPECT(std::fabs(weight.get() - 1.8) < 1e-10);
+    EXPECT(std::fabs(bias.get() - 3.0) < 1e-10);
+}
+
+static void panics_and_errors()  // alg.rs:110-119, 531-545; tensor/ops.rs:638-646
+{
+    Mat p({1.0}), g({1.0}), g2({1.0, 2.0});
+    AdamW opt(0.1, {{1, 1}}, NBO_DT_F64);
+    std::string what;
+    try {
+        opt.step({p.tensor()}, {g.tensor(), g.tensor()});
+    } catch (const Panic &e) {
+        what = e.what();
+    }
+    EXPECT(what == "nabla-train: AdamW params/grads length mismatch");
+    what.clear();
+    try {
+        opt.step({p.tensor(), p.tensor()}, {g.tensor(), g.tensor()});
+    } catch (const Panic &e) {
+        what = e.what();
+    }
+    EXPECT(what == "nabla-train: AdamW params count mismatch");
+    what.clear();
+    try {
+        opt.step({p.tensor()}, {g2.tensor()});
+    } catch (const Panic &e) {
+        what = e.what();
+    }
+    EXPECT(what.find("shapes must match") != std::string::npos);
+    what.clear();
+    try {
+        opt.load_meta(OptimMeta{OptimKind::Sgd, 0.1, 0, 0, 0, 0, 0, 0});
+    } catch (const StateError &e) {
+        what = e.what();
+    }
+    EXPECT(what == "optim kind mismatch");
+    what.clear();
+    double buf = 0;
+    try {
+        opt.state_read("m7", &buf, 1, false);
+    } catch (const StateError &e) {
+        what = e.what();
+    }
+    EXPECT(what == "m index out of range: 7");
+    what.clear();
+    try {
+        opt.state_read("mx", &buf, 1, false);
+    } catch (const StateError &e) {
+        what = e.what();
+    }
+    EXPECT(what == "bad tensor key: mx");
+    EXPECT(p.get() == 1.0);  // nothing ran
+}
+
+int main()
+{
+    struct {
+        const char *name;
+        void (*fn)();
+    } tests[] = {{"sgd_step_updates_param", sgd_step_updates_param},
+                 {"adam_step_updates_param", adam_step_updates_param},
+                 {"adamw_step_updates_param", adamw_step_updates_param},
+                 {"grad_scaler_unscale", grad_scaler_unscale},
+                 {"grad_scaler_detects_inf", grad_scaler_detects_inf},
+                 {"clip_grad_norm_scales", clip_grad_norm_scales},
+                 {"group_optimizer_weight_decay_exclusion", weight_decay_exclusion},
+                 {"panics_and_errors", panics_and_errors}};
+    try {
+        check(nbo_init());
+        for (auto &t : tests) {
+            const int before = failures;
+            t.fn();
+            std::printf("%s %s\n", failures == before ? "ok    " : "FAILED", t.name);
+        }
+    } catch (const std::exception &e) {
+        std::printf("unexpected exception: %s\n", e.what());
+        return 2;
+    }
+    std::printf("%d failure(s)\n", failures);
+    return failures ? 1 : 0;
+}
