@@ -154,8 +154,10 @@ void Runtime::launch_copy(const void *src, void *dst, uint64_t nvec)
 
 double Runtime::probe_pair_gbps(void *a, void *b, size_t bytes)
 {
-    const uint64_t nvec = bytes / 16;
-    const uint32_t grid = (uint32_t)(nvec / 2048); // 8 rows of 256 vectors per workgroup
+    // each workgroup covers 8 rows of NBO_BLOCK 128-bit vectors of both buffers; a tail
+    // that does not fill a workgroup is left out, so nothing is touched past `bytes`
+    const uint64_t per_wg = 8ull * NBO_BLOCK;
+    const uint32_t grid = (uint32_t)(bytes / 16 / per_wg);
     if (grid == 0) return 0.0;
     void *args[2] = {(void *)&a, (void *)&b};
     hipEvent_t e0, e1;
@@ -174,7 +176,7 @@ double Runtime::probe_pair_gbps(void *a, void *b, size_t bytes)
     }
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
-    return best > 0.0f ? 4.0 * (double)grid * 2048 * 16 / best / 1e6 : 0.0;
+    return best > 0.0f ? 4.0 * (double)grid * (double)per_wg * 16 / best / 1e6 : 0.0;
 }
 
 void Runtime::read_back(void *host_dst, const void *dev_src, size_t bytes)

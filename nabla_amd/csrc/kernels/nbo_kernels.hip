@@ -766,23 +766,25 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_copy_f32x4(const f32
         __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
-// Placement probe: reads and rewrites the same 2048 vectors per workgroup of two
-// buffers together.  Two buffers in the same region of HBM run measurably slower than
-// two in different regions; the host times this to classify freshly created chunks
-// (their contents do not matter yet).
+// Placement probe: every workgroup reads and rewrites the same 8 rows of NBO_BLOCK
+// 128-bit vectors of two buffers together.  Two buffers in the same region of HBM run
+// measurably slower than two in different regions; the host times this to classify
+// freshly created chunks (their contents do not matter yet).  The host launches
+// bytes / (16 * 8 * NBO_BLOCK) workgroups of NBO_BLOCK threads, so every access stays
+// inside the two windows.
 extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_probe_rmw2(f32x4 *a, f32x4 *b)
 {
-    const uint64_t c0 = (uint64_t)blockIdx.x * 2048;
+    const uint64_t c0 = (uint64_t)blockIdx.x * (8 * NBO_BLOCK);
     f32x4 va[8], vb[8];
 #pragma unroll
     for (int u = 0; u < 8; u++) {
-        const uint64_t i = c0 + u * 256 + threadIdx.x;
+        const uint64_t i = c0 + u * NBO_BLOCK + threadIdx.x;
         va[u] = __builtin_nontemporal_load(a + i);
         vb[u] = __builtin_nontemporal_load(b + i);
     }
 #pragma unroll
     for (int u = 0; u < 8; u++) {
-        const uint64_t i = c0 + u * 256 + threadIdx.x;
+        const uint64_t i = c0 + u * NBO_BLOCK + threadIdx.x;
         __builtin_nontemporal_store(va[u] + 1.0f, a + i);
         __builtin_nontemporal_store(vb[u] + 1.0f, b + i);
     }
