@@ -417,12 +417,19 @@ int nbo_optim_step(nbo_optim *opt, nbo_list *params, nbo_list *grads)
     return guarded([&] {
         check_step_args(opt, params, grads);
         Runtime &rt = Runtime::get();
-        NboPrepArgs p = {};
-        p.opt = opt->dev;
-        p.gf = nullptr;
-        p.hyper = hyper_of(opt);
-        rt.launch(K_PREP, 1, 64, p);
-        const NboUpdateArgs a = update_args(opt, params, grads, false, false);
+        NboUpdateArgs a = update_args(opt, params, grads, false, false);
+        if (opt->meta.kind == NBO_KIND_SGD) {
+            // no step_count, no skip: one launch, scalars in the argument block
+            a.direct = 1;
+            a.sgd_lr = opt->meta.lr;
+            a.sgd_momentum = opt->meta.momentum;
+            a.sgd_weight_decay = opt->meta.weight_decay;
+        } else {
+            NboPrepArgs p = {};
+            p.opt = opt->dev;
+            p.hyper = hyper_of(opt);
+            rt.launch(K_PREP, 1, 64, p);
+        }
         rt.launch(update_kernel(opt, params), opt->layout.nchunks, NBO_BLOCK, a);
     });
 }

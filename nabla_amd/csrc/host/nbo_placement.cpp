@@ -16,6 +16,8 @@ constexpr size_t kMapGranule = (size_t)2 << 20;
 // Two buffers of 1-2 GiB read-modify-written together run at 5.0-5.9 TB/s when both
 // lie in the same 96 GiB region of MI355X's HBM and at 6.3-6.5 TB/s when they do not.
 constexpr double kSameRegionBelowGBps = 6100.0;
+// Below this size per part the step is too short for placement to matter.
+constexpr size_t kMinPlacedBytes = (size_t)128 << 20;
 
 size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
@@ -67,7 +69,7 @@ void StatePlacement::allocate(uint32_t nparts, size_t bytes, void **out)
     for (uint32_t k = 0; k < 3; k++) out[k] = nullptr;
     const char *env = std::getenv("NBO_STATE_SPREAD");
     const bool spread = !(env && env[0] == '0');
-    if (spread && nparts > 1 && bytes >= kGiB && try_placed(nparts, bytes, out)) return;
+    if (spread && nparts > 1 && bytes >= kMinPlacedBytes && try_placed(nparts, bytes, out)) return;
     Runtime &rt = Runtime::get();
     try {
         for (uint32_t k = 0; k < nparts; k++) {
@@ -85,8 +87,10 @@ bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
     Runtime &rt = Runtime::get();
     const size_t chunk = bytes >= 16 * kGiB ? 2 * kGiB : kGiB;
     const size_t window = chunk; // probe size: whole chunks against each other
-    const size_t full = bytes / chunk;
-    const size_t tail = round_up(bytes - full * chunk, kMapGranule);
+    // a part smaller than one chunk still gets a whole chunk of its own (regions can
+    // only be told apart at this granularity); larger parts are whole chunks plus a tail
+    const size_t full = bytes < chunk ? 1 : bytes / chunk;
+    const size_t tail = bytes < chunk ? 0 : round_up(bytes - full * chunk, kMapGranule);
     const size_t part_va = full * chunk + tail;
     const size_t total_full = full * nparts;
     size_t free_b = 0, total_b = 0;
@@ -140,13 +144,17 @@ bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
         }
         std::vector<std::vector<size_t>> region_chunks; // chunk indices per region
         std::vector<char *> region_rep;                 // one mapped chunk per region
-        const size_t need_each = (total_full + 2) / 3;
+        // Which regions the parts will use.  Three parts rotate over all three regions.
+        // Two parts use the two regions found last: the first region found is where this
+        // process's most recent allocations went, and the caller's parameters and
+        // gradients -- read and written in the same kernel -- are most likely there.
+        const size_t first_used = nparts == 2 ? 1 : 0;
+        const size_t need_each = (total_full + (3 - first_used) - 1) / (3 - first_used);
         auto enough = [&]() {
             if (region_chunks.size() < 3) return false;
-            std::vector<size_t> sizes;
-            for (const auto &r : region_chunks) sizes.push_back(r.size());
-            std::sort(sizes.rbegin(), sizes.rend());
-            return sizes[2] >= need_each;
+            for (size_t r = first_used; r < 3; r++)
+                if (region_chunks[r].size() < need_each) return false;
+            return true;
         };
         while (chunks.size() < budget && !enough()) {
             Chunk c = {};
@@ -197,17 +205,23 @@ bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
             for (const auto &r : region_chunks) std::fprintf(stderr, " %zu", r.size());
             std::fprintf(stderr, "; %zu needed\n", total_full);
         }
-        // regions by size, largest first; chunk i of part j prefers region (i + j) mod R
-        std::sort(region_chunks.begin(), region_chunks.end(),
-                  [](const std::vector<size_t> &a, const std::vector<size_t> &b) { return a.size() > b.size(); });
-        while (!region_chunks.empty() && region_chunks.back().empty()) region_chunks.pop_back();
+        // chunk i of part j prefers the ((i + j) mod U)-th of the U regions in use; when
+        // that one has run dry, whichever region still has most chunks
         const size_t R = region_chunks.size();
+        std::vector<size_t> use;
+        for (size_t r = (R == 3 ? first_used : 0); r < R; r++) use.push_back(r);
+        size_t in_use = 0;
+        for (size_t r : use) in_use += region_chunks[r].size();
+        if (in_use < total_full) { // not enough there: every region is fair game
+            use.clear();
+            for (size_t r = 0; r < R; r++) use.push_back(r);
+        }
         std::vector<std::vector<size_t>> pick(nparts);
         for (size_t i = 0; i < full; i++)
             for (uint32_t j = 0; j < nparts; j++) {
-                size_t r = (i + j) % R;
+                size_t r = use[(i + j) % use.size()];
                 if (region_chunks[r].empty())
-                    for (size_t q = 0; q < R; q++)
+                    for (size_t q : use)
                         if (region_chunks[q].size() > region_chunks[r].size()) r = q;
                 pick[j].push_back(region_chunks[r].back());
                 region_chunks[r].pop_back();
@@ -253,7 +267,7 @@ bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
             }
         }
         success = true;
-        regions_used_ = (int)R;
+        regions_used_ = (int)use.size();
         for (uint32_t j = 0; j < nparts; j++) {
             out[j] = part_ranges[j].va;
             ranges_.push_back({part_ranges[j].va, part_va});

@@ -25,12 +25,15 @@ namespace nbo {
 // created one at a time and each is classified by a pairwise bandwidth probe against
 // one representative chunk per region found so far -- two chunks of the same region
 // are measurably slower together than two of different regions.  Creation stops once
-// every region that can be reached holds a third of the chunks needed; chunk i of
-// part j then comes from region (i + j) mod R, so that at every position of the
-// update's walk the parts sit in different regions and each region serves an equal
-// share of the traffic.  Chunks that were created but not chosen are released again.
+// every region to be used holds its share of the chunks needed; chunk i of part j
+// then comes from the ((i + j) mod U)-th of the U regions in use, so that at every
+// position of the update's walk the parts sit in different regions and each region
+// serves an equal share of the traffic.  Three parts use all three regions; two parts
+// (Adam / AdamW without master weights) use the two regions found last and leave the
+// first to the caller's own tensors.  A part smaller than a chunk gets one whole chunk.
+// Chunks that were created but not chosen are released again.
 //
-// Small state (< 1 GiB per part), a single part, NBO_STATE_SPREAD=0, or any failure
+// Small state (< 128 MiB per part), a single part, NBO_STATE_SPREAD=0, or any failure
 // along the way fall back to plain hipMalloc.
 class StatePlacement {
 public:

@@ -185,6 +185,13 @@ template <> struct Scal<float> {
           use_mom(o->momentum != 0.0), use_wd(o->weight_decay != 0.0)
     {
     }
+    // Sgd::step's own narrowing (alg.rs:393-397)
+    __device__ Scal(double lr, double momentum, double weight_decay)
+        : b1(0), omb1(0), b2(0), omb2(0), eps(0), ss(0), ibc2(0), omw(0), neg_lr(-(float)lr),
+          mom((float)momentum), wd((float)weight_decay), inv(1.0f), clip(1.0f), use_mom(momentum != 0.0),
+          use_wd(weight_decay != 0.0)
+    {
+    }
 };
 template <> struct Scal<double> {
     double b1, omb1, b2, omb2, eps, ss, ibc2, omw, neg_lr, mom, wd, inv, clip;
@@ -194,6 +201,11 @@ template <> struct Scal<double> {
           ss(o->d_ss), ibc2(o->d_ibc2), omw(o->d_omw), neg_lr(o->d_neg_lr), mom(o->d_momentum),
           wd(o->d_wd), inv(f ? f->inv_scale64 : 1.0), clip(f ? f->clip64 : 1.0),
           use_mom(o->momentum != 0.0), use_wd(o->weight_decay != 0.0)
+    {
+    }
+    __device__ Scal(double lr, double momentum, double weight_decay)
+        : b1(0), omb1(0), b2(0), omb2(0), eps(0), ss(0), ibc2(0), omw(0), neg_lr(-lr), mom(momentum),
+          wd(weight_decay), inv(1.0), clip(1.0), use_mom(momentum != 0.0), use_wd(weight_decay != 0.0)
     {
     }
 };
@@ -296,14 +308,15 @@ template <int ST, int KIND> DEV void update_body(const NboUpdateArgs &a)
     const uint32_t vbytes = VEC * SB;
     const bool vec_ok = ((((uintptr_t)pp) | ((uintptr_t)pg)) & (vbytes - 1)) == 0;
 
-    if (a.opt->skip) {
+    const bool direct = KIND == NBO_SGD && a.direct != 0;
+    if (!direct && a.opt->skip) {
         // found_inf: parameters, moments and step_count stay untouched
         // (trainer.rs:230-236); the gradients become zeros (core.rs:372-375).
         if (zero_g)
             for (uint32_t i = tid; i < c.cnt; i += NBO_BLOCK) IO<ST>::st1(pg + (uint64_t)i * SB, (T)0);
         return;
     }
-    const Scal<T> s(a.opt, a.gf);
+    const Scal<T> s = direct ? Scal<T>(a.sgd_lr, a.sgd_momentum, a.sgd_weight_decay) : Scal<T>(a.opt, a.gf);
     const bool use_m = KIND != NBO_SGD || s.use_mom;
 
     if (c.cnt == NBO_CHUNK && vec_ok) {

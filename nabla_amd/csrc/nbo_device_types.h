@@ -123,7 +123,11 @@ struct NboUpdateArgs {
     const NboOptimDev *opt;
     const NboGradFactors *gf; // null: gradients are used as they are
     uint32_t zero_grads;      // write zeros over the gradients after reading them
-    uint32_t pad;
+    // SGD outside the fused tail needs no device-side state at all (it has no
+    // step_count and cannot be skipped): with `direct` set its three scalars come from
+    // here and `opt` is not read, which saves the scalar-preparation launch
+    uint32_t direct;
+    double sgd_lr, sgd_momentum, sgd_weight_decay;
 };
 
 struct NboNormArgs {
