@@ -19,7 +19,9 @@
 
 // The norm pass runs a fixed grid so that its per-block partial sums, and hence
 // the reduced norm, do not depend on anything but the tensor list itself.
+#ifndef NBO_NORM_GRID_MAX
 #define NBO_NORM_GRID_MAX 2048u
+#endif
 // Per-step trace ring kept on the device (found_inf / skipped / scale / step_count).
 #define NBO_TRACE_LEN 1024u
 

@@ -318,3 +318,72 @@ def test_unfused_scaler_clip_zero_in_place(gpu):
     nb.zero_grad(g_dev)
     for t in H.host_list(g_dev):
         assert not t.any()
+
+
+# ---- HIP graph capture -----------------------------------------------------------------------
+
+def test_fused_steps_replay_from_a_hip_graph(gpu):
+    """A fused step allocates nothing, reads nothing back and keeps step_count and the
+    scaler on the device, so a caller may capture it.  Two fused steps are captured once
+    and replayed three times, with eager steps in between; after every replay the state
+    is compared with the oracle stepping through the same sequence."""
+    import torch
+
+    from nabla_amd import _lib
+
+    shapes = [(5, 7), (1, 8200), (3, 1000)]
+    w0 = H.randn_list(shapes, 31, 0.02)
+    g_bits = [O.bf16_from_f32(a) for a in H.randn_list(shapes, 32, 1e-3 * 65536.0)]
+    p_dev = H.dev_list([O.bf16_from_f32(a) for a in w0], shapes)
+    g_dev = H.dev_list(g_bits, shapes)
+    opt = nb.AdamW.new(2e-4, shapes, master=True).beta2(0.95).weight_decay(0.1)
+    for i, a in enumerate(w0):
+        opt.write_state(f"w{i}", H.to_dev(a, shapes[i]))
+    scaler = nb.GradScaler.new()
+    scaler.load_state(nb.GradScalerState(65536.0, 2.0, 0.5, 3, 0))
+    plist, glist = nb.TensorList(p_dev), nb.TensorList(g_dev)
+
+    ref = dict(p=[O.bf16_from_f32(a) for a in w0], w=H.copy_list(w0), m=H.zeros_like_list(w0),
+               v=H.zeros_like_list(w0))
+    meta, s = O.adamw_meta(2e-4, 0.9, 0.95, 1e-8, 0.1), O.ScalerState(65536.0, 2.0, 0.5, 3, 0)
+
+    def oracle_steps(k):
+        O.set_pow_mode(O.POW_SQRT)
+        try:
+            for _ in range(k):
+                O.mixed_step(meta, s, 1.0, ref["p"], g_bits, ref["w"], ref["m"], ref["v"])
+        finally:
+            O.set_pow_mode(O.POW_LIBM)
+
+    def check(what):
+        assert opt.step_count() == meta.step_count, what
+        assert scaler.state().scale == s.scale and scaler.state().consecutive_ok == s.consecutive_ok, what
+        H.assert_bits_equal(H.host_list(p_dev), ref["p"], what + ": params")
+        H.assert_bits_equal(H.host_list(opt.moments()[1]), ref["v"], what + ": v")
+
+    stream = torch.cuda.Stream()
+    lib = _lib.load()
+    _lib.check(lib.nbo_set_stream(stream.cuda_stream))
+    try:
+        with torch.cuda.stream(stream):
+            opt.fused_step(plist, glist, scaler=scaler, max_norm=1.0)  # creates everything eagerly
+            stream.synchronize()
+            oracle_steps(1)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                opt.fused_step(plist, glist, scaler=scaler, max_norm=1.0)
+                opt.fused_step(plist, glist, scaler=scaler, max_norm=1.0)
+            stream.synchronize()
+            check("capture must not execute")
+            for replay in range(3):
+                graph.replay()
+                stream.synchronize()
+                oracle_steps(2)
+                check(f"replay {replay}")
+                opt.fused_step(plist, glist, scaler=scaler, max_norm=1.0)  # eager, between replays
+                stream.synchronize()
+                oracle_steps(1)
+                check(f"eager step after replay {replay}")
+    finally:
+        _lib.check(lib.nbo_set_stream(None))
+    assert meta.step_count == 10 and s.scale == 65536.0 * 8
