@@ -231,7 +231,8 @@ def measure(name, steps, warmup):
             traffic = json.load(f).get(f"{name}:{dom}")
 
     out = {
-        "metric": "AdamW step HBM GB/s (bf16-mixed, whole step: unscale+found_inf+clip+update)"
+        "metric": "AdamW step HBM GB/s (% of peak) + params/s, bf16-mixed, whole step "
+                  "(unscale + found_inf + clip + update)"
         if cfg["kind"] == "adamw" else f"{cfg['kind']} step HBM GB/s",
         "value": round(gbps, 1),
         "unit": "GB/s",
@@ -244,7 +245,8 @@ def measure(name, steps, warmup):
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16 params/grads, f32 master/m/v" if cfg["mixed"] else "f32",
+        "dtype": "f32",
+        "storage": "bf16 params/grads, f32 master/m/v" if cfg["mixed"] else "f32 params/grads/m/v",
         "data": "synthetic (random-init parameters and gradients of the named shapes, resident in HBM)",
         "config": {"workload": name, "tensors": len(shapes), "params": n,
                    "bytes_per_param_step": upd_b + nrm_b, "optimizer": cfg["kind"],

@@ -603,6 +603,23 @@ def scale_grad(grads, factor: float) -> None:
     _call(_lib.load().nbo_scale_grad(g._h, float(factor)))
 
 
+def adamw_step(param, grad, m, v, lr, beta1, beta2, eps, weight_decay, step: int) -> None:
+    """The free function `adamw_step` (alg.rs:431-469): one AdamW update of one tensor
+    with caller-held moments and the step number passed in.  `param`, `grad`, `m`, `v`
+    are device tensors of one dtype (f32 or f64); `param`, `m`, `v` are updated in place."""
+    import torch
+
+    dtype = {torch.float32: "f32", torch.float64: "f64"}[param.dtype]
+    opt = AdamW.new(lr, [_shape2(param)], dtype=dtype).beta1(beta1).beta2(beta2).eps(eps) \
+        .weight_decay(weight_decay)
+    opt._meta.step_count = int(step) - 1  # step() increments before use (alg.rs:120)
+    opt.write_state("m0", m)
+    opt.write_state("v0", v)
+    opt.step([param], [grad])
+    m.copy_(opt.read_state("m0").reshape(m.shape))
+    v.copy_(opt.read_state("v0").reshape(v.shape))
+
+
 def accumulate(accum, grads, zero_grads: bool = False) -> None:
     """buf[i] = &buf[i] + g (nabla-train/src/trainer.rs:262-266), optionally clearing g."""
     a = _free_cache.get("accum_a", accum)

@@ -387,3 +387,51 @@ def test_fused_steps_replay_from_a_hip_graph(gpu):
     finally:
         _lib.check(lib.nbo_set_stream(None))
     assert meta.step_count == 10 and s.scale == 65536.0 * 8
+
+
+def test_adamw_step_free_function(gpu):
+    """adamw_step (alg.rs:431-469): caller-held moments, step number passed in."""
+    shape = (3, 1001)
+    p0, g0 = H.randn_list([shape], 41, 0.02)[0], H.randn_list([shape], 42, 1e-3)[0]
+    m0, v0 = np.abs(H.randn_list([shape], 43, 1e-4)[0]), np.abs(H.randn_list([shape], 44, 1e-7)[0])
+    p, g, m, v = (H.to_dev(a, shape) for a in (p0, g0, m0, v0))
+    nb.adamw_step(p, g, m, v, 1e-3, 0.9, 0.999, 1e-8, 0.01, 5)
+    pr, mr, vr = p0.copy(), m0.copy(), v0.copy()
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        O.adamw_step_single(pr, g0, mr, vr, 1e-3, 0.9, 0.999, 1e-8, 0.01, 5)
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+    H.assert_bits_equal([H.to_host(p), H.to_host(m), H.to_host(v)], [pr, mr, vr], "adamw_step")
+
+
+def test_nan_policy_skip_without_scaler(gpu):
+    """GradNanPolicy::Skip (trainer.rs:239-245, tests/trainer.rs:148-169): a non-finite
+    gradient drops the step -- params, moments and step_count stay as they were -- and
+    a finite one afterwards steps normally."""
+    shapes = [(2, 3), (1, 5000)]
+    p0 = H.randn_list(shapes, 51, 0.05)
+    p = H.dev_list(p0, shapes)
+    bad = H.randn_list(shapes, 52, 1e-2)
+    bad[1][4321] = np.nan
+    good = H.randn_list(shapes, 53, 1e-2)
+    opt = nb.Adam.new(1e-3, shapes)
+    opt.fused_step(p, H.dev_list(bad, shapes), skip_nonfinite=True)
+    info = opt.last_step()
+    assert (info.found_inf, info.step_count) == (1, 0)
+    H.assert_bits_equal(H.host_list(p), p0, "params after a skipped step")
+    assert not any(t.any() for t in H.host_list(opt.moments()[0]))
+    opt.fused_step(p, H.dev_list(good, shapes), skip_nonfinite=True)
+    pr, m, v, meta = H.copy_list(p0), H.zeros_like_list(p0), H.zeros_like_list(p0), O.adam_meta(1e-3)
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        O.adam_step(meta, pr, good, m, v)
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+    assert opt.step_count() == 1
+    H.assert_bits_equal(H.host_list(p), pr, "params after the next, finite step")
+    # without the policy the reference steps on regardless (trainer.rs:249)
+    opt2 = nb.Adam.new(1e-3, shapes)
+    p2 = H.dev_list(p0, shapes)
+    opt2.fused_step(p2, H.dev_list(bad, shapes))
+    assert opt2.step_count() == 1 and np.isnan(H.to_host(p2[1])[4321])
