@@ -120,7 +120,10 @@ int nbo_list_destroy(nbo_list *list);
  * meta->step_count seeds step_count).  Moments are created zero-filled.
  * state_dtype: NBO_DT_F32 or NBO_DT_F64 -- the arithmetic type T.
  * keep_master != 0: additionally hold f32 master weights so that the caller's
- * parameters and gradients may be bf16 (T = f32). */
+ * parameters and gradients may be bf16 (T = f32).
+ * State of 128 MiB per array or more is assembled from physical chunks chosen so that
+ * the arrays lie in different regions of the HBM (nbo_optim_state_regions tells the
+ * outcome); that takes up to a few seconds here and nothing per step. */
 int nbo_optim_create(const nbo_meta *meta, uint64_t n_tensors, const uint64_t *rows,
                      const uint64_t *cols, int state_dtype, int keep_master, nbo_optim **out);
 int nbo_optim_destroy(nbo_optim *opt);
