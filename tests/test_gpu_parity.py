@@ -435,3 +435,63 @@ def test_nan_policy_skip_without_scaler(gpu):
     p2 = H.dev_list(p0, shapes)
     opt2.fused_step(p2, H.dev_list(bad, shapes))
     assert opt2.step_count() == 1 and np.isnan(H.to_host(p2[1])[4321])
+
+
+def test_reset_set_lr_and_load_meta(gpu):
+    """Optimizer::reset (alg.rs:152-162), set_lr (:164-166), OptimState::load_meta
+    (:531-545) and load_state_tensors (:487-516) against the oracle doing the same."""
+    shapes = [(1, 3), (2, 4500)]
+    p0 = H.randn_list(shapes, 61, 0.02)
+    grads = [H.randn_list(shapes, 62 + k, 1e-3) for k in range(6)]
+    p = H.dev_list(p0, shapes)
+    opt = nb.AdamW.new(1e-3, shapes).weight_decay(0.05)
+    pr, m, v = H.copy_list(p0), H.zeros_like_list(p0), H.zeros_like_list(p0)
+    meta = O.adamw_meta(1e-3, weight_decay=0.05)
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        for k in range(2):
+            opt.step(p, H.dev_list(grads[k], shapes))
+            O.adam_step(meta, pr, grads[k], m, v)
+        # set_lr takes effect with the next step (the schedule calls it every step)
+        opt.set_lr(5e-4)
+        meta.lr = 5e-4
+        opt.step(p, H.dev_list(grads[2], shapes))
+        O.adam_step(meta, pr, grads[2], m, v)
+        assert opt.lr() == 5e-4 and opt.meta().lr == 5e-4 and opt.step_count() == 3
+        H.assert_bits_equal(H.host_list(p), pr, "after set_lr")
+        # reset: moments to zero, step_count to zero, params and hyper-parameters stay
+        opt.reset()
+        assert opt.step_count() == 0 and opt.meta().lr == 5e-4
+        assert not any(t.any() for t in H.host_list(opt.moments()[0] + opt.moments()[1]))
+        m, v = H.zeros_like_list(p0), H.zeros_like_list(p0)
+        meta.step_count = 0
+        opt.step(p, H.dev_list(grads[3], shapes))
+        O.adam_step(meta, pr, grads[3], m, v)
+        H.assert_bits_equal(H.host_list(p), pr, "after reset")
+        # load_meta: every field of set_state (alg.rs:90-105), including step_count
+        opt.load_meta(nb.OptimMeta("adamw", 2e-3, 0.8, 0.9, 1e-6, 0.2, 0.0, 40))
+        meta = O.adamw_meta(2e-3, 0.8, 0.9, 1e-6, 0.2, step_count=40)
+        # load_state_tensors: replace the moments
+        m = [np.abs(a) for a in H.randn_list(shapes, 70, 1e-4)]
+        v = [np.abs(a) for a in H.randn_list(shapes, 71, 1e-8)]
+        opt.load_state_tensors([(f"m{i}", H.to_dev(a, shapes[i])) for i, a in enumerate(m)] +
+                               [(f"v{i}", H.to_dev(a, shapes[i])) for i, a in enumerate(v)] +
+                               [("ignored", None)])
+        opt.step(p, H.dev_list(grads[4], shapes))
+        O.adam_step(meta, pr, grads[4], m, v)
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+    assert opt.step_count() == 41 == meta.step_count
+    got = opt.meta()
+    assert (got.beta1, got.beta2, got.eps, got.weight_decay, got.lr) == (0.8, 0.9, 1e-6, 0.2, 2e-3)
+    H.assert_bits_equal(H.host_list(p), pr, "after load_meta + load_state_tensors")
+    H.assert_bits_equal(H.host_list(opt.moments()[0]), m, "m")
+    H.assert_bits_equal(H.host_list(opt.moments()[1]), v, "v")
+    with pytest.raises(nb.OptimStateError, match="optim kind mismatch"):
+        opt.load_meta(nb.OptimMeta("adam", 1e-3, 0.9, 0.999, 1e-8, 0.0, 0.0, 0))
+    with pytest.raises(nb.NablaPanic, match="AdamW params/grads length mismatch"):
+        opt.step(p, H.dev_list(grads[5], shapes)[:1])
+    with pytest.raises(nb.NablaPanic, match="AdamW params count mismatch"):
+        opt.step(p[:1], H.dev_list(grads[5], shapes)[:1])
+    with pytest.raises(nb.NablaPanic, match="shapes must match"):
+        opt.step(p, [H.dev_list(grads[5], shapes)[0], H.to_dev(grads[5][1][:100], (1, 100))])
