@@ -759,13 +759,22 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_cast_master(const Nb
 {
     const ChunkRef c = chunk_ref(a.L, blockIdx.x);
     float *aw = state_part<float>(a.arena, c, a.arena.part_w);
-    if (a.mode == 0) {
-        const uint16_t *src = (const uint16_t *)a.src_ptrs[c.t] + c.base;
-        for (uint32_t e = threadIdx.x; e < c.cnt; e += NBO_BLOCK) aw[e] = bf16_bits_to_f32(src[e]);
-    } else {
-        uint16_t *dst = (uint16_t *)a.dst_ptrs[c.t] + c.base;
-        for (uint32_t e = threadIdx.x; e < c.cnt; e += NBO_BLOCK)
-            dst[e] = (uint16_t)f32_to_bf16_bits(aw[e]);
+    char *pt = (char *)(a.mode == 0 ? a.src_ptrs[c.t] : a.dst_ptrs[c.t]) + c.base * 2;
+    // whole 4-element vectors while the caller's address allows, then single elements
+    const uint32_t nvec = (((uintptr_t)pt) & 7u) == 0 ? c.cnt / 4 : 0;
+    for (uint32_t q = threadIdx.x; q < nvec; q += NBO_BLOCK) {
+        float x[4];
+        if (a.mode == 0) {
+            IO<NBO_BF16>::ldv(pt + (uint64_t)q * 8, x);
+            st_state(aw + q * 4, x);
+        } else {
+            ld_state(aw + q * 4, x);
+            IO<NBO_BF16>::stv(pt + (uint64_t)q * 8, x);
+        }
+    }
+    for (uint32_t e = nvec * 4 + threadIdx.x; e < c.cnt; e += NBO_BLOCK) {
+        if (a.mode == 0) aw[e] = IO<NBO_BF16>::ld1(pt + (uint64_t)e * 2);
+        else IO<NBO_BF16>::st1(pt + (uint64_t)e * 2, aw[e]);
     }
 }
 

@@ -87,8 +87,11 @@ def _mixed_full(gpu, shapes, steps, seed):
         del w
     opt.params_from_master(params)
     ref_m, ref_v = H.zeros_like_list(ref_w), H.zeros_like_list(ref_w)
+    # second reference: the reference-faithful libm powf variant (2 ulp / 1 bf16 ulp bar)
+    lib_w, lib_m, lib_v = H.copy_list(ref_w), H.zeros_like_list(ref_w), H.zeros_like_list(ref_w)
     scaler = nb.GradScaler.new()
     meta = O.adamw_meta(lr, 0.9, 0.95, 1e-8, wd)
+    lib_meta = O.adamw_meta(lr, 0.9, 0.95, 1e-8, wd)
     inv = np.float32(1.0 / 65536.0)
     O.set_pow_mode(O.POW_SQRT)
     try:
@@ -111,6 +114,9 @@ def _mixed_full(gpu, shapes, steps, seed):
             c = np.float32(1.0 / info.norm)
             g32 = [(O.bf16_to_f32(_take(g, s[0] * s[1])) * inv) * c for g, s in zip(grads, shapes)]
             O.adam_step(meta, ref_w, g32, ref_m, ref_v)
+            O.set_pow_mode(O.POW_LIBM)
+            O.adam_step(lib_meta, lib_w, g32, lib_m, lib_v)
+            O.set_pow_mode(O.POW_SQRT)
             del grads
     finally:
         O.set_pow_mode(O.POW_LIBM)
@@ -123,6 +129,15 @@ def _mixed_full(gpu, shapes, steps, seed):
     del w
     H.assert_bits_equal(_take_list(params, shapes), [O.bf16_from_f32(a) for a in ref_w],
                         "bf16 param slices")
+    # against libm powf: moments identical, master within 2 ulp (or the cancellation
+    # bound |d| <= steps * 8 * lr * 2^-23), bf16 params within 1 ulp
+    H.assert_bits_equal(lib_m, ref_m, "m, libm variant")
+    H.assert_bits_equal(lib_v, ref_v, "v, libm variant")
+    for a, b in zip(ref_w, lib_w):
+        ulp = O.ulp_distance_f32(a, b)
+        absd = np.abs(a.astype(np.float64) - b.astype(np.float64))
+        assert not ((ulp > 2) & (absd > steps * 8 * lr * 2.0 ** -23)).any()
+    assert H.max_ulp_bf16([O.bf16_from_f32(a) for a in ref_w], [O.bf16_from_f32(a) for a in lib_w]) <= 1
     # idempotence of the narrowing: params == bf16(master) everywhere, checked on the device
     for i in range(0, n_t, 37):
         wi = opt.read_state(f"w{i}")
