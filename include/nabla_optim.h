@@ -47,7 +47,7 @@ typedef enum nbo_status {
     NBO_ERR_DTYPE = 7,          /* element types of the lists / optimizer do not fit */
     NBO_ERR_ARG = 8,            /* null pointer, zero-sized list, bad enum value */
     NBO_ERR_NO_MASTER = 9,      /* bf16 step before master weights were set */
-    NBO_ERR_TOO_LARGE = 10,     /* more than 2^32-1 work chunks */
+    NBO_ERR_TOO_LARGE = 10,     /* more than 2^24-1 chunks of 8192 elements (1.4e11 elements) */
     NBO_ERR_NO_DEVICE = 11,     /* no gfx950 device / code object not loadable */
     NBO_ERR_HIP = 1000          /* NBO_ERR_HIP + hipError_t */
 } nbo_status;

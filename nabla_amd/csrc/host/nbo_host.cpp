@@ -246,8 +246,9 @@ void Layout::build(uint64_t nt, const uint64_t *r, const uint64_t *c, bool with_
         n[t] = rows[t] * cols[t];
         chunk_begin[t] = (uint32_t)chunks;
         chunks += (n[t] + NBO_CHUNK - 1) / NBO_CHUNK;
-        if (chunks > 0xFFFFFFFFull)
-            fail(NBO_ERR_TOO_LARGE, "tensor list has more than 2^32-1 work chunks");
+        // one workgroup per chunk: the launch's total thread count has to stay below 2^32
+        if (chunks * NBO_BLOCK > 0xFFFFFFFFull)
+            fail(NBO_ERR_TOO_LARGE, "tensor list too large for one launch (more than 2^32 threads)");
         // every tensor is padded to whole chunks, so a chunk never straddles two
         // state tiles
         soff[t] = off;
