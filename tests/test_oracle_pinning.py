@@ -492,3 +492,69 @@ def test_found_inf_leaves_everything_but_the_scaler_untouched():
     assert s.scale == 32768.0 and s.consecutive_ok == 0
     for a, b in zip(before, master + m + v + p):
         assert np.array_equal(a, b)
+
+
+def test_mixed_step_composition_in_exact_arithmetic():
+    """The Trainer tail for bf16 params / grads with f32 master (cast -> unscale -> clip ->
+    AdamW -> cast, trainer.rs:230-283) evaluated in exact rationals with a rounding after
+    every reference operation: pins the order of the stages (the norm is taken of the
+    unscaled gradients, the clip factor multiplies after the unscale factor, params are
+    the RNE narrowing of the updated master)."""
+    rng = np.random.default_rng(11)
+    sizes = [3, 4]
+    lr, b1, b2, eps, wd, max_norm, scale = 1e-3, 0.9, 0.95, 1e-8, 0.1, 0.5, 3.0
+    master = [(rng.standard_normal(n) * 0.02).astype(np.float32) for n in sizes]
+    p_bits = [O.bf16_from_f32(a) for a in master]
+    m = [np.zeros(n, np.float32) for n in sizes]
+    v = [np.zeros(n, np.float32) for n in sizes]
+    meta, s = O.adamw_meta(lr, b1, b2, eps, wd), O.ScalerState(scale, 2.0, 0.5, 2000, 0)
+    we = [[f32_exact(x) for x in a] for a in master]
+    me = [[Fraction(0)] * n for n in sizes]
+    ve = [[Fraction(0)] * n for n in sizes]
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        for t in (1, 2):
+            g_bits = [O.bf16_from_f32((rng.standard_normal(n) * 2.0).astype(np.float32)) for n in sizes]
+            ran, norm = O.mixed_step(meta, s, max_norm, p_bits, g_bits, master, m, v)
+            assert ran
+            # exact: g32 = widen(bf16) ; g = r32(g32 * r32(1/scale)) ; norm over all in list order
+            inv = r32(r64(Fraction(1) / Fraction(scale)))
+            ge = [[r32(Fraction(float(x)) * inv) for x in O.bf16_to_f32(gb)] for gb in g_bits]
+            acc = Fraction(0)
+            for t_ in ge:
+                for x in t_:
+                    acc = r64(acc + r64(x * x))
+            assert norm == math.sqrt(float(acc)) and norm > max_norm
+            c = r32(r64(Fraction(max_norm) / Fraction(norm)))
+            ge = [[r32(x * c) for x in t_] for t_ in ge]
+            # AdamW on the master in exact arithmetic (same chain as _exact_adam, step t)
+            def powi(a, n):
+                r, a = Fraction(1), Fraction(a)
+                while True:
+                    if n & 1:
+                        r = r64(r * a)
+                    n >>= 1
+                    if n == 0:
+                        return r
+                    a = r64(a * a)
+            bc1, bc2 = r64(1 - powi(b1, t)), r64(1 - powi(b2, t))
+            ss, ibc2 = r32(r64(Fraction(lr) / bc1)), r32(r64(1 / bc2))
+            fb1, fomb1, fb2, fomb2 = r32(b1), r32(r64(1 - Fraction(b1))), r32(b2), r32(r64(1 - Fraction(b2)))
+            omw = r32(1 - r32(r64(Fraction(wd) * Fraction(lr))))
+            for k in range(len(sizes)):
+                for i in range(sizes[k]):
+                    g = ge[k][i]
+                    me[k][i] = r32(r32(me[k][i] * fb1) + r32(fomb1 * g))
+                    ve[k][i] = r32(r32(ve[k][i] * fb2) + r32(fomb2 * r32(g * g)))
+                    denom = r32(sqrt_r32(r32(ve[k][i] * ibc2)) + r32(eps))
+                    upd = r32(r32(me[k][i] * ss) / denom)
+                    we[k][i] = r32(r32(we[k][i] * omw) + (-upd))
+            for k in range(len(sizes)):
+                for i in range(sizes[k]):
+                    assert f32_exact(master[k][i]) == we[k][i] and f32_exact(m[k][i]) == me[k][i]
+                    assert f32_exact(v[k][i]) == ve[k][i]
+                    # param = RNE narrowing of the master to 8 significand bits
+                    assert Fraction(float(O.bf16_to_f32(p_bits[k][i:i + 1])[0])) == rne(we[k][i], 8, -133)
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+    assert meta.step_count == 2 and s.consecutive_ok == 2 and s.scale == scale
