@@ -32,6 +32,9 @@ def parse_args():
     ap.add_argument("--workload", default="llama3-8b",
                     choices=["llama3-8b", "llama-1.1b", "gpt2-small-f32", "mlp-sgd-f32", "ragged-4096"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--zero-grads", choices=["off", "fused", "separate"], default="off",
+                    help="also clear the gradients every step (trainer.rs:285-290): inside the update "
+                         "kernel, or as a separate pass; +2 B/param of writes, reported in the config")
     ap.add_argument("--primary-only", action="store_true",
                     help="with the default workload, skip the additional llama-1.1b measurement")
     ap.add_argument("--calibrate-copy", type=float, default=0.0, metavar="GiB",
@@ -137,7 +140,7 @@ def cpu_baseline(cfg, budget_s):
     }
 
 
-def measure(name, steps, warmup):
+def measure(name, steps, warmup, zero_grads="off"):
     """Builds the workload on the device, runs `warmup` + `steps` steps, returns the
     result record (without the CPU baseline)."""
     import ctypes as C
@@ -183,11 +186,14 @@ def measure(name, steps, warmup):
 
     def step():
         if fused:
-            opt.fused_step(plist, glist, scaler=scaler, max_norm=cfg["clip"])
+            opt.fused_step(plist, glist, scaler=scaler, max_norm=cfg["clip"], zero_grads=zero_grads == "fused")
         else:
             opt.step(plist, glist)
+        if zero_grads == "separate" or (zero_grads == "fused" and not fused):
+            nb.zero_grad(glist)
 
     upd_b, nrm_b = bytes_per_param(cfg)
+    zero_b = 0 if zero_grads == "off" else (2 if cfg["mixed"] else 4)
     dom = f"nbo_update_{'bf16' if cfg['mixed'] else 'f32'}_{cfg['kind']}"
     names = [dom] + ([f"nbo_norm_{'bf16' if cfg['mixed'] else 'f32'}", "nbo_finalize"] if fused
                      else ([] if cfg["kind"] == "sgd" else ["nbo_prep"]))
@@ -219,9 +225,10 @@ def measure(name, steps, warmup):
     _lib.check(L.nbo_profile_enable(0))
 
     ms_step = (t1 - t0) / steps * 1e3
-    gbps = n * (upd_b + nrm_b) / (ms_step * 1e-3) / 1e9
+    gbps = n * (upd_b + nrm_b + zero_b) / (ms_step * 1e-3) / 1e9
     dom_ms = per_kernel[dom][1] / max(per_kernel[dom][0], 1)
-    dom_gbps = n * upd_b / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
+    dom_b = upd_b + (zero_b if zero_grads == "fused" and fused else 0)  # fused zeroing: the update kernel writes g too
+    dom_gbps = n * dom_b / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
     info = opt.last_step() if fused else None
 
     traffic = None
@@ -249,7 +256,8 @@ def measure(name, steps, warmup):
         "storage": "bf16 params/grads, f32 master/m/v" if cfg["mixed"] else "f32 params/grads/m/v",
         "data": "synthetic (random-init parameters and gradients of the named shapes, resident in HBM)",
         "config": {"workload": name, "tensors": len(shapes), "params": n,
-                   "bytes_per_param_step": upd_b + nrm_b, "optimizer": cfg["kind"],
+                   "bytes_per_param_step": upd_b + nrm_b + zero_b, "zero_grads": zero_grads,
+                   "optimizer": cfg["kind"],
                    "loss_scale": scale if cfg["scaler"] else None, "clip_max_norm": cfg["clip"] or None,
                    "state_hbm_regions": opt.state_regions()},
         "roofline": {
@@ -260,7 +268,7 @@ def measure(name, steps, warmup):
             "unit": "GB/s",
             "frac": round(dom_gbps / HBM_PEAK_GBPS, 4),
             "traffic": traffic,
-            "algorithmic_bytes_per_launch": n * upd_b,
+            "algorithmic_bytes_per_launch": n * dom_b,
             "avg_launch_ms": round(dom_ms, 4),
             "launches": per_kernel[dom][0],
         },
@@ -307,7 +315,7 @@ def main():
                           "launches": cnt.value, "avg_launch_ms": round(ms.value / max(cnt.value, 1), 4),
                           "GBps": round(2 * nbytes / (ms.value / max(cnt.value, 1)) / 1e6, 1)}))
         return
-    out, cfg = measure(args.workload, args.steps, args.warmup)
+    out, cfg = measure(args.workload, args.steps, args.warmup, args.zero_grads)
     if args.workload == "llama3-8b" and not args.primary_only:
         # the metric is quoted on the 1.1B and the 8B shapes: the smaller one rides along
         small, _ = measure("llama-1.1b", 10, 2)
