@@ -1,6 +1,7 @@
 // extern "C" entry points of include/nabla_optim.h.
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 
 #include "nbo_host.hpp"
@@ -9,9 +10,15 @@ using namespace nbo;
 
 namespace {
 
+// The runtime's stream, staging buffer and reduction scratch are shared by every
+// handle, so entry points run one at a time; the device work they enqueue is ordered
+// by the one stream.
+std::recursive_mutex g_api_mutex;
+
 // Runs `body`, mapping internal errors to status codes; nothing escapes the C ABI.
 template <typename F> int guarded(F &&body)
 {
+    std::lock_guard<std::recursive_mutex> lock(g_api_mutex);
     try {
         body();
         return NBO_OK;

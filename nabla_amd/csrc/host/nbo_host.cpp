@@ -36,7 +36,7 @@ static const char *const kKernelNames[K_COUNT] = {
     "nbo_scale_f32",         "nbo_scale_bf16",       "nbo_scale_f64",
     "nbo_prep",              "nbo_finalize",         "nbo_cast_master",
     "nbo_copy_f32x4",        "nbo_probe_rmw2",       "nbo_accum_f32",
-    "nbo_accum_bf16",        "nbo_accum_f64",
+    "nbo_accum_bf16",        "nbo_accum_f64",        "nbo_fill_zero",
 };
 
 Runtime &Runtime::get()
@@ -225,7 +225,13 @@ void Runtime::dfree(void *p)
 
 void Runtime::dzero(void *p, size_t bytes)
 {
-    if (bytes) hip_check(hipMemsetAsync(p, 0, bytes, stream_), "hipMemsetAsync");
+    if (bytes == 0) return;
+    NboFillArgs a = {p, bytes};
+    // eight 128-bit stores per thread for large ranges; the kernel strides over the rest
+    uint64_t grid = (bytes / 16 + 8ull * NBO_BLOCK - 1) / (8ull * NBO_BLOCK);
+    if (grid < 1) grid = 1;
+    if (grid > (1u << 20)) grid = 1u << 20;
+    launch(K_FILL_ZERO, (uint32_t)grid, NBO_BLOCK, a);
 }
 
 // ---------------------------------------------------------------------------------

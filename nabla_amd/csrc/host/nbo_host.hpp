@@ -1,6 +1,6 @@
 // Host runtime of the fused optimizer-step engine: internal classes behind the C ABI
 // of include/nabla_optim.h.  Device work goes through hipModuleLaunchKernel on
-// kernels of the embedded gfx950 code object and hipMemcpyAsync / hipMemsetAsync;
+// kernels of the embedded gfx950 code object and hipMemcpyAsync;
 // nothing here computes optimizer arithmetic on the host.
 #ifndef NBO_HOST_HPP
 #define NBO_HOST_HPP
@@ -38,7 +38,8 @@ enum KernelId {
     K_COPY = 18,
     K_PROBE = 19,
     K_ACCUM_BASE = 20, // + st
-    K_COUNT = 23
+    K_FILL_ZERO = 23,
+    K_COUNT = 24
 };
 
 // Process-wide runtime: device 0, the loaded module, the stream, scratch buffers.
@@ -65,7 +66,7 @@ public:
 
     void *dmalloc(size_t bytes);
     void dfree(void *p);
-    void dzero(void *p, size_t bytes); // asynchronous on the stream
+    void dzero(void *p, size_t bytes); // a fill kernel, asynchronous on the stream
 
     // Per-kernel timing with HIP events recorded on the launch stream, for the
     // benchmark's roofline figure.  Off by default.

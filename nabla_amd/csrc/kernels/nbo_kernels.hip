@@ -788,6 +788,26 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_copy_f32x4(const f32
         __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
+// Zero-fill of an arbitrary byte range: single bytes up to the first 16-byte boundary,
+// 128-bit stores for the body, single bytes for the rest.  Takes the place of
+// hipMemsetAsync so that everything the library enqueues is a kernel launch (a caller
+// may capture a reset or a step into a HIP graph).
+extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_fill_zero(const NboFillArgs a)
+{
+    char *p = (char *)a.p;
+    const uint64_t to_boundary = (16u - (uint32_t)((uintptr_t)p & 15u)) & 15u;
+    const uint64_t head = to_boundary < a.bytes ? to_boundary : a.bytes;
+    const uint64_t nvec = (a.bytes - head) / 16;
+    const uint64_t tail0 = head + nvec * 16;
+    const uint64_t gid = (uint64_t)blockIdx.x * NBO_BLOCK + threadIdx.x;
+    const uint64_t stride = (uint64_t)gridDim.x * NBO_BLOCK;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    for (uint64_t i = gid; i < nvec; i += stride)
+        __builtin_nontemporal_store(z, GLOBAL_PTR(u32x4, p + head) + i);
+    if (gid < head) p[gid] = 0;
+    if (gid < a.bytes - tail0) p[tail0 + gid] = 0;
+}
+
 // Placement probe: every workgroup reads and rewrites the same 8 rows of NBO_BLOCK
 // 128-bit vectors of two buffers together.  Two buffers in the same region of HBM run
 // measurably slower than two in different regions; the host times this to classify

@@ -191,4 +191,9 @@ struct NboCastArgs {
     uint32_t pad;
 };
 
+struct NboFillArgs {
+    void *p;
+    uint64_t bytes;
+};
+
 #endif

@@ -389,6 +389,71 @@ def test_fused_steps_replay_from_a_hip_graph(gpu):
     assert meta.step_count == 10 and s.scale == 65536.0 * 8
 
 
+def test_reset_and_steps_replay_from_a_hip_graph(gpu):
+    """Optimizer::reset clears the moments and step_count with a fill kernel (no memset
+    nodes), so it can sit in a captured graph with the steps that follow it.  The graph
+    [reset, step, step] is replayed twice with an eager step in between; the oracle does
+    the same sequence."""
+    import torch
+
+    from nabla_amd import _lib
+
+    shapes = [(3, 5), (1, 9000), (7, 11)]
+    p0 = H.randn_list(shapes, 81, 0.02)
+    g0 = H.randn_list(shapes, 82, 1e-3)
+    p_dev, g_dev = H.dev_list(p0, shapes), H.dev_list(g0, shapes)
+    plist, glist = nb.TensorList(p_dev), nb.TensorList(g_dev)
+    opt = nb.Adam.new(1e-3, shapes)
+    pr, m, v, meta = H.copy_list(p0), H.zeros_like_list(p0), H.zeros_like_list(p0), O.adam_meta(1e-3)
+
+    def oracle(reset, steps):
+        nonlocal m, v
+        if reset:
+            m, v = H.zeros_like_list(p0), H.zeros_like_list(p0)
+            meta.step_count = 0
+        O.set_pow_mode(O.POW_SQRT)
+        try:
+            for _ in range(steps):
+                O.adam_step(meta, pr, g0, m, v)
+        finally:
+            O.set_pow_mode(O.POW_LIBM)
+
+    def check(what):
+        assert opt.step_count() == meta.step_count, what
+        H.assert_bits_equal(H.host_list(p_dev), pr, what + ": params")
+        H.assert_bits_equal(H.host_list(opt.moments()[0]), m, what + ": m")
+        H.assert_bits_equal(H.host_list(opt.moments()[1]), v, what + ": v")
+
+    stream = torch.cuda.Stream()
+    lib = _lib.load()
+    _lib.check(lib.nbo_set_stream(stream.cuda_stream))
+    try:
+        with torch.cuda.stream(stream):
+            opt.step(plist, glist)
+            opt.step(plist, glist)
+            stream.synchronize()
+            oracle(False, 2)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                opt.reset()
+                opt.step(plist, glist)
+                opt.step(plist, glist)
+            stream.synchronize()
+            check("capture must not execute")
+            for replay in range(2):
+                graph.replay()
+                stream.synchronize()
+                oracle(True, 2)
+                check(f"replay {replay}")
+                opt.step(plist, glist)
+                stream.synchronize()
+                oracle(False, 1)
+                check(f"eager step after replay {replay}")
+    finally:
+        _lib.check(lib.nbo_set_stream(None))
+    assert meta.step_count == 3
+
+
 def test_adamw_step_free_function(gpu):
     """adamw_step (alg.rs:431-469): caller-held moments, step number passed in."""
     shape = (3, 1001)
