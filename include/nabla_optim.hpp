@@ -178,6 +178,26 @@ public:
         TensorList p(params), g(grads);
         step(p, g);
     }
+    // optim/core.rs:18-39.  `module.parameters_mut()` yields a std::vector<Tensor>; each
+    // variable's `grad()` yields a `const Tensor *`, null when backward has not run.
+    template <typename Module, typename Var> void step_with_vars(Module &module, const std::vector<Var> &param_vars)
+    {
+        const std::vector<Tensor> params = module.parameters_mut();
+        if (params.size() != param_vars.size())
+            throw Panic("nabla-train: step_with_vars param_vars length (" +
+                                                  std::to_string(param_vars.size()) +
+                                                  ") doesn't match module parameters count (" +
+                                                  std::to_string(params.size()) + ")");
+        std::vector<Tensor> grads;
+        for (size_t i = 0; i < param_vars.size(); i++) {
+            const Tensor *g = param_vars[i].grad();
+            if (!g)
+                throw Panic("nabla-train: step_with_vars: param_vars[" + std::to_string(i) +
+                                             "] has no gradient (call backward first)");
+            grads.push_back(*g);
+        }
+        step(params, grads);
+    }
     void reset() { check(nbo_optim_reset(handle())); }
     void set_lr(double lr)
     {

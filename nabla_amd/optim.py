@@ -292,6 +292,25 @@ class _Optimizer:
 
     step_slices = step
 
+    def step_with_vars(self, module, param_vars) -> None:
+        """optim/core.rs:18-39: parameters from `module.parameters_mut()`, gradients from
+        each variable's `grad()` (None, or an exception, means "no gradient")."""
+        params = list(module.parameters_mut())
+        if len(params) != len(param_vars):
+            raise NablaPanic(f"nabla-train: step_with_vars param_vars length ({len(param_vars)}) doesn't "
+                             f"match module parameters count ({len(params)})")
+        grads = []
+        for i, v in enumerate(param_vars):
+            try:
+                g = v.grad()
+            except Exception:
+                g = None
+            if g is None:
+                raise NablaPanic(f"nabla-train: step_with_vars: param_vars[{i}] has no gradient "
+                                 "(call backward first)")
+            grads.append(g)
+        self.step(params, grads)
+
     def reset(self) -> None:
         _call(_lib.load().nbo_optim_reset(self._handle()))
 

@@ -52,6 +52,39 @@ static void sgd_step_updates_param()  // optim.rs:47-57
     EXPECT(std::fabs(param.get() - 0.9) < 1e-10);
 }
 
+static void step_with_vars_pulls_params_and_grads()  // optim/core.rs:18-39 on the same values
+{
+    Mat param({1.0}), grad({1.0});
+    struct Module {
+        std::vector<Tensor> p;
+        std::vector<Tensor> parameters_mut() { return p; }
+    } module{{param.tensor()}};
+    struct Var {
+        Tensor g;
+        bool has;
+        const Tensor *grad() const { return has ? &g : nullptr; }
+    };
+    Sgd opt(0.1, {{1, 1}}, NBO_DT_F64);
+    opt.step_with_vars(module, std::vector<Var>{{grad.tensor(), true}});
+    EXPECT(std::fabs(param.get() - 0.9) < 1e-10);
+    bool panicked = false;
+    try {
+        opt.step_with_vars(module, std::vector<Var>{{grad.tensor(), false}});
+    } catch (const Panic &e) {
+        panicked = std::string(e.what()).find("param_vars[0] has no gradient (call backward first)") != std::string::npos;
+    }
+    EXPECT(panicked);
+    panicked = false;
+    try {
+        opt.step_with_vars(module, std::vector<Var>{});
+    } catch (const Panic &e) {
+        panicked = std::string(e.what()).find("param_vars length (0) doesn't match module parameters count (1)") !=
+                   std::string::npos;
+    }
+    EXPECT(panicked);
+    EXPECT(std::fabs(param.get() - 0.9) < 1e-10);
+}
+
 static void adam_step_updates_param()  // optim.rs:59-69
 {
     Mat param({1.0}), grad({1.0});
@@ -170,6 +203,7 @@ int main()
         const char *name;
         void (*fn)();
     } tests[] = {{"sgd_step_updates_param", sgd_step_updates_param},
+                 {"step_with_vars_pulls_params_and_grads", step_with_vars_pulls_params_and_grads},
                  {"adam_step_updates_param", adam_step_updates_param},
                  {"adamw_step_updates_param", adamw_step_updates_param},
                  {"grad_scaler_unscale", grad_scaler_unscale},

@@ -148,3 +148,30 @@ def test_meta_before_first_use_reports_constructor_defaults():
     g = nb.GradScaler.new().state()
     assert (g.scale, g.growth_factor, g.backoff_factor, g.growth_interval, g.consecutive_ok) == \
         (65536.0, 2.0, 0.5, 2000, 0)
+
+
+class _Module:
+    def __init__(self, params):
+        self._p = params
+
+    def parameters_mut(self):
+        return self._p
+
+
+class _Var:
+    def __init__(self, grad):
+        self._g = grad
+
+    def grad(self):
+        if self._g is None:
+            raise RuntimeError("no grad")
+        return self._g
+
+
+def test_step_with_vars_panics_like_the_reference():
+    """optim/core.rs:18-39: both asserts fire before anything reaches the device."""
+    opt = nb.Sgd.new(0.1, [(1, 1), (1, 1)])
+    with pytest.raises(nb.NablaPanic, match=r"param_vars length \(1\) doesn't match module parameters count \(2\)"):
+        opt.step_with_vars(_Module([object(), object()]), [_Var(object())])
+    with pytest.raises(nb.NablaPanic, match=r"param_vars\[1\] has no gradient \(call backward first\)"):
+        opt.step_with_vars(_Module([object(), object()]), [_Var(object()), _Var(None)])

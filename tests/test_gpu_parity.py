@@ -55,6 +55,30 @@ def test_sgd_mlp_100_steps_bit_exact(gpu):
     H.assert_bits_equal(H.host_list(p_dev), p_ref, "SGD params after 100 steps")
 
 
+def test_step_with_vars_takes_params_from_the_module_and_grads_from_the_variables(gpu):
+    """Optimizer::step_with_vars (optim/core.rs:18-39) on the reference's SGD known
+    answer (tests/optim.rs:47-57): p = 1, g = 1, lr = 0.1 gives 0.9."""
+    class Module:
+        def __init__(self, params):
+            self.params = params
+
+        def parameters_mut(self):
+            return self.params
+
+    class Var:
+        def __init__(self, grad):
+            self._grad = grad
+
+        def grad(self):
+            return self._grad
+
+    one = np.ones(1, dtype=np.float32)
+    module = Module([H.to_dev(one, (1, 1))])
+    nb.Sgd.new(0.1, [(1, 1)]).step_with_vars(module, [Var(H.to_dev(one, (1, 1)))])
+    assert H.to_host(module.params[0])[0] == np.float32(1.0) + np.float32(-0.1) * np.float32(1.0)
+    assert abs(float(H.to_host(module.params[0])[0]) - 0.9) < 1e-6
+
+
 @pytest.mark.parametrize("momentum,wd", [(0.9, 0.0), (0.0, 0.01), (0.9, 0.01)])
 def test_sgd_momentum_weight_decay_bit_exact(gpu, momentum, wd):
     shapes = RAGGED
