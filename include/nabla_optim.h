@@ -209,6 +209,35 @@ int nbo_fused_step_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *c
 /* Gradient accumulation of the Trainer, buf[i] = &buf[i] + g (trainer.rs:262-266),
  * optionally zeroing the gradients in the same pass.  Asynchronous. */
 int nbo_accumulate(nbo_list *accum, nbo_list *grads, int zero_grads);
+/* ---- Backend primitives on tensor lists ------------------------------------------------
+ * The single passes the reference's optimizers are chains of, as multi-tensor launches:
+ * BackendCore::{scale, axpy_inplace, add, zeros, clone_storage}
+ * (nabla-core/src/common/backend/mod.rs:82-216; CPU semantics nabla-core/src/cpu/mod.rs:137-139,
+ * 181, 211-232), BackendMath::{powf, emul, ediv} (backend/mod.rs:275-279; cpu/mod.rs:264-272) and
+ * Tensor::map(|x| x + s) (nabla-train/src/optim/alg.rs:133).  One IEEE operation per element
+ * in the lists' element type (bf16: the f32 operation, then bf16::from_f32,
+ * common/scalar/mod.rs:253-351); `s` is narrowed with T::from_f64.  All lists share shapes and
+ * element type; `out` may alias an operand.  powf with s = 0.5 is the correctly rounded
+ * square root, other exponents use the device math library (within 2 ulp of libm).  The
+ * generalisation of the reference's unused k_multi_axpy3 kernel
+ * (cuda_hip/common/kernels/k_ops.cuh:541-575) is NBO_BACKEND_AXPY.  Asynchronous. */
+typedef enum nbo_backend_op {
+    NBO_BACKEND_SCALE = 0,      /* out = a * s */
+    NBO_BACKEND_AXPY = 1,       /* out = out + s * a   (product and sum each rounded) */
+    NBO_BACKEND_ADD = 2,        /* out = a + b */
+    NBO_BACKEND_EMUL = 3,       /* out = a * b */
+    NBO_BACKEND_EDIV = 4,       /* out = a / b */
+    NBO_BACKEND_POWF = 5,       /* out = powf(a, s) */
+    NBO_BACKEND_ADD_SCALAR = 6, /* out = a + s */
+    NBO_BACKEND_ZEROS = 7,      /* out = 0             (a, b unused) */
+    NBO_BACKEND_CLONE = 8       /* out = a */
+} nbo_backend_op;
+int nbo_backend_apply(int op, nbo_list *out, nbo_list *a, nbo_list *b, double s);
+/* BackendCore::cast, default implementation (backend/mod.rs:157-160): dst = U::from_f64(
+ * src.to_f64()) per element, between any two of f32 / bf16 / f64 (f64 -> bf16 rounds to f32
+ * first, as bf16::from_f64 does).  Asynchronous. */
+int nbo_backend_cast(nbo_list *dst, nbo_list *src);
+
 /* Outcome of the optimizer's most recent fused step.  Synchronous. */
 int nbo_optim_last_step(nbo_optim *opt, nbo_step_info *out);
 /* The last `max_entries` (at most 1024) fused-step outcomes, oldest first; *n_out

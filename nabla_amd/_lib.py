@@ -107,6 +107,8 @@ SYMBOLS = {
     "nbo_fused_step_groups": (C.c_int, [C.c_uint64, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), _P, _P,
                                         C.c_double, C.c_uint32]),
     "nbo_accumulate": (C.c_int, [_P, _P, C.c_int]),
+    "nbo_backend_apply": (C.c_int, [C.c_int, _P, _P, _P, C.c_double]),
+    "nbo_backend_cast": (C.c_int, [_P, _P]),
     "nbo_optim_last_step": (C.c_int, [_P, C.POINTER(StepInfo)]),
     "nbo_optim_trace_read": (C.c_int, [_P, C.POINTER(StepInfo), C.c_uint64, _U64P, _U64P]),
     "nbo_copy_bytes": (C.c_int, [_P, _P, C.c_uint64]),

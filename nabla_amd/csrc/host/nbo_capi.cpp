@@ -791,6 +791,75 @@ int nbo_accumulate(nbo_list *accum, nbo_list *grads, int zero_grads)
     });
 }
 
+// ---- Backend primitives on tensor lists ----------------------------------------------------
+
+// The shape assert every binary Backend operation of the reference starts with
+// (tensor/ops.rs:638-646 for axpy_inplace; add / emul / ediv likewise).
+static void require_same_shapes(const nbo_list *x, const nbo_list *y, const char *op)
+{
+    if (x->layout.nt() != y->layout.nt())
+        fail(NBO_ERR_LEN_MISMATCH, std::string("nabla: ") + op + " -- tensor lists differ in length");
+    for (uint64_t t = 0; t < x->layout.nt(); t++)
+        if (x->layout.rows[t] != y->layout.rows[t] || x->layout.cols[t] != y->layout.cols[t])
+            fail(NBO_ERR_SHAPE, std::string("nabla: ") + op + " (" + std::to_string(x->layout.rows[t]) + "x" +
+                                    std::to_string(x->layout.cols[t]) + ") vs (" +
+                                    std::to_string(y->layout.rows[t]) + "x" +
+                                    std::to_string(y->layout.cols[t]) + ") -- shapes must match (tensor " +
+                                    std::to_string(t) + ")");
+}
+
+static_assert((int)NBO_BACKEND_SCALE == (int)NBO_EW_SCALE && (int)NBO_BACKEND_AXPY == (int)NBO_EW_AXPY &&
+                  (int)NBO_BACKEND_ADD == (int)NBO_EW_ADD && (int)NBO_BACKEND_EMUL == (int)NBO_EW_EMUL &&
+                  (int)NBO_BACKEND_EDIV == (int)NBO_EW_EDIV && (int)NBO_BACKEND_POWF == (int)NBO_EW_POWF &&
+                  (int)NBO_BACKEND_ADD_SCALAR == (int)NBO_EW_ADD_SCALAR &&
+                  (int)NBO_BACKEND_ZEROS == (int)NBO_EW_ZEROS && (int)NBO_BACKEND_CLONE == (int)NBO_EW_COPY,
+              "public operation codes and the kernels' must agree");
+
+int nbo_backend_apply(int op, nbo_list *out, nbo_list *a, nbo_list *b, double s)
+{
+    return guarded([&] {
+        static const char *const names[NBO_EW_COUNT] = {"scale", "axpy_inplace", "add",   "emul", "ediv",
+                                                        "powf",  "map",          "zeros", "clone_storage"};
+        require(op >= 0 && op < (int)NBO_EW_COUNT, NBO_ERR_ARG, "unknown backend operation");
+        require(out != nullptr, NBO_ERR_ARG, "null output list");
+        const bool needs_a = op != NBO_EW_ZEROS;
+        const bool needs_b = op == NBO_EW_ADD || op == NBO_EW_EMUL || op == NBO_EW_EDIV;
+        require(!needs_a || a != nullptr, NBO_ERR_ARG, "null operand list");
+        require(!needs_b || b != nullptr, NBO_ERR_ARG, "null second operand list");
+        if (needs_a) {
+            require_same_shapes(out, a, names[op]);
+            require(a->dtype == out->dtype, NBO_ERR_DTYPE, "operand and output differ in element type");
+        }
+        if (needs_b) {
+            require_same_shapes(out, b, names[op]);
+            require(b->dtype == out->dtype, NBO_ERR_DTYPE, "operands differ in element type");
+        }
+        NboEwArgs e = {};
+        e.L = out->layout.dev;
+        e.out_ptrs = out->ptrs_dev;
+        e.a_ptrs = needs_a ? a->ptrs_dev : nullptr;
+        e.b_ptrs = needs_b ? b->ptrs_dev : nullptr;
+        e.s = s;
+        e.op = (uint32_t)op;
+        Runtime::get().launch(K_EW_BASE + out->dtype, out->layout.nchunks, NBO_BLOCK, e);
+    });
+}
+
+int nbo_backend_cast(nbo_list *dst, nbo_list *src)
+{
+    return guarded([&] {
+        require(dst && src, NBO_ERR_ARG, "null list");
+        require_same_shapes(dst, src, "cast");
+        NboCastListArgs c = {};
+        c.L = dst->layout.dev;
+        c.dst_ptrs = dst->ptrs_dev;
+        c.src_ptrs = src->ptrs_dev;
+        c.dst_type = (uint32_t)dst->dtype;
+        c.src_type = (uint32_t)src->dtype;
+        Runtime::get().launch(K_CAST_LIST, dst->layout.nchunks, NBO_BLOCK, c);
+    });
+}
+
 int nbo_optim_last_step(nbo_optim *opt, nbo_step_info *out)
 {
     return guarded([&] {

@@ -39,7 +39,9 @@ enum KernelId {
     K_PROBE = 19,
     K_ACCUM_BASE = 20, // + st
     K_FILL_ZERO = 23,
-    K_COUNT = 24
+    K_EW_BASE = 24, // + st
+    K_CAST_LIST = 27,
+    K_COUNT = 28
 };
 
 // Process-wide runtime: device 0, the loaded module, the stream, scratch buffers.

@@ -778,6 +778,119 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_cast_master(const Nb
     }
 }
 
+// ---------------------------------------------------------------------------------
+// Backend primitives on tensor lists: the single passes the reference's optimizers are
+// chains of (BackendCore::{scale, axpy_inplace, add, zeros, clone_storage},
+// BackendMath::{powf, emul, ediv}, nabla-core/src/cpu/mod.rs:137-139, 181, 211-232,
+// 264-272; Tensor::map(|x| x + s) as used at nabla-train/src/optim/alg.rs:133).  Every
+// operation is one IEEE operation in the arithmetic type, rounded to the element type:
+// for bf16 that is the f32 operation followed by bf16::from_f32
+// (common/scalar/mod.rs:253-351), including the product inside axpy.
+template <int ST> DEV typename Traits<ST>::T to_storage_precision(typename Traits<ST>::T x) { return x; }
+template <> __device__ __forceinline__ float to_storage_precision<NBO_BF16>(float x)
+{
+    return bf16_bits_to_f32(f32_to_bf16_bits(x));
+}
+
+// powf(x, 0.5) is taken as the correctly rounded square root with C's pow special
+// cases (pow(-0, 0.5) = +0, pow(-inf, 0.5) = +inf); other exponents use the device
+// math library's pow.
+DEV float pow_elem(float x, float p)
+{
+    if (p == 0.5f) return x == -__builtin_inff() ? __builtin_inff() : __builtin_fabsf(__builtin_sqrtf(x));
+    return powf(x, p);
+}
+DEV double pow_elem(double x, double p)
+{
+    if (p == 0.5) return x == -__builtin_inf() ? __builtin_inf() : __builtin_fabs(__builtin_sqrt(x));
+    return pow(x, p);
+}
+
+template <int ST, typename T> DEV T ew_elem(uint32_t op, T o, T a, T b, T s)
+{
+    switch (op) {
+    case NBO_EW_SCALE: return a * s;
+    case NBO_EW_AXPY: return o + to_storage_precision<ST>(s * a);
+    case NBO_EW_ADD: return a + b;
+    case NBO_EW_EMUL: return a * b;
+    case NBO_EW_EDIV: return a / b;
+    case NBO_EW_POWF: return pow_elem(a, s);
+    case NBO_EW_ADD_SCALAR: return a + s;
+    case NBO_EW_COPY: return a;
+    default: return (T)0; // NBO_EW_ZEROS
+    }
+}
+
+template <int ST> DEV void ew_body(const NboEwArgs &a)
+{
+    typedef typename Traits<ST>::T T;
+    enum { SB = Traits<ST>::SBYTES, VEC = Traits<ST>::VEC };
+    const uint32_t tid = threadIdx.x;
+    const ChunkRef c = chunk_ref(a.L, blockIdx.x);
+    const uint32_t op = a.op;
+    const bool use_a = op != NBO_EW_ZEROS;
+    const bool use_b = op == NBO_EW_ADD || op == NBO_EW_EMUL || op == NBO_EW_EDIV;
+    const bool use_o = op == NBO_EW_AXPY;
+    char *po = (char *)a.out_ptrs[c.t] + c.base * SB;
+    const char *pa = use_a ? (const char *)a.a_ptrs[c.t] + c.base * SB : po;
+    const char *pb = use_b ? (const char *)a.b_ptrs[c.t] + c.base * SB : po;
+    const T s = to_storage_precision<ST>((T)a.s);
+    const bool vec_ok = ((((uintptr_t)po) | ((uintptr_t)pa) | ((uintptr_t)pb)) & (VEC * SB - 1)) == 0;
+    const uint32_t nvec = vec_ok ? c.cnt / VEC : 0;
+    for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
+        const uint64_t off = (uint64_t)q * VEC * SB;
+        T o[VEC] = {}, x[VEC] = {}, y[VEC] = {};
+        if (use_a) IO<ST>::ldv(pa + off, x);
+        if (use_b) IO<ST>::ldv(pb + off, y);
+        if (use_o) IO<ST>::ldv(po + off, o);
+#pragma unroll
+        for (int k = 0; k < VEC; k++) o[k] = ew_elem<ST, T>(op, o[k], x[k], y[k], s);
+        IO<ST>::stv(po + off, o);
+    }
+    for (uint32_t e = nvec * VEC + tid; e < c.cnt; e += NBO_BLOCK) {
+        const uint64_t off = (uint64_t)e * SB;
+        const T x = use_a ? IO<ST>::ld1(pa + off) : (T)0;
+        const T y = use_b ? IO<ST>::ld1(pb + off) : (T)0;
+        const T o = use_o ? IO<ST>::ld1(po + off) : (T)0;
+        IO<ST>::st1(po + off, ew_elem<ST, T>(op, o, x, y, s));
+    }
+}
+
+#define NBO_EW_KERNEL(name, ST)                                                             \
+    extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboEwArgs a)         \
+    {                                                                                       \
+        ew_body<ST>(a);                                                                     \
+    }
+NBO_EW_KERNEL(nbo_ew_f32, NBO_F32)
+NBO_EW_KERNEL(nbo_ew_bf16, NBO_BF16)
+NBO_EW_KERNEL(nbo_ew_f64, NBO_F64)
+
+// BackendCore::cast, default implementation (common/backend/mod.rs:157-160):
+// U::from_f64(x.to_f64()) per element.  Widening is exact; f64 -> f32 rounds to nearest
+// even; anything -> bf16 goes through f32 first (bf16::from_f64 = from_f32(v as f32),
+// scalar/mod.rs:338-340), so f64 -> bf16 rounds twice, as the reference does.
+DEV double cast_load(const char *p, uint32_t type, uint64_t e)
+{
+    if (type == NBO_F32) return (double)IO<NBO_F32>::ld1(p + e * 4);
+    if (type == NBO_BF16) return (double)IO<NBO_BF16>::ld1(p + e * 2);
+    return IO<NBO_F64>::ld1(p + e * 8);
+}
+
+extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_cast_list(const NboCastListArgs a)
+{
+    const ChunkRef c = chunk_ref(a.L, blockIdx.x);
+    const uint32_t ssz = a.src_type == NBO_F64 ? 8 : a.src_type == NBO_F32 ? 4 : 2;
+    const uint32_t dsz = a.dst_type == NBO_F64 ? 8 : a.dst_type == NBO_F32 ? 4 : 2;
+    const char *ps = (const char *)a.src_ptrs[c.t] + c.base * ssz;
+    char *pd = (char *)a.dst_ptrs[c.t] + c.base * dsz;
+    for (uint32_t e = threadIdx.x; e < c.cnt; e += NBO_BLOCK) {
+        const double v = cast_load(ps, a.src_type, e);
+        if (a.dst_type == NBO_F64) IO<NBO_F64>::st1(pd + (uint64_t)e * 8, v);
+        else if (a.dst_type == NBO_F32) IO<NBO_F32>::st1(pd + (uint64_t)e * 4, (float)v);
+        else IO<NBO_BF16>::st1(pd + (uint64_t)e * 2, (float)v);
+    }
+}
+
 // Plain streaming copy used only to calibrate the HBM byte counters of a profile
 // against a transfer of known size.
 extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_copy_f32x4(const f32x4 *src, f32x4 *dst,

@@ -196,4 +196,38 @@ struct NboFillArgs {
     uint64_t bytes;
 };
 
+// Backend primitives on tensor lists (nabla-core/src/common/backend/mod.rs:82-216,
+// 275-279): one IEEE operation per element, every result rounded to the element type.
+enum {
+    NBO_EW_SCALE = 0,      // out = a * s
+    NBO_EW_AXPY = 1,       // out = out + s * a      (two roundings, in place on out)
+    NBO_EW_ADD = 2,        // out = a + b
+    NBO_EW_EMUL = 3,       // out = a * b
+    NBO_EW_EDIV = 4,       // out = a / b
+    NBO_EW_POWF = 5,       // out = powf(a, s)
+    NBO_EW_ADD_SCALAR = 6, // out = a + s
+    NBO_EW_ZEROS = 7,      // out = 0
+    NBO_EW_COPY = 8,       // out = a
+    NBO_EW_COUNT = 9
+};
+
+struct NboEwArgs {
+    NboLayoutDev L;
+    const uint64_t *out_ptrs;
+    const uint64_t *a_ptrs; // null for NBO_EW_ZEROS
+    const uint64_t *b_ptrs; // null unless the operation has two tensor operands
+    double s;               // narrowed to the element type on the device
+    uint32_t op;
+    uint32_t pad;
+};
+
+// Element-type conversion of a tensor list through f64, as BackendCore::cast's default
+// (backend/mod.rs:157-160).
+struct NboCastListArgs {
+    NboLayoutDev L;
+    const uint64_t *dst_ptrs;
+    const uint64_t *src_ptrs;
+    uint32_t dst_type, src_type; // NBO_F32 / NBO_BF16 / NBO_F64
+};
+
 #endif

@@ -110,6 +110,8 @@ def _declare(L):
     L.orc_powi.argtypes = [C.c_double, C.c_int]
     L.orc_bf16_from_f32.restype = C.c_uint16
     L.orc_bf16_from_f32.argtypes = [C.c_float]
+    L.orc_bf16_from_f64.restype = C.c_uint16
+    L.orc_bf16_from_f64.argtypes = [C.c_double]
     L.orc_bf16_to_f32.restype = C.c_float
     L.orc_bf16_to_f32.argtypes = [C.c_uint16]
     L.orc_lr_at_step.restype = C.c_double
@@ -140,6 +142,8 @@ def _suffix(arr: np.ndarray) -> str:
         return "f32"
     if arr.dtype == np.float64:
         return "f64"
+    if arr.dtype == np.uint16:  # bf16 bit patterns
+        return "bf16"
     raise TypeError(f"oracle: unsupported dtype {arr.dtype}")
 
 
@@ -155,6 +159,10 @@ def _sizes(arrs):
 
 
 def _ctype(arr):
+    """Constructor of the C scalar that goes with `arr`'s element type; for bf16 (uint16
+    patterns) the Python float is narrowed with bf16::from_f64 first."""
+    if arr.dtype == np.uint16:
+        return lambda s: C.c_uint16(lib().orc_bf16_from_f64(C.c_double(s)))
     return C.c_float if arr.dtype == np.float32 else C.c_double
 
 
@@ -211,6 +219,26 @@ def powf(a, p):
     out = np.empty_like(a)
     getattr(lib(), f"orc_powf_{_suffix(a)}")(C.c_void_p(a.ctypes.data), _ctype(a)(p),
                                              C.c_void_p(out.ctypes.data), C.c_size_t(a.size))
+    return out
+
+
+def map_add(a, c):
+    """Tensor::map(|x| x + c)."""
+    out = np.empty_like(a)
+    getattr(lib(), f"orc_map_add_{_suffix(a)}")(C.c_void_p(a.ctypes.data), _ctype(a)(c),
+                                                C.c_void_p(out.ctypes.data), C.c_size_t(a.size))
+    return out
+
+
+_CAST_TYPE = {np.dtype(np.float32): 0, np.dtype(np.uint16): 1, np.dtype(np.float64): 2}
+
+
+def cast(src: np.ndarray, dst_dtype) -> np.ndarray:
+    """B::cast default (backend/mod.rs:157-160); np.uint16 stands for bf16 patterns."""
+    src = np.ascontiguousarray(src)
+    out = np.empty(src.shape, dtype=dst_dtype)
+    lib().orc_cast(C.c_void_p(src.ctypes.data), C.c_int(_CAST_TYPE[src.dtype]),
+                   C.c_void_p(out.ctypes.data), C.c_int(_CAST_TYPE[out.dtype]), C.c_size_t(src.size))
     return out
 
 

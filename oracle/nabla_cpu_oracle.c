@@ -168,21 +168,99 @@ double orc_lr_at_step(const orc_schedule *s, double base_lr, uint64_t step)
 #define FN(x) x##_f32
 #define POW_T powf
 #define SQRT_T sqrtf
+#define FABS_T fabsf
 #include "oracle_impl.inc"
 #undef T
 #undef FN
 #undef POW_T
 #undef SQRT_T
+#undef FABS_T
 
 #define T double
 #define FN(x) x##_f64
 #define POW_T pow
 #define SQRT_T sqrt
+#define FABS_T fabs
 #include "oracle_impl.inc"
 #undef T
 #undef FN
 #undef POW_T
 #undef SQRT_T
+#undef FABS_T
+
+/* ---- T = half::bf16 --------------------------------------------------------------------
+ * Every operation on bf16 is the f32 operation followed by bf16::from_f32: the
+ * reference's MathOps for half types (scalar/mod.rs:256-283: math_mul, math_div,
+ * math_powf) and the half crate's own `+` and `*` operators (half 2.7.1, not vendored;
+ * its documented software path converts to f32, operates and converts back). */
+uint16_t orc_bf16_from_f64(double v) { return orc_bf16_from_f32((float)v); } /* scalar/mod.rs:338-340 */
+
+static float pow_f32_mode(float x, float p)
+{
+    if (g_pow_mode == ORC_POW_SQRT && p == 0.5f) {
+        float r = fabsf(sqrtf(x));
+        return x == -INFINITY ? INFINITY : r;
+    }
+    return powf(x, p);
+}
+
+#define BF(x) orc_bf16_to_f32(x)
+#define RB(x) orc_bf16_from_f32(x)
+void orc_scale_bf16(const uint16_t *a, uint16_t s, uint16_t *out, size_t n)
+{
+    size_t i;
+    for (i = 0; i < n; i++) out[i] = RB(BF(a[i]) * BF(s));
+}
+void orc_axpy_inplace_bf16(uint16_t *y, uint16_t alpha, const uint16_t *x, size_t n)
+{
+    size_t i;
+    for (i = 0; i < n; i++) {
+        uint16_t t = RB(BF(alpha) * BF(x[i])); /* alpha * xi is a bf16 value */
+        y[i] = RB(BF(y[i]) + BF(t));
+    }
+}
+void orc_emul_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n)
+{
+    size_t i;
+    for (i = 0; i < n; i++) out[i] = RB(BF(a[i]) * BF(b[i]));
+}
+void orc_ediv_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n)
+{
+    size_t i;
+    for (i = 0; i < n; i++) out[i] = RB(BF(a[i]) / BF(b[i]));
+}
+void orc_add_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n)
+{
+    size_t i;
+    for (i = 0; i < n; i++) out[i] = RB(BF(a[i]) + BF(b[i]));
+}
+void orc_powf_bf16(const uint16_t *a, uint16_t p, uint16_t *out, size_t n)
+{
+    size_t i;
+    for (i = 0; i < n; i++) out[i] = RB(pow_f32_mode(BF(a[i]), BF(p)));
+}
+void orc_map_add_bf16(const uint16_t *a, uint16_t c, uint16_t *out, size_t n)
+{
+    size_t i;
+    for (i = 0; i < n; i++) out[i] = RB(BF(a[i]) + BF(c));
+}
+#undef BF
+#undef RB
+
+/* B::cast default (backend/mod.rs:157-160): U::from_f64(x.to_f64()) per element.
+ * Types: 0 = f32, 1 = bf16, 2 = f64. */
+void orc_cast(const void *src, int src_type, void *dst, int dst_type, size_t n)
+{
+    size_t i;
+    for (i = 0; i < n; i++) {
+        double v = src_type == 0   ? (double)((const float *)src)[i]
+                   : src_type == 1 ? (double)orc_bf16_to_f32(((const uint16_t *)src)[i])
+                                   : ((const double *)src)[i];
+        if (dst_type == 0) ((float *)dst)[i] = (float)v;
+        else if (dst_type == 1) ((uint16_t *)dst)[i] = orc_bf16_from_f64(v);
+        else ((double *)dst)[i] = v;
+    }
+}
 
 int orc_f32_step(orc_meta *meta, orc_scaler_state *scaler, double max_norm, size_t nt,
                  const uint64_t *sizes, float **params, float **grads, float **m, float **v,

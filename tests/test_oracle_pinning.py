@@ -558,3 +558,100 @@ def test_mixed_step_composition_in_exact_arithmetic():
     finally:
         O.set_pow_mode(O.POW_LIBM)
     assert meta.step_count == 2 and s.consecutive_ok == 2 and s.scale == scale
+
+
+# ---- 7. T = bf16 primitives and the generic cast ---------------------------------------
+
+def rbf(q):  # bfloat16: 8 significand bits, f32's exponent range
+    return rne(Fraction(q), 8, -133)
+
+
+def _bf_exact(h) -> Fraction:
+    return Fraction(float(O.bf16_to_f32(np.array([h], dtype=np.uint16))[0]))
+
+
+def test_bf16_primitives_are_the_f32_operation_then_one_rounding_to_bf16():
+    """scalar/mod.rs:256-283 and the half crate's operators: convert to f32, operate in
+    f32, bf16::from_f32.  Checked in exact arithmetic: RNE to 24 bits, then RNE to 8 bits.
+    (For +, * and / of 8-bit significands the two-step rounding provably equals the direct
+    one; where a shortcut would show is the inner rounding of axpy, checked below, and the
+    f64 -> bf16 cast, checked in the next test.)"""
+    rng = np.random.default_rng(7)
+    a = O.bf16_from_f32(_rand_f32(rng, 4000, -3, 2))
+    b = O.bf16_from_f32(_rand_f32(rng, 4000, -3, 2))
+    s = 0.3
+    sb = _bf_exact(O.bf16_from_f32(np.array([np.float32(s)]))[0])
+    cases = {
+        "scale": (O.scale(a, s), lambda x, y: x * sb),
+        "emul": (O.emul(a, b), lambda x, y: x * y),
+        "ediv": (O.ediv(a, b), lambda x, y: x / y),
+        "add": (O.add(a, b), lambda x, y: x + y),
+        "map_add": (O.map_add(a, s), lambda x, y: x + sb),
+    }
+    for name, (out, f) in cases.items():
+        for i in range(a.size):
+            exact = f(_bf_exact(a[i]), _bf_exact(b[i]))
+            assert _bf_exact(out[i]) == rbf(r32(exact)), (name, i)
+    # axpy: the product is itself a bf16 value before the sum (two bf16 roundings)
+    y = a.copy()
+    O.axpy_inplace(y, s, b)
+    skipped_inner_rounding_differs = 0
+    for i in range(a.size):
+        t = rbf(r32(sb * _bf_exact(b[i])))
+        want = rbf(r32(_bf_exact(a[i]) + t))
+        assert _bf_exact(y[i]) == want, i
+        skipped_inner_rounding_differs += want != rbf(r32(_bf_exact(a[i]) + r32(sb * _bf_exact(b[i]))))
+    assert skipped_inner_rounding_differs > 10
+
+
+def test_bf16_powf_follows_the_pow_mode():
+    a = O.bf16_from_f32(np.array([0.0, 0.25, 2.0, 3.0, 1e-6, 7e4], dtype=np.float32))
+    for mode in (O.POW_LIBM, O.POW_SQRT):
+        O.set_pow_mode(mode)
+        try:
+            out = O.powf(a, 0.5)
+        finally:
+            O.set_pow_mode(O.POW_LIBM)
+        for i in range(a.size):
+            # sqrt of a bf16 value, correctly rounded to f32, then to bf16: both candidate
+            # lowerings of powf agree after the second rounding on these inputs
+            assert _bf_exact(out[i]) == rbf(sqrt_r32(_bf_exact(a[i]))), (mode, i)
+
+
+def test_cast_goes_through_f64_and_narrows_to_bf16_in_two_steps():
+    """backend/mod.rs:157-160 with scalar/mod.rs:219, 338-344: widening is exact,
+    f64 -> f32 is one RNE, anything -> bf16 is `from_f32(v as f32)`."""
+    rng = np.random.default_rng(8)
+    x64 = rng.standard_normal(3000) * 10.0 ** rng.uniform(-6, 6, 3000)
+    # exact ties of the second rounding that the first rounding creates
+    x64[:4] = [1.0 + 2.0 ** -8 + 2.0 ** -30, 1.0 + 2.0 ** -8 - 2.0 ** -30, -(1.0 + 3 * 2.0 ** -8 - 2.0 ** -40), 0.0]
+    to32 = O.cast(x64, np.float32)
+    to16 = O.cast(x64, np.uint16)
+    two_step_differs = 0
+    for i in range(x64.size):
+        q = Fraction(float(x64[i]))
+        assert f32_exact(to32[i]) == r32(q)
+        assert _bf_exact(to16[i]) == rbf(r32(q))
+        two_step_differs += rbf(r32(q)) != rbf(q)
+    assert two_step_differs >= 2
+    assert to16[0] == 0x3F80 and rbf(Fraction(float(x64[0]))) == Fraction(1) + Fraction(1, 128)
+    x32 = _rand_f32(rng, 1000)
+    assert np.array_equal(O.cast(x32, np.float64), x32.astype(np.float64))
+    assert np.array_equal(O.cast(x32, np.uint16), O.bf16_from_f32(x32))
+    h = O.bf16_from_f32(x32)
+    assert np.array_equal(O.cast(h, np.float32), O.bf16_to_f32(h))
+    assert np.array_equal(O.cast(h, np.float64), O.bf16_to_f32(h).astype(np.float64))
+    assert np.array_equal(O.cast(h, np.uint16), h) and np.array_equal(O.cast(x32, np.float32), x32)
+
+
+def test_powf_half_of_negative_zero_and_minus_infinity():
+    """C's pow: pow(-0, 0.5) = +0 and pow(-inf, 0.5) = +inf; the sqrt lowering keeps both
+    (fabs, select) -- the oracle's two modes must agree on them."""
+    x = np.array([-0.0, -np.inf, np.inf, 0.0, 4.0], dtype=np.float32)
+    for mode in (O.POW_LIBM, O.POW_SQRT):
+        O.set_pow_mode(mode)
+        try:
+            out = O.powf(x, np.float32(0.5))
+        finally:
+            O.set_pow_mode(O.POW_LIBM)
+        assert np.array_equal(out.view(np.uint32), np.array([0.0, np.inf, np.inf, 0.0, 2.0], dtype=np.float32).view(np.uint32)), mode
