@@ -177,6 +177,9 @@ int nbo_scaler_unscale_and_update(nbo_scaler *s, nbo_list *grads, int *ok);
 /* clip_grad_norm (nabla-train/src/trainer.rs:500-523), in place on f32 / f64
  * gradients; *norm receives the pre-clip norm (0 when max_norm <= 0).  Synchronous. */
 int nbo_clip_grad_norm(nbo_list *grads, double max_norm, double *norm);
+/* Trainer::has_non_finite (nabla-train/src/trainer.rs:387-400): *found = 1 if any gradient
+ * element is inf or NaN.  One read-only pass; synchronous (the Trainer branches on it). */
+int nbo_has_non_finite(nbo_list *grads, int *found);
 /* zero_grad (nabla-ml/src/autograd/ops.rs:1668-1673; trainer.rs:285-290). */
 int nbo_zero_grad(nbo_list *grads);
 /* scale_grad (autograd/ops.rs:1675-1680), f32 / f64 gradients. */

@@ -101,6 +101,7 @@ SYMBOLS = {
     "nbo_scaler_load_state": (C.c_int, [_P, C.POINTER(ScalerState)]),
     "nbo_scaler_unscale_and_update": (C.c_int, [_P, _P, C.POINTER(C.c_int)]),
     "nbo_clip_grad_norm": (C.c_int, [_P, C.c_double, C.POINTER(C.c_double)]),
+    "nbo_has_non_finite": (C.c_int, [_P, C.POINTER(C.c_int)]),
     "nbo_zero_grad": (C.c_int, [_P]),
     "nbo_scale_grad": (C.c_int, [_P, C.c_double]),
     "nbo_fused_step": (C.c_int, [_P, _P, _P, _P, C.c_double, C.c_uint32]),

@@ -683,6 +683,24 @@ int nbo_clip_grad_norm(nbo_list *grads, double max_norm, double *norm)
     });
 }
 
+int nbo_has_non_finite(nbo_list *grads, int *found)
+{
+    return guarded([&] {
+        require(grads && found, NBO_ERR_ARG, "null list or output");
+        Runtime &rt = Runtime::get();
+        NboFinalizeArgs f = {};
+        f.partial_sumsq = rt.partial_sumsq();
+        f.partial_flag = rt.partial_flag();
+        f.grid = launch_norm(grads, nullptr);
+        f.check_finite = 1;
+        f.gf = rt.gf_scratch();
+        rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
+        NboGradFactors g;
+        rt.read_back(&g, rt.gf_scratch(), sizeof(g));
+        *found = g.found_inf ? 1 : 0;
+    });
+}
+
 int nbo_zero_grad(nbo_list *grads)
 {
     return guarded([&] {

@@ -610,6 +610,14 @@ def clip_grad_norm(grads, max_norm: float) -> float:
     return norm.value
 
 
+def has_non_finite(grads) -> bool:
+    """Trainer::has_non_finite (nabla-train/src/trainer.rs:387-400)."""
+    g = _free_cache.get("finite", grads)
+    found = C.c_int(0)
+    _call(_lib.load().nbo_has_non_finite(g._h, C.byref(found)))
+    return bool(found.value)
+
+
 def zero_grad(grads) -> None:
     """nabla-ml/src/autograd/ops.rs:1668-1673."""
     g = _free_cache.get("zero", grads)
