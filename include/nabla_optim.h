@@ -118,9 +118,11 @@ int nbo_list_destroy(nbo_list *list);
 /* Sgd::new / Adam::new / AdamW::new (alg.rs:319-330, 181-199, 20-39) + the builder
  * setters, all at once through `meta` (meta->kind selects the algorithm;
  * meta->step_count seeds step_count).  Moments are created zero-filled.
- * state_dtype: NBO_DT_F32 or NBO_DT_F64 -- the arithmetic type T.
- * keep_master != 0: additionally hold f32 master weights so that the caller's
- * parameters and gradients may be bf16 (T = f32).
+ * state_dtype: NBO_DT_F32, NBO_DT_F64 or NBO_DT_BF16 -- the arithmetic type T, which is
+ * also the type of the moments and of the caller's tensors (T = bf16: every operation is
+ * the f32 operation followed by bf16::from_f32, common/scalar/mod.rs:253-351).
+ * keep_master != 0 (f32 state only): additionally hold f32 master weights so that the
+ * caller's parameters and gradients may be bf16 while the arithmetic stays T = f32.
  * State of 128 MiB per array or more is assembled from physical chunks chosen so that
  * the arrays lie in different regions of the HBM (nbo_optim_state_regions tells the
  * outcome); that takes up to a few seconds here and nothing per step. */
@@ -167,22 +169,22 @@ int nbo_scaler_create(const nbo_scaler_state *state, nbo_scaler **out);
 int nbo_scaler_destroy(nbo_scaler *s);
 int nbo_scaler_state_get(nbo_scaler *s, nbo_scaler_state *out); /* GradScaler::state */
 int nbo_scaler_load_state(nbo_scaler *s, const nbo_scaler_state *state);
-/* GradScaler::unscale_and_update (core.rs:351-388) on f32 / f64 gradients, in place.
+/* GradScaler::unscale_and_update (core.rs:351-388), in place, in the gradients' own type.
  * *ok = 1 if all gradients were finite (they are now unscaled), 0 otherwise (they
  * are now zeros, scale was backed off).  Synchronous. */
 int nbo_scaler_unscale_and_update(nbo_scaler *s, nbo_list *grads, int *ok);
 
 /* ---- gradient utilities ------------------------------------------------------------ */
 
-/* clip_grad_norm (nabla-train/src/trainer.rs:500-523), in place on f32 / f64
- * gradients; *norm receives the pre-clip norm (0 when max_norm <= 0).  Synchronous. */
+/* clip_grad_norm (nabla-train/src/trainer.rs:500-523), in place, in the gradients'
+ * own type; *norm receives the pre-clip norm (0 when max_norm <= 0).  Synchronous. */
 int nbo_clip_grad_norm(nbo_list *grads, double max_norm, double *norm);
 /* Trainer::has_non_finite (nabla-train/src/trainer.rs:387-400): *found = 1 if any gradient
  * element is inf or NaN.  One read-only pass; synchronous (the Trainer branches on it). */
 int nbo_has_non_finite(nbo_list *grads, int *found);
 /* zero_grad (nabla-ml/src/autograd/ops.rs:1668-1673; trainer.rs:285-290). */
 int nbo_zero_grad(nbo_list *grads);
-/* scale_grad (autograd/ops.rs:1675-1680), f32 / f64 gradients. */
+/* scale_grad (autograd/ops.rs:1675-1680), in the gradients' own type. */
 int nbo_scale_grad(nbo_list *grads, double factor);
 
 /* ---- the fused Trainer tail ---------------------------------------------------------- */

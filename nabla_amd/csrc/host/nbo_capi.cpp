@@ -83,9 +83,11 @@ void check_step_args(const nbo_optim *opt, const nbo_list *params, const nbo_lis
                      std::to_string(t) + ")");
     }
     require(params->dtype == grads->dtype, NBO_ERR_DTYPE, "params and grads differ in element type");
-    if (params->dtype == NBO_DT_BF16) {
+    if (params->dtype == NBO_DT_BF16 && opt->state_dtype == NBO_DT_BF16) {
+        // Optimizer<bf16>: state and arithmetic in bf16, no master copy
+    } else if (params->dtype == NBO_DT_BF16) {
         require(opt->state_dtype == NBO_DT_F32 && opt->keep_master, NBO_ERR_DTYPE,
-                "bf16 tensors need an optimizer created with f32 state and keep_master");
+                "bf16 tensors need an optimizer created with bf16 state, or with f32 state and keep_master");
         require(opt->master_valid, NBO_ERR_NO_MASTER,
                 "bf16 step before the master weights were set (nbo_optim_master_from_params or "
                 "nbo_optim_state_write \"w{i}\")");
@@ -109,8 +111,11 @@ NboUpdateArgs update_args(nbo_optim *opt, nbo_list *params, nbo_list *grads, boo
     return a;
 }
 
+bool pure_bf16(const nbo_optim *opt) { return opt->state_dtype == NBO_DT_BF16; }
+
 int update_kernel(const nbo_optim *opt, const nbo_list *params)
 {
+    if (pure_bf16(opt)) return K_UPDATE_PBF16_BASE + opt->meta.kind;
     return K_UPDATE_BASE + params->dtype * 3 + opt->meta.kind;
 }
 
@@ -121,7 +126,7 @@ uint32_t norm_grid(const Layout &L)
 
 // First stage of the norm / found_inf pass over `grads`; partials land in the
 // runtime's scratch.  Returns the grid used (0 for an empty list).
-uint32_t launch_norm(nbo_list *grads, const NboScalerDev *scaler)
+uint32_t launch_norm(nbo_list *grads, const NboScalerDev *scaler, bool bf16_arithmetic = false)
 {
     Runtime &rt = Runtime::get();
     NboNormArgs a = {};
@@ -131,7 +136,10 @@ uint32_t launch_norm(nbo_list *grads, const NboScalerDev *scaler)
     a.partial_sumsq = rt.partial_sumsq();
     a.partial_flag = rt.partial_flag();
     a.grid = norm_grid(grads->layout);
-    rt.launch(K_NORM_BASE + grads->dtype, a.grid, NBO_BLOCK, a);
+    // bf16 gradients are unscaled in f32 when they feed f32 state (the mixed-precision
+    // composition) and in bf16 when the optimizer itself is bf16 or they are scaled in place
+    const bool pbf16 = bf16_arithmetic && grads->dtype == NBO_DT_BF16;
+    rt.launch(pbf16 ? (int)K_NORM_PBF16 : K_NORM_BASE + grads->dtype, a.grid, NBO_BLOCK, a);
     return a.grid;
 }
 
@@ -359,8 +367,8 @@ int nbo_optim_create(const nbo_meta *meta, uint64_t n_tensors, const uint64_t *r
         require(n_tensors == 0 || (rows && cols), NBO_ERR_ARG, "null shape array");
         require(meta->kind >= NBO_KIND_ADAMW && meta->kind <= NBO_KIND_SGD, NBO_ERR_ARG,
                 "unknown optimizer kind");
-        require(state_dtype == NBO_DT_F32 || state_dtype == NBO_DT_F64, NBO_ERR_DTYPE,
-                "optimizer state is f32 or f64");
+        require(state_dtype == NBO_DT_F32 || state_dtype == NBO_DT_F64 || state_dtype == NBO_DT_BF16,
+                NBO_ERR_DTYPE, "optimizer state is f32, f64 or bf16");
         require(!keep_master || state_dtype == NBO_DT_F32, NBO_ERR_DTYPE,
                 "master weights are f32: keep_master needs f32 state");
         require(n_tensors < (1ull << 31), NBO_ERR_TOO_LARGE, "too many tensors");
@@ -635,13 +643,11 @@ int nbo_scaler_unscale_and_update(nbo_scaler *s, nbo_list *grads, int *ok)
 {
     return guarded([&] {
         require(s && grads && ok, NBO_ERR_ARG, "null scaler, list or output");
-        require(grads->dtype != NBO_DT_BF16, NBO_ERR_DTYPE,
-                "in-place unscale takes f32 / f64 gradients; bf16 gradients go through nbo_fused_step");
         Runtime &rt = Runtime::get();
         NboFinalizeArgs f = {};
         f.partial_sumsq = rt.partial_sumsq();
         f.partial_flag = rt.partial_flag();
-        f.grid = launch_norm(grads, s->dev);
+        f.grid = launch_norm(grads, s->dev, true);
         f.check_finite = 1;
         f.scaler = s->dev;
         f.gf = rt.gf_scratch();
@@ -662,8 +668,6 @@ int nbo_clip_grad_norm(nbo_list *grads, double max_norm, double *norm)
 {
     return guarded([&] {
         require(grads && norm, NBO_ERR_ARG, "null list or output");
-        require(grads->dtype != NBO_DT_BF16, NBO_ERR_DTYPE,
-                "in-place clip takes f32 / f64 gradients; bf16 gradients go through nbo_fused_step");
         *norm = 0.0;
         if (max_norm <= 0.0) return; // trainer.rs:501-503
         Runtime &rt = Runtime::get();
@@ -713,7 +717,6 @@ int nbo_scale_grad(nbo_list *grads, double factor)
 {
     return guarded([&] {
         require(grads != nullptr, NBO_ERR_ARG, "null list");
-        require(grads->dtype != NBO_DT_BF16, NBO_ERR_DTYPE, "scale_grad takes f32 / f64 gradients");
         launch_scale(grads, nullptr, factor, 2);
     });
 }
@@ -731,7 +734,7 @@ int nbo_fused_step(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, nbo_lis
         f.partial_flag = rt.partial_flag();
         // without scaler, clipping and nan policy the pass has nothing to decide, but
         // it still runs so that the trace records every step
-        f.grid = launch_norm(grads, scaler ? scaler->dev : nullptr);
+        f.grid = launch_norm(grads, scaler ? scaler->dev : nullptr, pure_bf16(opt));
         f.check_finite = (scaler || (flags & NBO_STEP_SKIP_NONFINITE)) ? 1u : 0u;
         f.scaler = scaler ? scaler->dev : nullptr;
         f.gf = opt->gf;
@@ -758,6 +761,8 @@ int nbo_fused_step_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *c
             check_step_args(opts[g], params[g], grads[g]);
             require(grads[g]->dtype == all_grads->dtype, NBO_ERR_DTYPE,
                     "group gradients differ in element type from the whole list");
+            require(pure_bf16(opts[g]) == pure_bf16(opts[0]), NBO_ERR_DTYPE,
+                    "groups mix bf16 and f32 optimizer state");
             covered += grads[g]->layout.nt();
         }
         if (covered != all_grads->layout.nt())
@@ -768,7 +773,7 @@ int nbo_fused_step_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *c
         NboFinalizeArgs f = {};
         f.partial_sumsq = rt.partial_sumsq();
         f.partial_flag = rt.partial_flag();
-        f.grid = launch_norm(all_grads, scaler ? scaler->dev : nullptr);
+        f.grid = launch_norm(all_grads, scaler ? scaler->dev : nullptr, n_groups > 0 && pure_bf16(opts[0]));
         f.check_finite = (scaler || (flags & NBO_STEP_SKIP_NONFINITE)) ? 1u : 0u;
         f.scaler = scaler ? scaler->dev : nullptr;
         f.gf = rt.gf_scratch();

@@ -38,7 +38,8 @@ static const char *const kKernelNames[K_COUNT] = {
     "nbo_copy_f32x4",        "nbo_probe_rmw2",       "nbo_accum_f32",
     "nbo_accum_bf16",        "nbo_accum_f64",        "nbo_fill_zero",
     "nbo_ew_f32",            "nbo_ew_bf16",          "nbo_ew_f64",
-    "nbo_cast_list",
+    "nbo_cast_list",         "nbo_update_pbf16_adamw", "nbo_update_pbf16_adam",
+    "nbo_update_pbf16_sgd",  "nbo_norm_pbf16",
 };
 
 Runtime &Runtime::get()

@@ -41,7 +41,9 @@ enum KernelId {
     K_FILL_ZERO = 23,
     K_EW_BASE = 24, // + st
     K_CAST_LIST = 27,
-    K_COUNT = 28
+    K_UPDATE_PBF16_BASE = 28, // + kind: bf16 tensors with bf16 state and arithmetic
+    K_NORM_PBF16 = 31,
+    K_COUNT = 32
 };
 
 // Process-wide runtime: device 0, the loaded module, the stream, scratch buffers.
@@ -134,7 +136,7 @@ struct nbo_optim {
     NboOptimDev *dev = nullptr; // step_count lives here: the device decides skips
     NboGradFactors *gf = nullptr;
     NboTraceDev *trace = nullptr;
-    size_t elem_bytes() const { return state_dtype == NBO_DT_F64 ? 8 : 4; }
+    size_t elem_bytes() const { return state_dtype == NBO_DT_F64 ? 8 : state_dtype == NBO_DT_BF16 ? 2 : 4; }
 };
 
 #endif

@@ -83,6 +83,29 @@ DEV bool nonfinite_f64(double d)
     return ((uint32_t)(__double_as_longlong(d) >> 32) & 0x7FF00000u) == 0x7FF00000u;
 }
 
+// T = half::bf16 as an arithmetic type: a 16-bit pattern whose every operation is the
+// f32 operation followed by bf16::from_f32 (common/scalar/mod.rs:253-351 and the half
+// crate's operators).  Conversion from float / double is T::from_f64 = from_f32(v as f32).
+struct BF {
+    uint16_t bits;
+    __device__ __forceinline__ BF() : bits(0) {}
+    __device__ __forceinline__ BF(float x) : bits((uint16_t)f32_to_bf16_bits(x)) {}
+    __device__ __forceinline__ BF(double x) : bits((uint16_t)f32_to_bf16_bits((float)x)) {}
+    __device__ __forceinline__ BF(int x) : bits((uint16_t)f32_to_bf16_bits((float)x)) {}
+    __device__ __forceinline__ float f() const { return bf16_bits_to_f32(bits); }
+    __device__ __forceinline__ explicit operator double() const { return (double)f(); }
+};
+DEV BF operator*(BF a, BF b) { return BF(a.f() * b.f()); }
+DEV BF operator+(BF a, BF b) { return BF(a.f() + b.f()); }
+DEV BF operator-(BF a, BF b) { return BF(a.f() - b.f()); }
+DEV BF operator/(BF a, BF b) { return BF(a.f() / b.f()); }
+DEV BF bf_from_bits(uint32_t b)
+{
+    BF r;
+    r.bits = (uint16_t)b;
+    return r;
+}
+
 // f64::powi as compiler-rt's __powidf2 (alg.rs:122-123).
 DEV double powi_f64(double a, int n)
 {
@@ -116,6 +139,11 @@ template <> struct Traits<NBO_F64> {
     enum { VEC = 2, SBYTES = 8 };
 };
 
+template <> struct Traits<NBO_PBF16> {
+    typedef BF T;
+    enum { VEC = 4, SBYTES = 2 };
+};
+
 // arena (engine-owned, always 16-byte aligned) vectors of T
 DEV void ld_state(const float *p, float (&x)[4])
 {
@@ -136,6 +164,20 @@ DEV void st_state(double *p, const double (&x)[2])
 {
     f64x2 v = {x[0], x[1]};
     NBO_STORE(v, GLOBAL_PTR(f64x2, p));
+}
+
+DEV void ld_state(const BF *p, BF (&x)[4])
+{
+    u32x2 v = NBO_LOAD(GLOBAL_PTR(const u32x2, p));
+    x[0] = bf_from_bits(v.x & 0xFFFFu); x[1] = bf_from_bits(v.x >> 16);
+    x[2] = bf_from_bits(v.y & 0xFFFFu); x[3] = bf_from_bits(v.y >> 16);
+}
+DEV void st_state(BF *p, const BF (&x)[4])
+{
+    u32x2 v;
+    v.x = (uint32_t)x[0].bits | ((uint32_t)x[1].bits << 16);
+    v.y = (uint32_t)x[2].bits | ((uint32_t)x[3].bits << 16);
+    NBO_STORE(v, GLOBAL_PTR(u32x2, p));
 }
 
 // caller tensors: vector of VEC storage elements at byte address p
@@ -170,6 +212,13 @@ template <> struct IO<NBO_BF16> {
     }
     DEV float ld1(const char *p) { return bf16_bits_to_f32(*GLOBAL_PTR(const uint16_t, p)); }
     DEV void st1(char *p, float x) { *GLOBAL_PTR(uint16_t, p) = (uint16_t)f32_to_bf16_bits(x); }
+};
+
+template <> struct IO<NBO_PBF16> {
+    DEV void ldv(const char *p, BF (&x)[4]) { ld_state((const BF *)p, x); }
+    DEV void stv(char *p, const BF (&x)[4]) { st_state((BF *)p, x); }
+    DEV BF ld1(const char *p) { return bf_from_bits(*GLOBAL_PTR(const uint16_t, p)); }
+    DEV void st1(char *p, BF x) { *GLOBAL_PTR(uint16_t, p) = x.bits; }
 };
 
 // ---------------------------------------------------------------------------------
@@ -210,6 +259,26 @@ template <> struct Scal<double> {
     }
 };
 
+// T = bf16: T::from_f64(x) is from_f32(x as f32), so every scalar is the f32-narrowed one
+// rounded once more; `T::one() - wd_lr` is a bf16 subtraction (alg.rs:135).
+template <> struct Scal<BF> {
+    BF b1, omb1, b2, omb2, eps, ss, ibc2, omw, neg_lr, mom, wd, inv, clip;
+    bool use_mom, use_wd;
+    __device__ Scal(const NboOptimDev *o, const NboGradFactors *f)
+        : b1(o->b1), omb1(o->omb1), b2(o->b2), omb2(o->omb2), eps(o->eps_t), ss(o->ss), ibc2(o->ibc2),
+          omw(BF(1.0f) - BF(o->wd_lr_t)), neg_lr(o->neg_lr), mom(o->momentum_t), wd(o->wd_t),
+          inv(f ? f->inv_scale32 : 1.0f), clip(f ? f->clip32 : 1.0f), use_mom(o->momentum != 0.0),
+          use_wd(o->weight_decay != 0.0)
+    {
+    }
+    __device__ Scal(double lr, double momentum, double weight_decay)
+        : b1(), omb1(), b2(), omb2(), eps(), ss(), ibc2(), omw(), neg_lr(-(float)lr), mom(momentum),
+          wd(weight_decay), inv(1.0f), clip(1.0f), use_mom(momentum != 0.0), use_wd(weight_decay != 0.0)
+    {
+    }
+};
+
+DEV BF sqrt_rn(BF x) { return BF(__builtin_sqrtf(x.f())); }
 DEV float sqrt_rn(float x) { return __builtin_sqrtf(x); }
 DEV double sqrt_rn(double x) { return __builtin_sqrt(x); }
 
@@ -401,6 +470,9 @@ NBO_UPDATE_KERNEL(nbo_update_bf16_sgd, NBO_BF16, NBO_SGD)
 NBO_UPDATE_KERNEL(nbo_update_f64_adamw, NBO_F64, NBO_ADAMW)
 NBO_UPDATE_KERNEL(nbo_update_f64_adam, NBO_F64, NBO_ADAM)
 NBO_UPDATE_KERNEL(nbo_update_f64_sgd, NBO_F64, NBO_SGD)
+NBO_UPDATE_KERNEL(nbo_update_pbf16_adamw, NBO_PBF16, NBO_ADAMW)
+NBO_UPDATE_KERNEL(nbo_update_pbf16_adam, NBO_PBF16, NBO_ADAM)
+NBO_UPDATE_KERNEL(nbo_update_pbf16_sgd, NBO_PBF16, NBO_SGD)
 
 // ---------------------------------------------------------------------------------
 // Deterministic block reduction: xor-butterfly inside each 64-lane wavefront, then
@@ -455,6 +527,7 @@ template <int ST> DEV bool nonfinite(typename Traits<ST>::T x);
 template <> __device__ __forceinline__ bool nonfinite<NBO_F32>(float x) { return nonfinite_f32(x); }
 template <> __device__ __forceinline__ bool nonfinite<NBO_BF16>(float x) { return nonfinite_f32(x); }
 template <> __device__ __forceinline__ bool nonfinite<NBO_F64>(double x) { return nonfinite_f64(x); }
+template <> __device__ __forceinline__ bool nonfinite<NBO_PBF16>(BF x) { return (x.bits & 0x7F80u) == 0x7F80u; }
 
 template <int ST> DEV void norm_body(const NboNormArgs &a)
 {
@@ -526,6 +599,9 @@ template <int ST> DEV void norm_body(const NboNormArgs &a)
 NBO_NORM_KERNEL(nbo_norm_f32, NBO_F32)
 NBO_NORM_KERNEL(nbo_norm_bf16, NBO_BF16)
 NBO_NORM_KERNEL(nbo_norm_f64, NBO_F64)
+// bf16 gradients of a bf16 optimizer: the unscaled gradient is itself a bf16 value
+// (g * bf16(1/scale), rounded to bf16) before it is squared.
+NBO_NORM_KERNEL(nbo_norm_pbf16, NBO_PBF16)
 
 // ---------------------------------------------------------------------------------
 // Per-step scalars (alg.rs:120-135 AdamW, 265-277 Adam, 393-395 Sgd).  A skipped
@@ -571,6 +647,7 @@ DEV void prep_step(NboOptimDev *o, const NboHyper &h, const NboGradFactors *f)
     o->ss = (float)step_size;
     o->ibc2 = (float)ibc2;
     const float wd_lr_t = (float)wd_lr;
+    o->wd_lr_t = wd_lr_t;
     o->omw = 1.0f - wd_lr_t; // T::one() - wd_lr, in T (alg.rs:135)
     o->d_b1 = o->beta1;
     o->d_omb1 = omb1;
@@ -708,7 +785,9 @@ template <int ST> DEV void scale_body(const NboScaleArgs &a)
         scale_body<ST>(a);                                                                  \
     }
 NBO_SCALE_KERNEL(nbo_scale_f32, NBO_F32)
-NBO_SCALE_KERNEL(nbo_scale_bf16, NBO_BF16)
+// in place on bf16 tensors the arithmetic is bf16's: factor narrowed to bf16, product
+// rounded to bf16
+NBO_SCALE_KERNEL(nbo_scale_bf16, NBO_PBF16)
 NBO_SCALE_KERNEL(nbo_scale_f64, NBO_F64)
 
 // Gradient accumulation of the Trainer: buf[i] = &buf[i] + g (trainer.rs:262-266 ->

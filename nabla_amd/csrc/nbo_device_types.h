@@ -25,8 +25,10 @@
 // Per-step trace ring kept on the device (found_inf / skipped / scale / step_count).
 #define NBO_TRACE_LEN 1024u
 
-// Element storage types of caller tensors.
-enum { NBO_F32 = 0, NBO_BF16 = 1, NBO_F64 = 2 };
+// Element storage types of caller tensors.  NBO_PBF16 is bf16 storage with bf16
+// arithmetic (the reference's Optimizer<bf16>: every operation rounds to bf16), as
+// opposed to NBO_BF16 = bf16 tensors over f32 state; it only selects kernels.
+enum { NBO_F32 = 0, NBO_BF16 = 1, NBO_F64 = 2, NBO_PBF16 = 3 };
 // OptimKind order of the reference (nabla-train/src/optim/core.rs:46-51).
 enum { NBO_ADAMW = 0, NBO_ADAM = 1, NBO_SGD = 2 };
 
@@ -73,7 +75,8 @@ struct NboOptimDev {
     uint32_t skip; // this step is skipped (found_inf)
     // scalars narrowed to T exactly as the reference narrows them
     float b1, omb1, b2, omb2, eps_t, ss, ibc2, omw;
-    float neg_lr, momentum_t, wd_t, pad0;
+    float neg_lr, momentum_t, wd_t;
+    float wd_lr_t; // T::from_f64(weight_decay * lr) for T = f32 (bf16 narrows it once more)
     double d_b1, d_omb1, d_b2, d_omb2, d_eps, d_ss, d_ibc2, d_omw;
     double d_neg_lr, d_momentum, d_wd;
 };

@@ -244,7 +244,10 @@ class _Optimizer:
     def __init__(self, lr: float, param_shapes: Sequence[Tuple[int, int]], *, dtype: str = "f32",
                  master: bool = False):
         self._shapes = [(int(r), int(c)) for r, c in param_shapes]
-        self._state_dtype = {"f32": DT_F32, "f64": DT_F64}[dtype]
+        # "bf16" is the reference's Optimizer<bf16>: tensors, state and arithmetic all bf16
+        self._state_dtype = {"f32": DT_F32, "f64": DT_F64, "bf16": DT_BF16}[dtype]
+        if master and dtype != "f32":
+            raise ValueError("master weights are f32: master=True goes with dtype='f32'")
         self._master = bool(master)
         self._meta = _lib.Meta(self.KIND, 0, float(lr), 0.0, 0.0, 0.0, 0.0, 0.0, 0)
         self._h = None
@@ -376,7 +379,7 @@ class _Optimizer:
 
     def _torch_dtype(self):
         import torch
-        return torch.float64 if self._state_dtype == DT_F64 else torch.float32
+        return {DT_F64: torch.float64, DT_BF16: torch.bfloat16}.get(self._state_dtype, torch.float32)
 
     def read_state(self, name: str):
         """One state tensor as a new device tensor (a clone, like state_tensors())."""
@@ -636,7 +639,7 @@ def adamw_step(param, grad, m, v, lr, beta1, beta2, eps, weight_decay, step: int
     are device tensors of one dtype (f32 or f64); `param`, `m`, `v` are updated in place."""
     import torch
 
-    dtype = {torch.float32: "f32", torch.float64: "f64"}[param.dtype]
+    dtype = {torch.float32: "f32", torch.float64: "f64", torch.bfloat16: "bf16"}[param.dtype]
     opt = AdamW.new(lr, [_shape2(param)], dtype=dtype).beta1(beta1).beta2(beta2).eps(eps) \
         .weight_decay(weight_decay)
     opt._meta.step_count = int(step) - 1  # step() increments before use (alg.rs:120)

@@ -118,7 +118,7 @@ def _declare(L):
     L.orc_lr_at_step.argtypes = [C.POINTER(Schedule), C.c_double, C.c_uint64]
     L.orc_get_pow_mode.restype = C.c_int
     L.orc_get_threads.restype = C.c_int
-    for suf in ("f32", "f64"):
+    for suf in ("f32", "f64", "bf16"):
         getattr(L, f"orc_clip_grad_norm_{suf}").restype = C.c_double
         getattr(L, f"orc_clip_grad_norm_{suf}").argtypes = [
             C.c_size_t, C.c_void_p, C.c_void_p, C.c_double]

@@ -169,24 +169,40 @@ double orc_lr_at_step(const orc_schedule *s, double base_lr, uint64_t step)
 #define POW_T powf
 #define SQRT_T sqrtf
 #define FABS_T fabsf
+#define FROM_F64(x) ((float)(x))
+#define TO_F64(x) ((double)(x))
+#define NEG_T(x) (-(x))
+#define SUB_T(a, b) ((a) - (b))
 #include "oracle_impl.inc"
 #undef T
 #undef FN
 #undef POW_T
 #undef SQRT_T
 #undef FABS_T
+#undef FROM_F64
+#undef TO_F64
+#undef NEG_T
+#undef SUB_T
 
 #define T double
 #define FN(x) x##_f64
 #define POW_T pow
 #define SQRT_T sqrt
 #define FABS_T fabs
+#define FROM_F64(x) ((double)(x))
+#define TO_F64(x) ((double)(x))
+#define NEG_T(x) (-(x))
+#define SUB_T(a, b) ((a) - (b))
 #include "oracle_impl.inc"
 #undef T
 #undef FN
 #undef POW_T
 #undef SQRT_T
 #undef FABS_T
+#undef FROM_F64
+#undef TO_F64
+#undef NEG_T
+#undef SUB_T
 
 /* ---- T = half::bf16 --------------------------------------------------------------------
  * Every operation on bf16 is the f32 operation followed by bf16::from_f32: the
@@ -244,6 +260,29 @@ void orc_map_add_bf16(const uint16_t *a, uint16_t c, uint16_t *out, size_t n)
     size_t i;
     for (i = 0; i < n; i++) out[i] = RB(BF(a[i]) + BF(c));
 }
+void orc_map_mul_bf16(const uint16_t *a, uint16_t c, uint16_t *out, size_t n)
+{
+    size_t i;
+    for (i = 0; i < n; i++) out[i] = RB(BF(a[i]) * BF(c));
+}
+
+/* Sgd / Adam / AdamW / GradScaler / clip_grad_norm for T = bf16: the same bodies as for
+ * f32 and f64, over the bf16 primitive passes above. */
+#define T uint16_t
+#define FN(x) x##_bf16
+#define FROM_F64(x) orc_bf16_from_f64(x)
+#define TO_F64(x) ((double)orc_bf16_to_f32(x))
+#define NEG_T(x) ((uint16_t)((x) ^ 0x8000u))           /* Neg on half types flips the sign bit */
+#define SUB_T(a, b) RB(BF(a) - BF(b))
+#define ORC_PRIMITIVES_ELSEWHERE
+#include "oracle_impl.inc"
+#undef ORC_PRIMITIVES_ELSEWHERE
+#undef T
+#undef FN
+#undef FROM_F64
+#undef TO_F64
+#undef NEG_T
+#undef SUB_T
 #undef BF
 #undef RB
 

@@ -131,16 +131,11 @@ double orc_lr_at_step(const orc_schedule *s, double base_lr, uint64_t step);
 ORC_DECLARE(f32, float)
 ORC_DECLARE(f64, double)
 
-/* Backend primitives for T = half::bf16 (values passed as their 16-bit patterns):
- * the f32 operation, then bf16::from_f32 (scalar/mod.rs:253-351). */
+/* T = half::bf16, values passed as their 16-bit patterns: every operation is the f32
+ * operation followed by bf16::from_f32 (scalar/mod.rs:253-351); scalars are narrowed with
+ * bf16::from_f64 = from_f32(v as f32).  The same functions as for f32 / f64. */
+ORC_DECLARE(bf16, uint16_t)
 uint16_t orc_bf16_from_f64(double v);
-void orc_scale_bf16(const uint16_t *a, uint16_t s, uint16_t *out, size_t n);
-void orc_axpy_inplace_bf16(uint16_t *y, uint16_t alpha, const uint16_t *x, size_t n);
-void orc_emul_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n);
-void orc_ediv_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n);
-void orc_add_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n);
-void orc_powf_bf16(const uint16_t *a, uint16_t p, uint16_t *out, size_t n);
-void orc_map_add_bf16(const uint16_t *a, uint16_t c, uint16_t *out, size_t n);
 /* B::cast default, backend/mod.rs:157-160.  Types: 0 = f32, 1 = bf16, 2 = f64. */
 void orc_cast(const void *src, int src_type, void *dst, int dst_type, size_t n);
 

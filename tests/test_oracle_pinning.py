@@ -192,10 +192,13 @@ def test_axpy_is_multiply_then_add_not_fma():
     assert fused_differs > 10
 
 
-def _exact_adam(kind, lr, b1, b2, eps, wd, steps, p0, grads):
-    """Adam / AdamW on f32 in exact arithmetic with RNE after each operation of
-    alg.rs:120-148, taking the correctly rounded sqrt for powf(x, 0.5)."""
-    p = [f32_exact(x) for x in p0]
+def _exact_adam(kind, lr, b1, b2, eps, wd, steps, p0, grads, rt=None, exact=None):
+    """Adam / AdamW in exact arithmetic with one rounding `rt` (to the element type T,
+    default f32) after each operation of alg.rs:120-148, taking the correctly rounded
+    f32 sqrt for powf(x, 0.5).  `exact` turns an input element into a Fraction."""
+    rt = rt or r32
+    exact = exact or f32_exact
+    p = [exact(x) for x in p0]
     m = [Fraction(0)] * len(p)
     v = [Fraction(0)] * len(p)
     B1, B2, LR, EPS, WD = (Fraction(x) for x in (b1, b2, lr, eps, wd))
@@ -212,21 +215,21 @@ def _exact_adam(kind, lr, b1, b2, eps, wd, steps, p0, grads):
                 a = r64(a * a)
         bc1 = r64(1 - powi(B1, t))
         bc2 = r64(1 - powi(B2, t))
-        ss = r32(r64(LR / bc1))
-        ibc2 = r32(r64(1 / bc2))
-        fb1, fomb1 = r32(B1), r32(r64(1 - B1))
-        fb2, fomb2 = r32(B2), r32(r64(1 - B2))
-        feps = r32(EPS)
-        omw = r32(1 - r32(r64(WD * LR)))
-        g = [f32_exact(x) for x in grads[t - 1]]
+        ss = rt(r64(LR / bc1))
+        ibc2 = rt(r64(1 / bc2))
+        fb1, fomb1 = rt(B1), rt(r64(1 - B1))
+        fb2, fomb2 = rt(B2), rt(r64(1 - B2))
+        feps = rt(EPS)
+        omw = rt(1 - rt(r64(WD * LR)))
+        g = [exact(x) for x in grads[t - 1]]
         for i in range(len(p)):
-            m[i] = r32(r32(m[i] * fb1) + r32(fomb1 * g[i]))
-            v[i] = r32(r32(v[i] * fb2) + r32(fomb2 * r32(g[i] * g[i])))
-            denom = r32(sqrt_r32(r32(v[i] * ibc2)) + feps)
-            upd = r32(r32(m[i] * ss) / denom)
+            m[i] = rt(rt(m[i] * fb1) + rt(fomb1 * g[i]))
+            v[i] = rt(rt(v[i] * fb2) + rt(fomb2 * rt(g[i] * g[i])))
+            denom = rt(rt(sqrt_r32(rt(v[i] * ibc2))) + feps)
+            upd = rt(rt(m[i] * ss) / denom)
             if kind == "adamw":
-                p[i] = r32(p[i] * omw)
-            p[i] = r32(p[i] + (-upd))
+                p[i] = rt(p[i] * omw)
+            p[i] = rt(p[i] + (-upd))
     return p, m, v
 
 
@@ -655,3 +658,66 @@ def test_powf_half_of_negative_zero_and_minus_infinity():
         finally:
             O.set_pow_mode(O.POW_LIBM)
         assert np.array_equal(out.view(np.uint32), np.array([0.0, np.inf, np.inf, 0.0, 2.0], dtype=np.float32).view(np.uint32)), mode
+
+
+@pytest.mark.parametrize("kind", ["adam", "adamw"])
+def test_bf16_adam_chain_bit_exact_against_exact_arithmetic(kind):
+    """Optimizer<bf16>: the same chain with every result -- scalars included -- rounded to
+    f32 and then to bf16 (T::from_f64 = from_f32(v as f32); each operation = f32 operation +
+    from_f32)."""
+    rng = np.random.default_rng(12)
+    n, steps = 16, 4
+    lr, b1, b2, eps, wd = 1e-2, 0.9, 0.95, 1e-8, 0.1
+    rt = lambda q: rbf(r32(q))
+    p0 = O.bf16_from_f32((rng.standard_normal(n) * 0.5).astype(np.float32))
+    grads = [O.bf16_from_f32((rng.standard_normal(n) * 1e-2).astype(np.float32)) for _ in range(steps)]
+    pe, me, ve = _exact_adam(kind, lr, b1, b2, eps, wd, steps, p0, grads, rt=rt, exact=_bf_exact)
+    p, m, v = [p0.copy()], [np.zeros(n, np.uint16)], [np.zeros(n, np.uint16)]
+    meta = O.adam_meta(lr, b1, b2, eps) if kind == "adam" else O.adamw_meta(lr, b1, b2, eps, wd)
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        for t in range(steps):
+            O.adam_step(meta, p, [grads[t]], m, v)
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+    for i in range(n):
+        assert _bf_exact(m[0][i]) == me[i], f"m[{i}]"
+        assert _bf_exact(v[0][i]) == ve[i], f"v[{i}]"
+        assert _bf_exact(p[0][i]) == pe[i], f"p[{i}]"
+    assert meta.step_count == steps and any(x != 0 for x in m[0]) and any(x != 0 for x in v[0])
+
+
+def test_bf16_sgd_scaler_and_clip_in_exact_arithmetic():
+    rt = lambda q: rbf(r32(q))
+    rng = np.random.default_rng(13)
+    n = 32
+    p0 = O.bf16_from_f32((rng.standard_normal(n) * 0.5).astype(np.float32))
+    g0 = O.bf16_from_f32((rng.standard_normal(n) * 3.0).astype(np.float32))
+    # Sgd with momentum and weight decay (alg.rs:403-414), two steps
+    lr, mom, wd = 0.05, 0.9, 0.01
+    p, vel = [p0.copy()], [np.zeros(n, np.uint16)]
+    meta = O.sgd_meta(lr, momentum=mom, weight_decay=wd)
+    pe, ve = [_bf_exact(x) for x in p0], [Fraction(0)] * n
+    flr, fmom, fwd = rt(Fraction(lr)), rt(Fraction(mom)), rt(Fraction(wd))
+    for _ in range(2):
+        O.sgd_step(meta, p, [g0], vel)
+        for i in range(n):
+            ge = rt(_bf_exact(g0[i]) + rt(pe[i] * fwd))
+            ve[i] = rt(rt(ve[i] * fmom) + ge)
+            pe[i] = rt(pe[i] + rt(-flr * ve[i]))
+    for i in range(n):
+        assert _bf_exact(p[0][i]) == pe[i] and _bf_exact(vel[0][i]) == ve[i], i
+    # unscale by a scale that is not a power of two, then clip (core.rs:355,379; trainer.rs:504-521)
+    g = [g0.copy()]
+    st = O.ScalerState(3.0, 2.0, 0.5, 2, 0)
+    assert O.scaler_unscale_and_update(st, g)
+    inv = rt(r64(Fraction(1) / 3))
+    un = [rt(_bf_exact(x) * inv) for x in g0]
+    assert [_bf_exact(x) for x in g[0]] == un
+    norm = O.clip_grad_norm(g, 0.5)
+    total = Fraction(0)
+    for x in un:
+        total = r64(total + r64(x * x))
+    assert abs(norm - math.sqrt(float(total))) <= 1e-12 * norm
+    c = rt(r64(Fraction(0.5) / Fraction(norm)))
+    assert [_bf_exact(x) for x in g[0]] == [rt(x * c) for x in un]
