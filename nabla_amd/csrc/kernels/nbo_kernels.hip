@@ -70,12 +70,10 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // gets the quiet bit, everything else rounds to nearest even).
 DEV float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
-DEV uint32_t f32_to_bf16_bits(float f)
-{
-    uint32_t x = __float_as_uint(f);
-    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (x >> 16) | 0x0040u;
-    return (x + 0x7FFFu + ((x >> 16) & 1u)) >> 16;
-}
+// gfx950 converts f32 to bf16 in hardware (v_cvt_pk_bf16_f32); the instruction gives
+// half::bf16::from_f32's result for every one of the 2^32 inputs, NaN payloads included
+// (the rule: `(x >> 16) | 0x40` for NaN, else `(x + 0x7FFF + ((x >> 16) & 1)) >> 16`).
+DEV uint32_t f32_to_bf16_bits(float f) { return (uint32_t)__builtin_bit_cast(unsigned short, (__bf16)f); }
 
 DEV bool nonfinite_f32(float f) { return (__float_as_uint(f) & 0x7F800000u) == 0x7F800000u; }
 DEV bool nonfinite_f64(double d)
@@ -141,7 +139,7 @@ template <> struct Traits<NBO_F64> {
 
 template <> struct Traits<NBO_PBF16> {
     typedef BF T;
-    enum { VEC = 4, SBYTES = 2 };
+    enum { VEC = 8, SBYTES = 2 };
 };
 
 // arena (engine-owned, always 16-byte aligned) vectors of T
@@ -166,18 +164,24 @@ DEV void st_state(double *p, const double (&x)[2])
     NBO_STORE(v, GLOBAL_PTR(f64x2, p));
 }
 
-DEV void ld_state(const BF *p, BF (&x)[4])
+DEV void ld_state(const BF *p, BF (&x)[8])
 {
-    u32x2 v = NBO_LOAD(GLOBAL_PTR(const u32x2, p));
-    x[0] = bf_from_bits(v.x & 0xFFFFu); x[1] = bf_from_bits(v.x >> 16);
-    x[2] = bf_from_bits(v.y & 0xFFFFu); x[3] = bf_from_bits(v.y >> 16);
+    const u32x4 v = NBO_LOAD(GLOBAL_PTR(const u32x4, p));
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        x[2 * k] = bf_from_bits(w[k] & 0xFFFFu);
+        x[2 * k + 1] = bf_from_bits(w[k] >> 16);
+    }
 }
-DEV void st_state(BF *p, const BF (&x)[4])
+DEV void st_state(BF *p, const BF (&x)[8])
 {
-    u32x2 v;
+    u32x4 v;
     v.x = (uint32_t)x[0].bits | ((uint32_t)x[1].bits << 16);
     v.y = (uint32_t)x[2].bits | ((uint32_t)x[3].bits << 16);
-    NBO_STORE(v, GLOBAL_PTR(u32x2, p));
+    v.z = (uint32_t)x[4].bits | ((uint32_t)x[5].bits << 16);
+    v.w = (uint32_t)x[6].bits | ((uint32_t)x[7].bits << 16);
+    NBO_STORE(v, GLOBAL_PTR(u32x4, p));
 }
 
 // caller tensors: vector of VEC storage elements at byte address p
@@ -215,8 +219,8 @@ template <> struct IO<NBO_BF16> {
 };
 
 template <> struct IO<NBO_PBF16> {
-    DEV void ldv(const char *p, BF (&x)[4]) { ld_state((const BF *)p, x); }
-    DEV void stv(char *p, const BF (&x)[4]) { st_state((BF *)p, x); }
+    DEV void ldv(const char *p, BF (&x)[8]) { ld_state((const BF *)p, x); }
+    DEV void stv(char *p, const BF (&x)[8]) { st_state((BF *)p, x); }
     DEV BF ld1(const char *p) { return bf_from_bits(*GLOBAL_PTR(const uint16_t, p)); }
     DEV void st1(char *p, BF x) { *GLOBAL_PTR(uint16_t, p) = x.bits; }
 };

@@ -181,3 +181,20 @@ def test_adamw_as_a_chain_of_primitives_equals_the_fused_kernel(gpu):
         H.assert_bits_equal(H.host_list(p), H.host_list(fused_p), f"params after step {step}")
         H.assert_bits_equal(H.host_list(m), H.host_list(opt.moments()[0]), f"m after step {step}")
         H.assert_bits_equal(H.host_list(v), H.host_list(opt.moments()[1]), f"v after step {step}")
+
+
+def test_f32_to_bf16_rounding_for_every_high_half_and_boundary_low_half(gpu):
+    """The device narrows f32 to bf16 with gfx950's conversion instruction.  Every 16-bit
+    high half (all signs, exponents, top mantissa bits, infinities and NaNs) is combined
+    with the low halves that decide a rounding -- 0, 1, just below the tie, the tie, just
+    above it, all ones -- and must give half::bf16::from_f32's bits, NaN payloads included."""
+    hi = np.arange(1 << 16, dtype=np.uint32) << 16
+    lows = np.array([0x0000, 0x0001, 0x7FFF, 0x8000, 0x8001, 0xFFFF], dtype=np.uint32)
+    bits = (hi[:, None] | lows[None, :]).reshape(-1)
+    x = bits.view(np.float32)
+    n = x.size
+    src = H.to_dev(x, (1, n))
+    dst = H.to_dev(np.zeros(n, dtype=np.uint16), (1, n))
+    B.cast([src], [dst])
+    got, want = H.to_host(dst), O.bf16_from_f32(x)
+    assert np.array_equal(got, want), f"first difference at input bits {bits[np.nonzero(got != want)[0][0]]:#010x}"
