@@ -8,13 +8,17 @@
 //   Sgd / Adam / AdamW (alg.rs)         -> same names, same builder setters
 //   trait OptimState  (core.rs:64-79)   -> kind, state_read / state_write, meta, load_meta
 //   GradScaler        (core.rs:334-413) -> same methods
-//   clip_grad_norm, zero_grad, scale_grad -> free functions
+//   clip_grad_norm, zero_grad, scale_grad, has_non_finite, accumulate -> free functions
+//   LrSchedule / lr_at_step (core.rs:81-173)        -> same names (host arithmetic, f64)
+//   Trainer's loop body after backward (trainer.rs:216-291) -> TrainerTail, GradNanPolicy
+//   Backend primitives (nabla-core backend/mod.rs:82-216, 275-279) -> namespace backend
 // Where the reference panics (assert_eq! on list lengths, shape asserts) this throws
 // nabla::optim::Panic with the reference's message; where it returns Err(String) this
 // throws nabla::optim::StateError.
 #ifndef NABLA_OPTIM_HPP
 #define NABLA_OPTIM_HPP
 
+#include <cmath>
 #include <cstddef>
 #include <cstdint>
 #include <stdexcept>
@@ -335,6 +339,187 @@ inline double clip_grad_norm(TensorList &grads, double max_norm)
 inline void zero_grad(TensorList &grads) { check(nbo_zero_grad(grads.handle())); }
 inline void scale_grad(TensorList &grads, double factor) { check(nbo_scale_grad(grads.handle(), factor)); }
 inline void sync() { check(nbo_sync()); }
+// Trainer::has_non_finite, trainer.rs:387-400
+inline bool has_non_finite(TensorList &grads)
+{
+    int found = 0;
+    check(nbo_has_non_finite(grads.handle(), &found));
+    return found != 0;
+}
+// buf[i] = &buf[i] + g, trainer.rs:262-266
+inline void accumulate(TensorList &accum, TensorList &grads, bool zero_grads = false)
+{
+    check(nbo_accumulate(accum.handle(), grads.handle(), zero_grads ? 1 : 0));
+}
+
+// ---- LrSchedule (optim/core.rs:81-173): host arithmetic in f64 -------------------------
+struct LrSchedule {
+    enum Kind { Cosine, Linear, OneCycle, Step } kind;
+    uint64_t warmup_steps = 0, total_steps = 0, step_size = 0;
+    double min_lr = 0.0, max_lr = 0.0, pct_start = 0.0, gamma = 0.0;
+    static LrSchedule cosine(uint64_t warmup, uint64_t total, double min_lr)
+    {
+        LrSchedule s{Cosine};
+        s.warmup_steps = warmup, s.total_steps = total, s.min_lr = min_lr;
+        return s;
+    }
+    static LrSchedule linear(uint64_t warmup, uint64_t total)
+    {
+        LrSchedule s{Linear};
+        s.warmup_steps = warmup, s.total_steps = total;
+        return s;
+    }
+    static LrSchedule one_cycle(double max_lr, uint64_t total, double pct_start)
+    {
+        LrSchedule s{OneCycle};
+        s.max_lr = max_lr, s.total_steps = total, s.pct_start = pct_start;
+        return s;
+    }
+    static LrSchedule step(uint64_t step_size, double gamma)
+    {
+        LrSchedule s{Step};
+        s.step_size = step_size, s.gamma = gamma;
+        return s;
+    }
+};
+
+namespace detail {
+// f64::powi as compiler-rt's __powidf2: square-and-multiply from the low bit
+inline double powi(double a, int n)
+{
+    const bool recip = n < 0;
+    unsigned b = recip ? 0u - (unsigned)n : (unsigned)n;
+    double r = 1.0;
+    for (;;) {
+        if (b & 1u) r *= a;
+        b >>= 1;
+        if (b == 0) break;
+        a *= a;
+    }
+    return recip ? 1.0 / r : r;
+}
+inline double warmup_lr(double base_lr, uint64_t step, uint64_t warmup)
+{
+    return base_lr * (double)step / (double)(warmup > 1 ? warmup : 1);
+}
+inline double decay_progress(uint64_t step, uint64_t start, uint64_t total)
+{
+    const uint64_t d = total - start; // usize subtraction, as the reference writes it
+    return (double)(step - start) / (double)(d > 1 ? d : 1);
+}
+inline double cosine_decay(double high, double low, double progress)
+{
+    return low + 0.5 * (high - low) * (1.0 + std::cos(3.14159265358979323846264338327950288 * progress));
+}
+} // namespace detail
+
+inline double lr_at_step(const LrSchedule &s, double base_lr, uint64_t step)
+{
+    using namespace detail;
+    switch (s.kind) {
+    case LrSchedule::Cosine:
+        if (step < s.warmup_steps) return warmup_lr(base_lr, step, s.warmup_steps);
+        return cosine_decay(base_lr, s.min_lr, decay_progress(step, s.warmup_steps, s.total_steps));
+    case LrSchedule::Linear: {
+        if (step < s.warmup_steps) return warmup_lr(base_lr, step, s.warmup_steps);
+        const double p = 1.0 - decay_progress(step, s.warmup_steps, s.total_steps);
+        return base_lr * (p > 0.0 ? p : 0.0);
+    }
+    case LrSchedule::OneCycle: {
+        const uint64_t up = (uint64_t)((double)s.total_steps * s.pct_start);
+        if (step < up) return base_lr + (s.max_lr - base_lr) * (double)step / (double)(up > 1 ? up : 1);
+        return cosine_decay(s.max_lr, base_lr, decay_progress(step, up, s.total_steps));
+    }
+    default: {
+        const uint64_t sz = s.step_size > 1 ? s.step_size : 1;
+        return base_lr * powi(s.gamma, (int)(step / sz));
+    }
+    }
+}
+
+// ---- Backend primitives on tensor lists (nbo_backend_apply / nbo_backend_cast) ----------
+namespace backend {
+inline void apply(nbo_backend_op op, TensorList &out, TensorList *a, TensorList *b, double s)
+{
+    check(nbo_backend_apply(op, out.handle(), a ? a->handle() : nullptr, b ? b->handle() : nullptr, s));
+}
+inline void scale(TensorList &a, double s, TensorList &out) { apply(NBO_BACKEND_SCALE, out, &a, nullptr, s); }
+inline void axpy_inplace(TensorList &y, double alpha, TensorList &x) { apply(NBO_BACKEND_AXPY, y, &x, nullptr, alpha); }
+inline void add(TensorList &a, TensorList &b, TensorList &out) { apply(NBO_BACKEND_ADD, out, &a, &b, 0.0); }
+inline void emul(TensorList &a, TensorList &b, TensorList &out) { apply(NBO_BACKEND_EMUL, out, &a, &b, 0.0); }
+inline void ediv(TensorList &a, TensorList &b, TensorList &out) { apply(NBO_BACKEND_EDIV, out, &a, &b, 0.0); }
+inline void powf(TensorList &a, double p, TensorList &out) { apply(NBO_BACKEND_POWF, out, &a, nullptr, p); }
+inline void map_add(TensorList &a, double c, TensorList &out) { apply(NBO_BACKEND_ADD_SCALAR, out, &a, nullptr, c); }
+inline void zeros(TensorList &out) { apply(NBO_BACKEND_ZEROS, out, nullptr, nullptr, 0.0); }
+inline void clone_storage(TensorList &a, TensorList &out) { apply(NBO_BACKEND_CLONE, out, &a, nullptr, 0.0); }
+inline void cast(TensorList &src, TensorList &dst) { check(nbo_backend_cast(dst.handle(), src.handle())); }
+} // namespace backend
+
+// ---- the Trainer's loop body after backward (trainer.rs:216-291) --------------------------
+enum class GradNanPolicy { Skip, Stop }; // trainer.rs:403-406
+struct TrainError : std::runtime_error { // TrainError::EvalError
+    using std::runtime_error::runtime_error;
+};
+
+// Per micro-batch: scaler -> nan policy -> accumulate -> (every grad_accum-th) schedule,
+// clip, step, zero.  `accum` is caller-provided zero-filled storage shaped like the
+// gradients (the reference allocates it; this library allocates nothing per step).
+class TrainerTail {
+public:
+    TrainerTail(Optimizer &optimizer, TensorList &params, TensorList &accum)
+        : opt_(optimizer), params_(params), accum_(accum)
+    {
+    }
+    TrainerTail &with_schedule(const LrSchedule &s, double base_lr) { schedule_ = s, base_lr_ = base_lr, has_schedule_ = true; return *this; }
+    TrainerTail &with_grad_scaler(GradScaler &s) { scaler_ = &s; return *this; }
+    TrainerTail &with_grad_accum(uint64_t steps) { grad_accum_ = steps > 1 ? steps : 1; return *this; }
+    TrainerTail &with_nan_policy(GradNanPolicy p) { policy_ = p, has_policy_ = true; return *this; }
+    TrainerTail &with_grad_clip(double max_norm) { grad_clip_ = max_norm > 0.0 ? max_norm : 0.0; return *this; }
+    uint64_t step() const { return step_; }
+    double loss_scale() { return scaler_ ? scaler_->scale_factor() : 1.0; } // trainer.rs:218-221
+
+    // returns true if the optimizer stepped; grads are modified in place like the reference's
+    bool after_backward(TensorList &grads)
+    {
+        if (scaler_ && !scaler_->unscale_and_update(grads)) return drop(); // :230-237
+        if (has_policy_ && has_non_finite(grads)) {                        // :239-251
+            if (policy_ == GradNanPolicy::Skip) return drop();
+            throw TrainError("non-finite gradient");
+        }
+        if (accum_count_ == 0 && dirty_) { // a dropped accumulation starts again from zeros (:253-260)
+            zero_grad(accum_);
+            dirty_ = false;
+        }
+        accumulate(accum_, grads); // :262-266
+        dirty_ = true;
+        accum_count_ += 1;
+        if (accum_count_ < grad_accum_) return false;
+        if (has_schedule_) opt_.set_lr(lr_at_step(schedule_, base_lr_, step_)); // :270-273
+        if (grad_clip_ > 0.0) clip_grad_norm(accum_, grad_clip_);              // :274-278
+        opt_.step(params_, accum_);                                            // :279-283
+        accum_count_ = 0;
+        zero_grad(accum_); // :285-290
+        dirty_ = false;
+        step_ += 1;
+        return true;
+    }
+
+private:
+    bool drop()
+    {
+        accum_count_ = 0; // accum_grads = None: the buffer is cleared before its next use
+        return false;
+    }
+    Optimizer &opt_;
+    TensorList &params_;
+    TensorList &accum_;
+    GradScaler *scaler_ = nullptr;
+    LrSchedule schedule_{LrSchedule::Linear};
+    double base_lr_ = 0.0, grad_clip_ = 0.0;
+    bool has_schedule_ = false, has_policy_ = false, dirty_ = false;
+    GradNanPolicy policy_ = GradNanPolicy::Skip;
+    uint64_t grad_accum_ = 1, accum_count_ = 0, step_ = 0;
+};
 
 } // namespace optim
 } // namespace nabla

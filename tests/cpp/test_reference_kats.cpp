@@ -147,6 +147,71 @@ static void weight_decay_exclusion()  // optim.rs:140-165, the two groups as two
     EXPECT(std::fabs(bias.get() - 3.0) < 1e-10);
 }
 
+static void lr_schedules()  // optim.rs:83-118
+{
+    const LrSchedule lin = LrSchedule::linear(0, 10);
+    EXPECT(std::fabs(lr_at_step(lin, 1.0, 0) - 1.0) < 1e-10);
+    EXPECT(lr_at_step(lin, 1.0, 10) <= 1e-10);
+    const LrSchedule stp = LrSchedule::step(2, 0.1);
+    EXPECT(std::fabs(lr_at_step(stp, 1.0, 0) - 1.0) < 1e-10);
+    EXPECT(std::fabs(lr_at_step(stp, 1.0, 2) - 0.1) < 1e-10);
+    EXPECT(std::fabs(lr_at_step(stp, 1.0, 4) - 0.01) < 1e-10);
+    const LrSchedule one = LrSchedule::one_cycle(1.0, 10, 0.5);
+    EXPECT(lr_at_step(one, 0.1, 3) > 0.1);
+    const LrSchedule cosine = LrSchedule::cosine(10, 110, 0.1);  // closed forms: ramp, mid-point, end
+    EXPECT(std::fabs(lr_at_step(cosine, 1.0, 5) - 0.5) < 1e-12);
+    EXPECT(std::fabs(lr_at_step(cosine, 1.0, 60) - 0.55) < 1e-12);
+    EXPECT(std::fabs(lr_at_step(cosine, 1.0, 110) - 0.1) < 1e-12);
+}
+
+static void nan_policy_skip_drops_step()  // trainer.rs tests :148-169
+{
+    Mat w({1.0}), buf({0.0}), nan_grad({std::numeric_limits<double>::quiet_NaN()}), good({1.0});
+    Sgd opt(0.1, {{1, 1}}, NBO_DT_F64);
+    TensorList params({w.tensor()}), accum({buf.tensor()}), bad({nan_grad.tensor()}), ok({good.tensor()});
+    TrainerTail trainer(opt, params, accum);
+    trainer.with_nan_policy(GradNanPolicy::Skip);
+    EXPECT(!trainer.after_backward(bad));
+    EXPECT(trainer.step() == 0 && w.get() == 1.0);
+    EXPECT(trainer.after_backward(ok));  // and a finite gradient afterwards steps
+    EXPECT(trainer.step() == 1 && std::fabs(w.get() - 0.9) < 1e-12);
+    TrainerTail stopper(opt, params, accum);
+    stopper.with_nan_policy(GradNanPolicy::Stop);
+    bool raised = false;
+    try {
+        stopper.after_backward(bad);
+    } catch (const TrainError &e) {
+        raised = std::string(e.what()) == "non-finite gradient";
+    }
+    EXPECT(raised);
+}
+
+static void trainer_accumulates_then_clips_and_steps()  // trainer.rs:253-291 on hand-checked values
+{
+    Mat w({1.0}), buf({0.0}), g1({3.0}), g2({5.0});
+    Sgd opt(0.5, {{1, 1}}, NBO_DT_F64);
+    TensorList params({w.tensor()}), accum({buf.tensor()}), a({g1.tensor()}), b({g2.tensor()});
+    TrainerTail trainer(opt, params, accum);
+    trainer.with_grad_accum(2).with_grad_clip(4.0).with_schedule(LrSchedule::step(1, 0.5), 0.5);
+    EXPECT(!trainer.after_backward(a));
+    EXPECT(buf.get() == 3.0 && w.get() == 1.0);
+    EXPECT(trainer.after_backward(b));  // buf = 8, clipped to 4, lr(step 0) = 0.5: w = 1 - 0.5 * 4
+    EXPECT(std::fabs(w.get() + 1.0) < 1e-12 && buf.get() == 0.0 && trainer.step() == 1);
+    EXPECT(!trainer.after_backward(a));
+    EXPECT(trainer.after_backward(a));  // buf = 6 -> 4, lr(step 1) = 0.25: w = -1 - 0.25 * 4
+    EXPECT(std::fabs(w.get() + 2.0) < 1e-12 && trainer.step() == 2);
+}
+
+static void backend_axpy_is_multiply_then_add()  // cpu/mod.rs:216-223
+{
+    Mat y({1.0, 0.1}), x({3.0, 0.3});
+    TensorList ly({y.tensor()}), lx({x.tensor()});
+    backend::axpy_inplace(ly, 0.1, lx);
+    EXPECT(y.get(0) == 1.0 + 0.1 * 3.0);
+    const double prod = 0.1 * 0.3;  // rounded product, then rounded sum
+    EXPECT(y.get(1) == 0.1 + prod);
+}
+
 static void panics_and_errors()  // alg.rs:110-119, 531-545; tensor/ops.rs:638-646
 {
     Mat p({1.0}), g({1.0}), g2({1.0, 2.0});
@@ -210,6 +275,10 @@ int main()
                  {"grad_scaler_detects_inf", grad_scaler_detects_inf},
                  {"clip_grad_norm_scales", clip_grad_norm_scales},
                  {"group_optimizer_weight_decay_exclusion", weight_decay_exclusion},
+                 {"lr_schedules", lr_schedules},
+                 {"nan_policy_skip_drops_step", nan_policy_skip_drops_step},
+                 {"trainer_accumulates_then_clips_and_steps", trainer_accumulates_then_clips_and_steps},
+                 {"backend_axpy_is_multiply_then_add", backend_axpy_is_multiply_then_add},
                  {"panics_and_errors", panics_and_errors}};
     try {
         check(nbo_init());

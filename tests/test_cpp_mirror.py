@@ -18,4 +18,4 @@ def test_cpp_replay_of_reference_tests(gpu):
     r = subprocess.run([BIN], capture_output=True, text=True, timeout=120)
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count("ok    ") == 9 and "0 failure(s)" in r.stdout
+    assert r.stdout.count("ok    ") == 13 and "0 failure(s)" in r.stdout

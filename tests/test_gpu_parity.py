@@ -243,6 +243,20 @@ def test_mixed_adamw_no_clip_no_scaler(gpu):
     _check_mixed(dev, refs, 1e-3, 4)
 
 
+def test_fused_steps_are_reproducible_run_to_run(gpu):
+    """The norm is reduced in a fixed order (fixed grid, butterfly inside a wave, waves
+    and blocks in index order), so two runs over the same inputs agree in every bit,
+    the reported norms included."""
+    shapes = RAGGED + [(257, 1023), (1, 70001)]
+    state = dict(scale=1024.0, growth_factor=2.0, backoff_factor=0.5, growth_interval=3, consecutive_ok=0)
+    a, _ = _mixed_case(shapes, 6, 2e-4, 0.1, 0.5, state, 1e-3, seed=9)
+    b, _ = _mixed_case(shapes, 6, 2e-4, 0.1, 0.5, state, 1e-3, seed=9)
+    for key in ("p", "w", "m", "v"):
+        H.assert_bits_equal(a[key], b[key], key)
+    assert [np.float64(t[3]).tobytes() for t in a["trace"]] == [np.float64(t[3]).tobytes() for t in b["trace"]]
+    assert a["trace"] == b["trace"]
+
+
 def test_dynamic_loss_scale_ragged_trace_bit_exact(gpu):
     """Config 4 at reduced tensor count: ragged sizes, growth every 4 clean steps,
     inf/NaN injected every 4th step (scale only backs off) and, in a second run,
