@@ -217,3 +217,54 @@ def test_ragged_4096_dynamic_scale_64_steps(gpu):
     H.assert_bits_equal(H.host_list(v), ref_v, "v")
     H.assert_bits_equal(H.host_list([opt.read_state(f"w{i}") for i in range(len(sizes))]), ref_w, "master")
     H.assert_bits_equal([H.to_host(flat_p)], [ref_p_flat], "bf16 params")
+
+
+def test_one_tensor_longer_than_2_pow_32_elements(gpu):
+    """Element offsets are 64-bit throughout (the reference's own kernels take
+    `unsigned n`).  One bf16 tensor of 2^32 + 3 * 8192 + 5 elements -- its chunk indices
+    and byte offsets pass 2^32 and 2^33 -- plus a small tensor after it, through two fused
+    AdamW steps (bf16 arithmetic, so the state stays at 26 GB): slices at the head,
+    around element 2^32, in the last full chunk and in the ragged tail must match the
+    oracle bit for bit, and the global norm an independent f64 reduction."""
+    import torch
+
+    n_big = (1 << 32) + 3 * 8192 + 5
+    shapes = [(1, n_big), (3, 1000)]
+    cuts = [[(0, SL), ((1 << 32) - SL // 2, (1 << 32) + SL // 2), (n_big - 5 - 8192, n_big - 5 - 8192 + SL),
+             (n_big - SL, n_big)], [(0, 3000)]]
+
+    def take(t, k):
+        flat = t.reshape(-1)
+        return H.to_host(torch.cat([flat[a:b] for a, b in cuts[k]]))
+
+    torch.manual_seed(77)
+    params = [(torch.randn(s, device=gpu, dtype=torch.bfloat16) * 0.5) for s in shapes]
+    ref_p = [take(t, k) for k, t in enumerate(params)]
+    ref_m, ref_v = [np.zeros_like(a) for a in ref_p], [np.zeros_like(a) for a in ref_p]
+    opt = nb.AdamW.new(1e-2, shapes, dtype="bf16").beta2(0.95).weight_decay(0.1)
+    meta = O.adamw_meta(1e-2, 0.9, 0.95, 1e-8, 0.1)
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        for step in range(2):
+            grads = [(torch.randn(s, device=gpu, dtype=torch.bfloat16) * 1e-2) for s in shapes]
+            sumsq = sum((g.double() ** 2).sum() for g in grads)
+            opt.fused_step(params, grads, max_norm=1.0)
+            info = opt.last_step()
+            norm_ref = float(torch.sqrt(sumsq))
+            assert info.norm == pytest.approx(norm_ref, rel=1e-9) and info.clipped == 1
+            assert info.step_count == step + 1
+            # the clip factor is a bf16 value; the slices then follow the reference's chain
+            g_sl = [take(g, k) for k, g in enumerate(grads)]
+            c = 1.0 / info.norm
+            g_sl = [O.scale(a, c) for a in g_sl]  # g.map(|x| x * scale_t), trainer.rs:519
+            O.adam_step(meta, ref_p, g_sl, ref_m, ref_v)
+            del grads
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+    m = [opt.read_state("m0"), opt.read_state("m1")]
+    v = [opt.read_state("v0"), opt.read_state("v1")]
+    H.assert_bits_equal([take(t, k) for k, t in enumerate(params)], ref_p, "param slices")
+    H.assert_bits_equal([take(t, k) for k, t in enumerate(m)], ref_m, "m slices")
+    H.assert_bits_equal([take(t, k) for k, t in enumerate(v)], ref_v, "v slices")
+    # a chunk nobody should have touched twice or skipped: every element moved
+    assert bool((params[0].reshape(-1)[(1 << 32) - 8:(1 << 32) + 8] != 0).all())
