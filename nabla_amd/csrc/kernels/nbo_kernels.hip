@@ -952,26 +952,72 @@ NBO_EW_KERNEL(nbo_ew_f64, NBO_F64)
 // U::from_f64(x.to_f64()) per element.  Widening is exact; f64 -> f32 rounds to nearest
 // even; anything -> bf16 goes through f32 first (bf16::from_f64 = from_f32(v as f32),
 // scalar/mod.rs:338-340), so f64 -> bf16 rounds twice, as the reference does.
-DEV double cast_load(const char *p, uint32_t type, uint64_t e)
+template <int ST> DEV double cast_load1(const char *p, uint64_t e)
 {
-    if (type == NBO_F32) return (double)IO<NBO_F32>::ld1(p + e * 4);
-    if (type == NBO_BF16) return (double)IO<NBO_BF16>::ld1(p + e * 2);
-    return IO<NBO_F64>::ld1(p + e * 8);
+    return (double)IO<ST>::ld1(p + e * Traits<ST>::SBYTES);
+}
+template <int ST> DEV void cast_store1(char *p, uint64_t e, double v)
+{
+    typedef typename Traits<ST>::T T;
+    IO<ST>::st1(p + e * Traits<ST>::SBYTES, (T)v); // (float)v rounds to nearest even; bf16 narrows once more
+}
+// four consecutive elements at element index e (a multiple of 4) of a suitably aligned tensor
+template <int ST> DEV void cast_load4(const char *p, uint64_t e, double (&v)[4])
+{
+    typedef typename Traits<ST>::T T;
+    enum { VEC = Traits<ST>::VEC };
+#pragma unroll
+    for (int h = 0; h < 4 / VEC; h++) {
+        T x[VEC];
+        IO<ST>::ldv(p + (e + h * VEC) * Traits<ST>::SBYTES, x);
+#pragma unroll
+        for (int k = 0; k < VEC; k++) v[h * VEC + k] = (double)x[k];
+    }
+}
+template <int ST> DEV void cast_store4(char *p, uint64_t e, const double (&v)[4])
+{
+    typedef typename Traits<ST>::T T;
+    enum { VEC = Traits<ST>::VEC };
+#pragma unroll
+    for (int h = 0; h < 4 / VEC; h++) {
+        T x[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; k++) x[k] = (T)v[h * VEC + k];
+        IO<ST>::stv(p + (e + h * VEC) * Traits<ST>::SBYTES, x);
+    }
+}
+
+template <int SRC, int DST> DEV void cast_body(const NboCastListArgs &a)
+{
+    enum { SS = Traits<SRC>::SBYTES, DS = Traits<DST>::SBYTES };
+    const ChunkRef c = chunk_ref(a.L, blockIdx.x);
+    const char *ps = (const char *)a.src_ptrs[c.t] + c.base * SS;
+    char *pd = (char *)a.dst_ptrs[c.t] + c.base * DS;
+    // groups of four while both addresses allow whole vectors (16 bytes at most per access)
+    const uint32_t sa = SS * 4 > 16 ? 16 : SS * 4, da = DS * 4 > 16 ? 16 : DS * 4;
+    const bool vec_ok = (((uintptr_t)ps & (sa - 1)) | ((uintptr_t)pd & (da - 1))) == 0;
+    const uint32_t nquad = vec_ok ? c.cnt / 4 : 0;
+    for (uint32_t q = threadIdx.x; q < nquad; q += NBO_BLOCK) {
+        double v[4];
+        cast_load4<SRC>(ps, (uint64_t)q * 4, v);
+        cast_store4<DST>(pd, (uint64_t)q * 4, v);
+    }
+    for (uint32_t e = nquad * 4 + threadIdx.x; e < c.cnt; e += NBO_BLOCK)
+        cast_store1<DST>(pd, e, cast_load1<SRC>(ps, e));
+}
+
+template <int SRC> DEV void cast_from(const NboCastListArgs &a)
+{
+    if (a.dst_type == NBO_F32) cast_body<SRC, NBO_F32>(a);
+    else if (a.dst_type == NBO_BF16) cast_body<SRC, NBO_BF16>(a);
+    else cast_body<SRC, NBO_F64>(a);
 }
 
 extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_cast_list(const NboCastListArgs a)
 {
-    const ChunkRef c = chunk_ref(a.L, blockIdx.x);
-    const uint32_t ssz = a.src_type == NBO_F64 ? 8 : a.src_type == NBO_F32 ? 4 : 2;
-    const uint32_t dsz = a.dst_type == NBO_F64 ? 8 : a.dst_type == NBO_F32 ? 4 : 2;
-    const char *ps = (const char *)a.src_ptrs[c.t] + c.base * ssz;
-    char *pd = (char *)a.dst_ptrs[c.t] + c.base * dsz;
-    for (uint32_t e = threadIdx.x; e < c.cnt; e += NBO_BLOCK) {
-        const double v = cast_load(ps, a.src_type, e);
-        if (a.dst_type == NBO_F64) IO<NBO_F64>::st1(pd + (uint64_t)e * 8, v);
-        else if (a.dst_type == NBO_F32) IO<NBO_F32>::st1(pd + (uint64_t)e * 4, (float)v);
-        else IO<NBO_BF16>::st1(pd + (uint64_t)e * 2, (float)v);
-    }
+    if (a.src_type == NBO_F32) cast_from<NBO_F32>(a);
+    else if (a.src_type == NBO_BF16) cast_from<NBO_BF16>(a);
+    else cast_from<NBO_F64>(a);
 }
 
 // Plain streaming copy used only to calibrate the HBM byte counters of a profile
