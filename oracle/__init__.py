@@ -197,6 +197,14 @@ def randn_f32(n: int, seed: int, sigma: float = 1.0) -> np.ndarray:
     return out
 
 
+def bench_rand_f32(n: int, state: int = 42):
+    """benchmarks/src/lib.rs:7-22; returns (values, next state)."""
+    out = np.empty(n, dtype=np.float32)
+    st = C.c_uint64(state)
+    lib().orc_bench_rand_f32(C.c_void_p(out.ctypes.data), C.c_size_t(n), C.byref(st))
+    return out, st.value
+
+
 def lr_at_step(sched: Schedule, base_lr: float, step: int) -> float:
     return lib().orc_lr_at_step(C.byref(sched), base_lr, step)
 

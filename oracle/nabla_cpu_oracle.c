@@ -100,6 +100,21 @@ void orc_randn_f64(double *out, size_t n, uint64_t seed)
     }
 }
 
+/* rand_tensor of the reference's benchmarks (benchmarks/src/lib.rs:7-22): a 64-bit LCG
+ * (Knuth's MMIX constants) whose top 31 bits, over 2^31, minus one become the value
+ * (so it lies in [-1, 0)).  *state is the
+ * thread-local SEED, 42 at program start. */
+void orc_bench_rand_f32(float *out, size_t n, uint64_t *state)
+{
+    uint64_t x = *state;
+    size_t i;
+    for (i = 0; i < n; i++) {
+        x = x * 6364136223846793005ull + 1442695040888963407ull;
+        out[i] = (float)(x >> 33) / (float)(1ull << 31) - 1.0f;
+    }
+    *state = x;
+}
+
 void orc_randn_scaled_f32(float *out, size_t n, uint64_t seed, double sigma)
 {
     double *tmp = (double *)malloc((n ? n : 1) * sizeof(double));

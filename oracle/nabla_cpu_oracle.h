@@ -68,6 +68,9 @@ void orc_cast_f32_to_bf16(const float *src, uint16_t *dst, size_t n);
  * tensor/constructors.rs:14-41,206-223. */
 void orc_randn_f64(double *out, size_t n, uint64_t seed);
 void orc_randn_scaled_f32(float *out, size_t n, uint64_t seed, double sigma);
+/* rand_tensor of the reference's benchmarks -- benchmarks/src/lib.rs:7-22.  *state is
+ * the LCG state (42 at program start), advanced by n draws. */
+void orc_bench_rand_f32(float *out, size_t n, uint64_t *state);
 
 /* OptimMeta -- optim/core.rs:53-62.  kind: 0 AdamW, 1 Adam, 2 Sgd (enum order
  * of OptimKind, core.rs:46-51). */

@@ -721,3 +721,20 @@ def test_bf16_sgd_scaler_and_clip_in_exact_arithmetic():
     assert abs(norm - math.sqrt(float(total))) <= 1e-12 * norm
     c = rt(r64(Fraction(0.5) / Fraction(norm)))
     assert [_bf_exact(x) for x in g[0]] == [rt(x * c) for x in un]
+
+
+def test_bench_lcg_rand_tensor_in_exact_arithmetic():
+    """benchmarks/src/lib.rs:7-22: x' = x * 6364136223846793005 + 1442695040888963407 mod
+    2^64; value = ((x' >> 33) as f32) / 2^31 - 1, each conversion / operation one rounding."""
+    vals, state = O.bench_rand_f32(500, 42)
+    x = 42
+    for i in range(500):
+        x = (x * 6364136223846793005 + 1442695040888963407) % (1 << 64)
+        want = r32(r32(r32(Fraction(x >> 33)) / (1 << 31)) - 1)
+        assert f32_exact(vals[i]) == want, i
+    assert state == x
+    # 31 bits over 2^31 lie in [0, 1), so the values lie in [-1, 0): as written in the reference
+    assert -1.0 <= vals.min() and vals.max() < 0.0 and abs(float(vals.mean()) + 0.5) < 0.1
+    more, _ = O.bench_rand_f32(3, state)  # the stream continues across tensors
+    x = (x * 6364136223846793005 + 1442695040888963407) % (1 << 64)
+    assert f32_exact(more[0]) == r32(r32(r32(Fraction(x >> 33)) / (1 << 31)) - 1)
