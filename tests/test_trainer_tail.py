@@ -127,3 +127,41 @@ def test_builders_follow_the_reference():
     tail = TrainerTail(nb.Sgd.new(0.1, [(1, 1)]), []).with_grad_accum(0).with_grad_clip(0.0)
     assert tail.state.grad_accum == 1 and tail.grad_clip is None and tail.loss_scale() == 1.0
     assert tail.with_grad_clip(2.5).grad_clip == 2.5 and tail.with_grad_accum(4).state.grad_accum == 4
+
+
+# ---- the reference's own Trainer tests (nabla-train/tests/trainer.rs), replayed ------------
+
+@pytest.mark.gpu
+def test_reference_train_epoch_updates_weight(gpu):
+    """trainer.rs tests :108-132: one f64 weight of 1.0, loss = mse(w, 0) so the gradient is
+    2w, Sgd(0.1), two batches -> two steps and a smaller weight (exactly 0.8, then 0.64)."""
+    w = H.to_dev(np.ones(1, dtype=np.float64), (1, 1))
+    trainer = TrainerTail(nb.Sgd.new(0.1, [(1, 1)], dtype="f64"), [w])
+    steps = 0
+    for _batch in (0, 1):
+        grad = (2.0 * w).contiguous()  # backward of mean((w - 0)^2)
+        steps += int(trainer.after_backward([grad]))
+    assert steps == 2 and trainer.state.step == 2
+    new_w = float(H.to_host(w)[0])
+    assert new_w < 1.0 and abs(new_w - 0.64) < 1e-12
+
+
+@pytest.mark.gpu
+def test_reference_checkpoint_roundtrip_with_schedule(gpu, tmp_path):
+    """trainer.rs tests :249-304: Sgd(0.1) over two 1x1 parameters, a default GradScaler, a
+    Step{1, 0.9} schedule and TrainState{2, 3, 1, Some(42)} survive save -> load."""
+    from nabla_amd import checkpoint as ck
+    from nabla_amd.schedule import ScheduleState, Step
+
+    shapes = [(1, 1), (1, 1)]
+    module = [("w", H.to_dev(np.array([1.5]), (1, 1))), ("b", H.to_dev(np.array([-0.5]), (1, 1)))]
+    opt = nb.Sgd.new(0.1, shapes, dtype="f64")
+    ck.save_checkpoint(str(tmp_path), module, opt, nb.GradScaler.new(),
+                       ScheduleState(base_lr=0.1, schedule=Step(step_size=1, gamma=0.9)),
+                       ck.TrainState(epoch=2, step=3, grad_accum=1, rng_state=42))
+    opt2, scaler2 = nb.Sgd.new(0.1, shapes, dtype="f64"), nb.GradScaler.new()
+    params, state2, schedule2 = ck.load_checkpoint(str(tmp_path), opt2, scaler2)
+    assert (state2.epoch, state2.step, state2.rng_state, state2.grad_accum) == (2, 3, 42, 1)
+    assert schedule2 is not None and schedule2.base_lr == 0.1 and schedule2.schedule == Step(1, 0.9)
+    assert [k for k, _ in params] == ["w", "b"] and float(params[0][1].reshape(-1)[0]) == 1.5
+    assert scaler2.state().scale == 65536.0 and opt2.meta().lr == 0.1
