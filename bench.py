@@ -30,7 +30,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="llama3-8b",
-                    choices=["llama3-8b", "llama-1.1b", "gpt2-small-f32", "mlp-sgd-f32", "ragged-4096"])
+                    choices=["llama3-8b", "llama-1.1b", "gpt2-small-f32", "mlp-sgd-f32", "ragged-4096",
+                             "llama-1.1b-bf16"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--zero-grads", choices=["off", "fused", "separate"], default="off",
                     help="also clear the gradients every step (trainer.rs:285-290): inside the update "
@@ -55,6 +56,9 @@ def workload(name):
     if name == "llama-1.1b":
         return dict(shapes=W.llama_1b_shapes(), mixed=True, kind="adamw", lr=2e-4, wd=0.1,
                     betas=(0.9, 0.95), scaler=True, clip=1.0, p_sigma=0.02, g_sigma=1e-3)
+    if name == "llama-1.1b-bf16":  # Optimizer<bf16>: tensors, moments and arithmetic all bf16
+        return dict(shapes=W.llama_1b_shapes(), mixed=False, pure_bf16=True, kind="adamw", lr=2e-4, wd=0.1,
+                    betas=(0.9, 0.95), scaler=True, clip=1.0, p_sigma=0.02, g_sigma=1e-3)
     if name == "ragged-4096":
         return dict(shapes=[(1, n) for n in W.ragged_sizes()], mixed=True, kind="adamw", lr=2e-4,
                     wd=0.1, betas=(0.9, 0.95), scaler=True, clip=1.0, p_sigma=0.02, g_sigma=1e-3)
@@ -66,6 +70,8 @@ def workload(name):
 
 
 def bytes_per_param(cfg):
+    if cfg.get("pure_bf16"):
+        return 14, 2  # R p, g, m, v + W p, m, v at 2 B each; norm pass R g
     if cfg["kind"] == "sgd":
         return 12, 0
     if cfg["mixed"]:
@@ -109,7 +115,17 @@ def cpu_baseline(cfg, budget_s):
     else:
         meta = O.adamw_meta(cfg["lr"], *cfg["betas"], weight_decay=cfg["wd"])
     scaler = O.default_scaler() if cfg["scaler"] else None
-    if cfg["mixed"]:
+    if cfg.get("pure_bf16"):
+        p = [O.bf16_from_f32(a) for a in master]
+        m, v = [np.zeros_like(a) for a in p], [np.zeros_like(a) for a in p]
+        g16 = [O.bf16_from_f32(a) for a in g32]
+
+        def run():  # trainer.rs:230-283 with T = bf16
+            gg = [a.copy() for a in g16]
+            if O.scaler_unscale_and_update(scaler, gg):
+                O.clip_grad_norm(gg, cfg["clip"])
+                O.adam_step(meta, p, gg, m, v)
+    elif cfg["mixed"]:
         g = [O.bf16_from_f32(a) for a in g32]
         p = [O.bf16_from_f32(a) for a in master]
         run = lambda: O.mixed_step(meta, scaler, cfg["clip"], p, g, master, m, v)  # noqa: E731
@@ -157,7 +173,8 @@ def measure(name, steps, warmup, zero_grads="off"):
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
 
-    pdt = torch.bfloat16 if cfg["mixed"] else torch.float32
+    pure = bool(cfg.get("pure_bf16"))
+    pdt = torch.bfloat16 if (cfg["mixed"] or pure) else torch.float32
     params = [torch.empty(s, dtype=pdt, device=dev) for s in shapes]
     grads = [torch.empty(s, dtype=pdt, device=dev) for s in shapes]
     if cfg["kind"] == "sgd":
@@ -165,8 +182,8 @@ def measure(name, steps, warmup, zero_grads="off"):
     elif cfg["kind"] == "adam":
         opt = nb.Adam.new(cfg["lr"], shapes).beta1(cfg["betas"][0]).beta2(cfg["betas"][1])
     else:
-        opt = nb.AdamW.new(cfg["lr"], shapes, master=cfg["mixed"]).beta1(cfg["betas"][0]) \
-            .beta2(cfg["betas"][1]).weight_decay(cfg["wd"])
+        opt = nb.AdamW.new(cfg["lr"], shapes, master=cfg["mixed"], dtype="bf16" if pure else "f32") \
+            .beta1(cfg["betas"][0]).beta2(cfg["betas"][1]).weight_decay(cfg["wd"])
     scale = 65536.0 if cfg["scaler"] else 1.0
     for i, s in enumerate(shapes):  # synthetic, random-init
         w = torch.randn(s, dtype=torch.float32, device=dev) * cfg["p_sigma"]
@@ -193,9 +210,10 @@ def measure(name, steps, warmup, zero_grads="off"):
             nb.zero_grad(glist)
 
     upd_b, nrm_b = bytes_per_param(cfg)
-    zero_b = 0 if zero_grads == "off" else (2 if cfg["mixed"] else 4)
-    dom = f"nbo_update_{'bf16' if cfg['mixed'] else 'f32'}_{cfg['kind']}"
-    names = [dom] + ([f"nbo_norm_{'bf16' if cfg['mixed'] else 'f32'}", "nbo_finalize"] if fused
+    zero_b = 0 if zero_grads == "off" else (2 if (cfg["mixed"] or pure) else 4)
+    fam = "pbf16" if pure else "bf16" if cfg["mixed"] else "f32"
+    dom = f"nbo_update_{fam}_{cfg['kind']}"
+    names = [dom] + ([f"nbo_norm_{fam}", "nbo_finalize"] if fused
                      else ([] if cfg["kind"] == "sgd" else ["nbo_prep"]))
     # A step of a few microseconds would be dominated by the event records around each
     # launch, so small workloads take their kernel durations from a second, untimed pass.
@@ -252,8 +270,9 @@ def measure(name, steps, warmup, zero_grads="off"):
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
-        "storage": "bf16 params/grads, f32 master/m/v" if cfg["mixed"] else "f32 params/grads/m/v",
+        "dtype": "bf16" if pure else "f32",
+        "storage": ("bf16 params/grads/m/v" if pure else
+                    "bf16 params/grads, f32 master/m/v" if cfg["mixed"] else "f32 params/grads/m/v"),
         "data": "synthetic (random-init parameters and gradients of the named shapes, resident in HBM)",
         "config": {"workload": name, "tensors": len(shapes), "params": n,
                    "bytes_per_param_step": upd_b + nrm_b + zero_b, "zero_grads": zero_grads,

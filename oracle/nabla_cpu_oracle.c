@@ -239,36 +239,42 @@ static float pow_f32_mode(float x, float p)
 #define RB(x) orc_bf16_from_f32(x)
 void orc_scale_bf16(const uint16_t *a, uint16_t s, uint16_t *out, size_t n)
 {
-    size_t i;
-    for (i = 0; i < n; i++) out[i] = RB(BF(a[i]) * BF(s));
+    long i, ln = (long)n;
+#pragma omp parallel for schedule(static) num_threads(g_threads) if (ln > PAR_MIN)
+    for (i = 0; i < ln; i++) out[i] = RB(BF(a[i]) * BF(s));
 }
 void orc_axpy_inplace_bf16(uint16_t *y, uint16_t alpha, const uint16_t *x, size_t n)
 {
-    size_t i;
-    for (i = 0; i < n; i++) {
+    long i, ln = (long)n;
+#pragma omp parallel for schedule(static) num_threads(g_threads) if (ln > PAR_MIN)
+    for (i = 0; i < ln; i++) {
         uint16_t t = RB(BF(alpha) * BF(x[i])); /* alpha * xi is a bf16 value */
         y[i] = RB(BF(y[i]) + BF(t));
     }
 }
 void orc_emul_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n)
 {
-    size_t i;
-    for (i = 0; i < n; i++) out[i] = RB(BF(a[i]) * BF(b[i]));
+    long i, ln = (long)n;
+#pragma omp parallel for schedule(static) num_threads(g_threads) if (ln > PAR_MIN)
+    for (i = 0; i < ln; i++) out[i] = RB(BF(a[i]) * BF(b[i]));
 }
 void orc_ediv_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n)
 {
-    size_t i;
-    for (i = 0; i < n; i++) out[i] = RB(BF(a[i]) / BF(b[i]));
+    long i, ln = (long)n;
+#pragma omp parallel for schedule(static) num_threads(g_threads) if (ln > PAR_MIN)
+    for (i = 0; i < ln; i++) out[i] = RB(BF(a[i]) / BF(b[i]));
 }
 void orc_add_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n)
 {
-    size_t i;
-    for (i = 0; i < n; i++) out[i] = RB(BF(a[i]) + BF(b[i]));
+    long i, ln = (long)n;
+#pragma omp parallel for schedule(static) num_threads(g_threads) if (ln > PAR_MIN)
+    for (i = 0; i < ln; i++) out[i] = RB(BF(a[i]) + BF(b[i]));
 }
 void orc_powf_bf16(const uint16_t *a, uint16_t p, uint16_t *out, size_t n)
 {
-    size_t i;
-    for (i = 0; i < n; i++) out[i] = RB(pow_f32_mode(BF(a[i]), BF(p)));
+    long i, ln = (long)n;
+#pragma omp parallel for schedule(static) num_threads(g_threads) if (ln > PAR_MIN)
+    for (i = 0; i < ln; i++) out[i] = RB(pow_f32_mode(BF(a[i]), BF(p)));
 }
 void orc_map_add_bf16(const uint16_t *a, uint16_t c, uint16_t *out, size_t n)
 {
