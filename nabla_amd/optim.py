@@ -100,6 +100,19 @@ class TensorList:
     def key(self):
         return tuple((t.data_ptr(), s) for t, s in zip(self.tensors, self.shapes))
 
+    def rebind(self, tensors: Sequence) -> None:
+        """Point the list at other tensors of the same shapes and dtype: only the address
+        table is uploaded again (nbo_list_set_ptrs), the descriptor stays."""
+        tensors = list(tensors)
+        if [_shape2(t) for t in tensors] != self.shapes or any(_dtype_code(t) != self.dtype for t in tensors):
+            raise ValueError("rebind needs tensors of the list's shapes and dtype")
+        for t in tensors:
+            if hasattr(t, "is_contiguous") and not t.is_contiguous():
+                raise ValueError("tensors must be contiguous (row-major, as in the reference)")
+        ptrs = (C.c_void_p * max(len(tensors), 1))(*[t.data_ptr() for t in tensors])
+        _call(_lib.load().nbo_list_set_ptrs(self._h, ptrs))
+        self.tensors = tensors
+
     def __len__(self):
         return len(self.tensors)
 
@@ -127,6 +140,10 @@ class _ListCache:
                 a is b or (a.data_ptr() == b.data_ptr() and _shape2(a) == _shape2(b)
                            and a.dtype == b.dtype)
                 for a, b in zip(cur.tensors, tensors)):
+            return cur
+        if cur is not None and len(cur) == len(tensors) and all(
+                _shape2(a) == _shape2(b) and a.dtype == b.dtype for a, b in zip(cur.tensors, tensors)):
+            cur.rebind(tensors)  # same layout, new addresses (fresh gradient tensors every step)
             return cur
         cur = TensorList(tensors)
         self._last[slot] = cur

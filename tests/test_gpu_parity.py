@@ -598,3 +598,26 @@ def test_reset_set_lr_and_load_meta(gpu):
         opt.step(p[:1], H.dev_list(grads[5], shapes)[:1])
     with pytest.raises(nb.NablaPanic, match="shapes must match"):
         opt.step(p, [H.dev_list(grads[5], shapes)[0], H.to_dev(grads[5][1][:100], (1, 100))])
+
+
+def test_list_rebind_follows_moved_tensors(gpu):
+    """nbo_list_set_ptrs: a list pointed at new tensors of the same shapes steps those, and
+    leaves the old ones alone; a list of other shapes is refused."""
+    shapes = [(2, 3), (1, 9000)]
+    p0 = H.randn_list(shapes, 91, 0.05)
+    g0, g1 = H.randn_list(shapes, 92, 1e-2), H.randn_list(shapes, 93, 1e-2)
+    p_a, p_b = H.dev_list(p0, shapes), H.dev_list(p0, shapes)
+    plist, glist = nb.TensorList(p_a), nb.TensorList(H.dev_list(g0, shapes))
+    opt = nb.Sgd.new(0.1, shapes)
+    opt.step(plist, glist)
+    plist.rebind(p_b)
+    g1_dev = H.dev_list(g1, shapes)
+    glist.rebind(g1_dev)
+    opt.step(plist, glist)
+    ra, rb, vel, meta = H.copy_list(p0), H.copy_list(p0), H.zeros_like_list(p0), O.sgd_meta(0.1)
+    O.sgd_step(meta, ra, g0, vel)
+    O.sgd_step(meta, rb, g1, vel)
+    H.assert_bits_equal(H.host_list(p_a), ra, "first tensors: one step with g0")
+    H.assert_bits_equal(H.host_list(p_b), rb, "second tensors: one step with g1")
+    with pytest.raises(ValueError, match="shapes"):
+        plist.rebind(H.dev_list([p0[0]], [shapes[0]]))
