@@ -49,6 +49,7 @@ typedef enum nbo_status {
     NBO_ERR_NO_MASTER = 9,      /* bf16 step before master weights were set */
     NBO_ERR_TOO_LARGE = 10,     /* more than 2^24-1 chunks of 8192 elements (1.4e11 elements) */
     NBO_ERR_NO_DEVICE = 11,     /* no gfx950 device / code object not loadable */
+    NBO_ERR_IO = 12,            /* checkpoint file: io::Error of save_tensors / load_tensors */
     NBO_ERR_HIP = 1000          /* NBO_ERR_HIP + hipError_t */
 } nbo_status;
 
@@ -249,6 +250,30 @@ int nbo_optim_last_step(nbo_optim *opt, nbo_step_info *out);
  * receives how many were written, *total how many fused steps ran in all. */
 int nbo_optim_trace_read(nbo_optim *opt, nbo_step_info *out, uint64_t max_entries,
                          uint64_t *n_out, uint64_t *total);
+
+/* ---- checkpoint tensor files (NBLA) ------------------------------------------------------
+ * nabla-train's checkpoints keep parameters and optimizer state in two tensor files,
+ * params.nbla and optim.nbla (nabla-train/src/checkpoint.rs:34-105), in the format of
+ * save_tensors / load_tensors (nabla-ml/src/module/core.rs:21,66-120): "NBLA", u32 count,
+ * per tensor u32 name length, UTF-8 name, u32 rows, u32 cols, rows*cols f64 values, all
+ * little-endian; values pass through T::to_f64 / T::from_f64.  Device memory is streamed
+ * through a bounded host buffer.  Synchronous. */
+
+/* save_tensors over the tensors of `list` under `names[i]` (params.nbla from a module's
+ * state_dict; for a mixed-precision optimizer pass a list of its f32 master weights). */
+int nbo_nbla_save_list(const char *path, nbo_list *list, const char *const *names);
+/* load_tensors + Module::load_state_dict (module/core.rs:281-304): every tensor of the
+ * file must carry one of `names` ("unknown parameter key: k") and that tensor's shape
+ * ("shape mismatch for 'k': expected (r, c), got (r, c)"); tensors of the list that the
+ * file does not mention keep their values.  Nothing is written unless the file checks out. */
+int nbo_nbla_load_list(const char *path, nbo_list *list, const char *const *names);
+/* optim.nbla: OptimState::state_tensors (alg.rs:476-485, 553-562, 623-629) -- m0.., v0..
+ * (Sgd: v0.. = velocity) -- written by save_tensors. */
+int nbo_optim_save_state(nbo_optim *opt, const char *path);
+/* load_tensors + OptimState::load_state_tensors (alg.rs:487-516, 564-593, 631-648):
+ * "bad tensor key: k", "m index out of range: i", "missing m{i}" / "missing v{i}"; other
+ * prefixes are ignored.  Nothing is written unless the whole file checks out. */
+int nbo_optim_load_state(nbo_optim *opt, const char *path);
 
 /* ---- measurement helpers --------------------------------------------------------------- */
 

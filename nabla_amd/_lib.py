@@ -26,6 +26,7 @@ ERR_ARG = 8
 ERR_NO_MASTER = 9
 ERR_TOO_LARGE = 10
 ERR_NO_DEVICE = 11
+ERR_IO = 12
 ERR_HIP = 1000
 
 DT_F32, DT_BF16, DT_F64 = 0, 1, 2
@@ -112,6 +113,10 @@ SYMBOLS = {
     "nbo_backend_cast": (C.c_int, [_P, _P]),
     "nbo_optim_last_step": (C.c_int, [_P, C.POINTER(StepInfo)]),
     "nbo_optim_trace_read": (C.c_int, [_P, C.POINTER(StepInfo), C.c_uint64, _U64P, _U64P]),
+    "nbo_nbla_save_list": (C.c_int, [C.c_char_p, _P, C.POINTER(C.c_char_p)]),
+    "nbo_nbla_load_list": (C.c_int, [C.c_char_p, _P, C.POINTER(C.c_char_p)]),
+    "nbo_optim_save_state": (C.c_int, [_P, C.c_char_p]),
+    "nbo_optim_load_state": (C.c_int, [_P, C.c_char_p]),
     "nbo_copy_bytes": (C.c_int, [_P, _P, C.c_uint64]),
     "nbo_profile_enable": (C.c_int, [C.c_int]),
     "nbo_profile_read": (C.c_int, [C.c_char_p, _U64P, C.POINTER(C.c_double)]),

@@ -189,29 +189,99 @@ def read_meta(path: str, optimizer):
     return scaler_state, TrainState(epoch, step, grad_accum, rng), schedule
 
 
+def _native(call, *args):
+    """Run one of the library's NBLA entry points; its errors become CheckpointError with
+    the reference's kinds (checkpoint.rs:14-20)."""
+    from . import _lib
+    from .optim import NablaPanic, _call
+
+    try:
+        _call(call(*args))
+    except _lib.NablaOptimError as e:
+        raise CheckpointError("Io" if e.status == _lib.ERR_IO else "State", e.message) from None
+    except NablaPanic as e:  # shape mismatch of load_state_dict
+        raise CheckpointError("State", str(e)) from None
+    except OptimStateError as e:
+        raise CheckpointError("Optim", str(e)) from None
+
+
+def _name_array(names):
+    import ctypes as C
+
+    return (C.c_char_p * max(len(names), 1))(*[n.encode("utf-8") for n in names])
+
+
+def save_params_native(path: str, named_tensors: Sequence[Tuple[str, object]]) -> None:
+    """params.nbla straight from device tensors (nbo_nbla_save_list): no host copy of the
+    whole model, no Python loop over elements."""
+    from . import _lib
+    from .optim import TensorList
+
+    lst = TensorList([t for _, t in named_tensors])
+    _native(_lib.load().nbo_nbla_save_list, path.encode(), lst._h, _name_array([n for n, _ in named_tensors]))
+
+
+def load_params_native(path: str, named_tensors: Sequence[Tuple[str, object]]) -> None:
+    """load_tensors + Module::load_state_dict into the given device tensors
+    (nbo_nbla_load_list)."""
+    from . import _lib
+    from .optim import TensorList
+
+    lst = TensorList([t for _, t in named_tensors])
+    _native(_lib.load().nbo_nbla_load_list, path.encode(), lst._h, _name_array([n for n, _ in named_tensors]))
+
+
+def save_optim_native(path: str, optimizer) -> None:
+    """optim.nbla from the optimizer's device state (nbo_optim_save_state)."""
+    from . import _lib
+
+    _native(_lib.load().nbo_optim_save_state, optimizer._handle(), path.encode())
+
+
+def load_optim_native(path: str, optimizer) -> None:
+    """load_tensors + load_state_tensors into the optimizer's device state
+    (nbo_optim_load_state)."""
+    from . import _lib
+
+    _native(_lib.load().nbo_optim_load_state, optimizer._handle(), path.encode())
+
+
 def save_checkpoint(directory: str, params: Sequence[Tuple[str, object]], optimizer,
                     scaler: Optional[GradScaler], schedule: Optional[ScheduleState],
-                    state: TrainState) -> None:
+                    state: TrainState, native: bool = False) -> None:
     """checkpoint.rs:38-69.  `params` is the module's state_dict: (name, tensor) pairs;
-    for a mixed-precision optimizer pass its f32 master weights."""
+    for a mixed-precision optimizer pass its f32 master weights.  With `native` the two
+    tensor files are written by the library straight from device memory."""
     os.makedirs(directory, exist_ok=True)
-    save_tensors(params, os.path.join(directory, PARAMS_FILE))
-    save_tensors(optimizer.state_tensors(), os.path.join(directory, OPTIM_FILE))
+    if native:
+        save_params_native(os.path.join(directory, PARAMS_FILE), params)
+        save_optim_native(os.path.join(directory, OPTIM_FILE), optimizer)
+    else:
+        save_tensors(params, os.path.join(directory, PARAMS_FILE))
+        save_tensors(optimizer.state_tensors(), os.path.join(directory, OPTIM_FILE))
     write_meta(os.path.join(directory, META_FILE), optimizer, scaler, schedule, state)
 
 
-def load_checkpoint(directory: str, optimizer, scaler: Optional[GradScaler] = None):
+def load_checkpoint(directory: str, optimizer, scaler: Optional[GradScaler] = None,
+                    into: Optional[Sequence[Tuple[str, object]]] = None):
     """checkpoint.rs:71-105 -> (params, TrainState, ScheduleState | None).  Optimizer
     tensors and meta are loaded into `optimizer`, the scaler state into `scaler`; the
-    parameters are returned for the caller's module to take (load_state_dict)."""
-    params = load_tensors(os.path.join(directory, PARAMS_FILE))
-    optim_tensors = load_tensors(os.path.join(directory, OPTIM_FILE))
-    try:
-        import torch
+    parameters are returned for the caller's module to take (load_state_dict) -- or, with
+    `into` = the module's named device tensors, read into those by the library itself
+    (then `params` is None)."""
+    if into is not None:
+        load_params_native(os.path.join(directory, PARAMS_FILE), into)
+        load_optim_native(os.path.join(directory, OPTIM_FILE), optimizer)
+        params = None
+    else:
+        params = load_tensors(os.path.join(directory, PARAMS_FILE))
+        optim_tensors = load_tensors(os.path.join(directory, OPTIM_FILE))
+        try:
+            import torch
 
-        optimizer.load_state_tensors([(k, torch.from_numpy(v)) for k, v in optim_tensors])
-    except OptimStateError as e:
-        raise CheckpointError("Optim", str(e)) from None
+            optimizer.load_state_tensors([(k, torch.from_numpy(v)) for k, v in optim_tensors])
+        except OptimStateError as e:
+            raise CheckpointError("Optim", str(e)) from None
     scaler_state, train_state, schedule = read_meta(os.path.join(directory, META_FILE), optimizer)
     if scaler is not None and scaler_state is not None:
         scaler.load_state(scaler_state)

@@ -286,6 +286,7 @@ const char *nbo_status_string(int status)
     case NBO_ERR_NO_MASTER: return "master weights not set";
     case NBO_ERR_TOO_LARGE: return "tensor list too large";
     case NBO_ERR_NO_DEVICE: return "no usable gfx950 device";
+    case NBO_ERR_IO: return "checkpoint file i/o error";
     default: return status >= NBO_ERR_HIP ? "HIP runtime error" : "unknown status";
     }
 }
@@ -919,6 +920,40 @@ int nbo_optim_trace_read(nbo_optim *opt, nbo_step_info *out, uint64_t max_entrie
         *n_out = have;
         if (total) *total = t->count;
         std::free(t);
+    });
+}
+
+// ---- checkpoint tensor files -------------------------------------------------------------------
+
+int nbo_nbla_save_list(const char *path, nbo_list *list, const char *const *names)
+{
+    return guarded([&] {
+        require(list != nullptr, NBO_ERR_ARG, "null list");
+        nbla_save_list(path, list, names);
+    });
+}
+
+int nbo_nbla_load_list(const char *path, nbo_list *list, const char *const *names)
+{
+    return guarded([&] {
+        require(list != nullptr, NBO_ERR_ARG, "null list");
+        nbla_load_list(path, list, names);
+    });
+}
+
+int nbo_optim_save_state(nbo_optim *opt, const char *path)
+{
+    return guarded([&] {
+        require(opt != nullptr, NBO_ERR_ARG, "null optimizer");
+        optim_save_state(opt, path);
+    });
+}
+
+int nbo_optim_load_state(nbo_optim *opt, const char *path)
+{
+    return guarded([&] {
+        require(opt != nullptr, NBO_ERR_ARG, "null optimizer");
+        optim_load_state(opt, path);
     });
 }
 

@@ -2,6 +2,7 @@
 // optimizer-step engine.
 #include "nbo_host.hpp"
 
+#include <algorithm>
 #include <cstdio>
 #include <cstring>
 #include <mutex>
@@ -74,8 +75,9 @@ Runtime::Runtime()
     }
     for (int k = 0; k < K_COUNT; k++)
         hip_check(hipModuleGetFunction(&fn_[k], module_, kKernelNames[k]), kKernelNames[k]);
-    pinned_bytes_ = 1 << 20;
+    pinned_bytes_ = 8 << 20; // two halves of 4 MiB
     hip_check(hipHostMalloc(&pinned_, pinned_bytes_, hipHostMallocDefault), "hipHostMalloc");
+    for (hipEvent_t &e : staged_) hip_check(hipEventCreateWithFlags(&e, hipEventDisableTiming), "hipEventCreate");
     partial_sumsq_ = (double *)dmalloc(NBO_NORM_GRID_MAX * sizeof(double));
     partial_flag_ = (uint32_t *)dmalloc(NBO_NORM_GRID_MAX * sizeof(uint32_t));
     gf_scratch_ = (NboGradFactors *)dmalloc(sizeof(NboGradFactors));
@@ -182,19 +184,25 @@ double Runtime::probe_pair_gbps(void *a, void *b, size_t bytes)
     return best > 0.0f ? 4.0 * (double)grid * (double)per_wg * 16 / best / 1e6 : 0.0;
 }
 
+// Both directions run the two halves of the pinned buffer as a pipeline: while the DMA
+// engine fills (or drains) one half, the host copies the other.
 void Runtime::read_back(void *host_dst, const void *dev_src, size_t bytes)
 {
     char *out = (char *)host_dst;
     const char *src = (const char *)dev_src;
-    while (bytes) {
-        size_t chunk = bytes < pinned_bytes_ ? bytes : pinned_bytes_;
-        hip_check(hipMemcpyAsync(pinned_, src, chunk, hipMemcpyDeviceToHost, stream_),
+    const size_t half = pinned_bytes_ / 2;
+    const size_t nchunks = (bytes + half - 1) / half;
+    auto issue = [&](size_t k) {
+        const size_t n = std::min(half, bytes - k * half);
+        hip_check(hipMemcpyAsync((char *)pinned_ + (k & 1) * half, src + k * half, n, hipMemcpyDeviceToHost, stream_),
                   "hipMemcpyAsync D2H");
-        sync();
-        std::memcpy(out, pinned_, chunk);
-        out += chunk;
-        src += chunk;
-        bytes -= chunk;
+        hip_check(hipEventRecord(staged_[k & 1], stream_), "hipEventRecord");
+    };
+    if (nchunks) issue(0);
+    for (size_t k = 0; k < nchunks; k++) {
+        if (k + 1 < nchunks) issue(k + 1);
+        hip_check(hipEventSynchronize(staged_[k & 1]), "hipEventSynchronize");
+        std::memcpy(out + k * half, (const char *)pinned_ + (k & 1) * half, std::min(half, bytes - k * half));
     }
 }
 
@@ -202,16 +210,19 @@ void Runtime::upload(void *dev_dst, const void *host_src, size_t bytes)
 {
     char *dst = (char *)dev_dst;
     const char *src = (const char *)host_src;
-    while (bytes) {
-        size_t chunk = bytes < pinned_bytes_ ? bytes : pinned_bytes_;
-        std::memcpy(pinned_, src, chunk);
-        hip_check(hipMemcpyAsync(dst, pinned_, chunk, hipMemcpyHostToDevice, stream_),
+    const size_t half = pinned_bytes_ / 2;
+    const size_t nchunks = (bytes + half - 1) / half;
+    for (size_t k = 0; k < nchunks; k++) {
+        const size_t n = std::min(half, bytes - k * half);
+        // the half is free again once the transfer issued from it two chunks ago is done
+        if (k >= 2) hip_check(hipEventSynchronize(staged_[k & 1]), "hipEventSynchronize");
+        std::memcpy((char *)pinned_ + (k & 1) * half, src + k * half, n);
+        hip_check(hipMemcpyAsync(dst + k * half, (const char *)pinned_ + (k & 1) * half, n, hipMemcpyHostToDevice,
+                                 stream_),
                   "hipMemcpyAsync H2D");
-        sync(); // the staging buffer is reused
-        dst += chunk;
-        src += chunk;
-        bytes -= chunk;
+        hip_check(hipEventRecord(staged_[k & 1], stream_), "hipEventRecord");
     }
+    if (nchunks) sync(); // the staging buffer is reused by the next call
 }
 
 void *Runtime::dmalloc(size_t bytes)

@@ -64,7 +64,7 @@ public:
     // b together: the probe StatePlacement classifies HBM regions with.  Synchronous.
     double probe_pair_gbps(void *a, void *b, size_t bytes);
 
-    // synchronous small transfers through a pinned staging buffer
+    // synchronous transfers through a double-buffered pinned staging buffer
     void read_back(void *host_dst, const void *dev_src, size_t bytes);
     void upload(void *dev_dst, const void *host_src, size_t bytes);
 
@@ -88,6 +88,7 @@ private:
     hipStream_t stream_ = nullptr;
     void *pinned_ = nullptr;
     size_t pinned_bytes_ = 0;
+    hipEvent_t staged_[2] = {}; // one per half of the staging buffer
     double *partial_sumsq_ = nullptr;
     uint32_t *partial_flag_ = nullptr;
     NboGradFactors *gf_scratch_ = nullptr;
@@ -138,5 +139,13 @@ struct nbo_optim {
     NboTraceDev *trace = nullptr;
     size_t elem_bytes() const { return state_dtype == NBO_DT_F64 ? 8 : state_dtype == NBO_DT_BF16 ? 2 : 4; }
 };
+
+namespace nbo {
+// NBLA tensor files (nbo_nbla.cpp)
+void nbla_save_list(const char *path, const nbo_list *list, const char *const *names);
+void nbla_load_list(const char *path, nbo_list *list, const char *const *names);
+void optim_save_state(const nbo_optim *opt, const char *path);
+void optim_load_state(nbo_optim *opt, const char *path);
+} // namespace nbo
 
 #endif

@@ -1,0 +1,301 @@
+// NBLA tensor files -- the bulk part of nabla-train's checkpoints (params.nbla,
+// optim.nbla; nabla-train/src/checkpoint.rs:34-105) in the format of
+// nabla-ml/src/module/core.rs:21,66-120: "NBLA", u32 count, then per tensor u32 name
+// length, UTF-8 name, u32 rows, u32 cols and rows*cols f64 values, all little-endian.
+// Values are f64 whatever the element type (T::to_f64 on save, T::from_f64 on load), so
+// f32 and bf16 state round-trips exactly.  Device memory is streamed through a bounded
+// host buffer; nothing here needs the whole tensor on the host.
+#include <cerrno>
+#include <cstdio>
+#include <cstring>
+#include <memory>
+
+#include "nbo_host.hpp"
+
+using namespace nbo;
+
+namespace {
+
+constexpr size_t kChunkElems = (size_t)1 << 20; // elements per streaming step
+
+struct FileCloser {
+    void operator()(std::FILE *f) const
+    {
+        if (f) std::fclose(f);
+    }
+};
+using FilePtr = std::unique_ptr<std::FILE, FileCloser>;
+
+FilePtr open_file(const char *path, const char *mode)
+{
+    if (!path) fail(NBO_ERR_ARG, "null path");
+    FilePtr f(std::fopen(path, mode));
+    if (!f) fail(NBO_ERR_IO, std::string(path) + ": " + std::strerror(errno));
+    return f;
+}
+
+void write_all(std::FILE *f, const void *p, size_t n)
+{
+    if (n && std::fwrite(p, 1, n, f) != n) fail(NBO_ERR_IO, std::string("write failed: ") + std::strerror(errno));
+}
+
+void read_exact(std::FILE *f, void *p, size_t n)
+{
+    if (n && std::fread(p, 1, n, f) != n) fail(NBO_ERR_IO, "failed to fill whole buffer"); // io::ErrorKind::UnexpectedEof
+}
+
+void write_u32(std::FILE *f, uint32_t v)
+{
+    const unsigned char b[4] = {(unsigned char)v, (unsigned char)(v >> 8), (unsigned char)(v >> 16),
+                                (unsigned char)(v >> 24)};
+    write_all(f, b, 4);
+}
+
+uint32_t read_u32(std::FILE *f)
+{
+    unsigned char b[4];
+    read_exact(f, b, 4);
+    return (uint32_t)b[0] | ((uint32_t)b[1] << 8) | ((uint32_t)b[2] << 16) | ((uint32_t)b[3] << 24);
+}
+
+size_t dtype_bytes(int dtype) { return dtype == NBO_DT_F64 ? 8 : dtype == NBO_DT_BF16 ? 2 : 4; }
+
+// half::bf16::from_f32 / f32::from(bf16) on the host (common/scalar/mod.rs:338-344)
+uint16_t bf16_from_f32(float v)
+{
+    uint32_t x;
+    std::memcpy(&x, &v, 4);
+    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((x >> 16) | 0x0040u);
+    return (uint16_t)((x + 0x7FFFu + ((x >> 16) & 1u)) >> 16);
+}
+
+float bf16_to_f32(uint16_t h)
+{
+    const uint32_t x = (uint32_t)h << 16;
+    float f;
+    std::memcpy(&f, &x, 4);
+    return f;
+}
+
+// T::to_f64 over `n` raw elements
+void widen(int dtype, const void *raw, double *out, size_t n)
+{
+    if (dtype == NBO_DT_F64) std::memcpy(out, raw, n * 8);
+    else if (dtype == NBO_DT_F32)
+        for (size_t i = 0; i < n; i++) out[i] = (double)((const float *)raw)[i];
+    else
+        for (size_t i = 0; i < n; i++) out[i] = (double)bf16_to_f32(((const uint16_t *)raw)[i]);
+}
+
+// T::from_f64 over `n` values (f32: one rounding; bf16: through f32, scalar/mod.rs:338-340)
+void narrow(int dtype, const double *in, void *raw, size_t n)
+{
+    if (dtype == NBO_DT_F64) std::memcpy(raw, in, n * 8);
+    else if (dtype == NBO_DT_F32)
+        for (size_t i = 0; i < n; i++) ((float *)raw)[i] = (float)in[i];
+    else
+        for (size_t i = 0; i < n; i++) ((uint16_t *)raw)[i] = bf16_from_f32((float)in[i]);
+}
+
+struct Buffers {
+    std::vector<unsigned char> raw;
+    std::vector<double> f64;
+    Buffers() : raw(kChunkElems * 8), f64(kChunkElems) {}
+};
+
+void write_header(std::FILE *f, const std::string &name, uint64_t rows, uint64_t cols)
+{
+    if (rows > 0xFFFFFFFFull || cols > 0xFFFFFFFFull || name.size() > 0xFFFFFFFFull)
+        fail(NBO_ERR_TOO_LARGE, "tensor '" + name + "' does not fit the file format's 32-bit fields");
+    write_u32(f, (uint32_t)name.size());
+    write_all(f, name.data(), name.size());
+    write_u32(f, (uint32_t)rows);
+    write_u32(f, (uint32_t)cols);
+}
+
+// device elements -> f64 little-endian values in the file
+void stream_out(std::FILE *f, const void *dev, int dtype, uint64_t n, Buffers &b)
+{
+    Runtime &rt = Runtime::get();
+    const size_t eb = dtype_bytes(dtype);
+    for (uint64_t done = 0; done < n;) {
+        const size_t k = (size_t)std::min<uint64_t>(kChunkElems, n - done);
+        rt.read_back(b.raw.data(), (const char *)dev + done * eb, k * eb);
+        widen(dtype, b.raw.data(), b.f64.data(), k);
+        write_all(f, b.f64.data(), k * 8); // the build targets little-endian hosts only
+        done += k;
+    }
+}
+
+// f64 values in the file -> device elements
+void stream_in(std::FILE *f, void *dev, int dtype, uint64_t n, Buffers &b)
+{
+    Runtime &rt = Runtime::get();
+    const size_t eb = dtype_bytes(dtype);
+    for (uint64_t done = 0; done < n;) {
+        const size_t k = (size_t)std::min<uint64_t>(kChunkElems, n - done);
+        read_exact(f, b.f64.data(), k * 8);
+        narrow(dtype, b.f64.data(), b.raw.data(), k);
+        rt.upload((char *)dev + done * eb, b.raw.data(), k * eb);
+        done += k;
+    }
+}
+
+struct Entry {
+    std::string name;
+    uint64_t rows, cols;
+    long data_offset;
+};
+
+// Reads the file's table of contents, skipping over the values.
+std::vector<Entry> read_index(std::FILE *f)
+{
+    char magic[4];
+    read_exact(f, magic, 4);
+    if (std::memcmp(magic, "NBLA", 4) != 0) fail(NBO_ERR_IO, "not a nabla tensor file");
+    const uint32_t count = read_u32(f);
+    std::vector<Entry> out;
+    for (uint32_t i = 0; i < count; i++) {
+        Entry e;
+        const uint32_t name_len = read_u32(f);
+        e.name.resize(name_len);
+        read_exact(f, e.name.empty() ? nullptr : &e.name[0], name_len);
+        e.rows = read_u32(f);
+        e.cols = read_u32(f);
+        e.data_offset = std::ftell(f);
+        const uint64_t bytes = e.rows * e.cols * 8;
+        if (e.data_offset < 0 || std::fseek(f, (long)bytes, SEEK_CUR) != 0) fail(NBO_ERR_IO, "seek failed");
+        out.push_back(std::move(e));
+    }
+    // a truncated last tensor shows up as a short file
+    const long end_of_index = std::ftell(f);
+    if (std::fseek(f, 0, SEEK_END) != 0 || std::ftell(f) < end_of_index) fail(NBO_ERR_IO, "failed to fill whole buffer");
+    return out;
+}
+
+void seek_to(std::FILE *f, long off)
+{
+    if (std::fseek(f, off, SEEK_SET) != 0) fail(NBO_ERR_IO, "seek failed");
+}
+
+} // namespace
+
+namespace nbo {
+
+void nbla_save_list(const char *path, const nbo_list *list, const char *const *names)
+{
+    const uint64_t nt = list->layout.nt();
+    if (nt && !names) fail(NBO_ERR_ARG, "null name array");
+    if (nt > 0xFFFFFFFFull) fail(NBO_ERR_TOO_LARGE, "too many tensors for the file format");
+    Runtime::get().sync(); // everything enqueued so far is part of what gets saved
+    FilePtr f = open_file(path, "wb");
+    Buffers b;
+    write_all(f.get(), "NBLA", 4);
+    write_u32(f.get(), (uint32_t)nt);
+    for (uint64_t t = 0; t < nt; t++) {
+        if (!names[t]) fail(NBO_ERR_ARG, "null tensor name");
+        write_header(f.get(), names[t], list->layout.rows[t], list->layout.cols[t]);
+        stream_out(f.get(), (const void *)(uintptr_t)list->ptrs[t], list->dtype, list->layout.n[t], b);
+    }
+    if (std::fflush(f.get()) != 0) fail(NBO_ERR_IO, std::string("write failed: ") + std::strerror(errno));
+}
+
+// Module::load_state_dict (nabla-ml/src/module/core.rs:281-304) over load_tensors: every
+// tensor of the file must name a tensor of the list and have its shape.
+void nbla_load_list(const char *path, nbo_list *list, const char *const *names)
+{
+    const uint64_t nt = list->layout.nt();
+    if (nt && !names) fail(NBO_ERR_ARG, "null name array");
+    FilePtr f = open_file(path, "rb");
+    const std::vector<Entry> index = read_index(f.get());
+    std::vector<uint64_t> target(index.size());
+    for (size_t k = 0; k < index.size(); k++) {
+        uint64_t t = 0;
+        while (t < nt && index[k].name != names[t]) t++;
+        if (t == nt) fail(NBO_ERR_STATE_KEY, "unknown parameter key: " + index[k].name);
+        if (index[k].rows != list->layout.rows[t] || index[k].cols != list->layout.cols[t])
+            fail(NBO_ERR_SHAPE, "shape mismatch for '" + index[k].name + "': expected (" +
+                                    std::to_string(list->layout.rows[t]) + ", " +
+                                    std::to_string(list->layout.cols[t]) + "), got (" +
+                                    std::to_string(index[k].rows) + ", " + std::to_string(index[k].cols) + ")");
+        target[k] = t;
+    }
+    Buffers b;
+    for (size_t k = 0; k < index.size(); k++) {
+        seek_to(f.get(), index[k].data_offset);
+        stream_in(f.get(), (void *)(uintptr_t)list->ptrs[target[k]], list->dtype, list->layout.n[target[k]], b);
+    }
+}
+
+// OptimState::state_tensors (alg.rs:476-485, 553-562, 623-629) written by save_tensors:
+// m0.., then v0.. (Sgd: v0.. = velocity).
+void optim_save_state(const nbo_optim *opt, const char *path)
+{
+    const uint64_t nt = opt->layout.nt();
+    const bool adam_like = opt->meta.kind != NBO_KIND_SGD;
+    Runtime::get().sync();
+    FilePtr f = open_file(path, "wb");
+    Buffers b;
+    write_all(f.get(), "NBLA", 4);
+    write_u32(f.get(), (uint32_t)(nt * (adam_like ? 2 : 1)));
+    const size_t eb = opt->elem_bytes();
+    for (int which = 0; which < (adam_like ? 2 : 1); which++) {
+        const char prefix = adam_like && which == 0 ? 'm' : 'v';
+        const uint32_t part = which == 0 ? 0u : opt->arena.part_v;
+        for (uint64_t t = 0; t < nt; t++) {
+            write_header(f.get(), prefix + std::to_string(t), opt->layout.rows[t], opt->layout.cols[t]);
+            const char *dev = (const char *)opt->arena.part[part] + (size_t)opt->layout.soff[t] * eb;
+            stream_out(f.get(), dev, opt->state_dtype, opt->layout.n[t], b);
+        }
+    }
+    if (std::fflush(f.get()) != 0) fail(NBO_ERR_IO, std::string("write failed: ") + std::strerror(errno));
+}
+
+// OptimState::load_state_tensors (alg.rs:487-516, 564-593, 631-648) over load_tensors:
+// other prefixes are ignored, every expected tensor must be present; nothing is written
+// unless the whole file checks out.
+void optim_load_state(nbo_optim *opt, const char *path)
+{
+    const uint64_t nt = opt->layout.nt();
+    const bool adam_like = opt->meta.kind != NBO_KIND_SGD;
+    FilePtr f = open_file(path, "rb");
+    const std::vector<Entry> index = read_index(f.get());
+    std::vector<long> m_at(nt, -1), v_at(nt, -1);
+    for (const Entry &e : index) {
+        const char c = e.name.empty() ? '\0' : e.name[0];
+        if (!(c == 'v' || (c == 'm' && adam_like))) continue;
+        // what Rust's str::parse::<usize> accepts: an optional '+', then decimal digits
+        const char *p = e.name.c_str() + 1;
+        if (*p == '+') p++;
+        if (*p == '\0') fail(NBO_ERR_STATE_KEY, "bad tensor key: " + e.name);
+        uint64_t idx = 0;
+        for (; *p; p++) {
+            if (*p < '0' || *p > '9' || idx > (UINT64_MAX - (uint64_t)(*p - '0')) / 10)
+                fail(NBO_ERR_STATE_KEY, "bad tensor key: " + e.name);
+            idx = idx * 10 + (uint64_t)(*p - '0');
+        }
+        if (idx >= nt) fail(NBO_ERR_STATE_INDEX, std::string(1, c) + " index out of range: " + std::to_string(idx));
+        if (e.rows * e.cols != opt->layout.n[idx])
+            fail(NBO_ERR_SHAPE, "state tensor " + e.name + " has " + std::to_string(opt->layout.n[idx]) +
+                                    " elements, file has " + std::to_string(e.rows * e.cols));
+        (c == 'm' ? m_at : v_at)[idx] = e.data_offset; // a later duplicate wins, as in the reference
+    }
+    if (adam_like)
+        for (uint64_t t = 0; t < nt; t++)
+            if (m_at[t] < 0) fail(NBO_ERR_STATE_KEY, "missing m" + std::to_string(t));
+    for (uint64_t t = 0; t < nt; t++)
+        if (v_at[t] < 0) fail(NBO_ERR_STATE_KEY, "missing v" + std::to_string(t));
+    Buffers b;
+    const size_t eb = opt->elem_bytes();
+    for (int which = 0; which < (adam_like ? 2 : 1); which++) {
+        const std::vector<long> &at = adam_like && which == 0 ? m_at : v_at;
+        const uint32_t part = which == 0 ? 0u : opt->arena.part_v;
+        for (uint64_t t = 0; t < nt; t++) {
+            seek_to(f.get(), at[t]);
+            char *dev = (char *)opt->arena.part[part] + (size_t)opt->layout.soff[t] * eb;
+            stream_in(f.get(), dev, opt->state_dtype, opt->layout.n[t], b);
+        }
+    }
+}
+
+} // namespace nbo

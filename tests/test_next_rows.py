@@ -281,3 +281,138 @@ def test_checkpoint_round_trip_restores_bit_identical_training(gpu, tmp_path):
     H.assert_bits_equal(H.host_list(o2.moments()[0]), H.host_list(o1.moments()[0]), "m after resume")
     H.assert_bits_equal(H.host_list(o2.moments()[1]), H.host_list(o1.moments()[1]), "v after resume")
     assert o2.step_count() == o1.step_count() == 5
+
+
+# ---- N1, native: NBLA files written and read by the library itself ------------------------------
+
+def _file_bytes(path):
+    with open(path, "rb") as f:
+        return f.read()
+
+
+@pytest.mark.gpu
+def test_native_nbla_writer_is_byte_identical_to_the_format_writer(gpu, tmp_path):
+    """nbo_nbla_save_list / nbo_optim_save_state against the Python writer whose byte layout
+    is checked against a hand-assembled file above: same bytes, for f32, bf16 and f64
+    tensors, an empty tensor and a tensor longer than the streaming chunk (2^20)."""
+    import torch
+
+    from nabla_amd import checkpoint as ck
+
+    shapes = [(3, 5), (1, 1), (0, 7), (1025, 1031)]
+    names = ["layer.weight", "b", "empty", "big"]
+    for dt in (torch.float32, torch.bfloat16, torch.float64):
+        torch.manual_seed(5)
+        tensors = [(torch.randn(s, device=gpu, dtype=torch.float32) * 3).to(dt) for s in shapes]
+        named = list(zip(names, tensors))
+        ck.save_tensors(named, str(tmp_path / "py.nbla"))
+        ck.save_params_native(str(tmp_path / "native.nbla"), named)
+        assert _file_bytes(tmp_path / "native.nbla") == _file_bytes(tmp_path / "py.nbla"), dt
+    for opt in (nb.AdamW.new(1e-3, shapes), nb.Sgd.new(0.1, shapes).momentum(0.9),
+                nb.Adam.new(1e-3, shapes, dtype="bf16")):
+        dt = torch.bfloat16 if opt._state_dtype == nb.DT_BF16 else torch.float32
+        p = [torch.randn(s, device=gpu, dtype=torch.float32).to(dt) for s in shapes]
+        g = [torch.randn(s, device=gpu, dtype=torch.float32).to(dt) for s in shapes]
+        opt.step(p, g)
+        ck.save_tensors(opt.state_tensors(), str(tmp_path / "py.nbla"))
+        ck.save_optim_native(str(tmp_path / "native.nbla"), opt)
+        assert _file_bytes(tmp_path / "native.nbla") == _file_bytes(tmp_path / "py.nbla"), opt.NAME
+
+
+@pytest.mark.gpu
+def test_native_nbla_reader_round_trip_and_errors(gpu, tmp_path):
+    import torch
+
+    from nabla_amd import checkpoint as ck
+
+    shapes = [(3, 5), (1, 1), (1025, 1031)]
+    names = ["w", "b", "big"]
+    torch.manual_seed(6)
+    src = [torch.randn(s, device=gpu) for s in shapes]
+    path = str(tmp_path / "params.nbla")
+    ck.save_params_native(path, list(zip(names, src)))
+    # load_state_dict: by name, any order, tensors the file does not mention keep their values
+    dst = [torch.zeros(s, device=gpu) for s in shapes]
+    extra = torch.full((2, 2), 7.0, device=gpu)
+    ck.load_params_native(path, [("extra", extra), ("big", dst[2]), ("w", dst[0]), ("b", dst[1])])
+    assert all(torch.equal(a, b) for a, b in zip(src, dst)) and bool((extra == 7.0).all())
+    # f64 values narrow with T::from_f64 on load: bf16 goes through f32
+    as_bf16 = [torch.zeros(s, device=gpu, dtype=torch.bfloat16) for s in shapes]
+    ck.load_params_native(path, list(zip(names, as_bf16)))
+    assert all(torch.equal(a.to(torch.bfloat16), b) for a, b in zip(src, as_bf16))
+    with pytest.raises(ck.CheckpointError, match="unknown parameter key: b"):
+        ck.load_params_native(path, [("w", dst[0]), ("big", dst[2])])
+    with pytest.raises(ck.CheckpointError, match=r"shape mismatch for 'w': expected \(5, 3\), got \(3, 5\)"):
+        ck.load_params_native(path, [("w", torch.zeros((5, 3), device=gpu)), ("b", dst[1]), ("big", dst[2])])
+    with pytest.raises(ck.CheckpointError, match="No such file"):
+        ck.load_params_native(str(tmp_path / "absent.nbla"), list(zip(names, dst)))
+    (tmp_path / "junk.nbla").write_bytes(b"NOPE" + bytes(16))
+    with pytest.raises(ck.CheckpointError, match="not a nabla tensor file"):
+        ck.load_params_native(str(tmp_path / "junk.nbla"), list(zip(names, dst)))
+    (tmp_path / "short.nbla").write_bytes(_file_bytes(path)[:-9])
+    with pytest.raises(ck.CheckpointError, match="failed to fill whole buffer"):
+        ck.load_params_native(str(tmp_path / "short.nbla"), list(zip(names, dst)))
+
+    # optimizer state: round trip, then the reference's load_state_tensors errors
+    opt = nb.AdamW.new(1e-3, shapes)
+    p = [torch.randn(s, device=gpu) for s in shapes]
+    opt.step(p, [torch.randn(s, device=gpu) for s in shapes])
+    opath = str(tmp_path / "optim.nbla")
+    ck.save_optim_native(opath, opt)
+    other = nb.AdamW.new(1e-3, shapes)
+    ck.load_optim_native(opath, other)
+    for a, b in zip(opt.moments()[0] + opt.moments()[1], other.moments()[0] + other.moments()[1]):
+        assert torch.equal(a, b)
+    tensors = ck.load_tensors(opath)
+    ck.save_tensors([t for t in tensors if t[0] != "v1"] + [("ignored.key", np.zeros((1, 1)))], opath)
+    with pytest.raises(ck.CheckpointError, match="missing v1"):
+        ck.load_optim_native(opath, other)
+    ck.save_tensors(tensors + [("m9", np.zeros((1, 1)))], opath)
+    with pytest.raises(ck.CheckpointError, match="m index out of range: 9"):
+        ck.load_optim_native(opath, other)
+    ck.save_tensors(tensors + [("mx", np.zeros((1, 1)))], opath)
+    with pytest.raises(ck.CheckpointError, match="bad tensor key: mx"):
+        ck.load_optim_native(opath, other)
+    # a failed load left the state alone
+    for a, b in zip(opt.moments()[1], other.moments()[1]):
+        assert torch.equal(a, b)
+    sgd = nb.Sgd.new(0.1, shapes)  # Sgd reads only v{i} and ignores m{i}
+    ck.save_tensors(tensors, opath)
+    ck.load_optim_native(opath, sgd)
+    assert all(torch.equal(a, b) for a, b in zip(sgd.velocity(), opt.moments()[1]))
+
+
+@pytest.mark.gpu
+def test_native_checkpoint_resumes_bit_identical_training(gpu, tmp_path):
+    """save_checkpoint(native=True) after two steps, load_checkpoint(into=...) into a fresh
+    optimizer and fresh tensors, two more steps on both: identical bits, and the files are
+    the ones the reference format prescribes (params.nbla, optim.nbla, meta.txt)."""
+    import os
+
+    import torch
+
+    from nabla_amd import checkpoint as ck
+    from nabla_amd.schedule import Cosine, ScheduleState
+
+    shapes = [(4, 9), (1, 20000), (1, 3)]
+    names = ["a.weight", "b.weight", "b.bias"]
+    torch.manual_seed(8)
+    p1 = [torch.randn(s, device=gpu) * 0.1 for s in shapes]
+    grads = [[torch.randn(s, device=gpu) * 1e-2 for s in shapes] for _ in range(4)]
+    o1 = nb.AdamW.new(1e-3, shapes).beta2(0.95).weight_decay(0.1)
+    for k in range(2):
+        o1.step(p1, grads[k])
+    sched = ScheduleState(base_lr=1e-3, schedule=Cosine(warmup_steps=1, total_steps=9, min_lr=1e-5))
+    ck.save_checkpoint(str(tmp_path), list(zip(names, p1)), o1, None, sched,
+                       ck.TrainState(epoch=1, step=2, grad_accum=1, rng_state=None), native=True)
+    assert sorted(os.listdir(tmp_path)) == ["meta.txt", "optim.nbla", "params.nbla"]
+    p2 = [torch.zeros(s, device=gpu) for s in shapes]
+    o2 = nb.AdamW.new(5.0, shapes)  # every hyper-parameter comes back from meta.txt
+    params, state, schedule = ck.load_checkpoint(str(tmp_path), o2, None, into=list(zip(names, p2)))
+    assert params is None and (state.epoch, state.step) == (1, 2) and schedule == sched
+    assert o2.step_count() == 2 and o2.meta().beta2 == 0.95 and o2.meta().weight_decay == 0.1
+    for k in range(2, 4):
+        o1.step(p1, grads[k])
+        o2.step(p2, grads[k])
+    assert all(torch.equal(a, b) for a, b in zip(p1, p2))
+    assert all(torch.equal(a, b) for a, b in zip(o1.moments()[1], o2.moments()[1]))
