@@ -250,6 +250,10 @@ public:
     {
         check(nbo_optim_state_write(handle(), name.c_str(), buf, n, on_device ? 1 : 0));
     }
+    // optim.nbla of a checkpoint (checkpoint.rs:59-62, 92-95): state_tensors() through
+    // save_tensors, load_tensors into load_state_tensors; errors as StateError / RuntimeError
+    void save_state(const std::string &path) { check(nbo_optim_save_state(handle(), path.c_str())); }
+    void load_state(const std::string &path) { check(nbo_optim_load_state(handle(), path.c_str())); }
     void master_from_params(TensorList &params_bf16) { check(nbo_optim_master_from_params(handle(), params_bf16.handle())); }
 
     nbo_optim *handle()
@@ -350,6 +354,21 @@ inline bool has_non_finite(TensorList &grads)
 inline void accumulate(TensorList &accum, TensorList &grads, bool zero_grads = false)
 {
     check(nbo_accumulate(accum.handle(), grads.handle(), zero_grads ? 1 : 0));
+}
+
+// params.nbla of a checkpoint: save_tensors / load_tensors + load_state_dict
+// (nabla-ml/src/module/core.rs:66-120, 281-304) over a list of device tensors
+inline void save_tensors(const std::string &path, TensorList &list, const std::vector<std::string> &names)
+{
+    std::vector<const char *> c;
+    for (const std::string &n : names) c.push_back(n.c_str());
+    check(nbo_nbla_save_list(path.c_str(), list.handle(), c.data()));
+}
+inline void load_state_dict(const std::string &path, TensorList &list, const std::vector<std::string> &names)
+{
+    std::vector<const char *> c;
+    for (const std::string &n : names) c.push_back(n.c_str());
+    check(nbo_nbla_load_list(path.c_str(), list.handle(), c.data()));
 }
 
 // ---- LrSchedule (optim/core.rs:81-173): host arithmetic in f64 -------------------------
