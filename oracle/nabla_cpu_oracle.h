@@ -33,6 +33,13 @@
  *     round-to-nearest-even algorithm is restated and cross-checked against
  *     torch's bf16 cast for all non-NaN inputs.  No reference test exercises
  *     bf16 (PARITY UNPINNED for NaN payloads).
+ *   - T = bf16 instantiations (primitives, Sgd / Adam / AdamW, scaler, clip): the
+ *     reference's tests never instantiate an optimizer at half::bf16.  Each operation
+ *     is restated from scalar/mod.rs:253-351 (f32 operation, then bf16::from_f32) and
+ *     the `half` crate's documented operators, and checked in exact arithmetic (round
+ *     to 24 bits, then to 8) including the inner rounding of axpy and the two-step
+ *     f64 -> bf16 cast.  PARITY UNPINNED against any output of the reference.
+ *   - the benchmarks' LCG rand_tensor (benchmarks/src/lib.rs:7-22): exact arithmetic.
  */
 #ifndef NABLA_CPU_ORACLE_H
 #define NABLA_CPU_ORACLE_H
