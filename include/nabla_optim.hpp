@@ -133,6 +133,11 @@ public:
         return ok != 0;
     }
     double scale_factor() { return state().scale; }
+    // core.rs:347-349: out = loss * T::from_f64(scale)
+    void scale_loss(TensorList &loss, TensorList &out)
+    {
+        check(nbo_backend_apply(NBO_BACKEND_SCALE, out.handle(), loss.handle(), nullptr, scale_factor()));
+    }
     GradScalerState state()
     {
         if (!h_) return init_;

@@ -112,6 +112,10 @@ static void grad_scaler_unscale()  // optim.rs:120-128
     EXPECT(scaler.unscale_and_update(grads));
     EXPECT(g.get() < 2.0);
     EXPECT(g.get() == 2.0 / 65536.0);
+    Mat loss({0.75}), scaled({0.0});  // scale_loss, core.rs:347-349
+    TensorList l({loss.tensor()}), o({scaled.tensor()});
+    scaler.scale_loss(l, o);
+    EXPECT(scaled.get() == 0.75 * 65536.0);
 }
 
 static void grad_scaler_detects_inf()  // optim.rs:130-138

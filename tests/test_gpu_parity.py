@@ -621,3 +621,45 @@ def test_list_rebind_follows_moved_tensors(gpu):
     H.assert_bits_equal(H.host_list(p_b), rb, "second tensors: one step with g1")
     with pytest.raises(ValueError, match="shapes"):
         plist.rebind(H.dev_list([p0[0]], [shapes[0]]))
+
+
+def test_two_host_threads_drive_two_optimizers(gpu):
+    """Entry points may be called from several threads (ctypes drops the GIL around each
+    call, so the calls do overlap in time); the library runs them one at a time and each
+    optimizer's result is what it would be alone."""
+    import threading
+
+    shapes = [(3, 5), (1, 9000)]
+    cases = []
+    for k in range(2):
+        p0 = H.randn_list(shapes, 600 + k, 0.05)
+        grads = [H.randn_list(shapes, 700 + 10 * k + s, 1e-2) for s in range(25)]
+        cases.append(dict(p0=p0, grads=grads, p_dev=H.dev_list(p0, shapes),
+                          g_dev=[H.dev_list(g, shapes) for g in grads],
+                          opt=nb.AdamW.new(1e-3, shapes).weight_decay(0.01 * (k + 1)), errors=[]))
+
+    def run(c):
+        try:
+            for g in c["g_dev"]:
+                c["opt"].fused_step(c["p_dev"], g, max_norm=0.5)
+                c["opt"].last_step()  # a synchronous call in between
+        except Exception as e:  # surfaced below, in the main thread
+            c["errors"].append(e)
+
+    threads = [threading.Thread(target=run, args=(c,)) for c in cases]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        for k, c in enumerate(cases):
+            assert not c["errors"], c["errors"]
+            pr, m, v = H.copy_list(c["p0"]), H.zeros_like_list(c["p0"]), H.zeros_like_list(c["p0"])
+            meta = O.adamw_meta(1e-3, weight_decay=0.01 * (k + 1))
+            for g in c["grads"]:
+                O.f32_step(meta, None, 0.5, pr, H.copy_list(g), m, v)
+            H.assert_bits_equal(H.host_list(c["p_dev"]), pr, f"thread {k}: params")
+            assert c["opt"].step_count() == 25
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
