@@ -78,6 +78,7 @@ Runtime::Runtime()
     pinned_bytes_ = 8 << 20; // two halves of 4 MiB
     hip_check(hipHostMalloc(&pinned_, pinned_bytes_, hipHostMallocDefault), "hipHostMalloc");
     for (hipEvent_t &e : staged_) hip_check(hipEventCreateWithFlags(&e, hipEventDisableTiming), "hipEventCreate");
+    for (hipEvent_t &e : probe_ev_) hip_check(hipEventCreate(&e), "hipEventCreate");
     partial_sumsq_ = (double *)dmalloc(NBO_NORM_GRID_MAX * sizeof(double));
     partial_flag_ = (uint32_t *)dmalloc(NBO_NORM_GRID_MAX * sizeof(uint32_t));
     gf_scratch_ = (NboGradFactors *)dmalloc(sizeof(NboGradFactors));
@@ -165,9 +166,7 @@ double Runtime::probe_pair_gbps(void *a, void *b, size_t bytes)
     const uint32_t grid = (uint32_t)(bytes / 16 / per_wg);
     if (grid == 0) return 0.0;
     void *args[2] = {(void *)&a, (void *)&b};
-    hipEvent_t e0, e1;
-    hip_check(hipEventCreate(&e0), "hipEventCreate");
-    hip_check(hipEventCreate(&e1), "hipEventCreate");
+    const hipEvent_t e0 = probe_ev_[0], e1 = probe_ev_[1];
     float best = 0.0f;
     for (int rep = 0; rep < 4; rep++) {
         hip_check(hipEventRecord(e0, stream_), "hipEventRecord");
@@ -179,8 +178,6 @@ double Runtime::probe_pair_gbps(void *a, void *b, size_t bytes)
         hip_check(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime");
         if (rep > 0 && (best == 0.0f || ms < best)) best = ms; // first run warms up
     }
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
     return best > 0.0f ? 4.0 * (double)grid * (double)per_wg * 16 / best / 1e6 : 0.0;
 }
 

@@ -89,6 +89,7 @@ private:
     void *pinned_ = nullptr;
     size_t pinned_bytes_ = 0;
     hipEvent_t staged_[2] = {}; // one per half of the staging buffer
+    hipEvent_t probe_ev_[2] = {}; // timing of the placement probe
     double *partial_sumsq_ = nullptr;
     uint32_t *partial_flag_ = nullptr;
     NboGradFactors *gf_scratch_ = nullptr;
