@@ -1,7 +1,8 @@
 // The reference's own tests for the optimizer step (nabla-train/tests/optim.rs:47-138,
 // nabla-train/tests/trainer.rs:171-203), replayed through the C++ mirror of its
 // interface (include/nabla_optim.hpp) on the device: f64, 1x1 tensors, the same
-// values and the same assertions.  Exit code 0 = all passed.
+// values and the same assertions.  Exit code 0 = all passed.  With a directory as its
+// argument the checkpoint test writes there (and leaves the files for the caller).
 #include <hip/hip_runtime_api.h>
 
 #include <cmath>
@@ -11,7 +12,7 @@
 #include <string>
 #include <vector>
 
-#include "../../include/nabla_optim.hpp"
+#include "../../include/nabla_checkpoint.hpp"
 
 using namespace nabla::optim;
 
@@ -216,6 +217,57 @@ static void backend_axpy_is_multiply_then_add()  // cpu/mod.rs:216-223
     EXPECT(y.get(1) == 0.1 + prod);
 }
 
+static std::string g_checkpoint_dir;
+
+static void checkpoint_roundtrip_with_schedule()  // trainer.rs tests :249-304
+{
+    std::string dir = g_checkpoint_dir;
+    if (dir.empty()) {
+        char tmpl[] = "/tmp/nbo_ckpt_XXXXXX";
+        const char *made = mkdtemp(tmpl);
+        EXPECT(made != nullptr);
+        dir = made ? made : "/tmp";
+    }
+    Mat w({1.5}), b({-0.5});
+    TensorList module({w.tensor(), b.tensor()});
+    const std::vector<std::string> names = {"w", "b"};
+    Sgd opt(0.1, {{1, 1}, {1, 1}}, NBO_DT_F64);
+    GradScaler scaler;
+    const ScheduleState schedule{0.1, LrSchedule::step(1, 0.9)};
+    TrainState state;
+    state.epoch = 2, state.step = 3, state.grad_accum = 1, state.rng_state = 42;
+    save_checkpoint(dir, module, names, opt, &scaler, &schedule, state);
+
+    Mat w2({0.0}), b2({0.0});
+    TensorList module2({w2.tensor(), b2.tensor()});
+    Sgd opt2(0.7, {{1, 1}, {1, 1}}, NBO_DT_F64);
+    GradScaler scaler2;
+    scaler2.load_state(GradScalerState{1.0, 3.0, 0.25, 7, 5});
+    TrainState state2;
+    std::optional<ScheduleState> schedule2;
+    load_checkpoint(dir, module2, names, opt2, &scaler2, schedule2, state2);
+    EXPECT(state2.epoch == 2);
+    EXPECT(state2.step == 3);
+    EXPECT(state2.rng_state && *state2.rng_state == 42);
+    EXPECT(schedule2.has_value());
+    EXPECT(schedule2 && schedule2->base_lr == 0.1 && schedule2->schedule.kind == LrSchedule::Step &&
+           schedule2->schedule.step_size == 1 && schedule2->schedule.gamma == 0.9);
+    EXPECT(w2.get() == 1.5 && b2.get() == -0.5);
+    EXPECT(opt2.lr() == 0.1 && scaler2.scale_factor() == 65536.0 && scaler2.state().growth_interval == 2000);
+    // Rust's f64 Display, which meta.txt is written with
+    EXPECT(rust_f64_str(0.1) == "0.1" && rust_f64_str(65536.0) == "65536" && rust_f64_str(1e-8) == "0.00000001");
+    EXPECT(rust_f64_str(1e21) == "1000000000000000000000" && rust_f64_str(-2.5) == "-2.5" && rust_f64_str(0.0) == "0");
+    // a checkpoint of another optimizer kind is refused with the reference's error
+    Adam other(0.1, {{1, 1}, {1, 1}}, NBO_DT_F64);
+    std::string what;
+    try {
+        load_checkpoint(dir, module2, names, other, nullptr, schedule2, state2);
+    } catch (const CheckpointError &e) {
+        what = e.what();
+    }
+    EXPECT(what.find("missing m0") != std::string::npos || what.find("optim kind mismatch") != std::string::npos);
+}
+
 static void panics_and_errors()  // alg.rs:110-119, 531-545; tensor/ops.rs:638-646
 {
     Mat p({1.0}), g({1.0}), g2({1.0, 2.0});
@@ -266,8 +318,9 @@ static void panics_and_errors()  // alg.rs:110-119, 531-545; tensor/ops.rs:638-6
     EXPECT(p.get() == 1.0);  // nothing ran
 }
 
-int main()
+int main(int argc, char **argv)
 {
+    if (argc > 1) g_checkpoint_dir = argv[1];
     struct {
         const char *name;
         void (*fn)();
@@ -283,6 +336,7 @@ int main()
                  {"nan_policy_skip_drops_step", nan_policy_skip_drops_step},
                  {"trainer_accumulates_then_clips_and_steps", trainer_accumulates_then_clips_and_steps},
                  {"backend_axpy_is_multiply_then_add", backend_axpy_is_multiply_then_add},
+                 {"checkpoint_roundtrip_with_schedule", checkpoint_roundtrip_with_schedule},
                  {"panics_and_errors", panics_and_errors}};
     try {
         check(nbo_init());

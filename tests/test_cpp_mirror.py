@@ -1,8 +1,10 @@
-"""The C++ mirror of the reference interface (include/nabla_optim.hpp) replays the
-reference's own optimizer tests on the device (tests/cpp/test_reference_kats.cpp)."""
+"""The C++ mirror of the reference interface (include/nabla_optim.hpp,
+include/nabla_checkpoint.hpp) replays the reference's own optimizer and trainer tests on
+the device (tests/cpp/test_reference_kats.cpp)."""
 import os
 import subprocess
 
+import numpy as np
 import pytest
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -14,8 +16,31 @@ def test_cpp_replay_is_built():
 
 
 @pytest.mark.gpu
-def test_cpp_replay_of_reference_tests(gpu):
-    r = subprocess.run([BIN], capture_output=True, text=True, timeout=120)
+def test_cpp_replay_of_reference_tests(gpu, tmp_path):
+    r = subprocess.run([BIN, str(tmp_path)], capture_output=True, text=True, timeout=120)
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count("ok    ") == 13 and "0 failure(s)" in r.stdout
+    assert r.stdout.count("ok    ") == 14 and "0 failure(s)" in r.stdout
+
+    # the checkpoint the C++ side left behind is the one the Python mirror writes and reads
+    from nabla_amd import checkpoint as ck
+    from nabla_amd import optim as nb
+    from nabla_amd.schedule import ScheduleState, Step
+    from tests import helpers as H
+
+    assert sorted(os.listdir(tmp_path)) == ["meta.txt", "optim.nbla", "params.nbla"]
+    shapes = [(1, 1), (1, 1)]
+    opt = nb.Sgd.new(0.7, shapes, dtype="f64")
+    scaler = nb.GradScaler.new()
+    params, state, schedule = ck.load_checkpoint(str(tmp_path), opt, scaler)
+    assert (state.epoch, state.step, state.grad_accum, state.rng_state) == (2, 3, 1, 42)
+    assert schedule == ScheduleState(base_lr=0.1, schedule=Step(step_size=1, gamma=0.9))
+    assert [(k, float(v[0, 0])) for k, v in params] == [("w", 1.5), ("b", -0.5)]
+    assert opt.meta().lr == 0.1 and scaler.state().scale == 65536.0
+    other = tmp_path / "py"
+    ck.save_checkpoint(str(other), [("w", H.to_dev(np.array([1.5]), (1, 1))), ("b", H.to_dev(np.array([-0.5]), (1, 1)))],
+                       nb.Sgd.new(0.1, shapes, dtype="f64"), nb.GradScaler.new(),
+                       ScheduleState(base_lr=0.1, schedule=Step(step_size=1, gamma=0.9)),
+                       ck.TrainState(epoch=2, step=3, grad_accum=1, rng_state=42))
+    for name in ("meta.txt", "params.nbla", "optim.nbla"):
+        assert (other / name).read_bytes() == (tmp_path / name).read_bytes(), name
