@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "../../include/nabla_checkpoint.hpp"
+#include "../../include/nabla_groups.hpp"
 
 using namespace nabla::optim;
 
@@ -141,15 +142,30 @@ static void clip_grad_norm_scales()  // trainer.rs:171-203
     EXPECT(clip_grad_norm(grads, 0.0) == 0.0);  // trainer.rs:501-503
 }
 
-static void weight_decay_exclusion()  // optim.rs:140-165, the two groups as two optimizers
+static void weight_decay_exclusion()  // optim.rs:140-165
 {
-    Mat weight({2.0}), bias({3.0}), zero({0.0});
-    Sgd decay(1.0, {{1, 1}}, NBO_DT_F64), no_decay(1.0, {{1, 1}}, NBO_DT_F64);
-    decay.weight_decay(0.1);
-    decay.step({weight.tensor()}, {zero.tensor()});
-    no_decay.step({bias.tensor()}, {zero.tensor()});
+    Mat weight({2.0}), bias({3.0}), zero_w({0.0}), zero_b({0.0});
+    const std::vector<std::pair<std::string, Tensor>> named = {{"weight", weight.tensor()}, {"bias", bias.tensor()}};
+    const ParamGroupConfig bias_group =
+        ParamGroupConfig::sgd("no_decay", ParamSelector::Any({{ParamMatch::Suffix, "bias"}}), 1.0, 0.0, 0.0);
+    const ParamGroupConfig decay_group = ParamGroupConfig::sgd("decay", ParamSelector::All(), 1.0, 0.0, 0.1);
+    GroupOptimizer opt = GroupOptimizer::from_named_params(named, {bias_group}, &decay_group, NBO_DT_F64);
+    EXPECT(opt.groups() == 2 && opt.group_indices(0) == std::vector<size_t>{1} && opt.group_indices(1) == std::vector<size_t>{0});
+    opt.step({weight.tensor(), bias.tensor()}, {zero_w.tensor(), zero_b.tensor()});
     EXPECT(std::fabs(weight.get() - 1.8) < 1e-10);
     EXPECT(std::fabs(bias.get() - 3.0) < 1e-10);
+    // set_lr keeps the groups' proportions (groups.rs:302-312); the fused tail decides once for all
+    opt.set_lr(0.5);
+    opt.fused_step({weight.tensor(), bias.tensor()}, {zero_w.tensor(), zero_b.tensor()}, nullptr, 1.0);
+    EXPECT(std::fabs(weight.get() - 1.8 * (1.0 - 0.5 * 0.1)) < 1e-12);
+    EXPECT(std::fabs(bias.get() - 3.0) < 1e-10);
+    bool refused = false;
+    try {
+        GroupOptimizer::from_named_params(named, {bias_group}, nullptr, NBO_DT_F64);
+    } catch (const StateError &e) {
+        refused = std::string(e.what()) == "nabla-train: group assignment incomplete";
+    }
+    EXPECT(refused);
 }
 
 static void lr_schedules()  // optim.rs:83-118
