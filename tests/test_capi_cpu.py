@@ -175,3 +175,26 @@ def test_step_with_vars_panics_like_the_reference():
         opt.step_with_vars(_Module([object(), object()]), [_Var(object())])
     with pytest.raises(nb.NablaPanic, match=r"param_vars\[1\] has no gradient \(call backward first\)"):
         opt.step_with_vars(_Module([object(), object()]), [_Var(object()), _Var(None)])
+
+
+def test_header_is_plain_c99_and_links_from_c(tmp_path):
+    """The boundary is a C ABI: a C99 translation unit that includes the header compiles
+    with -pedantic -Werror, links against the library and calls it."""
+    import subprocess
+
+    src = tmp_path / "t.c"
+    src.write_text('#include "nabla_optim.h"\n#include <stdio.h>\n#include <string.h>\n'
+                   "int main(void) {\n"
+                   "    nbo_meta m; nbo_scaler_state s; nbo_step_info i;\n"
+                   "    memset(&m, 0, sizeof m); memset(&s, 0, sizeof s); memset(&i, 0, sizeof i);\n"
+                   '    printf("%s|%s|%d\\n", nbo_version(), nbo_status_string(NBO_ERR_KIND), (int)NBO_BACKEND_AXPY);\n'
+                   "    return nbo_optim_step(0, 0, 0) == NBO_ERR_ARG ? 0 : 1;\n"
+                   "}\n")
+    exe = tmp_path / "t"
+    libdir = os.path.join(ROOT, "nabla_amd")
+    r = subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(ROOT, "include"),
+                        "-o", str(exe), str(src), "-L", libdir, "-l:libnabla_optim.so",
+                        f"-Wl,-rpath,{libdir}", "-Wl,-rpath,/opt/rocm/lib"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0 and r.stdout.strip() == "0.1.0|optim kind mismatch|1", r.stdout + r.stderr
