@@ -198,3 +198,51 @@ def test_header_is_plain_c99_and_links_from_c(tmp_path):
     assert r.returncode == 0, r.stderr
     r = subprocess.run([str(exe)], capture_output=True, text=True)
     assert r.returncode == 0 and r.stdout.strip() == "0.1.0|optim kind mismatch|1", r.stdout + r.stderr
+
+
+def test_null_arguments_are_errors_not_crashes():
+    """Every entry point checks its pointers before it touches the device: with nulls
+    they return NBO_ERR_ARG and leave a message, with or without a GPU."""
+    lib = _lib.load()
+    null = None
+    calls = [
+        lambda: lib.nbo_list_create(1, null, null, 0, null, null),
+        lambda: lib.nbo_list_set_ptrs(null, null),
+        lambda: lib.nbo_optim_create(null, 0, null, null, 0, 0, null),
+        lambda: lib.nbo_optim_step(null, null, null),
+        lambda: lib.nbo_optim_reset(null),
+        lambda: lib.nbo_optim_set_lr(null, 0.1),
+        lambda: lib.nbo_optim_get_meta(null, null),
+        lambda: lib.nbo_optim_load_meta(null, null),
+        lambda: lib.nbo_optim_state_read(null, b"m0", null, 0, 0),
+        lambda: lib.nbo_optim_state_write(null, b"m0", null, 0, 0),
+        lambda: lib.nbo_optim_master_from_params(null, null),
+        lambda: lib.nbo_optim_state_regions(null, null),
+        lambda: lib.nbo_scaler_create(null, null),
+        lambda: lib.nbo_scaler_state_get(null, null),
+        lambda: lib.nbo_scaler_load_state(null, null),
+        lambda: lib.nbo_scaler_unscale_and_update(null, null, null),
+        lambda: lib.nbo_clip_grad_norm(null, 1.0, null),
+        lambda: lib.nbo_has_non_finite(null, null),
+        lambda: lib.nbo_zero_grad(null),
+        lambda: lib.nbo_scale_grad(null, 1.0),
+        lambda: lib.nbo_fused_step(null, null, null, null, 1.0, 0),
+        lambda: lib.nbo_fused_step_groups(1, null, null, null, null, null, 1.0, 0),
+        lambda: lib.nbo_accumulate(null, null, 0),
+        lambda: lib.nbo_backend_apply(0, null, null, null, 1.0),
+        lambda: lib.nbo_backend_apply(99, null, null, null, 1.0),
+        lambda: lib.nbo_backend_cast(null, null),
+        lambda: lib.nbo_optim_last_step(null, null),
+        lambda: lib.nbo_optim_trace_read(null, null, 0, null, null),
+        lambda: lib.nbo_nbla_save_list(b"/nonexistent/x", null, null),
+        lambda: lib.nbo_nbla_load_list(b"/nonexistent/x", null, null),
+        lambda: lib.nbo_optim_save_state(null, b"/nonexistent/x"),
+        lambda: lib.nbo_optim_load_state(null, b"/nonexistent/x"),
+        lambda: lib.nbo_copy_bytes(null, null, 16),
+        lambda: lib.nbo_profile_read(null, null, null),
+    ]
+    for k, call in enumerate(calls):
+        assert call() == _lib.ERR_ARG, f"call {k}"
+        assert lib.nbo_last_error(), f"call {k} left no message"
+    # destroying nothing is fine, as free(NULL) is
+    assert lib.nbo_list_destroy(null) in (0, _lib.ERR_NO_DEVICE)
