@@ -8,6 +8,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <limits>
 #include <string>
 #include <vector>
@@ -334,8 +335,28 @@ static void panics_and_errors()  // alg.rs:110-119, 531-545; tensor/ops.rs:638-6
     EXPECT(p.get() == 1.0);  // nothing ran
 }
 
+// `--lr`: prints lr_at_step for a grid of schedules and steps as f64 bit patterns, for a
+// bit-for-bit comparison with the CPU oracle (needs no device).
+static int print_lr_grid()
+{
+    const LrSchedule scheds[] = {LrSchedule::cosine(10, 110, 1e-5), LrSchedule::cosine(0, 7, 0.0),
+                                 LrSchedule::linear(5, 50),         LrSchedule::linear(0, 1),
+                                 LrSchedule::one_cycle(1e-2, 100, 0.3), LrSchedule::one_cycle(0.5, 9, 0.0),
+                                 LrSchedule::step(3, 0.7),          LrSchedule::step(0, 0.5)};
+    for (size_t k = 0; k < sizeof(scheds) / sizeof(scheds[0]); k++)
+        for (uint64_t step = 0; step <= 120; step += (step < 12 ? 1 : 9)) {
+            const double lr = lr_at_step(scheds[k], 3e-4, step);
+            uint64_t bits;
+            static_assert(sizeof(bits) == sizeof(lr), "f64 is 64 bits");
+            std::memcpy(&bits, &lr, 8);
+            std::printf("%zu %llu %016llx\n", k, (unsigned long long)step, (unsigned long long)bits);
+        }
+    return 0;
+}
+
 int main(int argc, char **argv)
 {
+    if (argc > 1 && std::string(argv[1]) == "--lr") return print_lr_grid();
     if (argc > 1) g_checkpoint_dir = argv[1];
     struct {
         const char *name;

@@ -15,6 +15,26 @@ def test_cpp_replay_is_built():
     assert os.path.exists(BIN), "build it with `make -C tests/cpp` (or __graft_entry__.build())"
 
 
+def test_cpp_lr_at_step_matches_the_oracle_bit_for_bit():
+    """The C++ mirror's lr_at_step over a grid of schedules and steps against the oracle's
+    restatement of optim/core.rs:81-173 (no device involved)."""
+    import struct
+
+    import oracle as O
+
+    r = subprocess.run([BIN, "--lr"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0, r.stderr
+    scheds = [O.Schedule(0, 10, 110, 1e-5, 0.0), O.Schedule(0, 0, 7, 0.0, 0.0), O.Schedule(1, 5, 50, 0.0, 0.0),
+              O.Schedule(1, 0, 1, 0.0, 0.0), O.Schedule(2, 0, 100, 1e-2, 0.3), O.Schedule(2, 0, 9, 0.5, 0.0),
+              O.Schedule(3, 3, 0, 0.7, 0.0), O.Schedule(3, 0, 0, 0.5, 0.0)]
+    lines = r.stdout.split("\n")[:-1]
+    assert len(lines) == 8 * 25
+    for line in lines:
+        k, step, bits = line.split()
+        want = O.lr_at_step(scheds[int(k)], 3e-4, int(step))
+        assert struct.pack("<d", want) == struct.pack("<Q", int(bits, 16)), line
+
+
 @pytest.mark.gpu
 def test_cpp_replay_of_reference_tests(gpu, tmp_path):
     r = subprocess.run([BIN, str(tmp_path)], capture_output=True, text=True, timeout=120)
