@@ -112,13 +112,15 @@ def _declare(L):
     L.orc_bf16_from_f32.argtypes = [C.c_float]
     L.orc_bf16_from_f64.restype = C.c_uint16
     L.orc_bf16_from_f64.argtypes = [C.c_double]
+    L.orc_f16_from_f64.restype = C.c_uint16
+    L.orc_f16_from_f64.argtypes = [C.c_double]
     L.orc_bf16_to_f32.restype = C.c_float
     L.orc_bf16_to_f32.argtypes = [C.c_uint16]
     L.orc_lr_at_step.restype = C.c_double
     L.orc_lr_at_step.argtypes = [C.POINTER(Schedule), C.c_double, C.c_uint64]
     L.orc_get_pow_mode.restype = C.c_int
     L.orc_get_threads.restype = C.c_int
-    for suf in ("f32", "f64", "bf16"):
+    for suf in ("f32", "f64", "bf16", "f16"):
         getattr(L, f"orc_clip_grad_norm_{suf}").restype = C.c_double
         getattr(L, f"orc_clip_grad_norm_{suf}").argtypes = [
             C.c_size_t, C.c_void_p, C.c_void_p, C.c_double]
@@ -144,6 +146,8 @@ def _suffix(arr: np.ndarray) -> str:
         return "f64"
     if arr.dtype == np.uint16:  # bf16 bit patterns
         return "bf16"
+    if arr.dtype == np.float16:
+        return "f16"
     raise TypeError(f"oracle: unsupported dtype {arr.dtype}")
 
 
@@ -163,6 +167,8 @@ def _ctype(arr):
     patterns) the Python float is narrowed with bf16::from_f64 first."""
     if arr.dtype == np.uint16:
         return lambda s: C.c_uint16(lib().orc_bf16_from_f64(C.c_double(s)))
+    if arr.dtype == np.float16:
+        return lambda s: C.c_uint16(lib().orc_f16_from_f64(C.c_double(s)))
     return C.c_float if arr.dtype == np.float32 else C.c_double
 
 
@@ -238,11 +244,12 @@ def map_add(a, c):
     return out
 
 
-_CAST_TYPE = {np.dtype(np.float32): 0, np.dtype(np.uint16): 1, np.dtype(np.float64): 2}
+_CAST_TYPE = {np.dtype(np.float32): 0, np.dtype(np.uint16): 1, np.dtype(np.float64): 2, np.dtype(np.float16): 3}
 
 
 def cast(src: np.ndarray, dst_dtype) -> np.ndarray:
-    """B::cast default (backend/mod.rs:157-160); np.uint16 stands for bf16 patterns."""
+    """B::cast default (backend/mod.rs:157-160); np.uint16 stands for bf16 patterns,
+    np.float16 is f16."""
     src = np.ascontiguousarray(src)
     out = np.empty(src.shape, dtype=dst_dtype)
     lib().orc_cast(C.c_void_p(src.ctypes.data), C.c_int(_CAST_TYPE[src.dtype]),
@@ -331,18 +338,20 @@ def f32_step(meta, scaler, max_norm, params, grads, m, v):
     return bool(ran), norm.value
 
 
-def mixed_step(meta, scaler, max_norm, params_bf16, grads_bf16, master, m, v):
-    """Trainer tail for bf16 params/grads with f32 master/m/v. Returns (ran, norm)."""
-    for a in list(params_bf16) + list(grads_bf16):
-        if a.dtype != np.uint16:
-            raise TypeError("oracle.mixed_step: bf16 tensors are uint16 bit patterns")
+def mixed_step(meta, scaler, max_norm, params_half, grads_half, master, m, v):
+    """Trainer tail for bf16 (np.uint16 patterns) or f16 (np.float16) params/grads with f32
+    master/m/v. Returns (ran, norm)."""
+    kinds = {a.dtype for a in list(params_half) + list(grads_half)}
+    if kinds - {np.dtype(np.uint16)} and kinds - {np.dtype(np.float16)}:
+        raise TypeError("oracle.mixed_step: tensors are bf16 bit patterns (uint16) or float16, not a mix")
+    half_type = 3 if np.dtype(np.float16) in kinds else 1
     norm = C.c_double(0.0)
     L = lib()
-    L.orc_mixed_step.restype = C.c_int
-    ran = L.orc_mixed_step(C.byref(meta), C.byref(scaler) if scaler is not None else None,
-                           C.c_double(max_norm), C.c_size_t(len(master)), _sizes(master),
-                           _ptrs(params_bf16), _ptrs(grads_bf16), _ptrs(master), _ptrs(m),
-                           _ptrs(v), C.byref(norm))
+    L.orc_mixed_step_half.restype = C.c_int
+    ran = L.orc_mixed_step_half(C.byref(meta), C.byref(scaler) if scaler is not None else None,
+                                C.c_double(max_norm), C.c_size_t(len(master)), _sizes(master),
+                                _ptrs(params_half), _ptrs(grads_half), C.c_int(half_type), _ptrs(master),
+                                _ptrs(m), _ptrs(v), C.byref(norm))
     return bool(ran), norm.value
 
 

@@ -62,6 +62,54 @@ float orc_bf16_to_f32(uint16_t h)
     return f;
 }
 
+/* half::f16::from_f32 (crate half 2.7.1, software path `f32_to_f16_fallback`; the F16C
+ * instruction it uses where the CPU has it gives the same bits): IEEE binary16, round to
+ * nearest even, subnormals kept, overflow to infinity; NaN keeps its top ten payload
+ * bits and gets the quiet bit. */
+uint16_t orc_f16_from_f32(float v)
+{
+    uint32_t x;
+    memcpy(&x, &v, 4);
+    uint32_t sign = x & 0x80000000u, exp = x & 0x7F800000u, man = x & 0x007FFFFFu;
+    if (exp == 0x7F800000u) {
+        uint32_t nan_bit = man == 0 ? 0u : 0x0200u;
+        return (uint16_t)((sign >> 16) | 0x7C00u | nan_bit | (man >> 13));
+    }
+    uint32_t half_sign = sign >> 16;
+    int32_t half_exp = (int32_t)(exp >> 23) - 127 + 15;
+    if (half_exp >= 0x1F) return (uint16_t)(half_sign | 0x7C00u);
+    if (half_exp <= 0) {
+        if (14 - half_exp > 24) return (uint16_t)half_sign; /* too small: signed zero */
+        man |= 0x00800000u;
+        uint32_t half_man = man >> (14 - half_exp);
+        uint32_t round_bit = 1u << (13 - half_exp);
+        if ((man & round_bit) != 0 && (man & (3u * round_bit - 1u)) != 0) half_man += 1;
+        return (uint16_t)(half_sign | half_man);
+    }
+    uint32_t bits = half_sign | ((uint32_t)half_exp << 10) | (man >> 13);
+    uint32_t round_bit = 0x00001000u;
+    if ((man & round_bit) != 0 && (man & (3u * round_bit - 1u)) != 0) bits += 1; /* may carry into the exponent */
+    return (uint16_t)bits;
+}
+
+/* f32::from(f16) (software path `f16_to_f32_fallback`): exact. */
+float orc_f16_to_f32(uint16_t h)
+{
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16, exp = (h >> 10) & 0x1Fu, man = h & 0x03FFu, x;
+    float f;
+    if (exp == 0x1Fu) {
+        x = sign | 0x7F800000u | (man ? (0x00400000u | (man << 13)) : 0u);
+    } else if (exp == 0) {
+        f = ldexpf((float)man, -24); /* subnormal or zero: man * 2^-24, exact */
+        memcpy(&x, &f, 4);
+        x |= sign;
+    } else {
+        x = sign | ((exp + 112u) << 23) | (man << 13);
+    }
+    memcpy(&f, &x, 4);
+    return f;
+}
+
 /* Tensor::cast (tensor/shape.rs:489-493) -> default B::cast
  * (backend/mod.rs:157-160): U::from_f64(get().to_f64()), serial from_fn. */
 void orc_cast_bf16_to_f32(const uint16_t *src, float *dst, size_t n)
@@ -219,12 +267,9 @@ double orc_lr_at_step(const orc_schedule *s, double base_lr, uint64_t step)
 #undef NEG_T
 #undef SUB_T
 
-/* ---- T = half::bf16 --------------------------------------------------------------------
- * Every operation on bf16 is the f32 operation followed by bf16::from_f32: the
- * reference's MathOps for half types (scalar/mod.rs:256-283: math_mul, math_div,
- * math_powf) and the half crate's own `+` and `*` operators (half 2.7.1, not vendored;
- * its documented software path converts to f32, operates and converts back). */
+/* ---- T = half::bf16 and T = half::f16 (oracle_half.inc) ---------------------------------- */
 uint16_t orc_bf16_from_f64(double v) { return orc_bf16_from_f32((float)v); } /* scalar/mod.rs:338-340 */
+uint16_t orc_f16_from_f64(double v) { return orc_f16_from_f32((float)v); }
 
 static float pow_f32_mode(float x, float p)
 {
@@ -235,89 +280,35 @@ static float pow_f32_mode(float x, float p)
     return powf(x, p);
 }
 
-#define BF(x) orc_bf16_to_f32(x)
-#define RB(x) orc_bf16_from_f32(x)
-void orc_scale_bf16(const uint16_t *a, uint16_t s, uint16_t *out, size_t n)
-{
-    long i, ln = (long)n;
-#pragma omp parallel for schedule(static) num_threads(g_threads) if (ln > PAR_MIN)
-    for (i = 0; i < ln; i++) out[i] = RB(BF(a[i]) * BF(s));
-}
-void orc_axpy_inplace_bf16(uint16_t *y, uint16_t alpha, const uint16_t *x, size_t n)
-{
-    long i, ln = (long)n;
-#pragma omp parallel for schedule(static) num_threads(g_threads) if (ln > PAR_MIN)
-    for (i = 0; i < ln; i++) {
-        uint16_t t = RB(BF(alpha) * BF(x[i])); /* alpha * xi is a bf16 value */
-        y[i] = RB(BF(y[i]) + BF(t));
-    }
-}
-void orc_emul_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n)
-{
-    long i, ln = (long)n;
-#pragma omp parallel for schedule(static) num_threads(g_threads) if (ln > PAR_MIN)
-    for (i = 0; i < ln; i++) out[i] = RB(BF(a[i]) * BF(b[i]));
-}
-void orc_ediv_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n)
-{
-    long i, ln = (long)n;
-#pragma omp parallel for schedule(static) num_threads(g_threads) if (ln > PAR_MIN)
-    for (i = 0; i < ln; i++) out[i] = RB(BF(a[i]) / BF(b[i]));
-}
-void orc_add_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, size_t n)
-{
-    long i, ln = (long)n;
-#pragma omp parallel for schedule(static) num_threads(g_threads) if (ln > PAR_MIN)
-    for (i = 0; i < ln; i++) out[i] = RB(BF(a[i]) + BF(b[i]));
-}
-void orc_powf_bf16(const uint16_t *a, uint16_t p, uint16_t *out, size_t n)
-{
-    long i, ln = (long)n;
-#pragma omp parallel for schedule(static) num_threads(g_threads) if (ln > PAR_MIN)
-    for (i = 0; i < ln; i++) out[i] = RB(pow_f32_mode(BF(a[i]), BF(p)));
-}
-void orc_map_add_bf16(const uint16_t *a, uint16_t c, uint16_t *out, size_t n)
-{
-    size_t i;
-    for (i = 0; i < n; i++) out[i] = RB(BF(a[i]) + BF(c));
-}
-void orc_map_mul_bf16(const uint16_t *a, uint16_t c, uint16_t *out, size_t n)
-{
-    size_t i;
-    for (i = 0; i < n; i++) out[i] = RB(BF(a[i]) * BF(c));
-}
+#define HFN(x) x##_bf16
+#define H_TO_F32(h) orc_bf16_to_f32(h)
+#define H_FROM_F32(f) orc_bf16_from_f32(f)
+#include "oracle_half.inc"
+#undef HFN
+#undef H_TO_F32
+#undef H_FROM_F32
 
-/* Sgd / Adam / AdamW / GradScaler / clip_grad_norm for T = bf16: the same bodies as for
- * f32 and f64, over the bf16 primitive passes above. */
-#define T uint16_t
-#define FN(x) x##_bf16
-#define FROM_F64(x) orc_bf16_from_f64(x)
-#define TO_F64(x) ((double)orc_bf16_to_f32(x))
-#define NEG_T(x) ((uint16_t)((x) ^ 0x8000u))           /* Neg on half types flips the sign bit */
-#define SUB_T(a, b) RB(BF(a) - BF(b))
-#define ORC_PRIMITIVES_ELSEWHERE
-#include "oracle_impl.inc"
-#undef ORC_PRIMITIVES_ELSEWHERE
-#undef T
-#undef FN
-#undef FROM_F64
-#undef TO_F64
-#undef NEG_T
-#undef SUB_T
-#undef BF
-#undef RB
+#define HFN(x) x##_f16
+#define H_TO_F32(h) orc_f16_to_f32(h)
+#define H_FROM_F32(f) orc_f16_from_f32(f)
+#include "oracle_half.inc"
+#undef HFN
+#undef H_TO_F32
+#undef H_FROM_F32
 
 /* B::cast default (backend/mod.rs:157-160): U::from_f64(x.to_f64()) per element.
- * Types: 0 = f32, 1 = bf16, 2 = f64. */
+ * Types: 0 = f32, 1 = bf16, 2 = f64, 3 = f16. */
 void orc_cast(const void *src, int src_type, void *dst, int dst_type, size_t n)
 {
     size_t i;
     for (i = 0; i < n; i++) {
         double v = src_type == 0   ? (double)((const float *)src)[i]
                    : src_type == 1 ? (double)orc_bf16_to_f32(((const uint16_t *)src)[i])
+                   : src_type == 3 ? (double)orc_f16_to_f32(((const uint16_t *)src)[i])
                                    : ((const double *)src)[i];
         if (dst_type == 0) ((float *)dst)[i] = (float)v;
         else if (dst_type == 1) ((uint16_t *)dst)[i] = orc_bf16_from_f64(v);
+        else if (dst_type == 3) ((uint16_t *)dst)[i] = orc_f16_from_f64(v);
         else ((double *)dst)[i] = v;
     }
 }
@@ -340,22 +331,31 @@ int orc_f32_step(orc_meta *meta, orc_scaler_state *scaler, double max_norm, size
     return 1;
 }
 
-int orc_mixed_step(orc_meta *meta, orc_scaler_state *scaler, double max_norm, size_t nt,
-                   const uint64_t *sizes, uint16_t **params_bf16, uint16_t *const *grads_bf16,
-                   float **master, float **m, float **v, double *norm_out)
+/* half_type: 1 = bf16, 3 = f16 (the type codes of orc_cast) */
+int orc_mixed_step_half(orc_meta *meta, orc_scaler_state *scaler, double max_norm, size_t nt,
+                        const uint64_t *sizes, uint16_t **params_h, uint16_t *const *grads_h, int half_type,
+                        float **master, float **m, float **v, double *norm_out)
 {
     size_t i;
     float **g32 = (float **)malloc((nt ? nt : 1) * sizeof(float *));
     if (!g32) abort();
-    for (i = 0; i < nt; i++) { /* g32 = g_bf16.cast::<f32>() */
+    for (i = 0; i < nt; i++) { /* g32 = g_half.cast::<f32>() */
         g32[i] = alloc_f32((size_t)sizes[i]);
-        orc_cast_bf16_to_f32(grads_bf16[i], g32[i], (size_t)sizes[i]);
+        orc_cast(grads_h[i], half_type, g32[i], 0, (size_t)sizes[i]);
     }
     int ran = orc_f32_step(meta, scaler, max_norm, nt, sizes, master, g32, m, v, norm_out);
     if (ran)
-        for (i = 0; i < nt; i++) /* p_bf16 = master.cast::<bf16>() */
-            orc_cast_f32_to_bf16(master[i], params_bf16[i], (size_t)sizes[i]);
+        for (i = 0; i < nt; i++) /* p_half = master.cast::<half>() */
+            orc_cast(master[i], 0, params_h[i], half_type, (size_t)sizes[i]);
     for (i = 0; i < nt; i++) free(g32[i]);
     free(g32);
     return ran;
+}
+
+int orc_mixed_step(orc_meta *meta, orc_scaler_state *scaler, double max_norm, size_t nt,
+                   const uint64_t *sizes, uint16_t **params_bf16, uint16_t *const *grads_bf16,
+                   float **master, float **m, float **v, double *norm_out)
+{
+    return orc_mixed_step_half(meta, scaler, max_norm, nt, sizes, params_bf16, grads_bf16, 1, master, m, v,
+                               norm_out);
 }

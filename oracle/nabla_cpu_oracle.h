@@ -146,7 +146,12 @@ ORC_DECLARE(f64, double)
  * bf16::from_f64 = from_f32(v as f32).  The same functions as for f32 / f64. */
 ORC_DECLARE(bf16, uint16_t)
 uint16_t orc_bf16_from_f64(double v);
-/* B::cast default, backend/mod.rs:157-160.  Types: 0 = f32, 1 = bf16, 2 = f64. */
+/* T = half::f16 likewise (IEEE binary16 patterns). */
+ORC_DECLARE(f16, uint16_t)
+uint16_t orc_f16_from_f32(float v);
+float orc_f16_to_f32(uint16_t h);
+uint16_t orc_f16_from_f64(double v);
+/* B::cast default, backend/mod.rs:157-160.  Types: 0 = f32, 1 = bf16, 2 = f64, 3 = f16. */
 void orc_cast(const void *src, int src_type, void *dst, int dst_type, size_t n);
 
 /*
@@ -162,6 +167,11 @@ void orc_cast(const void *src, int src_type, void *dst, int dst_type, size_t n);
 int orc_mixed_step(orc_meta *meta, orc_scaler_state *scaler, double max_norm, size_t nt,
                    const uint64_t *sizes, uint16_t **params_bf16, uint16_t *const *grads_bf16,
                    float **master, float **m, float **v, double *norm_out);
+
+/* The same composition for f16 tensors over f32 state: half_type 1 = bf16, 3 = f16. */
+int orc_mixed_step_half(orc_meta *meta, orc_scaler_state *scaler, double max_norm, size_t nt,
+                        const uint64_t *sizes, uint16_t **params_h, uint16_t *const *grads_h, int half_type,
+                        float **master, float **m, float **v, double *norm_out);
 
 /* Same tail for T = f32 throughout (params are the f32 tensors themselves);
  * grads are modified in place like the reference does. */

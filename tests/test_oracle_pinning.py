@@ -738,3 +738,82 @@ def test_bench_lcg_rand_tensor_in_exact_arithmetic():
     more, _ = O.bench_rand_f32(3, state)  # the stream continues across tensors
     x = (x * 6364136223846793005 + 1442695040888963407) % (1 << 64)
     assert f32_exact(more[0]) == r32(r32(r32(Fraction(x >> 33)) / (1 << 31)) - 1)
+
+
+# ---- 8. T = f16 -------------------------------------------------------------------------------
+
+def r16(q):  # IEEE binary16: 11 significand bits, subnormals down to 2^-24
+    return rne(Fraction(q), 11, -24)
+
+
+def test_f16_conversions_match_ieee_binary16_everywhere():
+    """half::f16::from_f32 / f32::from(f16) restated from the half crate's software path:
+    every one of the 65536 patterns widens exactly (against numpy's float16), and every
+    f16 value's neighbourhood in f32 -- the value, both ties and one f32 ulp either side of
+    them -- narrows as IEEE round-to-nearest-even does, overflow and subnormals included.
+    NaN: top ten payload bits kept, quiet bit set."""
+    all16 = np.arange(1 << 16, dtype=np.uint16).view(np.float16)
+    wide = O.cast(all16, np.float32)
+    finite = ~np.isnan(all16)
+    assert np.array_equal(wide[finite].view(np.uint32), all16[finite].astype(np.float32).view(np.uint32))
+    assert np.isnan(wide[~finite]).all()
+    base = all16[finite].astype(np.float32).view(np.uint32).astype(np.int64)
+    cand = []
+    for off in (0, 0x0FFF, 0x1000, 0x1001, -0x0FFF, -0x1000, -0x1001, 1, -1, 0x1FFF):
+        cand.append(base + off)
+    bits = np.concatenate(cand)
+    bits = bits[(bits >= 0) & (bits < (1 << 32))].astype(np.uint32)
+    x = bits.view(np.float32)
+    x = x[~np.isnan(x)]
+    got = O.cast(x, np.float16)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    for i in range(0, x.size, 9973):  # and a sample against exact rational rounding
+        q = r16(Fraction(float(x[i])))
+        if abs(q) < 65520:
+            assert Fraction(float(got[i])) == q, hex(int(x[i:i + 1].view(np.uint32)[0]))
+    nan_in = np.array([0x7FC00000, 0xFFC00000, 0x7F800001, 0x7FA5A000, 0xFF80E000], dtype=np.uint32).view(np.float32)
+    nan_out = O.cast(nan_in, np.float16).view(np.uint16)
+    assert list(nan_out) == [0x7E00, 0xFE00, 0x7E00, 0x7F2D, 0xFE07]
+
+
+@pytest.mark.parametrize("kind", ["adam", "adamw"])
+def test_f16_adam_chain_bit_exact_against_exact_arithmetic(kind):
+    """Optimizer<f16>: every result rounded to f32 and then to f16."""
+    rng = np.random.default_rng(21)
+    n, steps = 16, 4
+    lr, b1, b2, eps, wd = 1e-2, 0.9, 0.95, 1e-4, 0.1  # eps representable in f16 (1e-8 narrows to 0)
+    rt = lambda q: r16(r32(q))
+    fx = lambda x: Fraction(float(x))
+    p0 = (rng.standard_normal(n) * 0.5).astype(np.float16)
+    grads = [(rng.standard_normal(n) * 1e-1).astype(np.float16) for _ in range(steps)]
+    pe, me, ve = _exact_adam(kind, lr, b1, b2, eps, wd, steps, p0, grads, rt=rt, exact=fx)
+    p, m, v = [p0.copy()], [np.zeros(n, np.float16)], [np.zeros(n, np.float16)]
+    meta = O.adam_meta(lr, b1, b2, eps) if kind == "adam" else O.adamw_meta(lr, b1, b2, eps, wd)
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        for t in range(steps):
+            O.adam_step(meta, p, [grads[t]], m, v)
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+    for i in range(n):
+        assert fx(m[0][i]) == me[i] and fx(v[0][i]) == ve[i] and fx(p[0][i]) == pe[i], i
+    assert any(x != 0 for x in v[0])
+
+
+def test_f16_mixed_step_is_the_f32_step_between_two_casts():
+    rng = np.random.default_rng(22)
+    n = 64
+    w0 = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    g16 = (rng.standard_normal(n) * 4.0).astype(np.float16)
+    meta, s = O.adamw_meta(1e-3, weight_decay=0.1), O.ScalerState(1024.0, 2.0, 0.5, 2, 0)
+    p, w, m, v = [w0.astype(np.float16)], [w0.copy()], [np.zeros(n, np.float32)], [np.zeros(n, np.float32)]
+    ran, norm = O.mixed_step(meta, s, 0.01, p, [g16], w, m, v)
+    meta2, s2 = O.adamw_meta(1e-3, weight_decay=0.1), O.ScalerState(1024.0, 2.0, 0.5, 2, 0)
+    w2, m2, v2 = [w0.copy()], [np.zeros(n, np.float32)], [np.zeros(n, np.float32)]
+    ran2, norm2 = O.f32_step(meta2, s2, 0.01, w2, [g16.astype(np.float32)], m2, v2)
+    assert ran and ran2 and norm == norm2
+    assert np.array_equal(w[0].view(np.uint32), w2[0].view(np.uint32))
+    with np.errstate(over="ignore"):
+        assert np.array_equal(p[0].view(np.uint16), w2[0].astype(np.float16).view(np.uint16))
