@@ -46,7 +46,7 @@ typedef enum nbo_status {
     NBO_ERR_KIND = 6,           /* "optim kind mismatch"               alg.rs:531-545 */
     NBO_ERR_DTYPE = 7,          /* element types of the lists / optimizer do not fit */
     NBO_ERR_ARG = 8,            /* null pointer, zero-sized list, bad enum value */
-    NBO_ERR_NO_MASTER = 9,      /* bf16 step before master weights were set */
+    NBO_ERR_NO_MASTER = 9,      /* bf16 / f16 step before master weights were set */
     NBO_ERR_TOO_LARGE = 10,     /* more than 2^24-1 chunks of 8192 elements (1.4e11 elements) */
     NBO_ERR_NO_DEVICE = 11,     /* no gfx950 device / code object not loadable */
     NBO_ERR_IO = 12,            /* checkpoint file: io::Error of save_tensors / load_tensors */
@@ -54,7 +54,7 @@ typedef enum nbo_status {
 } nbo_status;
 
 /* Element type of caller tensors. */
-typedef enum nbo_dtype { NBO_DT_F32 = 0, NBO_DT_BF16 = 1, NBO_DT_F64 = 2 } nbo_dtype;
+typedef enum nbo_dtype { NBO_DT_F32 = 0, NBO_DT_BF16 = 1, NBO_DT_F64 = 2, NBO_DT_F16 = 3 } nbo_dtype;
 
 /* OptimKind, in the reference's order (optim/core.rs:46-51). */
 typedef enum nbo_kind { NBO_KIND_ADAMW = 0, NBO_KIND_ADAM = 1, NBO_KIND_SGD = 2 } nbo_kind;
@@ -119,11 +119,11 @@ int nbo_list_destroy(nbo_list *list);
 /* Sgd::new / Adam::new / AdamW::new (alg.rs:319-330, 181-199, 20-39) + the builder
  * setters, all at once through `meta` (meta->kind selects the algorithm;
  * meta->step_count seeds step_count).  Moments are created zero-filled.
- * state_dtype: NBO_DT_F32, NBO_DT_F64 or NBO_DT_BF16 -- the arithmetic type T, which is
- * also the type of the moments and of the caller's tensors (T = bf16: every operation is
- * the f32 operation followed by bf16::from_f32, common/scalar/mod.rs:253-351).
+ * state_dtype: NBO_DT_F32, NBO_DT_F64, NBO_DT_BF16 or NBO_DT_F16 -- the arithmetic type T,
+ * which is also the type of the moments and of the caller's tensors (T = bf16 / f16: every
+ * operation is the f32 operation followed by T::from_f32, common/scalar/mod.rs:253-351).
  * keep_master != 0 (f32 state only): additionally hold f32 master weights so that the
- * caller's parameters and gradients may be bf16 while the arithmetic stays T = f32.
+ * caller's parameters and gradients may be bf16 or f16 while the arithmetic stays T = f32.
  * State of 128 MiB per array or more is assembled from physical chunks chosen so that
  * the arrays lie in different regions of the HBM (nbo_optim_state_regions tells the
  * outcome); that takes up to a few seconds here and nothing per step. */
@@ -153,10 +153,10 @@ int nbo_optim_state_read(nbo_optim *opt, const char *name, void *buf, uint64_t n
                          int on_device);
 int nbo_optim_state_write(nbo_optim *opt, const char *name, const void *buf, uint64_t n_elems,
                           int on_device);
-/* master = f32(params) for bf16 parameter lists (Tensor::cast, tensor/shape.rs:489-493),
- * and the converse params = bf16(master). */
-int nbo_optim_master_from_params(nbo_optim *opt, nbo_list *params_bf16);
-int nbo_optim_params_from_master(nbo_optim *opt, nbo_list *params_bf16);
+/* master = f32(params) for bf16 or f16 parameter lists (Tensor::cast, tensor/shape.rs:489-493),
+ * and the converse params = bf16(master) / f16(master). */
+int nbo_optim_master_from_params(nbo_optim *opt, nbo_list *params_half);
+int nbo_optim_params_from_master(nbo_optim *opt, nbo_list *params_half);
 
 /* How the optimizer's state arrays were placed in HBM: *regions = 0 for plain
  * allocations, otherwise the number of 96 GiB HBM regions their chunks were spread
@@ -197,7 +197,7 @@ int nbo_scale_grad(nbo_list *grads, double factor);
  *   scaler.unscale_and_update(grads)  -> found_inf, skip, scale update
  *   clip_grad_norm(grads, max_norm)   -> only when max_norm > 0
  *   optimizer.step(params, grads)     -> unscale and clip factors applied on the fly
- *   params = bf16(master)             -> for bf16 lists
+ *   params = bf16(master)             -> for bf16 lists (f16(master) for f16 lists)
  *   zero grads                        -> with NBO_STEP_ZERO_GRADS
  * `scaler` may be NULL.  Gradients are not modified (except for the optional
  * zeroing): the two factors are applied inside the update, element by element,
@@ -221,7 +221,7 @@ int nbo_accumulate(nbo_list *accum, nbo_list *grads, int zero_grads);
  * (nabla-core/src/common/backend/mod.rs:82-216; CPU semantics nabla-core/src/cpu/mod.rs:137-139,
  * 181, 211-232), BackendMath::{powf, emul, ediv} (backend/mod.rs:275-279; cpu/mod.rs:264-272) and
  * Tensor::map(|x| x + s) (nabla-train/src/optim/alg.rs:133).  One IEEE operation per element
- * in the lists' element type (bf16: the f32 operation, then bf16::from_f32,
+ * in the lists' element type (bf16 / f16: the f32 operation, then T::from_f32,
  * common/scalar/mod.rs:253-351); `s` is narrowed with T::from_f64.  All lists share shapes and
  * element type; `out` may alias an operand.  powf with s = 0.5 is the correctly rounded
  * square root, other exponents use the device math library (within 2 ulp of libm).  The
@@ -240,8 +240,8 @@ typedef enum nbo_backend_op {
 } nbo_backend_op;
 int nbo_backend_apply(int op, nbo_list *out, nbo_list *a, nbo_list *b, double s);
 /* BackendCore::cast, default implementation (backend/mod.rs:157-160): dst = U::from_f64(
- * src.to_f64()) per element, between any two of f32 / bf16 / f64 (f64 -> bf16 rounds to f32
- * first, as bf16::from_f64 does).  Asynchronous. */
+ * src.to_f64()) per element, between any two of f32 / bf16 / f16 / f64 (f64 -> bf16 or f16
+ * rounds to f32 first, as their from_f64 does).  Asynchronous. */
 int nbo_backend_cast(nbo_list *dst, nbo_list *src);
 
 /* Outcome of the optimizer's most recent fused step.  Synchronous. */

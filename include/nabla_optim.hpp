@@ -170,7 +170,7 @@ private:
 };
 
 // trait Optimizer + trait OptimState.  T is float or double (the arithmetic type);
-// with `master` the caller's tensors may be bf16 while the state stays f32.
+// with `master` the caller's tensors may be bf16 or f16 while the state stays f32.
 class Optimizer {
 public:
     Optimizer(const Optimizer &) = delete;
@@ -259,7 +259,7 @@ public:
     // save_tensors, load_tensors into load_state_tensors; errors as StateError / RuntimeError
     void save_state(const std::string &path) { check(nbo_optim_save_state(handle(), path.c_str())); }
     void load_state(const std::string &path) { check(nbo_optim_load_state(handle(), path.c_str())); }
-    void master_from_params(TensorList &params_bf16) { check(nbo_optim_master_from_params(handle(), params_bf16.handle())); }
+    void master_from_params(TensorList &params_half) { check(nbo_optim_master_from_params(handle(), params_half.handle())); }
 
     nbo_optim *handle()
     {

@@ -29,7 +29,7 @@ ERR_NO_DEVICE = 11
 ERR_IO = 12
 ERR_HIP = 1000
 
-DT_F32, DT_BF16, DT_F64 = 0, 1, 2
+DT_F32, DT_BF16, DT_F64, DT_F16 = 0, 1, 2, 3
 KIND_ADAMW, KIND_ADAM, KIND_SGD = 0, 1, 2
 
 STEP_ZERO_GRADS = 1

@@ -8,7 +8,7 @@ nabla-core/src/cpu/mod.rs:137-139, 181, 211-232, 264-272): `scale`, `axpy_inplac
 tensor list -- the generalisation of the reference's never-launched `k_multi_axpy3`
 (cuda_hip/common/kernels/k_ops.cuh:541-575) from three tensors to any number -- with the
 reference's rounding: one IEEE operation per element in the list's element type (for bf16
-the f32 operation followed by `bf16::from_f32`).
+and f16 the f32 operation followed by `T::from_f32`).
 
 Arguments are sequences of same-dtype device tensors (anything with `data_ptr()`,
 `shape`, `dtype`: torch tensors on cuda:0) or `TensorList`s.  Functions that produce a new
@@ -85,6 +85,6 @@ def clone_storage(a: Tensors, out: Tensors) -> None:
 
 def cast(src: Tensors, dst: Tensors) -> None:
     """B::cast default (backend/mod.rs:157-160): dst = U::from_f64(src.to_f64()), between
-    any two of f32 / bf16 / f64."""
+    any two of f32 / bf16 / f16 / f64."""
     ld, ls = _list(dst), _list(src)  # keep the descriptors alive across the call
     _call(_lib.load().nbo_backend_cast(ld._h, ls._h))

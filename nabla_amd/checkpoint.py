@@ -47,14 +47,14 @@ class TrainState:
 
 
 def _to_host_f64(t) -> np.ndarray:
-    """Tensor -> 2-D float64 array, through f32 for bf16 (scalar/mod.rs:342-344)."""
+    """Tensor -> 2-D float64 array, through f32 for bf16 / f16 (scalar/mod.rs:342-344)."""
     if isinstance(t, np.ndarray):
         a = t
     else:  # torch tensor
         import torch
 
         x = t.detach()
-        if x.dtype == torch.bfloat16:
+        if x.dtype in (torch.bfloat16, torch.float16):
             x = x.float()
         a = x.cpu().numpy()
     if a.ndim == 1:

@@ -83,13 +83,14 @@ void check_step_args(const nbo_optim *opt, const nbo_list *params, const nbo_lis
                      std::to_string(t) + ")");
     }
     require(params->dtype == grads->dtype, NBO_ERR_DTYPE, "params and grads differ in element type");
-    if (params->dtype == NBO_DT_BF16 && opt->state_dtype == NBO_DT_BF16) {
-        // Optimizer<bf16>: state and arithmetic in bf16, no master copy
-    } else if (params->dtype == NBO_DT_BF16) {
+    if (is_half(params->dtype) && opt->state_dtype == params->dtype) {
+        // Optimizer<bf16> / Optimizer<f16>: state and arithmetic in the tensors' type, no master copy
+    } else if (is_half(params->dtype)) {
         require(opt->state_dtype == NBO_DT_F32 && opt->keep_master, NBO_ERR_DTYPE,
-                "bf16 tensors need an optimizer created with bf16 state, or with f32 state and keep_master");
+                "bf16 / f16 tensors need an optimizer created with state of their own type, or with f32 "
+                "state and keep_master");
         require(opt->master_valid, NBO_ERR_NO_MASTER,
-                "bf16 step before the master weights were set (nbo_optim_master_from_params or "
+                "bf16 / f16 step before the master weights were set (nbo_optim_master_from_params or "
                 "nbo_optim_state_write \"w{i}\")");
     } else {
         require(params->dtype == opt->state_dtype, NBO_ERR_DTYPE,
@@ -111,12 +112,19 @@ NboUpdateArgs update_args(nbo_optim *opt, nbo_list *params, nbo_list *grads, boo
     return a;
 }
 
-bool pure_bf16(const nbo_optim *opt) { return opt->state_dtype == NBO_DT_BF16; }
+// the optimizer's own arithmetic type is a 16-bit one (Optimizer<bf16> / Optimizer<f16>)
+bool pure_half(const nbo_optim *opt) { return is_half(opt->state_dtype); }
+
+// kernel id for element type `dtype`: f32 / bf16 / f64 are `base + dtype`, f16 has its own
+int kernel_for(int base, int f16_id, int dtype) { return dtype == NBO_DT_F16 ? f16_id : base + dtype; }
 
 int update_kernel(const nbo_optim *opt, const nbo_list *params)
 {
-    if (pure_bf16(opt)) return K_UPDATE_PBF16_BASE + opt->meta.kind;
-    return K_UPDATE_BASE + params->dtype * 3 + opt->meta.kind;
+    const int kind = opt->meta.kind;
+    if (opt->state_dtype == NBO_DT_BF16) return K_UPDATE_PBF16_BASE + kind;
+    if (opt->state_dtype == NBO_DT_F16) return K_UPDATE_PF16_BASE + kind;
+    if (params->dtype == NBO_DT_F16) return K_UPDATE_F16_BASE + kind;
+    return K_UPDATE_BASE + params->dtype * 3 + kind;
 }
 
 uint32_t norm_grid(const Layout &L)
@@ -126,7 +134,7 @@ uint32_t norm_grid(const Layout &L)
 
 // First stage of the norm / found_inf pass over `grads`; partials land in the
 // runtime's scratch.  Returns the grid used (0 for an empty list).
-uint32_t launch_norm(nbo_list *grads, const NboScalerDev *scaler, bool bf16_arithmetic = false)
+uint32_t launch_norm(nbo_list *grads, const NboScalerDev *scaler, bool half_arithmetic = false)
 {
     Runtime &rt = Runtime::get();
     NboNormArgs a = {};
@@ -136,10 +144,13 @@ uint32_t launch_norm(nbo_list *grads, const NboScalerDev *scaler, bool bf16_arit
     a.partial_sumsq = rt.partial_sumsq();
     a.partial_flag = rt.partial_flag();
     a.grid = norm_grid(grads->layout);
-    // bf16 gradients are unscaled in f32 when they feed f32 state (the mixed-precision
-    // composition) and in bf16 when the optimizer itself is bf16 or they are scaled in place
-    const bool pbf16 = bf16_arithmetic && grads->dtype == NBO_DT_BF16;
-    rt.launch(pbf16 ? (int)K_NORM_PBF16 : K_NORM_BASE + grads->dtype, a.grid, NBO_BLOCK, a);
+    // bf16 / f16 gradients are unscaled in f32 when they feed f32 state (the mixed-precision
+    // composition) and in their own type when the optimizer itself is of that type or they are
+    // scaled in place
+    int k = kernel_for(K_NORM_BASE, K_NORM_F16, grads->dtype);
+    if (half_arithmetic && grads->dtype == NBO_DT_BF16) k = K_NORM_PBF16;
+    if (half_arithmetic && grads->dtype == NBO_DT_F16) k = K_NORM_PF16;
+    rt.launch(k, a.grid, NBO_BLOCK, a);
     return a.grid;
 }
 
@@ -151,7 +162,7 @@ void launch_scale(nbo_list *grads, const NboGradFactors *gf, double factor, uint
     a.gf = gf;
     a.factor = factor;
     a.mode = mode;
-    Runtime::get().launch(K_SCALE_BASE + grads->dtype, grads->layout.nchunks, NBO_BLOCK, a);
+    Runtime::get().launch(kernel_for(K_SCALE_BASE, K_SCALE_F16, grads->dtype), grads->layout.nchunks, NBO_BLOCK, a);
 }
 
 // "m12" -> ('m', 12) with the reference's parsing rules (alg.rs:491-507): the prefix
@@ -316,8 +327,8 @@ int nbo_list_create(uint64_t n_tensors, const uint64_t *rows, const uint64_t *co
         require(out != nullptr, NBO_ERR_ARG, "null output pointer");
         *out = nullptr;
         require(n_tensors == 0 || (rows && cols && dev_ptrs), NBO_ERR_ARG, "null shape or pointer array");
-        require(dtype == NBO_DT_F32 || dtype == NBO_DT_BF16 || dtype == NBO_DT_F64, NBO_ERR_ARG,
-                "unknown dtype");
+        require(dtype == NBO_DT_F32 || dtype == NBO_DT_BF16 || dtype == NBO_DT_F64 || dtype == NBO_DT_F16,
+                NBO_ERR_ARG, "unknown dtype");
         require(n_tensors < (1ull << 31), NBO_ERR_TOO_LARGE, "too many tensors");
         Runtime &rt = Runtime::get();
         nbo_list *l = new nbo_list();
@@ -368,8 +379,8 @@ int nbo_optim_create(const nbo_meta *meta, uint64_t n_tensors, const uint64_t *r
         require(n_tensors == 0 || (rows && cols), NBO_ERR_ARG, "null shape array");
         require(meta->kind >= NBO_KIND_ADAMW && meta->kind <= NBO_KIND_SGD, NBO_ERR_ARG,
                 "unknown optimizer kind");
-        require(state_dtype == NBO_DT_F32 || state_dtype == NBO_DT_F64 || state_dtype == NBO_DT_BF16,
-                NBO_ERR_DTYPE, "optimizer state is f32, f64 or bf16");
+        require(state_dtype == NBO_DT_F32 || state_dtype == NBO_DT_F64 || is_half(state_dtype),
+                NBO_ERR_DTYPE, "optimizer state is f32, f64, bf16 or f16");
         require(!keep_master || state_dtype == NBO_DT_F32, NBO_ERR_DTYPE,
                 "master weights are f32: keep_master needs f32 state");
         require(n_tensors < (1ull << 31), NBO_ERR_TOO_LARGE, "too many tensors");
@@ -527,7 +538,7 @@ static void cast_master(nbo_optim *opt, nbo_list *params, uint32_t mode)
 {
     require(opt && params, NBO_ERR_ARG, "null optimizer or list");
     require(opt->keep_master, NBO_ERR_DTYPE, "optimizer was created without master weights");
-    require(params->dtype == NBO_DT_BF16, NBO_ERR_DTYPE, "master casts take a bf16 list");
+    require(is_half(params->dtype), NBO_ERR_DTYPE, "master casts take a bf16 or f16 list");
     if (params->layout.nt() != opt->layout.nt())
         fail(NBO_ERR_COUNT_MISMATCH, "params count mismatch");
     for (uint64_t t = 0; t < opt->layout.nt(); t++)
@@ -539,22 +550,23 @@ static void cast_master(nbo_optim *opt, nbo_list *params, uint32_t mode)
     a.dst_ptrs = params->ptrs_dev;
     a.arena = opt->arena;
     a.mode = mode;
+    a.half_type = (uint32_t)params->dtype; // NBO_DT_BF16 / NBO_DT_F16 are the device's codes too
     Runtime::get().launch(K_CAST_MASTER, opt->layout.nchunks, NBO_BLOCK, a);
 }
 
-int nbo_optim_master_from_params(nbo_optim *opt, nbo_list *params_bf16)
+int nbo_optim_master_from_params(nbo_optim *opt, nbo_list *params_half)
 {
     return guarded([&] {
-        cast_master(opt, params_bf16, 0);
+        cast_master(opt, params_half, 0);
         opt->master_valid = true;
     });
 }
 
-int nbo_optim_params_from_master(nbo_optim *opt, nbo_list *params_bf16)
+int nbo_optim_params_from_master(nbo_optim *opt, nbo_list *params_half)
 {
     return guarded([&] {
         require(opt && opt->master_valid, NBO_ERR_NO_MASTER, "master weights not set");
-        cast_master(opt, params_bf16, 1);
+        cast_master(opt, params_half, 1);
     });
 }
 
@@ -735,7 +747,7 @@ int nbo_fused_step(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, nbo_lis
         f.partial_flag = rt.partial_flag();
         // without scaler, clipping and nan policy the pass has nothing to decide, but
         // it still runs so that the trace records every step
-        f.grid = launch_norm(grads, scaler ? scaler->dev : nullptr, pure_bf16(opt));
+        f.grid = launch_norm(grads, scaler ? scaler->dev : nullptr, pure_half(opt));
         f.check_finite = (scaler || (flags & NBO_STEP_SKIP_NONFINITE)) ? 1u : 0u;
         f.scaler = scaler ? scaler->dev : nullptr;
         f.gf = opt->gf;
@@ -762,7 +774,7 @@ int nbo_fused_step_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *c
             check_step_args(opts[g], params[g], grads[g]);
             require(grads[g]->dtype == all_grads->dtype, NBO_ERR_DTYPE,
                     "group gradients differ in element type from the whole list");
-            require(pure_bf16(opts[g]) == pure_bf16(opts[0]), NBO_ERR_DTYPE,
+            require(pure_half(opts[g]) == pure_half(opts[0]), NBO_ERR_DTYPE,
                     "groups mix bf16 and f32 optimizer state");
             covered += grads[g]->layout.nt();
         }
@@ -774,7 +786,7 @@ int nbo_fused_step_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *c
         NboFinalizeArgs f = {};
         f.partial_sumsq = rt.partial_sumsq();
         f.partial_flag = rt.partial_flag();
-        f.grid = launch_norm(all_grads, scaler ? scaler->dev : nullptr, n_groups > 0 && pure_bf16(opts[0]));
+        f.grid = launch_norm(all_grads, scaler ? scaler->dev : nullptr, n_groups > 0 && pure_half(opts[0]));
         f.check_finite = (scaler || (flags & NBO_STEP_SKIP_NONFINITE)) ? 1u : 0u;
         f.scaler = scaler ? scaler->dev : nullptr;
         f.gf = rt.gf_scratch();
@@ -811,7 +823,7 @@ int nbo_accumulate(nbo_list *accum, nbo_list *grads, int zero_grads)
         a.a_ptrs = accum->ptrs_dev;
         a.b_ptrs = grads->ptrs_dev;
         a.zero_b = zero_grads ? 1u : 0u;
-        Runtime::get().launch(K_ACCUM_BASE + accum->dtype, accum->layout.nchunks, NBO_BLOCK, a);
+        Runtime::get().launch(kernel_for(K_ACCUM_BASE, K_ACCUM_F16, accum->dtype), accum->layout.nchunks, NBO_BLOCK, a);
     });
 }
 
@@ -865,7 +877,7 @@ int nbo_backend_apply(int op, nbo_list *out, nbo_list *a, nbo_list *b, double s)
         e.b_ptrs = needs_b ? b->ptrs_dev : nullptr;
         e.s = s;
         e.op = (uint32_t)op;
-        Runtime::get().launch(K_EW_BASE + out->dtype, out->layout.nchunks, NBO_BLOCK, e);
+        Runtime::get().launch(kernel_for(K_EW_BASE, K_EW_F16, out->dtype), out->layout.nchunks, NBO_BLOCK, e);
     });
 }
 

@@ -41,6 +41,10 @@ static const char *const kKernelNames[K_COUNT] = {
     "nbo_ew_f32",            "nbo_ew_bf16",          "nbo_ew_f64",
     "nbo_cast_list",         "nbo_update_pbf16_adamw", "nbo_update_pbf16_adam",
     "nbo_update_pbf16_sgd",  "nbo_norm_pbf16",
+    "nbo_update_f16_adamw",  "nbo_update_f16_adam",  "nbo_update_f16_sgd",
+    "nbo_update_pf16_adamw", "nbo_update_pf16_adam", "nbo_update_pf16_sgd",
+    "nbo_norm_f16",          "nbo_norm_pf16",        "nbo_scale_f16",
+    "nbo_accum_f16",         "nbo_ew_f16",
 };
 
 Runtime &Runtime::get()

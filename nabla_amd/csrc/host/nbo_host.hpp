@@ -17,6 +17,12 @@
 
 namespace nbo {
 
+// 16-bit element types: bf16 and IEEE binary16
+inline bool is_half(int dtype) { return dtype == NBO_DT_BF16 || dtype == NBO_DT_F16; }
+static_assert((int)NBO_DT_F32 == (int)NBO_F32 && (int)NBO_DT_BF16 == (int)NBO_BF16 && (int)NBO_DT_F64 == (int)NBO_F64 &&
+                  (int)NBO_DT_F16 == (int)NBO_F16,
+              "the public element type codes are the device's storage codes");
+
 // Thrown internally, converted to a status code at the C boundary.
 struct Error {
     int status;
@@ -29,7 +35,7 @@ void set_last_error(const std::string &msg);
 const char *get_last_error();
 
 enum KernelId {
-    K_UPDATE_BASE = 0, // + st * 3 + kind
+    K_UPDATE_BASE = 0, // + st * 3 + kind, st = f32 / bf16 / f64 (f16 has ids of its own below)
     K_NORM_BASE = 9,   // + st
     K_SCALE_BASE = 12, // + st
     K_PREP = 15,
@@ -43,7 +49,14 @@ enum KernelId {
     K_CAST_LIST = 27,
     K_UPDATE_PBF16_BASE = 28, // + kind: bf16 tensors with bf16 state and arithmetic
     K_NORM_PBF16 = 31,
-    K_COUNT = 32
+    K_UPDATE_F16_BASE = 32,  // + kind: f16 tensors over f32 state and master weights
+    K_UPDATE_PF16_BASE = 35, // + kind: f16 tensors with f16 state and arithmetic
+    K_NORM_F16 = 38,
+    K_NORM_PF16 = 39,
+    K_SCALE_F16 = 40,
+    K_ACCUM_F16 = 41,
+    K_EW_F16 = 42,
+    K_COUNT = 43
 };
 
 // Process-wide runtime: device 0, the loaded module, the stream, scratch buffers.
@@ -138,7 +151,7 @@ struct nbo_optim {
     NboOptimDev *dev = nullptr; // step_count lives here: the device decides skips
     NboGradFactors *gf = nullptr;
     NboTraceDev *trace = nullptr;
-    size_t elem_bytes() const { return state_dtype == NBO_DT_F64 ? 8 : state_dtype == NBO_DT_BF16 ? 2 : 4; }
+    size_t elem_bytes() const { return state_dtype == NBO_DT_F64 ? 8 : nbo::is_half(state_dtype) ? 2 : 4; }
 };
 
 namespace nbo {

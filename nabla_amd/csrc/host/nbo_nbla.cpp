@@ -58,7 +58,7 @@ uint32_t read_u32(std::FILE *f)
     return (uint32_t)b[0] | ((uint32_t)b[1] << 8) | ((uint32_t)b[2] << 16) | ((uint32_t)b[3] << 24);
 }
 
-size_t dtype_bytes(int dtype) { return dtype == NBO_DT_F64 ? 8 : dtype == NBO_DT_BF16 ? 2 : 4; }
+size_t dtype_bytes(int dtype) { return dtype == NBO_DT_F64 ? 8 : is_half(dtype) ? 2 : 4; }
 
 // half::bf16::from_f32 / f32::from(bf16) on the host (common/scalar/mod.rs:338-344)
 uint16_t bf16_from_f32(float v)
@@ -77,22 +77,62 @@ float bf16_to_f32(uint16_t h)
     return f;
 }
 
+// half::f16::from_f32 / f32::from(f16) on the host: IEEE binary16, round to nearest even,
+// subnormals kept, overflow to infinity, NaN payloads truncated with the quiet bit set.
+uint16_t f16_from_f32(float v)
+{
+    uint32_t x;
+    std::memcpy(&x, &v, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u, ax = x & 0x7FFFFFFFu;
+    if (ax > 0x7F800000u) return (uint16_t)(sign | 0x7E00u | ((ax >> 13) & 0x03FFu));
+    if (ax >= 0x47800000u) return (uint16_t)(sign | 0x7C00u); // 65536 and above, infinity
+    if (ax >= 0x38800000u) {                                  // normal in binary16 (2^-14 and above)
+        const uint32_t r = ax - 0x38000000u;                  // exponent rebiased from 127 to 15
+        return (uint16_t)(sign | ((r + 0x0FFFu + ((r >> 13) & 1u)) >> 13)); // a carry into exponent 31 is infinity
+    }
+    if (ax <= 0x33000000u) return (uint16_t)sign; // up to 2^-25 (the tie to zero included)
+    const uint32_t man = (ax & 0x007FFFFFu) | 0x00800000u, shift = 126u - (ax >> 23); // 14..24
+    const uint32_t rem = man & ((1u << shift) - 1u), half_way = 1u << (shift - 1u);
+    uint32_t q = man >> shift; // multiples of 2^-24
+    if (rem > half_way || (rem == half_way && (q & 1u))) q++;
+    return (uint16_t)(sign | q);
+}
+
+float f16_to_f32(uint16_t h)
+{
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 0x1Fu, m = h & 0x03FFu;
+    uint32_t x;
+    if (e == 0) {
+        const float sub = (float)m * 5.9604644775390625e-08f; // m * 2^-24, exact
+        std::memcpy(&x, &sub, 4);
+        x |= sign;
+    } else if (e == 31) x = sign | 0x7F800000u | (m << 13);
+    else x = sign | ((e + 112u) << 23) | (m << 13);
+    float f;
+    std::memcpy(&f, &x, 4);
+    return f;
+}
+
 // T::to_f64 over `n` raw elements
 void widen(int dtype, const void *raw, double *out, size_t n)
 {
     if (dtype == NBO_DT_F64) std::memcpy(out, raw, n * 8);
     else if (dtype == NBO_DT_F32)
         for (size_t i = 0; i < n; i++) out[i] = (double)((const float *)raw)[i];
+    else if (dtype == NBO_DT_F16)
+        for (size_t i = 0; i < n; i++) out[i] = (double)f16_to_f32(((const uint16_t *)raw)[i]);
     else
         for (size_t i = 0; i < n; i++) out[i] = (double)bf16_to_f32(((const uint16_t *)raw)[i]);
 }
 
-// T::from_f64 over `n` values (f32: one rounding; bf16: through f32, scalar/mod.rs:338-340)
+// T::from_f64 over `n` values (f32: one rounding; bf16 / f16: through f32, scalar/mod.rs:338-340)
 void narrow(int dtype, const double *in, void *raw, size_t n)
 {
     if (dtype == NBO_DT_F64) std::memcpy(raw, in, n * 8);
     else if (dtype == NBO_DT_F32)
         for (size_t i = 0; i < n; i++) ((float *)raw)[i] = (float)in[i];
+    else if (dtype == NBO_DT_F16)
+        for (size_t i = 0; i < n; i++) ((uint16_t *)raw)[i] = f16_from_f32((float)in[i]);
     else
         for (size_t i = 0; i < n; i++) ((uint16_t *)raw)[i] = bf16_from_f32((float)in[i]);
 }

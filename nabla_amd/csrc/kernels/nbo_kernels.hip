@@ -81,25 +81,43 @@ DEV bool nonfinite_f64(double d)
     return ((uint32_t)(__double_as_longlong(d) >> 32) & 0x7FF00000u) == 0x7FF00000u;
 }
 
-// T = half::bf16 as an arithmetic type: a 16-bit pattern whose every operation is the
-// f32 operation followed by bf16::from_f32 (common/scalar/mod.rs:253-351 and the half
+// f16: the device's conversion instructions (v_cvt_f16_f32 / v_cvt_f32_f16) give
+// half::f16::from_f32's and f32::from(f16)'s bits for every input -- round to nearest even,
+// subnormals kept, overflow to infinity, NaN payloads truncated with the quiet bit set.
+DEV uint32_t f32_to_f16_bits(float f) { return (uint32_t)__builtin_bit_cast(unsigned short, (_Float16)f); }
+DEV float f16_bits_to_f32(uint32_t h) { return (float)__builtin_bit_cast(_Float16, (unsigned short)h); }
+
+// T = half::bf16 / half::f16 as an arithmetic type: a 16-bit pattern whose every operation
+// is the f32 operation followed by T::from_f32 (common/scalar/mod.rs:253-351 and the half
 // crate's operators).  Conversion from float / double is T::from_f64 = from_f32(v as f32).
-struct BF {
+enum { FMT_BF16 = 0, FMT_F16 = 1 };
+template <int FMT> struct Half16 {
     uint16_t bits;
-    __device__ __forceinline__ BF() : bits(0) {}
-    __device__ __forceinline__ BF(float x) : bits((uint16_t)f32_to_bf16_bits(x)) {}
-    __device__ __forceinline__ BF(double x) : bits((uint16_t)f32_to_bf16_bits((float)x)) {}
-    __device__ __forceinline__ BF(int x) : bits((uint16_t)f32_to_bf16_bits((float)x)) {}
-    __device__ __forceinline__ float f() const { return bf16_bits_to_f32(bits); }
+    static __device__ __forceinline__ uint16_t narrow(float x)
+    {
+        return (uint16_t)(FMT == FMT_BF16 ? f32_to_bf16_bits(x) : f32_to_f16_bits(x));
+    }
+    __device__ __forceinline__ Half16() : bits(0) {}
+    __device__ __forceinline__ Half16(float x) : bits(narrow(x)) {}
+    __device__ __forceinline__ Half16(double x) : bits(narrow((float)x)) {}
+    __device__ __forceinline__ Half16(int x) : bits(narrow((float)x)) {}
+    __device__ __forceinline__ float f() const { return FMT == FMT_BF16 ? bf16_bits_to_f32(bits) : f16_bits_to_f32(bits); }
     __device__ __forceinline__ explicit operator double() const { return (double)f(); }
+    // inf or NaN: all exponent bits set
+    __device__ __forceinline__ bool nonfinite() const
+    {
+        return FMT == FMT_BF16 ? (bits & 0x7F80u) == 0x7F80u : (bits & 0x7C00u) == 0x7C00u;
+    }
 };
-DEV BF operator*(BF a, BF b) { return BF(a.f() * b.f()); }
-DEV BF operator+(BF a, BF b) { return BF(a.f() + b.f()); }
-DEV BF operator-(BF a, BF b) { return BF(a.f() - b.f()); }
-DEV BF operator/(BF a, BF b) { return BF(a.f() / b.f()); }
-DEV BF bf_from_bits(uint32_t b)
+typedef Half16<FMT_BF16> BF;
+typedef Half16<FMT_F16> HF;
+template <int FMT> DEV Half16<FMT> operator*(Half16<FMT> a, Half16<FMT> b) { return Half16<FMT>(a.f() * b.f()); }
+template <int FMT> DEV Half16<FMT> operator+(Half16<FMT> a, Half16<FMT> b) { return Half16<FMT>(a.f() + b.f()); }
+template <int FMT> DEV Half16<FMT> operator-(Half16<FMT> a, Half16<FMT> b) { return Half16<FMT>(a.f() - b.f()); }
+template <int FMT> DEV Half16<FMT> operator/(Half16<FMT> a, Half16<FMT> b) { return Half16<FMT>(a.f() / b.f()); }
+template <int FMT> DEV Half16<FMT> half_from_bits(uint32_t b)
 {
-    BF r;
+    Half16<FMT> r;
     r.bits = (uint16_t)b;
     return r;
 }
@@ -141,6 +159,14 @@ template <> struct Traits<NBO_PBF16> {
     typedef BF T;
     enum { VEC = 8, SBYTES = 2 };
 };
+template <> struct Traits<NBO_F16> { // f16 tensors over f32 state
+    typedef float T;
+    enum { VEC = 4, SBYTES = 2 };
+};
+template <> struct Traits<NBO_PF16> { // f16 tensors, state and arithmetic
+    typedef HF T;
+    enum { VEC = 8, SBYTES = 2 };
+};
 
 // arena (engine-owned, always 16-byte aligned) vectors of T
 DEV void ld_state(const float *p, float (&x)[4])
@@ -164,17 +190,17 @@ DEV void st_state(double *p, const double (&x)[2])
     NBO_STORE(v, GLOBAL_PTR(f64x2, p));
 }
 
-DEV void ld_state(const BF *p, BF (&x)[8])
+template <int FMT> DEV void ld_state(const Half16<FMT> *p, Half16<FMT> (&x)[8])
 {
     const u32x4 v = NBO_LOAD(GLOBAL_PTR(const u32x4, p));
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-        x[2 * k] = bf_from_bits(w[k] & 0xFFFFu);
-        x[2 * k + 1] = bf_from_bits(w[k] >> 16);
+        x[2 * k] = half_from_bits<FMT>(w[k] & 0xFFFFu);
+        x[2 * k + 1] = half_from_bits<FMT>(w[k] >> 16);
     }
 }
-DEV void st_state(BF *p, const BF (&x)[8])
+template <int FMT> DEV void st_state(Half16<FMT> *p, const Half16<FMT> (&x)[8])
 {
     u32x4 v;
     v.x = (uint32_t)x[0].bits | ((uint32_t)x[1].bits << 16);
@@ -218,11 +244,33 @@ template <> struct IO<NBO_BF16> {
     DEV void st1(char *p, float x) { *GLOBAL_PTR(uint16_t, p) = (uint16_t)f32_to_bf16_bits(x); }
 };
 
-template <> struct IO<NBO_PBF16> {
-    DEV void ldv(const char *p, BF (&x)[8]) { ld_state((const BF *)p, x); }
-    DEV void stv(char *p, const BF (&x)[8]) { st_state((BF *)p, x); }
-    DEV BF ld1(const char *p) { return bf_from_bits(*GLOBAL_PTR(const uint16_t, p)); }
-    DEV void st1(char *p, BF x) { *GLOBAL_PTR(uint16_t, p) = x.bits; }
+template <int FMT> struct IOHalf16 {
+    typedef Half16<FMT> H;
+    DEV void ldv(const char *p, H (&x)[8]) { ld_state((const H *)p, x); }
+    DEV void stv(char *p, const H (&x)[8]) { st_state((H *)p, x); }
+    DEV H ld1(const char *p) { return half_from_bits<FMT>(*GLOBAL_PTR(const uint16_t, p)); }
+    DEV void st1(char *p, H x) { *GLOBAL_PTR(uint16_t, p) = x.bits; }
+};
+template <> struct IO<NBO_PBF16> : IOHalf16<FMT_BF16> {};
+template <> struct IO<NBO_PF16> : IOHalf16<FMT_F16> {};
+template <> struct IO<NBO_F16> {
+    DEV void ldv(const char *p, float (&x)[4])
+    {
+        u32x2 v = NBO_LOAD(GLOBAL_PTR(const u32x2, p));
+        x[0] = f16_bits_to_f32(v.x & 0xFFFFu);
+        x[1] = f16_bits_to_f32(v.x >> 16);
+        x[2] = f16_bits_to_f32(v.y & 0xFFFFu);
+        x[3] = f16_bits_to_f32(v.y >> 16);
+    }
+    DEV void stv(char *p, const float (&x)[4])
+    {
+        u32x2 v;
+        v.x = f32_to_f16_bits(x[0]) | (f32_to_f16_bits(x[1]) << 16);
+        v.y = f32_to_f16_bits(x[2]) | (f32_to_f16_bits(x[3]) << 16);
+        NBO_STORE(v, GLOBAL_PTR(u32x2, p));
+    }
+    DEV float ld1(const char *p) { return f16_bits_to_f32(*GLOBAL_PTR(const uint16_t, p)); }
+    DEV void st1(char *p, float x) { *GLOBAL_PTR(uint16_t, p) = (uint16_t)f32_to_f16_bits(x); }
 };
 
 // ---------------------------------------------------------------------------------
@@ -263,14 +311,15 @@ template <> struct Scal<double> {
     }
 };
 
-// T = bf16: T::from_f64(x) is from_f32(x as f32), so every scalar is the f32-narrowed one
-// rounded once more; `T::one() - wd_lr` is a bf16 subtraction (alg.rs:135).
-template <> struct Scal<BF> {
-    BF b1, omb1, b2, omb2, eps, ss, ibc2, omw, neg_lr, mom, wd, inv, clip;
+// T = bf16 / f16: T::from_f64(x) is from_f32(x as f32), so every scalar is the f32-narrowed
+// one rounded once more; `T::one() - wd_lr` is a subtraction in T (alg.rs:135).
+template <int FMT> struct Scal<Half16<FMT>> {
+    typedef Half16<FMT> H;
+    H b1, omb1, b2, omb2, eps, ss, ibc2, omw, neg_lr, mom, wd, inv, clip;
     bool use_mom, use_wd;
     __device__ Scal(const NboOptimDev *o, const NboGradFactors *f)
         : b1(o->b1), omb1(o->omb1), b2(o->b2), omb2(o->omb2), eps(o->eps_t), ss(o->ss), ibc2(o->ibc2),
-          omw(BF(1.0f) - BF(o->wd_lr_t)), neg_lr(o->neg_lr), mom(o->momentum_t), wd(o->wd_t),
+          omw(H(1.0f) - H(o->wd_lr_t)), neg_lr(o->neg_lr), mom(o->momentum_t), wd(o->wd_t),
           inv(f ? f->inv_scale32 : 1.0f), clip(f ? f->clip32 : 1.0f), use_mom(o->momentum != 0.0),
           use_wd(o->weight_decay != 0.0)
     {
@@ -282,7 +331,7 @@ template <> struct Scal<BF> {
     }
 };
 
-DEV BF sqrt_rn(BF x) { return BF(__builtin_sqrtf(x.f())); }
+template <int FMT> DEV Half16<FMT> sqrt_rn(Half16<FMT> x) { return Half16<FMT>(__builtin_sqrtf(x.f())); }
 DEV float sqrt_rn(float x) { return __builtin_sqrtf(x); }
 DEV double sqrt_rn(double x) { return __builtin_sqrt(x); }
 
@@ -367,7 +416,7 @@ template <int ST, int KIND> DEV void update_body(const NboUpdateArgs &a)
         ITERS = ROWS / U
     };
     static_assert(ROWS % U == 0 && ROWS * ROW == NBO_CHUNK, "chunk must be a whole number of unrolled rows");
-    const bool mixed = ST == NBO_BF16; // f32 master lives in the arena
+    const bool mixed = ST == NBO_BF16 || ST == NBO_F16; // f32 master lives in the arena
     const bool has_v = KIND != NBO_SGD;
     const uint32_t tid = threadIdx.x;
     const ChunkRef c = chunk_ref(a.L, blockIdx.x);
@@ -477,6 +526,12 @@ NBO_UPDATE_KERNEL(nbo_update_f64_sgd, NBO_F64, NBO_SGD)
 NBO_UPDATE_KERNEL(nbo_update_pbf16_adamw, NBO_PBF16, NBO_ADAMW)
 NBO_UPDATE_KERNEL(nbo_update_pbf16_adam, NBO_PBF16, NBO_ADAM)
 NBO_UPDATE_KERNEL(nbo_update_pbf16_sgd, NBO_PBF16, NBO_SGD)
+NBO_UPDATE_KERNEL(nbo_update_f16_adamw, NBO_F16, NBO_ADAMW)
+NBO_UPDATE_KERNEL(nbo_update_f16_adam, NBO_F16, NBO_ADAM)
+NBO_UPDATE_KERNEL(nbo_update_f16_sgd, NBO_F16, NBO_SGD)
+NBO_UPDATE_KERNEL(nbo_update_pf16_adamw, NBO_PF16, NBO_ADAMW)
+NBO_UPDATE_KERNEL(nbo_update_pf16_adam, NBO_PF16, NBO_ADAM)
+NBO_UPDATE_KERNEL(nbo_update_pf16_sgd, NBO_PF16, NBO_SGD)
 
 // ---------------------------------------------------------------------------------
 // Deterministic block reduction: xor-butterfly inside each 64-lane wavefront, then
@@ -531,7 +586,9 @@ template <int ST> DEV bool nonfinite(typename Traits<ST>::T x);
 template <> __device__ __forceinline__ bool nonfinite<NBO_F32>(float x) { return nonfinite_f32(x); }
 template <> __device__ __forceinline__ bool nonfinite<NBO_BF16>(float x) { return nonfinite_f32(x); }
 template <> __device__ __forceinline__ bool nonfinite<NBO_F64>(double x) { return nonfinite_f64(x); }
-template <> __device__ __forceinline__ bool nonfinite<NBO_PBF16>(BF x) { return (x.bits & 0x7F80u) == 0x7F80u; }
+template <> __device__ __forceinline__ bool nonfinite<NBO_PBF16>(BF x) { return x.nonfinite(); }
+template <> __device__ __forceinline__ bool nonfinite<NBO_F16>(float x) { return nonfinite_f32(x); }
+template <> __device__ __forceinline__ bool nonfinite<NBO_PF16>(HF x) { return x.nonfinite(); }
 
 template <int ST> DEV void norm_body(const NboNormArgs &a)
 {
@@ -548,8 +605,8 @@ template <int ST> DEV void norm_body(const NboNormArgs &a)
         const ChunkRef c = chunk_ref(a.L, ci);
         const char *pg = (const char *)a.g_ptrs[c.t] + c.base * SB;
         uint32_t done = 0;
-        if (ST == NBO_BF16) {
-            // 8 bf16 per 128-bit load
+        if constexpr (ST == NBO_BF16 || ST == NBO_F16) {
+            // 8 half-width elements per 128-bit load
             if ((((uintptr_t)pg) & 15u) == 0) {
                 const uint32_t nvec = c.cnt / 8;
                 for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
@@ -557,8 +614,8 @@ template <int ST> DEV void norm_body(const NboNormArgs &a)
                     const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
                     for (int k = 0; k < 4; k++) {
-                        const float lo = __uint_as_float(ww[k] << 16);
-                        const float hi = __uint_as_float(ww[k] & 0xFFFF0000u);
+                        const float lo = ST == NBO_BF16 ? __uint_as_float(ww[k] << 16) : f16_bits_to_f32(ww[k] & 0xFFFFu);
+                        const float hi = ST == NBO_BF16 ? __uint_as_float(ww[k] & 0xFFFF0000u) : f16_bits_to_f32(ww[k] >> 16);
                         bad |= (uint32_t)nonfinite_f32(lo) | (uint32_t)nonfinite_f32(hi);
                         acc = sq_acc<ST>(acc, (T)(lo * inv));
                         acc = sq_acc<ST>(acc, (T)(hi * inv));
@@ -606,6 +663,8 @@ NBO_NORM_KERNEL(nbo_norm_f64, NBO_F64)
 // bf16 gradients of a bf16 optimizer: the unscaled gradient is itself a bf16 value
 // (g * bf16(1/scale), rounded to bf16) before it is squared.
 NBO_NORM_KERNEL(nbo_norm_pbf16, NBO_PBF16)
+NBO_NORM_KERNEL(nbo_norm_f16, NBO_F16)
+NBO_NORM_KERNEL(nbo_norm_pf16, NBO_PF16)
 
 // ---------------------------------------------------------------------------------
 // Per-step scalars (alg.rs:120-135 AdamW, 265-277 Adam, 393-395 Sgd).  A skipped
@@ -792,6 +851,7 @@ NBO_SCALE_KERNEL(nbo_scale_f32, NBO_F32)
 // in place on bf16 tensors the arithmetic is bf16's: factor narrowed to bf16, product
 // rounded to bf16
 NBO_SCALE_KERNEL(nbo_scale_bf16, NBO_PBF16)
+NBO_SCALE_KERNEL(nbo_scale_f16, NBO_PF16)
 NBO_SCALE_KERNEL(nbo_scale_f64, NBO_F64)
 
 // Gradient accumulation of the Trainer: buf[i] = &buf[i] + g (trainer.rs:262-266 ->
@@ -834,11 +894,12 @@ template <int ST> DEV void accum_body(const NboAccumArgs &a)
 NBO_ACCUM_KERNEL(nbo_accum_f32, NBO_F32)
 NBO_ACCUM_KERNEL(nbo_accum_bf16, NBO_BF16)
 NBO_ACCUM_KERNEL(nbo_accum_f64, NBO_F64)
+NBO_ACCUM_KERNEL(nbo_accum_f16, NBO_F16)
 
 // ---------------------------------------------------------------------------------
-// Master-weight casts: arena f32 <- bf16 tensors (exact widening) and
-// bf16 tensors <- arena f32 (round to nearest even).
-extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_cast_master(const NboCastArgs a)
+// Master-weight casts: arena f32 <- bf16 / f16 tensors (exact widening) and
+// bf16 / f16 tensors <- arena f32 (round to nearest even).
+template <int ST> DEV void cast_master_body(const NboCastArgs &a)
 {
     const ChunkRef c = chunk_ref(a.L, blockIdx.x);
     float *aw = state_part<float>(a.arena, c, a.arena.part_w);
@@ -848,17 +909,22 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_cast_master(const Nb
     for (uint32_t q = threadIdx.x; q < nvec; q += NBO_BLOCK) {
         float x[4];
         if (a.mode == 0) {
-            IO<NBO_BF16>::ldv(pt + (uint64_t)q * 8, x);
+            IO<ST>::ldv(pt + (uint64_t)q * 8, x);
             st_state(aw + q * 4, x);
         } else {
             ld_state(aw + q * 4, x);
-            IO<NBO_BF16>::stv(pt + (uint64_t)q * 8, x);
+            IO<ST>::stv(pt + (uint64_t)q * 8, x);
         }
     }
     for (uint32_t e = nvec * 4 + threadIdx.x; e < c.cnt; e += NBO_BLOCK) {
-        if (a.mode == 0) aw[e] = IO<NBO_BF16>::ld1(pt + (uint64_t)e * 2);
-        else IO<NBO_BF16>::st1(pt + (uint64_t)e * 2, aw[e]);
+        if (a.mode == 0) aw[e] = IO<ST>::ld1(pt + (uint64_t)e * 2);
+        else IO<ST>::st1(pt + (uint64_t)e * 2, aw[e]);
     }
+}
+extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_cast_master(const NboCastArgs a)
+{
+    if (a.half_type == NBO_F16) cast_master_body<NBO_F16>(a);
+    else cast_master_body<NBO_BF16>(a);
 }
 
 // ---------------------------------------------------------------------------------
@@ -873,6 +939,10 @@ template <int ST> DEV typename Traits<ST>::T to_storage_precision(typename Trait
 template <> __device__ __forceinline__ float to_storage_precision<NBO_BF16>(float x)
 {
     return bf16_bits_to_f32(f32_to_bf16_bits(x));
+}
+template <> __device__ __forceinline__ float to_storage_precision<NBO_F16>(float x)
+{
+    return f16_bits_to_f32(f32_to_f16_bits(x));
 }
 
 // powf(x, 0.5) is taken as the correctly rounded square root with C's pow special
@@ -947,6 +1017,7 @@ template <int ST> DEV void ew_body(const NboEwArgs &a)
 NBO_EW_KERNEL(nbo_ew_f32, NBO_F32)
 NBO_EW_KERNEL(nbo_ew_bf16, NBO_BF16)
 NBO_EW_KERNEL(nbo_ew_f64, NBO_F64)
+NBO_EW_KERNEL(nbo_ew_f16, NBO_F16)
 
 // BackendCore::cast, default implementation (common/backend/mod.rs:157-160):
 // U::from_f64(x.to_f64()) per element.  Widening is exact; f64 -> f32 rounds to nearest
@@ -1010,6 +1081,7 @@ template <int SRC> DEV void cast_from(const NboCastListArgs &a)
 {
     if (a.dst_type == NBO_F32) cast_body<SRC, NBO_F32>(a);
     else if (a.dst_type == NBO_BF16) cast_body<SRC, NBO_BF16>(a);
+    else if (a.dst_type == NBO_F16) cast_body<SRC, NBO_F16>(a);
     else cast_body<SRC, NBO_F64>(a);
 }
 
@@ -1017,6 +1089,7 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_cast_list(const NboC
 {
     if (a.src_type == NBO_F32) cast_from<NBO_F32>(a);
     else if (a.src_type == NBO_BF16) cast_from<NBO_BF16>(a);
+    else if (a.src_type == NBO_F16) cast_from<NBO_F16>(a);
     else cast_from<NBO_F64>(a);
 }
 

@@ -27,8 +27,9 @@
 
 // Element storage types of caller tensors.  NBO_PBF16 is bf16 storage with bf16
 // arithmetic (the reference's Optimizer<bf16>: every operation rounds to bf16), as
-// opposed to NBO_BF16 = bf16 tensors over f32 state; it only selects kernels.
-enum { NBO_F32 = 0, NBO_BF16 = 1, NBO_F64 = 2, NBO_PBF16 = 3 };
+// opposed to NBO_BF16 = bf16 tensors over f32 state; it only selects kernels.  NBO_F16 /
+// NBO_PF16 are the same pair for IEEE binary16.
+enum { NBO_F32 = 0, NBO_BF16 = 1, NBO_F64 = 2, NBO_F16 = 3, NBO_PBF16 = 4, NBO_PF16 = 5 };
 // OptimKind order of the reference (nabla-train/src/optim/core.rs:46-51).
 enum { NBO_ADAMW = 0, NBO_ADAM = 1, NBO_SGD = 2 };
 
@@ -190,8 +191,8 @@ struct NboCastArgs {
     const uint64_t *src_ptrs;
     const uint64_t *dst_ptrs;
     NboArenaDev arena; // the master part is one side of the cast
-    uint32_t mode;     // 0: master(f32) <- src(bf16) widen; 1: dst(bf16) <- master(f32) narrow
-    uint32_t pad;
+    uint32_t mode;      // 0: master(f32) <- src widen; 1: dst <- master(f32) narrow
+    uint32_t half_type; // NBO_BF16 or NBO_F16: the tensors' element type
 };
 
 struct NboFillArgs {

@@ -18,7 +18,7 @@ from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
 from . import _lib
-from ._lib import (DT_BF16, DT_F32, DT_F64, KIND_ADAM, KIND_ADAMW, KIND_SGD, STEP_SKIP_NONFINITE,
+from ._lib import (DT_BF16, DT_F16, DT_F32, DT_F64, KIND_ADAM, KIND_ADAMW, KIND_SGD, STEP_SKIP_NONFINITE,
                    STEP_ZERO_GRADS, NablaOptimError)
 
 
@@ -53,6 +53,8 @@ def _dtype_code(t) -> int:
         return DT_BF16
     if name.endswith("float64"):
         return DT_F64
+    if name.endswith("float16"):  # after bfloat16, which ends the same way
+        return DT_F16
     raise TypeError(f"unsupported tensor dtype {name}")
 
 
@@ -261,8 +263,9 @@ class _Optimizer:
     def __init__(self, lr: float, param_shapes: Sequence[Tuple[int, int]], *, dtype: str = "f32",
                  master: bool = False):
         self._shapes = [(int(r), int(c)) for r, c in param_shapes]
-        # "bf16" is the reference's Optimizer<bf16>: tensors, state and arithmetic all bf16
-        self._state_dtype = {"f32": DT_F32, "f64": DT_F64, "bf16": DT_BF16}[dtype]
+        # "bf16" / "f16" are the reference's Optimizer<bf16> / Optimizer<f16>: tensors, state and
+        # arithmetic all of that type
+        self._state_dtype = {"f32": DT_F32, "f64": DT_F64, "bf16": DT_BF16, "f16": DT_F16}[dtype]
         if master and dtype != "f32":
             raise ValueError("master weights are f32: master=True goes with dtype='f32'")
         self._master = bool(master)
@@ -396,7 +399,8 @@ class _Optimizer:
 
     def _torch_dtype(self):
         import torch
-        return {DT_F64: torch.float64, DT_BF16: torch.bfloat16}.get(self._state_dtype, torch.float32)
+        return {DT_F64: torch.float64, DT_BF16: torch.bfloat16,
+                DT_F16: torch.float16}.get(self._state_dtype, torch.float32)
 
     def read_state(self, name: str):
         """One state tensor as a new device tensor (a clone, like state_tensors())."""
@@ -656,7 +660,7 @@ def adamw_step(param, grad, m, v, lr, beta1, beta2, eps, weight_decay, step: int
     are device tensors of one dtype (f32 or f64); `param`, `m`, `v` are updated in place."""
     import torch
 
-    dtype = {torch.float32: "f32", torch.float64: "f64", torch.bfloat16: "bf16"}[param.dtype]
+    dtype = {torch.float32: "f32", torch.float64: "f64", torch.bfloat16: "bf16", torch.float16: "f16"}[param.dtype]
     opt = AdamW.new(lr, [_shape2(param)], dtype=dtype).beta1(beta1).beta2(beta2).eps(eps) \
         .weight_decay(weight_decay)
     opt._meta.step_count = int(step) - 1  # step() increments before use (alg.rs:120)

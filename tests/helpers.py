@@ -71,6 +71,27 @@ def max_ulp_f32(a_list, b_list):
     return worst
 
 
+def narrow_list(arrs, half):
+    """f32 arrays -> the oracle's representation of `half` ("bf16": uint16 bit patterns,
+    "f16": np.float16), rounded as T::from_f32 does."""
+    return [O.bf16_from_f32(a) if half == "bf16" else O.cast(np.ascontiguousarray(a, dtype=np.float32), np.float16)
+            for a in arrs]
+
+
+def widen_list(arrs):
+    """bf16 patterns / float16 arrays -> f32 (exact)."""
+    return [O.bf16_to_f32(a) if a.dtype == np.uint16 else O.cast(a, np.float32) for a in arrs]
+
+
+def max_ulp_half(a_list, b_list):
+    """Largest distance in units of the last place between 16-bit patterns (bf16 or f16)."""
+    worst = 0
+    for a, b in zip(a_list, b_list):
+        if a.size:
+            worst = max(worst, int(O.ulp_distance_bf16(a.view(np.uint16), b.view(np.uint16)).max()))
+    return worst
+
+
 def max_ulp_bf16(a_list, b_list):
     worst = 0
     for a, b in zip(a_list, b_list):
@@ -81,10 +102,10 @@ def max_ulp_bf16(a_list, b_list):
 
 def assert_bits_equal(a_list, b_list, what):
     for i, (a, b) in enumerate(zip(a_list, b_list)):
-        av = a.view(np.uint32) if a.dtype == np.float32 else (
-            a.view(np.uint64) if a.dtype == np.float64 else a)
-        bv = b.view(np.uint32) if b.dtype == np.float32 else (
-            b.view(np.uint64) if b.dtype == np.float64 else b)
+        assert a.dtype == b.dtype, f"{what}: tensor {i}: {a.dtype} vs {b.dtype}"
+        bits = {np.dtype(np.float16): np.uint16, np.dtype(np.float32): np.uint32, np.dtype(np.float64): np.uint64}
+        av = a.view(bits[a.dtype]) if a.dtype in bits else a
+        bv = b.view(bits[b.dtype]) if b.dtype in bits else b
         if not np.array_equal(av, bv):
             bad = np.nonzero(av != bv)[0]
             raise AssertionError(

@@ -21,8 +21,8 @@ def _inputs(dtype, seed, sigma=1.0, positive=False):
     base = H.randn_list(SHAPES, seed, sigma, np.float64)
     if positive:
         base = [np.abs(a) + 1e-3 for a in base]
-    if dtype == "bf16":
-        return [O.cast(a, np.uint16) for a in base]
+    if dtype in ("bf16", "f16"):
+        return [O.cast(a, np.uint16 if dtype == "bf16" else np.float16) for a in base]
     return [a.astype(NP_DTYPE[dtype]) for a in base]
 
 
@@ -30,7 +30,7 @@ def _empty_like(arrs):
     return H.dev_list([np.zeros_like(a) for a in arrs], SHAPES)
 
 
-@pytest.mark.parametrize("dtype", ["f32", "bf16", "f64"])
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f64", "f16"])
 def test_every_primitive_bit_exact(gpu, dtype):
     a, b = _inputs(dtype, 900), _inputs(dtype, 950, positive=True)
     da, db = H.dev_list(a, SHAPES), H.dev_list(b, SHAPES)
@@ -104,9 +104,11 @@ def test_powf_half_special_cases_follow_c_pow(gpu):
 
 
 @pytest.mark.parametrize("src,dst", [("f64", "bf16"), ("f64", "f32"), ("f32", "bf16"), ("bf16", "f32"),
-                                     ("bf16", "f64"), ("f32", "f64"), ("f32", "f32")])
+                                     ("bf16", "f64"), ("f32", "f64"), ("f32", "f32"), ("f64", "f16"),
+                                     ("f32", "f16"), ("f16", "f32"), ("f16", "f64"), ("f16", "bf16"),
+                                     ("bf16", "f16")])
 def test_cast_bit_exact(gpu, src, dst):
-    np_of = {"f32": np.float32, "f64": np.float64, "bf16": np.uint16}
+    np_of = {"f32": np.float32, "f64": np.float64, "bf16": np.uint16, "f16": np.float16}
     a = H.randn_list(SHAPES, 970, 3.0, np.float64)
     a[3][:3] = [1.0 + 2.0 ** -8 + 2.0 ** -30, -(1.0 + 3 * 2.0 ** -8 - 2.0 ** -40), 1e-42]  # double-rounding ties, f32 subnormal
     a = [O.cast(x, np_of[src]) for x in a]
@@ -198,3 +200,28 @@ def test_f32_to_bf16_rounding_for_every_high_half_and_boundary_low_half(gpu):
     B.cast([src], [dst])
     got, want = H.to_host(dst), O.bf16_from_f32(x)
     assert np.array_equal(got, want), f"first difference at input bits {bits[np.nonzero(got != want)[0][0]]:#010x}"
+
+
+def test_f32_to_f16_and_back_for_every_high_half_and_boundary_low_bits(gpu):
+    """The device converts between f32 and f16 with gfx950's conversion instructions.  An f16
+    keeps 10 mantissa bits, so bit 12 of an f32 decides the rounding of a normal result;
+    every 16-bit high half (all signs, exponents, infinities, NaNs; the exponents that land
+    among f16's subnormals and beyond its largest value included) is combined with low halves
+    around that tie and must give half::f16::from_f32's bits, NaN payloads included.  Every
+    one of the 65536 f16 patterns must widen to f32::from(f16)'s bits."""
+    hi = np.arange(1 << 16, dtype=np.uint32) << 16
+    lows = np.array([0x0000, 0x0001, 0x0FFF, 0x1000, 0x1001, 0x2000, 0x2FFF, 0x3000, 0x3001, 0x7FFF, 0x8000,
+                     0xE000, 0xEFFF, 0xF000, 0xF001, 0xFFFF], dtype=np.uint32)
+    bits = (hi[:, None] | lows[None, :]).reshape(-1)
+    x = bits.view(np.float32)
+    n = x.size
+    dst = H.to_dev(np.zeros(n, dtype=np.float16), (1, n))
+    B.cast([H.to_dev(x, (1, n))], [dst])
+    got, want = H.to_host(dst).view(np.uint16), O.cast(x, np.float16).view(np.uint16)
+    assert np.array_equal(got, want), f"first difference at input bits {bits[np.nonzero(got != want)[0][0]]:#010x}"
+
+    h = np.arange(1 << 16, dtype=np.uint16).view(np.float16)
+    wide = H.to_dev(np.zeros(h.size, dtype=np.float32), (1, h.size))
+    B.cast([H.to_dev(h, (1, h.size))], [wide])
+    got, want = H.to_host(wide).view(np.uint32), O.cast(h, np.float32).view(np.uint32)
+    assert np.array_equal(got, want), f"first difference at f16 bits {np.nonzero(got != want)[0][0]:#06x}"

@@ -154,12 +154,13 @@ def test_adam_f64_bit_exact_vs_sqrt_variant(gpu):
 
 # ---- the fused Trainer tail: bf16 params/grads, f32 master/m/v -------------------------------
 
-def _mixed_case(shapes, steps, lr, wd, max_norm, scaler_state, grad_sigma, inject=None, seed=1):
+def _mixed_case(shapes, steps, lr, wd, max_norm, scaler_state, grad_sigma, inject=None, seed=1, half="bf16"):
     """Run `steps` fused steps on the device and the same Trainer tail on both oracle
-    variants.  inject(step, grads_bits) may poison gradients in place.  Returns the
-    device results and both references."""
+    variants, with parameters and gradients of the 16-bit type `half` over f32 master
+    weights and moments.  inject(step, grads_bits) may poison gradients in place.  Returns
+    the device results and both references."""
     master0 = H.randn_list(shapes, seed, 0.02)
-    p_bits0 = [O.bf16_from_f32(a) for a in master0]
+    p_bits0 = H.narrow_list(master0, half)
     p_dev = H.dev_list(p_bits0, shapes)
     opt = nb.AdamW.new(lr, shapes, master=True).beta2(0.95).weight_decay(wd)
     for i, a in enumerate(master0):
@@ -181,7 +182,7 @@ def _mixed_case(shapes, steps, lr, wd, max_norm, scaler_state, grad_sigma, injec
     scale_now = scaler_state["scale"] if scaler_state else 1.0
     for step in range(steps):
         g32 = H.randn_list(shapes, 5000 + 17 * step + seed, grad_sigma * scale_now)
-        g_bits = [O.bf16_from_f32(a) for a in g32]
+        g_bits = H.narrow_list(g32, half)
         if inject is not None:
             inject(step, g_bits)
         g_dev = H.dev_list(g_bits, shapes)
@@ -221,11 +222,11 @@ def _check_mixed(dev, refs, lr, steps):
     H.assert_bits_equal(dev["m"], sq["m"], "m vs sqrt-variant oracle")
     H.assert_bits_equal(dev["v"], sq["v"], "v vs sqrt-variant oracle")
     H.assert_bits_equal(dev["w"], sq["w"], "master vs sqrt-variant oracle")
-    H.assert_bits_equal(dev["p"], sq["p"], "bf16 params vs sqrt-variant oracle")
+    H.assert_bits_equal(dev["p"], sq["p"], "16-bit params vs sqrt-variant oracle")
     H.assert_bits_equal(dev["m"], libm["m"], "m vs libm-powf oracle")
     H.assert_bits_equal(dev["v"], libm["v"], "v vs libm-powf oracle")
     _param_close(dev["w"], libm["w"], lr, steps, "master vs libm-powf oracle")
-    assert H.max_ulp_bf16(dev["p"], libm["p"]) <= 1, "bf16 params vs libm-powf oracle"
+    assert H.max_ulp_half(dev["p"], libm["p"]) <= 1, "16-bit params vs libm-powf oracle"
 
 
 def test_mixed_adamw_scaler_clip_llama_like(gpu):
@@ -241,6 +242,24 @@ def test_mixed_adamw_scaler_clip_llama_like(gpu):
 def test_mixed_adamw_no_clip_no_scaler(gpu):
     dev, refs = _mixed_case(RAGGED, 4, 1e-3, 0.01, 0.0, None, 1e-3)
     _check_mixed(dev, refs, 1e-3, 4)
+
+
+def test_mixed_f16_adamw_with_dynamic_loss_scale(gpu):
+    """f16 parameters and gradients over f32 master weights -- what a GradScaler is for:
+    gradients that only survive f16 because they are scaled, an overflow to inf every fifth
+    step (the scale backs off, the step is skipped), growth every 3 clean steps."""
+    shapes = H.llama_shapes(2, 256, 64, 704, 1000) + RAGGED
+
+    def inject(step, g):
+        if step % 5 == 4:
+            g[3].view(np.uint16)[7] = [0x7C00, 0xFC00, 0x7E01][(step // 5) % 3]
+
+    scaler = dict(scale=65536.0, growth_factor=2.0, backoff_factor=0.5, growth_interval=3, consecutive_ok=0)
+    # sigma 1e-6: most unscaled gradients would be f16 subnormals or zero
+    dev, refs = _mixed_case(shapes, 12, 2e-4, 0.1, 1.0, scaler, 1e-6, inject=inject, seed=3, half="f16")
+    _check_mixed(dev, refs, 2e-4, 12)
+    assert [t[0] for t in dev["trace"]] == [1 if s % 5 == 4 else 0 for s in range(12)]
+    assert dev["p"][0].dtype == np.float16 and dev["step_count"] == 10
 
 
 def test_fused_steps_are_reproducible_run_to_run(gpu):

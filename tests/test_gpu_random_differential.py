@@ -24,8 +24,8 @@ def _carve(arrs, torch_dtype, rng):
 
     gaps = [int(rng.integers(0, 4)) for _ in arrs]
     total = sum(a.size + g for a, g in zip(arrs, gaps)) + 8
-    if torch_dtype == torch.bfloat16:
-        buf = torch.zeros(total, dtype=torch.int16, device="cuda:0").view(torch.bfloat16)
+    if torch_dtype in (torch.bfloat16, torch.float16):
+        buf = torch.zeros(total, dtype=torch.int16, device="cuda:0").view(torch_dtype)
     else:
         buf = torch.zeros(total, dtype=torch_dtype, device="cuda:0")
     views, off = [], 0
@@ -43,14 +43,20 @@ def _case(seed):
     import torch
 
     rng = np.random.default_rng(seed)
-    mode = ["f32", "f64", "mixed", "bf16"][int(rng.integers(0, 4))]
+    # "mixed" / "mixed16": bf16 / f16 tensors over f32 state and master weights;
+    # "bf16" / "f16": Optimizer<bf16> / Optimizer<f16>
+    mode = ["f32", "f64", "mixed", "bf16", "f16", "mixed16"][int(rng.integers(0, 6))]
+    half = {"mixed": "bf16", "bf16": "bf16", "f16": "f16", "mixed16": "f16"}.get(mode)
+    is_mixed, is_pure = mode in ("mixed", "mixed16"), mode in ("bf16", "f16")
     kind = ["sgd", "adam", "adamw"][int(rng.integers(0, 3))]
     nt = int(rng.integers(1, 9))
     sizes = [int(rng.choice(SIZES)) if rng.random() < 0.7 else int(rng.integers(1, 30000)) for _ in range(nt)]
     shapes = [(1, n) for n in sizes]
     lr = float(10.0 ** rng.uniform(-4, -1))
     b1, b2 = float(rng.choice([0.0, 0.8, 0.9])), float(rng.choice([0.9, 0.95, 0.999]))
-    eps = float(rng.choice([1e-8, 1e-6]))
+    # T = f16 turns an eps below 2^-25 into zero, and 0 / 0 gives NaNs whose sign depends on
+    # the machine
+    eps = float(rng.choice([1e-3, 1e-4] if mode == "f16" else [1e-8, 1e-6]))
     wd = float(rng.choice([0.0, 0.01, 0.1]))
     mom = float(rng.choice([0.0, 0.9]))
     steps = int(rng.integers(1, 6))
@@ -60,17 +66,17 @@ def _case(seed):
     nan_policy = bool(rng.random() < 0.3)
     if mode == "f64":
         # The reference adds the squares serially, the device in a fixed tree: the two f64 norms
-        # agree to ~1e-13 relative, not in the last bit.  T = f32 / bf16 narrow max_norm / norm
+        # agree to ~1e-13 relative, not in the last bit.  T = f32 / bf16 / f16 narrow max_norm / norm
         # before use, which hides that; T = f64 does not, so a clipped f64 step is only equal
         # up to the last ulp and is left to the directed test below.
         clip = 0.0
     what = f"seed {seed}: {mode} {kind} nt={nt} sizes={sizes} lr={lr:.3g} scaler={use_scaler}({scale0}) clip={clip}"
 
-    el = {"f32": np.float32, "f64": np.float64, "mixed": np.float32, "bf16": np.float32}[mode]
+    el = np.float64 if mode == "f64" else np.float32
     w0 = [(O.randn_f64(n, 100 * seed + i) * 0.5).astype(el) for i, n in enumerate(sizes)]
-    if mode == "bf16":
-        w0 = [O.bf16_from_f32(a) for a in w0]
-    tdt = {"f32": torch.float32, "f64": torch.float64, "mixed": torch.bfloat16, "bf16": torch.bfloat16}[mode]
+    if is_pure:
+        w0 = H.narrow_list(w0, half)
+    tdt = {"f32": torch.float32, "f64": torch.float64, "bf16": torch.bfloat16, "f16": torch.float16}[half or mode]
 
     if kind == "sgd":
         meta = O.sgd_meta(lr, momentum=mom, weight_decay=wd)
@@ -81,18 +87,18 @@ def _case(seed):
     else:
         meta = O.adamw_meta(lr, b1, b2, eps, wd)
         make = lambda **kw: nb.AdamW.new(lr, shapes, **kw).beta1(b1).beta2(b2).eps(eps).weight_decay(wd)  # noqa: E731
-    opt = make(master=True) if mode == "mixed" else make(dtype=mode)
+    opt = make(master=True) if is_mixed else make(dtype=mode)
 
     # reference state
-    if mode == "mixed":
+    if is_mixed:
         ref_w = H.copy_list(w0)
-        ref_p = [O.bf16_from_f32(a) for a in w0]
+        ref_p = H.narrow_list(w0, half)
     else:
         ref_w, ref_p = None, H.copy_list(w0)
-    state_like = ref_w if mode == "mixed" else ref_p
+    state_like = ref_w if is_mixed else ref_p
     ref_m, ref_v = [np.zeros_like(a) for a in state_like], [np.zeros_like(a) for a in state_like]
     p_dev, keep_p = _carve(ref_p, tdt, rng)
-    if mode == "mixed":
+    if is_mixed:
         for i, a in enumerate(w0):
             opt.write_state(f"w{i}", H.to_dev(a, shapes[i]))
     scaler = ref_scaler = None
@@ -117,11 +123,11 @@ def _case(seed):
             if bad:
                 t = int(rng.choice([i for i, n in enumerate(sizes) if n]))
                 g[t][int(rng.integers(0, sizes[t]))] = rng.choice([np.inf, -np.inf, np.nan])
-            if mode in ("mixed", "bf16"):
-                g = [O.bf16_from_f32(a.astype(np.float32)) for a in g]
+            if half:
+                g = H.narrow_list(g, half)
             g_dev, kg = _carve(g, tdt, rng)
             keep.append(kg)
-            fused = mode == "mixed" or rng.random() < 0.6
+            fused = is_mixed or rng.random() < 0.6
             zero = fused and rng.random() < 0.3
             if fused:
                 opt.fused_step(p_dev, g_dev, scaler=scaler, max_norm=clip, skip_nonfinite=nan_policy, zero_grads=zero)
@@ -134,15 +140,15 @@ def _case(seed):
                         nb.clip_grad_norm(g_dev, clip)
                     opt.step(p_dev, g_dev)
             # the reference's order (trainer.rs:230-283) on the oracle
-            if mode == "mixed":
-                skip = nan_policy and ref_scaler is None and any(not np.isfinite(O.bf16_to_f32(a)).all() for a in g)
+            if is_mixed:
+                skip = nan_policy and ref_scaler is None and any(not np.isfinite(a).all() for a in H.widen_list(g))
                 if not skip:
                     O.mixed_step(meta, ref_scaler, clip, ref_p, g, ref_w, ref_m, ref_v)
             else:
                 gr = H.copy_list(g)
                 ok = O.scaler_unscale_and_update(ref_scaler, gr) if ref_scaler else True
                 if ok and nan_policy:
-                    vals = [O.bf16_to_f32(a) if mode == "bf16" else a for a in gr]
+                    vals = H.widen_list(gr) if is_pure else gr
                     ok = all(np.isfinite(a).all() for a in vals)
                 if ok:
                     O.clip_grad_norm(gr, clip)
@@ -162,12 +168,12 @@ def _case(seed):
         H.assert_bits_equal(H.host_list(opt.moments()[0]), ref_m, what + ": m")
         H.assert_bits_equal(H.host_list(opt.moments()[1]), ref_v, what + ": v")
         assert opt.step_count() == meta.step_count, what
-    if mode == "mixed":
+    if is_mixed:
         H.assert_bits_equal(H.host_list([opt.read_state(f"w{i}") for i in range(nt)]), ref_w, what + ": master")
     if use_scaler:
         st = scaler.state()
         assert (st.scale, st.consecutive_ok) == (ref_scaler.scale, ref_scaler.consecutive_ok), what
-    start = [O.bf16_from_f32(a) for a in w0] if mode == "mixed" else w0
+    start = H.narrow_list(w0, half) if is_mixed else w0
     return any(not np.array_equal(a, b) for a, b in zip(ref_p, start))  # did any parameter move?
 
 

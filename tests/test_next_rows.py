@@ -293,7 +293,7 @@ def _file_bytes(path):
 @pytest.mark.gpu
 def test_native_nbla_writer_is_byte_identical_to_the_format_writer(gpu, tmp_path):
     """nbo_nbla_save_list / nbo_optim_save_state against the Python writer whose byte layout
-    is checked against a hand-assembled file above: same bytes, for f32, bf16 and f64
+    is checked against a hand-assembled file above: same bytes, for f32, bf16, f16 and f64
     tensors, an empty tensor and a tensor longer than the streaming chunk (2^20)."""
     import torch
 
@@ -301,7 +301,7 @@ def test_native_nbla_writer_is_byte_identical_to_the_format_writer(gpu, tmp_path
 
     shapes = [(3, 5), (1, 1), (0, 7), (1025, 1031)]
     names = ["layer.weight", "b", "empty", "big"]
-    for dt in (torch.float32, torch.bfloat16, torch.float64):
+    for dt in (torch.float32, torch.bfloat16, torch.float64, torch.float16):
         torch.manual_seed(5)
         tensors = [(torch.randn(s, device=gpu, dtype=torch.float32) * 3).to(dt) for s in shapes]
         named = list(zip(names, tensors))
@@ -309,8 +309,8 @@ def test_native_nbla_writer_is_byte_identical_to_the_format_writer(gpu, tmp_path
         ck.save_params_native(str(tmp_path / "native.nbla"), named)
         assert _file_bytes(tmp_path / "native.nbla") == _file_bytes(tmp_path / "py.nbla"), dt
     for opt in (nb.AdamW.new(1e-3, shapes), nb.Sgd.new(0.1, shapes).momentum(0.9),
-                nb.Adam.new(1e-3, shapes, dtype="bf16")):
-        dt = torch.bfloat16 if opt._state_dtype == nb.DT_BF16 else torch.float32
+                nb.Adam.new(1e-3, shapes, dtype="bf16"), nb.Adam.new(1e-3, shapes, dtype="f16").eps(1e-3)):
+        dt = {nb.DT_BF16: torch.bfloat16, nb.DT_F16: torch.float16}.get(opt._state_dtype, torch.float32)
         p = [torch.randn(s, device=gpu, dtype=torch.float32).to(dt) for s in shapes]
         g = [torch.randn(s, device=gpu, dtype=torch.float32).to(dt) for s in shapes]
         opt.step(p, g)
@@ -324,6 +324,7 @@ def test_native_nbla_reader_round_trip_and_errors(gpu, tmp_path):
     import torch
 
     from nabla_amd import checkpoint as ck
+    from tests import helpers as H
 
     shapes = [(3, 5), (1, 1), (1025, 1031)]
     names = ["w", "b", "big"]
@@ -340,6 +341,26 @@ def test_native_nbla_reader_round_trip_and_errors(gpu, tmp_path):
     as_bf16 = [torch.zeros(s, device=gpu, dtype=torch.bfloat16) for s in shapes]
     ck.load_params_native(path, list(zip(names, as_bf16)))
     assert all(torch.equal(a.to(torch.bfloat16), b) for a, b in zip(src, as_bf16))
+    # f16 narrows on the host in software: every f32 high half with the low bits that decide
+    # a rounding, as f64 values in the file, plus f64 values whose rounding to f32 creates a
+    # tie for the second rounding (the reference narrows through f32, scalar/mod.rs:338-340)
+    hi = np.arange(1 << 16, dtype=np.uint32) << 16
+    lows = np.array([0x0000, 0x0001, 0x0FFF, 0x1000, 0x1001, 0x2FFF, 0x3000, 0x3001, 0xFFFF], dtype=np.uint32)
+    with np.errstate(invalid="ignore"):  # signalling NaNs among the patterns
+        vals = (hi[:, None] | lows[None, :]).reshape(-1).view(np.float32).astype(np.float64)
+    vals[:3] = [1.0 + 2.0 ** -11 + 2.0 ** -40, -(1.0 + 3 * 2.0 ** -11 - 2.0 ** -40), 65519.999]
+    f16_path = str(tmp_path / "edge.nbla")
+    ck.save_tensors([("edge", vals.reshape(1, -1))], f16_path)
+    as_f16 = torch.zeros((1, vals.size), device=gpu, dtype=torch.float16)
+    ck.load_params_native(f16_path, [("edge", as_f16)])
+    got, want = H.to_host(as_f16).view(np.uint16), O.cast(vals, np.float16).view(np.uint16)
+    assert np.array_equal(got, want), f"first difference at value {vals[np.nonzero(got != want)[0][0]]!r}"
+    # and back: every f16 pattern widens exactly (NaNs keep their payload in the f64 file)
+    every = torch.from_numpy(np.arange(1 << 16, dtype=np.uint16).view(np.int16).copy()).view(torch.float16)
+    ck.save_params_native(f16_path, [("every", every.reshape(1, -1).to(gpu))])
+    back = ck.load_tensors(f16_path)[0][1].reshape(-1)
+    want = O.cast(O.cast(np.arange(1 << 16, dtype=np.uint16).view(np.float16), np.float32), np.float64)
+    assert np.array_equal(back.view(np.uint64), want.view(np.uint64))
     with pytest.raises(ck.CheckpointError, match="unknown parameter key: b"):
         ck.load_params_native(path, [("w", dst[0]), ("big", dst[2])])
     with pytest.raises(ck.CheckpointError, match=r"shape mismatch for 'w': expected \(5, 3\), got \(3, 5\)"):
