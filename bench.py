@@ -31,7 +31,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="llama3-8b",
                     choices=["llama3-8b", "llama-1.1b", "gpt2-small-f32", "mlp-sgd-f32", "ragged-4096",
-                             "llama-1.1b-bf16"])
+                             "llama-1.1b-bf16", "llama-1.1b-f16", "llama-1.1b-f16-mixed"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--zero-grads", choices=["off", "fused", "separate"], default="off",
                     help="also clear the gradients every step (trainer.rs:285-290): inside the update "
@@ -56,8 +56,12 @@ def workload(name):
     if name == "llama-1.1b":
         return dict(shapes=W.llama_1b_shapes(), mixed=True, kind="adamw", lr=2e-4, wd=0.1,
                     betas=(0.9, 0.95), scaler=True, clip=1.0, p_sigma=0.02, g_sigma=1e-3)
-    if name == "llama-1.1b-bf16":  # Optimizer<bf16>: tensors, moments and arithmetic all bf16
-        return dict(shapes=W.llama_1b_shapes(), mixed=False, pure_bf16=True, kind="adamw", lr=2e-4, wd=0.1,
+    if name in ("llama-1.1b-bf16", "llama-1.1b-f16"):  # Optimizer<bf16> / Optimizer<f16>: all in 16 bits
+        return dict(shapes=W.llama_1b_shapes(), mixed=False, pure=True, half=name[-4:].lstrip("-"), kind="adamw",
+                    lr=2e-4, wd=0.1, betas=(0.9, 0.95), eps=1e-8 if name.endswith("bf16") else 1e-4,
+                    scaler=True, clip=1.0, p_sigma=0.02, g_sigma=1e-3)
+    if name == "llama-1.1b-f16-mixed":  # f16 tensors over f32 master weights and moments
+        return dict(shapes=W.llama_1b_shapes(), mixed=True, half="f16", kind="adamw", lr=2e-4, wd=0.1,
                     betas=(0.9, 0.95), scaler=True, clip=1.0, p_sigma=0.02, g_sigma=1e-3)
     if name == "ragged-4096":
         return dict(shapes=[(1, n) for n in W.ragged_sizes()], mixed=True, kind="adamw", lr=2e-4,
@@ -70,7 +74,7 @@ def workload(name):
 
 
 def bytes_per_param(cfg):
-    if cfg.get("pure_bf16"):
+    if cfg.get("pure"):
         return 14, 2  # R p, g, m, v + W p, m, v at 2 B each; norm pass R g
     if cfg["kind"] == "sgd":
         return 12, 0
@@ -113,21 +117,22 @@ def cpu_baseline(cfg, budget_s):
     elif cfg["kind"] == "adam":
         meta = O.adam_meta(cfg["lr"], *cfg["betas"])
     else:
-        meta = O.adamw_meta(cfg["lr"], *cfg["betas"], weight_decay=cfg["wd"])
+        meta = O.adamw_meta(cfg["lr"], *cfg["betas"], eps=cfg.get("eps", 1e-8), weight_decay=cfg["wd"])
     scaler = O.default_scaler() if cfg["scaler"] else None
-    if cfg.get("pure_bf16"):
-        p = [O.bf16_from_f32(a) for a in master]
+    narrow = (lambda a: O.cast(a, np.float16)) if cfg.get("half") == "f16" else O.bf16_from_f32
+    if cfg.get("pure"):
+        p = [narrow(a) for a in master]
         m, v = [np.zeros_like(a) for a in p], [np.zeros_like(a) for a in p]
-        g16 = [O.bf16_from_f32(a) for a in g32]
+        g16 = [narrow(a) for a in g32]
 
-        def run():  # trainer.rs:230-283 with T = bf16
+        def run():  # trainer.rs:230-283 with T = bf16 / f16
             gg = [a.copy() for a in g16]
             if O.scaler_unscale_and_update(scaler, gg):
                 O.clip_grad_norm(gg, cfg["clip"])
                 O.adam_step(meta, p, gg, m, v)
     elif cfg["mixed"]:
-        g = [O.bf16_from_f32(a) for a in g32]
-        p = [O.bf16_from_f32(a) for a in master]
+        g = [narrow(a) for a in g32]
+        p = [narrow(a) for a in master]
         run = lambda: O.mixed_step(meta, scaler, cfg["clip"], p, g, master, m, v)  # noqa: E731
     else:
         def run():
@@ -173,8 +178,9 @@ def measure(name, steps, warmup, zero_grads="off"):
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
 
-    pure = bool(cfg.get("pure_bf16"))
-    pdt = torch.bfloat16 if (cfg["mixed"] or pure) else torch.float32
+    pure, half = bool(cfg.get("pure")), cfg.get("half", "bf16")
+    hdt = torch.float16 if half == "f16" else torch.bfloat16
+    pdt = hdt if (cfg["mixed"] or pure) else torch.float32
     params = [torch.empty(s, dtype=pdt, device=dev) for s in shapes]
     grads = [torch.empty(s, dtype=pdt, device=dev) for s in shapes]
     if cfg["kind"] == "sgd":
@@ -182,8 +188,8 @@ def measure(name, steps, warmup, zero_grads="off"):
     elif cfg["kind"] == "adam":
         opt = nb.Adam.new(cfg["lr"], shapes).beta1(cfg["betas"][0]).beta2(cfg["betas"][1])
     else:
-        opt = nb.AdamW.new(cfg["lr"], shapes, master=cfg["mixed"], dtype="bf16" if pure else "f32") \
-            .beta1(cfg["betas"][0]).beta2(cfg["betas"][1]).weight_decay(cfg["wd"])
+        opt = nb.AdamW.new(cfg["lr"], shapes, master=cfg["mixed"], dtype=half if pure else "f32") \
+            .beta1(cfg["betas"][0]).beta2(cfg["betas"][1]).eps(cfg.get("eps", 1e-8)).weight_decay(cfg["wd"])
     scale = 65536.0 if cfg["scaler"] else 1.0
     for i, s in enumerate(shapes):  # synthetic, random-init
         w = torch.randn(s, dtype=torch.float32, device=dev) * cfg["p_sigma"]
@@ -211,7 +217,7 @@ def measure(name, steps, warmup, zero_grads="off"):
 
     upd_b, nrm_b = bytes_per_param(cfg)
     zero_b = 0 if zero_grads == "off" else (2 if (cfg["mixed"] or pure) else 4)
-    fam = "pbf16" if pure else "bf16" if cfg["mixed"] else "f32"
+    fam = ("pf16" if half == "f16" else "pbf16") if pure else half if cfg["mixed"] else "f32"
     dom = f"nbo_update_{fam}_{cfg['kind']}"
     names = [dom] + ([f"nbo_norm_{fam}", "nbo_finalize"] if fused
                      else ([] if cfg["kind"] == "sgd" else ["nbo_prep"]))
@@ -270,9 +276,9 @@ def measure(name, steps, warmup, zero_grads="off"):
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if pure else "f32",
-        "storage": ("bf16 params/grads/m/v" if pure else
-                    "bf16 params/grads, f32 master/m/v" if cfg["mixed"] else "f32 params/grads/m/v"),
+        "dtype": half if pure else "f32",
+        "storage": (f"{half} params/grads/m/v" if pure else
+                    f"{half} params/grads, f32 master/m/v" if cfg["mixed"] else "f32 params/grads/m/v"),
         "data": "synthetic (random-init parameters and gradients of the named shapes, resident in HBM)",
         "config": {"workload": name, "tensors": len(shapes), "params": n,
                    "bytes_per_param_step": upd_b + nrm_b + zero_b, "zero_grads": zero_grads,
