@@ -590,6 +590,13 @@ template <> __device__ __forceinline__ bool nonfinite<NBO_PBF16>(BF x) { return 
 template <> __device__ __forceinline__ bool nonfinite<NBO_F16>(float x) { return nonfinite_f32(x); }
 template <> __device__ __forceinline__ bool nonfinite<NBO_PF16>(HF x) { return x.nonfinite(); }
 
+// A 16-bit pattern as the arithmetic type of storage ST (exact).
+template <int ST> DEV typename Traits<ST>::T from_half_bits(uint32_t b);
+template <> __device__ __forceinline__ float from_half_bits<NBO_BF16>(uint32_t b) { return bf16_bits_to_f32(b); }
+template <> __device__ __forceinline__ float from_half_bits<NBO_F16>(uint32_t b) { return f16_bits_to_f32(b); }
+template <> __device__ __forceinline__ BF from_half_bits<NBO_PBF16>(uint32_t b) { return half_from_bits<FMT_BF16>(b); }
+template <> __device__ __forceinline__ HF from_half_bits<NBO_PF16>(uint32_t b) { return half_from_bits<FMT_F16>(b); }
+
 template <int ST> DEV void norm_body(const NboNormArgs &a)
 {
     typedef typename Traits<ST>::T T;
@@ -605,22 +612,28 @@ template <int ST> DEV void norm_body(const NboNormArgs &a)
         const ChunkRef c = chunk_ref(a.L, ci);
         const char *pg = (const char *)a.g_ptrs[c.t] + c.base * SB;
         uint32_t done = 0;
-        if constexpr (ST == NBO_BF16 || ST == NBO_F16) {
-            // 8 half-width elements per 128-bit load
+        if constexpr (SB == 2) {
+            // 8 half-width elements per 128-bit load.  Inf / NaN test on both halves of a word
+            // at once: adding the exponent field's lowest bit to the masked exponent carries
+            // into the sign position exactly when the exponent is all ones.
+            constexpr bool is_bf = ST == NBO_BF16 || ST == NBO_PBF16;
+            constexpr uint32_t EXP_MASK = is_bf ? 0x7F807F80u : 0x7C007C00u;
+            constexpr uint32_t EXP_LSB = is_bf ? 0x00800080u : 0x04000400u;
             if ((((uintptr_t)pg) & 15u) == 0) {
                 const uint32_t nvec = c.cnt / 8;
+                uint32_t carries = 0;
                 for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
                     const u32x4 w = __builtin_nontemporal_load(GLOBAL_PTR(const u32x4, pg) + q);
                     const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
                     for (int k = 0; k < 4; k++) {
-                        const float lo = ST == NBO_BF16 ? __uint_as_float(ww[k] << 16) : f16_bits_to_f32(ww[k] & 0xFFFFu);
-                        const float hi = ST == NBO_BF16 ? __uint_as_float(ww[k] & 0xFFFF0000u) : f16_bits_to_f32(ww[k] >> 16);
-                        bad |= (uint32_t)nonfinite_f32(lo) | (uint32_t)nonfinite_f32(hi);
+                        carries |= (ww[k] & EXP_MASK) + EXP_LSB;
+                        const T lo = from_half_bits<ST>(ww[k] & 0xFFFFu), hi = from_half_bits<ST>(ww[k] >> 16);
                         acc = sq_acc<ST>(acc, (T)(lo * inv));
                         acc = sq_acc<ST>(acc, (T)(hi * inv));
                     }
                 }
+                bad |= (uint32_t)((carries & 0x80008000u) != 0);
                 done = nvec * 8;
             }
         } else {
