@@ -218,10 +218,11 @@ public:
 
     // the Trainer tail (trainer.rs:230-291) in one asynchronous call
     void fused_step(TensorList &params, TensorList &grads, GradScaler *scaler, double max_norm,
-                    bool zero_grads = false)
+                    bool zero_grads = false, bool skip_nonfinite = false)
     {
         check(nbo_fused_step(handle(), scaler ? scaler->handle() : nullptr, params.handle(), grads.handle(),
-                             max_norm, zero_grads ? NBO_STEP_ZERO_GRADS : 0u));
+                             max_norm,
+                             (zero_grads ? NBO_STEP_ZERO_GRADS : 0u) | (skip_nonfinite ? NBO_STEP_SKIP_NONFINITE : 0u)));
     }
     nbo_step_info last_step()
     {
@@ -488,6 +489,11 @@ struct TrainError : std::runtime_error { // TrainError::EvalError
 // Per micro-batch: scaler -> nan policy -> accumulate -> (every grad_accum-th) schedule,
 // clip, step, zero.  `accum` is caller-provided zero-filled storage shaped like the
 // gradients (the reference allocates it; this library allocates nothing per step).
+// Without accumulation and with at most one of scaler / nan policy the whole sequence is
+// one fused step whose skip is decided on the device (the decision is read back only
+// because step(), which the schedule is a function of, must not advance on a skipped step);
+// otherwise the decisions are the reference's synchronous ones and clip + step + zero over
+// the accumulation buffer are one fused step.
 class TrainerTail {
 public:
     TrainerTail(Optimizer &optimizer, TensorList &params, TensorList &accum)
@@ -505,6 +511,7 @@ public:
     // returns true if the optimizer stepped; grads are modified in place like the reference's
     bool after_backward(TensorList &grads)
     {
+        if (grad_accum_ == 1 && !(scaler_ && has_policy_)) return fused(grads);
         if (scaler_ && !scaler_->unscale_and_update(grads)) return drop(); // :230-237
         if (has_policy_ && has_non_finite(grads)) {                        // :239-251
             if (policy_ == GradNanPolicy::Skip) return drop();
@@ -519,16 +526,25 @@ public:
         accum_count_ += 1;
         if (accum_count_ < grad_accum_) return false;
         if (has_schedule_) opt_.set_lr(lr_at_step(schedule_, base_lr_, step_)); // :270-273
-        if (grad_clip_ > 0.0) clip_grad_norm(accum_, grad_clip_);              // :274-278
-        opt_.step(params_, accum_);                                            // :279-283
+        opt_.fused_step(params_, accum_, nullptr, grad_clip_, /*zero_grads=*/true); // :274-290
         accum_count_ = 0;
-        zero_grad(accum_); // :285-290
         dirty_ = false;
         step_ += 1;
         return true;
     }
 
 private:
+    bool fused(TensorList &grads)
+    {
+        if (has_schedule_) opt_.set_lr(lr_at_step(schedule_, base_lr_, step_)); // harmless if the step is skipped
+        opt_.fused_step(params_, grads, scaler_, grad_clip_, false, has_policy_);
+        if ((scaler_ || has_policy_) && opt_.last_step().found_inf) {
+            if (!scaler_ && policy_ == GradNanPolicy::Stop) throw TrainError("non-finite gradient");
+            return false;
+        }
+        step_ += 1;
+        return true;
+    }
     bool drop()
     {
         accum_count_ = 0; // accum_grads = None: the buffer is cleared before its next use

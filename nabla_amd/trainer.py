@@ -14,8 +14,10 @@ Per micro-batch, in the reference's order:
 With `grad_accum == 1` and at most one of scaler / nan policy, steps 1-4 are one
 `fused_step` (three launches, the skip decided on the device); the decision is read back
 afterwards only because `state.step` -- which the schedule is a function of -- must not
-advance on a skipped step.  Otherwise the unfused entry points run in the order above,
-with the reference's synchronous decisions after steps 1 and 2.
+advance on a skipped step.  Otherwise the unfused entry points run steps 1-3 in the order
+above, with the reference's synchronous decisions after steps 1 and 2, and step 4 is one
+`fused_step` over the accumulation buffer (norm pass, then clip + update + zeroing in one
+kernel) instead of the reference's four passes.
 """
 from __future__ import annotations
 
@@ -129,10 +131,9 @@ class TrainerTail:
         if self._accum_count < self.state.grad_accum:
             return False
         self._set_lr()
-        if self.grad_clip is not None:
-            nb.clip_grad_norm(self._accum, self.grad_clip)
-        self.optimizer.step(self.params, self._accum)
+        # clip_grad_norm, step and the re-zeroing of the buffer (:274-290)
+        self.optimizer.fused_step(self.params, self._accum, scaler=None, max_norm=self.grad_clip or 0.0,
+                                  zero_grads=True)
         self._accum_count = 0
-        nb.zero_grad(self._accum)
         self.state.step += 1
         return True
