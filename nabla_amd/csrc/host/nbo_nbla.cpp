@@ -187,9 +187,19 @@ struct Entry {
     long data_offset;
 };
 
-// Reads the file's table of contents, skipping over the values.
+// Reads the file's table of contents, skipping over the values.  Lengths come from the
+// file, so each is checked against what is left of it before anything is sized by it; a
+// file that ends early is the reference's read_exact error.
 std::vector<Entry> read_index(std::FILE *f)
 {
+    if (std::fseek(f, 0, SEEK_END) != 0) fail(NBO_ERR_IO, "seek failed");
+    const long file_size = std::ftell(f);
+    if (file_size < 0 || std::fseek(f, 0, SEEK_SET) != 0) fail(NBO_ERR_IO, "seek failed");
+    const auto left = [&]() -> uint64_t {
+        const long pos = std::ftell(f);
+        if (pos < 0) fail(NBO_ERR_IO, "seek failed");
+        return pos < file_size ? (uint64_t)(file_size - pos) : 0;
+    };
     char magic[4];
     read_exact(f, magic, 4);
     if (std::memcmp(magic, "NBLA", 4) != 0) fail(NBO_ERR_IO, "not a nabla tensor file");
@@ -198,18 +208,18 @@ std::vector<Entry> read_index(std::FILE *f)
     for (uint32_t i = 0; i < count; i++) {
         Entry e;
         const uint32_t name_len = read_u32(f);
+        if (name_len > left()) fail(NBO_ERR_IO, "failed to fill whole buffer");
         e.name.resize(name_len);
         read_exact(f, e.name.empty() ? nullptr : &e.name[0], name_len);
         e.rows = read_u32(f);
         e.cols = read_u32(f);
         e.data_offset = std::ftell(f);
-        const uint64_t bytes = e.rows * e.cols * 8;
-        if (e.data_offset < 0 || std::fseek(f, (long)bytes, SEEK_CUR) != 0) fail(NBO_ERR_IO, "seek failed");
+        if (e.data_offset < 0) fail(NBO_ERR_IO, "seek failed");
+        const uint64_t elems = e.rows * e.cols; // both below 2^32
+        if (elems > left() / 8) fail(NBO_ERR_IO, "failed to fill whole buffer");
+        if (std::fseek(f, (long)(elems * 8), SEEK_CUR) != 0) fail(NBO_ERR_IO, "seek failed");
         out.push_back(std::move(e));
     }
-    // a truncated last tensor shows up as a short file
-    const long end_of_index = std::ftell(f);
-    if (std::fseek(f, 0, SEEK_END) != 0 || std::ftell(f) < end_of_index) fail(NBO_ERR_IO, "failed to fill whole buffer");
     return out;
 }
 

@@ -373,6 +373,13 @@ def test_native_nbla_reader_round_trip_and_errors(gpu, tmp_path):
     (tmp_path / "short.nbla").write_bytes(_file_bytes(path)[:-9])
     with pytest.raises(ck.CheckpointError, match="failed to fill whole buffer"):
         ck.load_params_native(str(tmp_path / "short.nbla"), list(zip(names, dst)))
+    # lengths a corrupt header claims are checked against the file before anything is sized by them
+    (tmp_path / "name.nbla").write_bytes(b"NBLA" + struct.pack("<II", 1, 0xFFFFFFF0) + b"x" * 8)
+    (tmp_path / "data.nbla").write_bytes(b"NBLA" + struct.pack("<II", 1, 1) + b"w" +
+                                         struct.pack("<II", 0xFFFFFFFF, 0xFFFFFFFF) + bytes(16))
+    for bad in ("name.nbla", "data.nbla"):
+        with pytest.raises(ck.CheckpointError, match="failed to fill whole buffer"):
+            ck.load_params_native(str(tmp_path / bad), list(zip(names, dst)))
 
     # optimizer state: round trip, then the reference's load_state_tensors errors
     opt = nb.AdamW.new(1e-3, shapes)
