@@ -39,6 +39,14 @@
  *     the `half` crate's documented operators, and checked in exact arithmetic (round
  *     to 24 bits, then to 8) including the inner rounding of axpy and the two-step
  *     f64 -> bf16 cast.  PARITY UNPINNED against any output of the reference.
+ *   - f16 conversions and the T = f16 instantiations: half::f16::from_f32 /
+ *     f32::from(f16) are restated from the same crate's published algorithm and
+ *     checked against IEEE binary16 as numpy's float16 implements it (every one of the
+ *     65536 patterns widened; narrowing on random values, every tie and the subnormal
+ *     and overflow boundaries); the pass chains are the same source as for bf16,
+ *     checked in exact arithmetic (round to 24 bits, then to 11).  No reference test
+ *     runs f16 on this path: PARITY UNPINNED for NaN payloads and against any output
+ *     of the reference.
  *   - the benchmarks' LCG rand_tensor (benchmarks/src/lib.rs:7-22): exact arithmetic.
  */
 #ifndef NABLA_CPU_ORACLE_H
