@@ -187,6 +187,8 @@ public:
         TensorList p(params), g(grads);
         step(p, g);
     }
+    // optim/core.rs:12-16: the default forwards to step
+    void step_slices(const std::vector<Tensor> &params, const std::vector<Tensor> &grads) { step(params, grads); }
     // optim/core.rs:18-39.  `module.parameters_mut()` yields a std::vector<Tensor>; each
     // variable's `grad()` yields a `const Tensor *`, null when backward has not run.
     template <typename Module, typename Var> void step_with_vars(Module &module, const std::vector<Var> &param_vars)
@@ -261,6 +263,16 @@ public:
     void save_state(const std::string &path) { check(nbo_optim_save_state(handle(), path.c_str())); }
     void load_state(const std::string &path) { check(nbo_optim_load_state(handle(), path.c_str())); }
     void master_from_params(TensorList &params_half) { check(nbo_optim_master_from_params(handle(), params_half.handle())); }
+    void params_from_master(TensorList &params_half) { check(nbo_optim_params_from_master(handle(), params_half.handle())); }
+    // names of state_tensors() in their order (alg.rs:476-485, 553-562, 623-629)
+    std::vector<std::string> state_names() const
+    {
+        std::vector<std::string> out;
+        if (meta_.kind != NBO_KIND_SGD)
+            for (size_t i = 0; i < shapes_.size(); i++) out.push_back("m" + std::to_string(i));
+        for (size_t i = 0; i < shapes_.size(); i++) out.push_back("v" + std::to_string(i));
+        return out;
+    }
 
     nbo_optim *handle()
     {
@@ -298,6 +310,14 @@ private:
 
 using Shapes = std::vector<std::pair<uint64_t, uint64_t>>;
 
+// `X::from_params(lr, params)` is `X(lr, shapes_of(params))` (alg.rs:41-45, 201-205, 332-336)
+inline Shapes shapes_of(const std::vector<Tensor> &params)
+{
+    Shapes out;
+    for (const Tensor &p : params) out.push_back(p.shape());
+    return out;
+}
+
 // alg.rs:310-428
 class Sgd : public Optimizer {
 public:
@@ -309,6 +329,12 @@ public:
     Sgd &weight_decay(double wd) { builder_guard(); meta_.weight_decay = wd; return *this; }
     double momentum_value() const { return meta_.momentum; }
     double weight_decay_value() const { return meta_.weight_decay; }
+    // alg.rs:374-378
+    void set_state(double lr, double momentum, double weight_decay)
+    {
+        load_meta({OptimKind::Sgd, lr, 0.0, 0.0, 0.0, weight_decay, momentum, 0});
+        meta_.momentum = momentum, meta_.weight_decay = weight_decay;
+    }
 };
 
 // alg.rs:169-308
@@ -322,6 +348,12 @@ public:
     Adam &beta1(double b) { builder_guard(); meta_.beta1 = b; return *this; }
     Adam &beta2(double b) { builder_guard(); meta_.beta2 = b; return *this; }
     Adam &eps(double e) { builder_guard(); meta_.eps = e; return *this; }
+    // alg.rs:244-250
+    void set_state(uint64_t step_count, double beta1, double beta2, double eps, double lr)
+    {
+        load_meta({OptimKind::Adam, lr, beta1, beta2, eps, 0.0, 0.0, step_count});
+        meta_.beta1 = beta1, meta_.beta2 = beta2, meta_.eps = eps;
+    }
 };
 
 // alg.rs:7-167
@@ -336,6 +368,12 @@ public:
     AdamW &beta2(double b) { builder_guard(); meta_.beta2 = b; return *this; }
     AdamW &eps(double e) { builder_guard(); meta_.eps = e; return *this; }
     AdamW &weight_decay(double wd) { builder_guard(); meta_.weight_decay = wd; return *this; }
+    // alg.rs:90-105
+    void set_state(uint64_t step_count, double beta1, double beta2, double eps, double weight_decay, double lr)
+    {
+        load_meta({OptimKind::AdamW, lr, beta1, beta2, eps, weight_decay, 0.0, step_count});
+        meta_.beta1 = beta1, meta_.beta2 = beta2, meta_.eps = eps, meta_.weight_decay = weight_decay;
+    }
 };
 
 // nabla-train/src/trainer.rs:500-523; returns the pre-clip norm

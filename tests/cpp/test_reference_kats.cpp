@@ -335,6 +335,36 @@ static void panics_and_errors()  // alg.rs:110-119, 531-545; tensor/ops.rs:638-6
     EXPECT(p.get() == 1.0);  // nothing ran
 }
 
+static void constructors_and_set_state()  // alg.rs:41-45, 90-105, 244-250, 374-378; core.rs:12-16
+{
+    Mat p({1.0, 2.0}), g({1.0, 1.0});
+    const std::vector<Tensor> params = {p.tensor()}, grads = {g.tensor()};
+    EXPECT(shapes_of(params) == (Shapes{{1, 2}}));
+    AdamW opt(0.1, shapes_of(params), NBO_DT_F64);  // AdamW::from_params(0.1, &params)
+    EXPECT((opt.state_names() == std::vector<std::string>{"m0", "v0"}));
+    opt.step_slices(params, grads);
+    EXPECT(opt.step_count() == 1);
+    opt.set_state(41, 0.8, 0.9, 1e-6, 0.25, 0.5);
+    const OptimMeta m = opt.meta();
+    EXPECT(m.step_count == 41 && m.beta1 == 0.8 && m.beta2 == 0.9 && m.eps == 1e-6 && m.weight_decay == 0.25 &&
+           m.lr == 0.5 && opt.lr() == 0.5);
+    opt.step_slices(params, grads);
+    EXPECT(opt.step_count() == 42);
+    Adam adam(0.1, shapes_of(params), NBO_DT_F64);
+    adam.set_state(7, 0.5, 0.75, 1e-3, 0.125);
+    const OptimMeta a = adam.meta();
+    EXPECT(a.step_count == 7 && a.beta1 == 0.5 && a.beta2 == 0.75 && a.eps == 1e-3 && a.lr == 0.125 &&
+           a.weight_decay == 0.0);
+    Sgd sgd(0.1, shapes_of(params), NBO_DT_F64);
+    EXPECT((sgd.state_names() == std::vector<std::string>{"v0"}));
+    sgd.set_state(0.5, 0.0, 0.5);  // p <- p - 0.5 * (g + 0.5 * p)
+    const double before = p.get(1);
+    sgd.step_slices(params, grads);
+    EXPECT(p.get(1) == before - 0.5 * (1.0 + before * 0.5));
+    const OptimMeta sm = sgd.meta();
+    EXPECT(sm.lr == 0.5 && sm.momentum == 0.0 && sm.weight_decay == 0.5 && sm.step_count == 0);
+}
+
 // `--lr`: prints lr_at_step for a grid of schedules and steps as f64 bit patterns, for a
 // bit-for-bit comparison with the CPU oracle (needs no device).
 static int print_lr_grid()
@@ -374,7 +404,8 @@ int main(int argc, char **argv)
                  {"trainer_accumulates_then_clips_and_steps", trainer_accumulates_then_clips_and_steps},
                  {"backend_axpy_is_multiply_then_add", backend_axpy_is_multiply_then_add},
                  {"checkpoint_roundtrip_with_schedule", checkpoint_roundtrip_with_schedule},
-                 {"panics_and_errors", panics_and_errors}};
+                 {"panics_and_errors", panics_and_errors},
+                 {"constructors_and_set_state", constructors_and_set_state}};
     try {
         check(nbo_init());
         for (auto &t : tests) {
