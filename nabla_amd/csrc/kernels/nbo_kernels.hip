@@ -12,7 +12,9 @@
 //                   (trainer.rs:514-517) and the per-step scalars (alg.rs:120-135)
 //   nbo_scale_*     the in-place gradient rescale / zero of core.rs:372-380,
 //                   trainer.rs:518-520, autograd/ops.rs:1668-1680
-//   nbo_cast_*      bf16 <-> f32 casts (common/scalar/mod.rs:338-344)
+//   nbo_cast_*      bf16 / f16 <-> f32 casts (common/scalar/mod.rs:338-344), casts between lists
+//   nbo_ew_*        the Backend primitives as single passes (nabla-core/src/cpu/mod.rs:211-272)
+//   nbo_accum_*     gradient accumulation buf += g (trainer.rs:253-267)
 //
 // Numerics contract: every arithmetic operation of the reference is one IEEE
 // round-to-nearest operation here, in the same order, never contracted into an
@@ -138,9 +140,11 @@ DEV double powi_f64(double a, int n)
 }
 
 // ---------------------------------------------------------------------------------
-// Storage access.  ST is the caller-tensor element type (NBO_F32 / NBO_BF16 /
-// NBO_F64); the arithmetic type T is float for the first two and double for the
-// last.  One "vector" is VEC consecutive elements = 16 bytes of T.
+// Storage access.  ST names the caller-tensor element type together with the arithmetic
+// type T: NBO_F32 (float), NBO_F64 (double), NBO_BF16 / NBO_F16 (16-bit tensors, T = float:
+// the f32-master composition), NBO_PBF16 / NBO_PF16 (16-bit tensors with T the same 16-bit
+// type, every operation rounded to it).  One "vector" is VEC consecutive elements = 16 bytes
+// of T.
 template <int ST> struct Traits;
 template <> struct Traits<NBO_F32> {
     typedef float T;
