@@ -215,6 +215,27 @@ int nbo_fused_step_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *c
 /* Gradient accumulation of the Trainer, buf[i] = &buf[i] + g (trainer.rs:262-266),
  * optionally zeroing the gradients in the same pass.  Asynchronous. */
 int nbo_accumulate(nbo_list *accum, nbo_list *grads, int zero_grads);
+/* One micro-batch of the accumulating Trainer in a single pass over the gradients
+ * (trainer.rs:230-267): the finite scan and loss-scale update of
+ * GradScaler::unscale_and_update (core.rs:351-388; `scaler` may be null: no unscale),
+ * buf[i] = &buf[i] + T(g * T(1 / scale)), and the sum of squares of the new buffer, which
+ * the clip of the last micro-batch needs (trainer.rs:504-513; hand it to
+ * nbo_fused_step_norm).  *ok = 0 on a non-finite gradient (with a scaler, or with
+ * NBO_ACC_CHECK_FINITE for GradNanPolicy): the buffer then holds garbage, as the Trainer
+ * discards the accumulation (trainer.rs:232-236, 241-245).  The gradients themselves stay
+ * as they were unless NBO_ACC_WRITE_GRADS asks for the reference's in-place result
+ * (unscaled, or zeros when non-finite).  Results are those of
+ * nbo_scaler_unscale_and_update followed by nbo_accumulate, bit for bit.  Synchronous. */
+#define NBO_ACC_CHECK_FINITE 1u
+#define NBO_ACC_WRITE_GRADS 2u
+int nbo_unscale_accumulate(nbo_scaler *scaler, nbo_list *accum, nbo_list *grads, uint32_t flags, int *ok,
+                           double *accum_sumsq);
+/* clip_grad_norm + Optimizer::step (+ zeroing with NBO_STEP_ZERO_GRADS) over gradients whose
+ * sum of squares is already known -- from nbo_unscale_accumulate, if nothing has written the
+ * buffer since -- so the norm pass is not run again (trainer.rs:274-290).  No scaler and no
+ * finite check: both belong to the micro-batches.  Asynchronous. */
+int nbo_fused_step_norm(nbo_optim *opt, nbo_list *params, nbo_list *grads, double max_norm, double sumsq,
+                        uint32_t flags);
 /* ---- Backend primitives on tensor lists ------------------------------------------------
  * The single passes the reference's optimizers are chains of, as multi-tensor launches:
  * BackendCore::{scale, axpy_inplace, add, zeros, clone_storage}

@@ -226,6 +226,12 @@ public:
                              max_norm,
                              (zero_grads ? NBO_STEP_ZERO_GRADS : 0u) | (skip_nonfinite ? NBO_STEP_SKIP_NONFINITE : 0u)));
     }
+    // clip + step (+ zeroing) over gradients whose sum of squares is already known
+    void fused_step_norm(TensorList &params, TensorList &grads, double sumsq, double max_norm, bool zero_grads = false)
+    {
+        check(nbo_fused_step_norm(handle(), params.handle(), grads.handle(), max_norm, sumsq,
+                                  zero_grads ? NBO_STEP_ZERO_GRADS : 0u));
+    }
     nbo_step_info last_step()
     {
         nbo_step_info info;
@@ -399,6 +405,18 @@ inline void accumulate(TensorList &accum, TensorList &grads, bool zero_grads = f
 {
     check(nbo_accumulate(accum.handle(), grads.handle(), zero_grads ? 1 : 0));
 }
+// One micro-batch of the accumulating Trainer in a single pass (trainer.rs:230-267): finite
+// scan + loss-scale update, buf[i] = &buf[i] + g / scale, and the new buffer's sum of squares.
+// Returns false on a non-finite gradient (the buffer then holds garbage, the Trainer discards it).
+inline bool unscale_accumulate(TensorList &accum, TensorList &grads, GradScaler *scaler, double *sumsq,
+                               bool check_finite = false, bool write_grads = false)
+{
+    int ok = 0;
+    check(nbo_unscale_accumulate(scaler ? scaler->handle() : nullptr, accum.handle(), grads.handle(),
+                                 (check_finite ? NBO_ACC_CHECK_FINITE : 0u) | (write_grads ? NBO_ACC_WRITE_GRADS : 0u),
+                                 &ok, sumsq));
+    return ok != 0;
+}
 
 // params.nbla of a checkpoint: save_tensors / load_tensors + load_state_dict
 // (nabla-ml/src/module/core.rs:66-120, 281-304) over a list of device tensors
@@ -530,8 +548,10 @@ struct TrainError : std::runtime_error { // TrainError::EvalError
 // Without accumulation and with at most one of scaler / nan policy the whole sequence is
 // one fused step whose skip is decided on the device (the decision is read back only
 // because step(), which the schedule is a function of, must not advance on a skipped step);
-// otherwise the decisions are the reference's synchronous ones and clip + step + zero over
-// the accumulation buffer are one fused step.
+// otherwise the decisions are the reference's synchronous ones: scan, unscale and
+// accumulation are one pass over the gradients, which also yields the buffer's sum of
+// squares, and clip + step + zero over the accumulation buffer are one fused step.
+// The reference unscales the gradients in place on the way; here they are only read.
 class TrainerTail {
 public:
     TrainerTail(Optimizer &optimizer, TensorList &params, TensorList &accum)
@@ -546,25 +566,37 @@ public:
     uint64_t step() const { return step_; }
     double loss_scale() { return scaler_ ? scaler_->scale_factor() : 1.0; } // trainer.rs:218-221
 
-    // returns true if the optimizer stepped; grads are modified in place like the reference's
+    // returns true if the optimizer stepped
     bool after_backward(TensorList &grads)
     {
         if (grad_accum_ == 1 && !(scaler_ && has_policy_)) return fused(grads);
-        if (scaler_ && !scaler_->unscale_and_update(grads)) return drop(); // :230-237
-        if (has_policy_ && has_non_finite(grads)) {                        // :239-251
-            if (policy_ == GradNanPolicy::Skip) return drop();
-            throw TrainError("non-finite gradient");
-        }
         if (accum_count_ == 0 && dirty_) { // a dropped accumulation starts again from zeros (:253-260)
             zero_grad(accum_);
             dirty_ = false;
         }
-        accumulate(accum_, grads); // :262-266
-        dirty_ = true;
+        double sumsq = -1.0;
+        if (scaler_ && has_policy_) {
+            // both decisions, in the reference's order: a micro-batch whose unscaled gradients
+            // overflow is the nan policy's, not the scaler's
+            if (!scaler_->unscale_and_update(grads)) return drop(); // :230-237
+            if (has_non_finite(grads)) {                            // :239-251
+                if (policy_ == GradNanPolicy::Skip) return drop();
+                throw TrainError("non-finite gradient");
+            }
+            accumulate(accum_, grads); // :262-266
+            dirty_ = true;
+        } else {
+            dirty_ = true; // a non-finite micro-batch leaves garbage in the buffer
+            if (!unscale_accumulate(accum_, grads, scaler_, &sumsq, has_policy_)) {
+                if (!scaler_ && policy_ == GradNanPolicy::Stop) throw TrainError("non-finite gradient");
+                return drop();
+            }
+        }
         accum_count_ += 1;
         if (accum_count_ < grad_accum_) return false;
         if (has_schedule_) opt_.set_lr(lr_at_step(schedule_, base_lr_, step_)); // :270-273
-        opt_.fused_step(params_, accum_, nullptr, grad_clip_, /*zero_grads=*/true); // :274-290
+        if (sumsq < 0.0) opt_.fused_step(params_, accum_, nullptr, grad_clip_, /*zero_grads=*/true); // :274-290
+        else opt_.fused_step_norm(params_, accum_, sumsq, grad_clip_, /*zero_grads=*/true);
         accum_count_ = 0;
         dirty_ = false;
         step_ += 1;

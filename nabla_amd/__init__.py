@@ -13,6 +13,6 @@ multi-tensor launches.
 from . import _lib  # noqa: F401
 from .optim import (Adam, AdamW, GradScaler, GradScalerState, NablaPanic, OptimMeta,  # noqa: F401
                     OptimStateError, Sgd, TensorList, accumulate, clip_grad_norm, has_non_finite,
-                    scale_grad, sync, zero_grad)
+                    scale_grad, sync, unscale_accumulate, zero_grad)
 
 __version__ = "0.1.0"

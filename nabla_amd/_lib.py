@@ -34,6 +34,8 @@ KIND_ADAMW, KIND_ADAM, KIND_SGD = 0, 1, 2
 
 STEP_ZERO_GRADS = 1
 STEP_SKIP_NONFINITE = 2
+ACC_CHECK_FINITE = 1
+ACC_WRITE_GRADS = 2
 
 
 class Meta(C.Structure):
@@ -109,6 +111,8 @@ SYMBOLS = {
     "nbo_fused_step_groups": (C.c_int, [C.c_uint64, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), _P, _P,
                                         C.c_double, C.c_uint32]),
     "nbo_accumulate": (C.c_int, [_P, _P, C.c_int]),
+    "nbo_unscale_accumulate": (C.c_int, [_P, _P, _P, C.c_uint32, C.POINTER(C.c_int), C.POINTER(C.c_double)]),
+    "nbo_fused_step_norm": (C.c_int, [_P, _P, _P, C.c_double, C.c_double, C.c_uint32]),
     "nbo_backend_apply": (C.c_int, [C.c_int, _P, _P, _P, C.c_double]),
     "nbo_backend_cast": (C.c_int, [_P, _P]),
     "nbo_optim_last_step": (C.c_int, [_P, C.POINTER(StepInfo)]),

@@ -807,23 +807,87 @@ int nbo_fused_step_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *c
     });
 }
 
+// The asserts of the accumulation `&buf[i] + g` (trainer.rs:262-266 -> tensor/ops.rs add).
+static void check_accum_args(const nbo_list *accum, const nbo_list *grads)
+{
+    require(accum && grads, NBO_ERR_ARG, "null list");
+    if (accum->layout.nt() != grads->layout.nt())
+        fail(NBO_ERR_LEN_MISMATCH, "nabla-train: accumulation buffers / grads length mismatch");
+    for (uint64_t t = 0; t < accum->layout.nt(); t++)
+        if (accum->layout.rows[t] != grads->layout.rows[t] || accum->layout.cols[t] != grads->layout.cols[t])
+            fail(NBO_ERR_SHAPE, "nabla: add -- shapes are not broadcast-compatible (tensor " +
+                                    std::to_string(t) + ")");
+    require(accum->dtype == grads->dtype, NBO_ERR_DTYPE, "lists differ in element type");
+}
+
 int nbo_accumulate(nbo_list *accum, nbo_list *grads, int zero_grads)
 {
     return guarded([&] {
-        require(accum && grads, NBO_ERR_ARG, "null list");
-        if (accum->layout.nt() != grads->layout.nt())
-            fail(NBO_ERR_LEN_MISMATCH, "nabla-train: accumulation buffers / grads length mismatch");
-        for (uint64_t t = 0; t < accum->layout.nt(); t++)
-            if (accum->layout.rows[t] != grads->layout.rows[t] || accum->layout.cols[t] != grads->layout.cols[t])
-                fail(NBO_ERR_SHAPE, "nabla: add -- shapes are not broadcast-compatible (tensor " +
-                                        std::to_string(t) + ")");
-        require(accum->dtype == grads->dtype, NBO_ERR_DTYPE, "lists differ in element type");
+        check_accum_args(accum, grads);
         NboAccumArgs a = {};
         a.L = accum->layout.dev;
         a.a_ptrs = accum->ptrs_dev;
         a.b_ptrs = grads->ptrs_dev;
         a.zero_b = zero_grads ? 1u : 0u;
         Runtime::get().launch(kernel_for(K_ACCUM_BASE, K_ACCUM_F16, accum->dtype), accum->layout.nchunks, NBO_BLOCK, a);
+    });
+}
+
+int nbo_unscale_accumulate(nbo_scaler *scaler, nbo_list *accum, nbo_list *grads, uint32_t flags, int *ok,
+                           double *accum_sumsq)
+{
+    return guarded([&] {
+        check_accum_args(accum, grads);
+        require(ok != nullptr, NBO_ERR_ARG, "null output");
+        Runtime &rt = Runtime::get();
+        NboAccNormArgs a = {};
+        a.L = accum->layout.dev;
+        a.acc_ptrs = accum->ptrs_dev;
+        a.g_ptrs = grads->ptrs_dev;
+        a.scaler = scaler ? scaler->dev : nullptr;
+        a.partial_sumsq = rt.partial_sumsq();
+        a.partial_flag = rt.partial_flag();
+        a.grid = norm_grid(accum->layout);
+        a.write_grads = (flags & NBO_ACC_WRITE_GRADS) ? 1u : 0u;
+        rt.launch(kernel_for(K_ACCNORM_BASE, K_ACCNORM_F16, accum->dtype), a.grid, NBO_BLOCK, a);
+        NboFinalizeArgs f = {};
+        f.partial_sumsq = rt.partial_sumsq();
+        f.partial_flag = rt.partial_flag();
+        f.grid = a.grid;
+        f.check_finite = (scaler || (flags & NBO_ACC_CHECK_FINITE)) ? 1u : 0u;
+        f.scaler = scaler ? scaler->dev : nullptr;
+        f.gf = rt.gf_scratch();
+        rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
+        if (a.write_grads && f.check_finite) launch_scale(grads, rt.gf_scratch(), 1.0, 4);
+        NboGradFactors g;
+        rt.read_back(&g, rt.gf_scratch(), sizeof(g));
+        *ok = g.found_inf ? 0 : 1;
+        if (accum_sumsq) *accum_sumsq = g.sumsq;
+    });
+}
+
+int nbo_fused_step_norm(nbo_optim *opt, nbo_list *params, nbo_list *grads, double max_norm, double sumsq,
+                        uint32_t flags)
+{
+    return guarded([&] {
+        check_step_args(opt, params, grads);
+        require(sumsq >= 0.0, NBO_ERR_ARG, "the sum of squares is negative or NaN");
+        Runtime &rt = Runtime::get();
+        NboFinalizeArgs f = {};
+        f.partial_sumsq = rt.partial_sumsq();
+        f.partial_flag = rt.partial_flag();
+        f.grid = 0; // nothing to reduce: the sum of squares comes with the call
+        f.use_sumsq_in = 1;
+        f.sumsq_in = sumsq;
+        f.gf = opt->gf;
+        f.opt = opt->dev;
+        f.trace = opt->trace;
+        f.max_norm = max_norm;
+        f.hyper = hyper_of(opt);
+        rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
+        const NboUpdateArgs a =
+            update_args(opt, params, grads, true, (flags & NBO_STEP_ZERO_GRADS) != 0);
+        rt.launch(update_kernel(opt, params), opt->layout.nchunks, NBO_BLOCK, a);
     });
 }
 

@@ -44,7 +44,8 @@ static const char *const kKernelNames[K_COUNT] = {
     "nbo_update_f16_adamw",  "nbo_update_f16_adam",  "nbo_update_f16_sgd",
     "nbo_update_pf16_adamw", "nbo_update_pf16_adam", "nbo_update_pf16_sgd",
     "nbo_norm_f16",          "nbo_norm_pf16",        "nbo_scale_f16",
-    "nbo_accum_f16",         "nbo_ew_f16",
+    "nbo_accum_f16",         "nbo_ew_f16",           "nbo_accnorm_f32",
+    "nbo_accnorm_bf16",      "nbo_accnorm_f64",      "nbo_accnorm_f16",
 };
 
 Runtime &Runtime::get()

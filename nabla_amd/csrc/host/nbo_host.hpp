@@ -56,7 +56,9 @@ enum KernelId {
     K_SCALE_F16 = 40,
     K_ACCUM_F16 = 41,
     K_EW_F16 = 42,
-    K_COUNT = 43
+    K_ACCNORM_BASE = 43, // + st (f32 / bf16 / f64)
+    K_ACCNORM_F16 = 46,
+    K_COUNT = 47
 };
 
 // Process-wide runtime: device 0, the loaded module, the stream, scratch buffers.

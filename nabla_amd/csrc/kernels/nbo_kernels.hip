@@ -773,11 +773,12 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_finalize(const NboFi
         acc = acc + a.partial_sumsq[i];
         bad |= a.partial_flag[i];
     }
-    const double sumsq = block_sum(acc, lds_d);
+    const double reduced = block_sum(acc, lds_d);
     const uint32_t any_bad = block_or(bad, lds_u);
     if (tid != 0) return;
 
     NboGradFactors f;
+    const double sumsq = a.use_sumsq_in ? a.sumsq_in : reduced;
     f.sumsq = sumsq;
     const bool found = a.check_finite && any_bad;
     double inv = 1.0;
@@ -838,6 +839,9 @@ template <int ST> DEV void scale_body(const NboScaleArgs &a)
         } else if (a.mode == 1) {
             if (!a.gf->clipped) return; // trainer.rs:515: untouched when norm <= max_norm
             f = sizeof(T) == 4 ? (T)a.gf->clip32 : (T)a.gf->clip64;
+        } else if (a.mode == 4) {
+            if (!a.gf->found_inf) return; // core.rs:372-375 alone: zeros on a non-finite gradient
+            zero = true;
         }
     }
     const bool vec_ok = (((uintptr_t)pg) & (VEC * SB - 1)) == 0;
@@ -912,6 +916,75 @@ NBO_ACCUM_KERNEL(nbo_accum_f32, NBO_F32)
 NBO_ACCUM_KERNEL(nbo_accum_bf16, NBO_BF16)
 NBO_ACCUM_KERNEL(nbo_accum_f64, NBO_F64)
 NBO_ACCUM_KERNEL(nbo_accum_f16, NBO_F16)
+
+// One micro-batch of the accumulating Trainer in one pass (trainer.rs:230-267): the finite
+// scan of GradScaler::unscale_and_update over g (core.rs:357-368), u = g * T(1 / scale)
+// (core.rs:376-380), buf = buf + u (trainer.rs:262-266), and the first stage of the sum of
+// squares of the new buf, which clip_grad_norm needs once the last micro-batch is in
+// (trainer.rs:504-513).  Same fixed grid, chunk striding and reduction as the norm pass.  On
+// a non-finite gradient buf receives garbage: the Trainer discards the accumulation then.
+template <int ST> DEV void accnorm_body(const NboAccNormArgs &a)
+{
+    typedef typename Traits<ST>::T T;
+    enum { SB = Traits<ST>::SBYTES, VEC = Traits<ST>::VEC };
+    __shared__ double lds_d[NBO_BLOCK / 64];
+    __shared__ uint32_t lds_u[NBO_BLOCK / 64];
+    const uint32_t tid = threadIdx.x;
+    const T inv = a.scaler ? (T)(1.0 / a.scaler->scale) : (T)1; // core.rs:355
+    const bool write_g = a.write_grads != 0;
+    double acc = 0.0;
+    uint32_t bad = 0;
+
+    for (uint32_t ci = blockIdx.x; ci < a.L.nchunks; ci += a.grid) {
+        const ChunkRef c = chunk_ref(a.L, ci);
+        char *pa = (char *)a.acc_ptrs[c.t] + c.base * SB;
+        char *pg = (char *)a.g_ptrs[c.t] + c.base * SB;
+        const bool vec_ok = ((((uintptr_t)pa) | ((uintptr_t)pg)) & 15u) == 0;
+        const uint32_t nvec = vec_ok ? c.cnt / VEC : 0;
+        for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
+            const uint64_t off = (uint64_t)q * VEC * SB;
+            T g[VEC], b[VEC];
+            IO<ST>::ldv(pg + off, g);
+            IO<ST>::ldv(pa + off, b);
+#pragma unroll
+            for (int k = 0; k < VEC; k++) {
+                bad |= (uint32_t)nonfinite<ST>(g[k]);
+                g[k] = g[k] * inv;
+                b[k] = b[k] + g[k];
+                acc = sq_acc<ST>(acc, b[k]);
+            }
+            IO<ST>::stv(pa + off, b);
+            if (write_g) IO<ST>::stv(pg + off, g);
+        }
+        for (uint32_t e = nvec * VEC + tid; e < c.cnt; e += NBO_BLOCK) {
+            const uint64_t off = (uint64_t)e * SB;
+            const T g = IO<ST>::ld1(pg + off);
+            bad |= (uint32_t)nonfinite<ST>(g);
+            const T u = g * inv;
+            const T b = IO<ST>::ld1(pa + off) + u;
+            acc = sq_acc<ST>(acc, b);
+            IO<ST>::st1(pa + off, b);
+            if (write_g) IO<ST>::st1(pg + off, u);
+        }
+    }
+    const double bs = block_sum(acc, lds_d);
+    const uint32_t bo = block_or(bad, lds_u);
+    if (tid == 0) {
+        a.partial_sumsq[blockIdx.x] = bs;
+        a.partial_flag[blockIdx.x] = bo;
+    }
+}
+
+#define NBO_ACCNORM_KERNEL(name, ST)                                                        \
+    extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboAccNormArgs a)    \
+    {                                                                                       \
+        accnorm_body<ST>(a);                                                                \
+    }
+// 16-bit lists: unscale and add in the lists' own type, as the in-place passes do
+NBO_ACCNORM_KERNEL(nbo_accnorm_f32, NBO_F32)
+NBO_ACCNORM_KERNEL(nbo_accnorm_bf16, NBO_PBF16)
+NBO_ACCNORM_KERNEL(nbo_accnorm_f64, NBO_F64)
+NBO_ACCNORM_KERNEL(nbo_accnorm_f16, NBO_PF16)
 
 // ---------------------------------------------------------------------------------
 // Master-weight casts: arena f32 <- bf16 / f16 tensors (exact widening) and

@@ -157,6 +157,9 @@ struct NboFinalizeArgs {
     NboTraceDev *trace;    // may be null
     double max_norm;       // <= 0 disables clipping (trainer.rs:501-503)
     NboHyper hyper;        // copied into *opt before the scalars are derived
+    double sumsq_in;       // with use_sumsq_in: the sum of squares, already known (grid = 0)
+    uint32_t use_sumsq_in;
+    uint32_t pad;
 };
 
 struct NboPrepArgs {
@@ -165,6 +168,19 @@ struct NboPrepArgs {
     const NboScalerDev *scaler; // may be null; only read, for the trace entry
     NboTraceDev *trace;         // may be null
     NboHyper hyper;
+};
+
+// One micro-batch of the accumulating Trainer in a single pass (trainer.rs:230-267): finite
+// scan of g, acc[i] = acc[i] + T(g[i] * inv_scale), and the sum of squares of the new acc.
+struct NboAccNormArgs {
+    NboLayoutDev L;
+    const uint64_t *acc_ptrs;
+    const uint64_t *g_ptrs;
+    const NboScalerDev *scaler; // null: no unscale, inv_scale = 1
+    double *partial_sumsq;      // [grid]
+    uint32_t *partial_flag;     // [grid]
+    uint32_t grid;
+    uint32_t write_grads;       // also store the unscaled gradients in place, as the reference does
 };
 
 // a[i] = a[i] + b[i] over two lists of the same shapes (gradient accumulation).

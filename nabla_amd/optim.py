@@ -359,6 +359,15 @@ class _Optimizer:
         _call(_lib.load().nbo_fused_step(self._handle(), scaler._handle() if scaler else None,
                                          p._h, g._h, float(max_norm), flags))
 
+    def fused_step_norm(self, params, grads, sumsq: float, max_norm: float = 0.0,
+                        zero_grads: bool = False) -> None:
+        """clip_grad_norm + step (+ zeroing) over gradients whose sum of squares is already
+        known (from `unscale_accumulate`), without another norm pass (trainer.rs:274-290)."""
+        p = self._cache.get("p", params)
+        g = self._cache.get("g", grads)
+        _call(_lib.load().nbo_fused_step_norm(self._handle(), p._h, g._h, float(max_norm), float(sumsq),
+                                              STEP_ZERO_GRADS if zero_grads else 0))
+
     def last_step(self) -> _lib.StepInfo:
         info = _lib.StepInfo()
         _call(_lib.load().nbo_optim_last_step(self._handle(), C.byref(info)))
@@ -676,6 +685,22 @@ def accumulate(accum, grads, zero_grads: bool = False) -> None:
     a = _free_cache.get("accum_a", accum)
     g = _free_cache.get("accum_g", grads)
     _call(_lib.load().nbo_accumulate(a._h, g._h, int(zero_grads)))
+
+
+def unscale_accumulate(accum, grads, scaler: Optional["GradScaler"] = None, check_finite: bool = False,
+                       write_grads: bool = False) -> Tuple[bool, float]:
+    """One micro-batch of the accumulating Trainer in a single pass (trainer.rs:230-267):
+    finite scan + loss-scale update, buf[i] = &buf[i] + g / scale, and the sum of squares of
+    the new buffer.  Returns (ok, sumsq); on ok == False the buffer holds garbage (the
+    Trainer discards the accumulation then).  The gradients stay as they were unless
+    `write_grads` asks for the reference's in-place result."""
+    a = _free_cache.get("accum_a", accum)
+    g = _free_cache.get("accum_g", grads)
+    ok, sumsq = C.c_int(0), C.c_double(0.0)
+    flags = (_lib.ACC_CHECK_FINITE if check_finite else 0) | (_lib.ACC_WRITE_GRADS if write_grads else 0)
+    _call(_lib.load().nbo_unscale_accumulate(scaler._handle() if scaler else None, a._h, g._h, flags,
+                                             C.byref(ok), C.byref(sumsq)))
+    return bool(ok.value), sumsq.value
 
 
 def sync() -> None:

@@ -14,10 +14,11 @@ Per micro-batch, in the reference's order:
 With `grad_accum == 1` and at most one of scaler / nan policy, steps 1-4 are one
 `fused_step` (three launches, the skip decided on the device); the decision is read back
 afterwards only because `state.step` -- which the schedule is a function of -- must not
-advance on a skipped step.  Otherwise the unfused entry points run steps 1-3 in the order
-above, with the reference's synchronous decisions after steps 1 and 2, and step 4 is one
-`fused_step` over the accumulation buffer (norm pass, then clip + update + zeroing in one
-kernel) instead of the reference's four passes.
+advance on a skipped step.  With accumulation, steps 1-3 are one pass over the gradients
+(`unscale_accumulate`: finite scan, unscale, add into the buffer, and the buffer's sum of
+squares for the clip) with the reference's synchronous decision after it, and step 4 is
+clip + update + zeroing in one kernel (`fused_step_norm`); with a scaler *and* a nan policy
+the two decisions stay separate entry points in the reference's order.
 """
 from __future__ import annotations
 
@@ -85,8 +86,9 @@ class TrainerTail:
 
     # -- one micro-batch -------------------------------------------------------------------
     def after_backward(self, grads: Sequence) -> bool:
-        """Consume one micro-batch's gradients (modified in place like the reference's);
-        returns True if the optimizer stepped."""
+        """Consume one micro-batch's gradients; returns True if the optimizer stepped.  The
+        reference unscales the gradients in place on the way; here they are only read (nothing
+        uses them afterwards), except on the path with both a scaler and a nan policy."""
         grads = grads if isinstance(grads, nb.TensorList) else list(grads)
         fusable = self.state.grad_accum == 1 and not (self.scaler and self.nan_policy)
         if fusable:
@@ -117,23 +119,41 @@ class TrainerTail:
     def _unfused(self, grads) -> bool:
         import torch
 
-        if self.scaler is not None and not self.scaler.unscale_and_update(grads):
-            return self._drop()
-        if self.nan_policy is not None and nb.has_non_finite(grads):
-            if self.nan_policy is GradNanPolicy.SKIP:
-                return self._drop()
-            raise TrainError("non-finite gradient")
         tensors = grads.tensors if isinstance(grads, nb.TensorList) else grads
-        if self._accum is None:
+        fresh = self._accum is None
+        if fresh:
             self._accum = [torch.zeros_like(g) for g in tensors]
-        nb.accumulate(self._accum, grads)
+        if self.scaler is not None and self.nan_policy is not None:
+            # both decisions, in the reference's order: a micro-batch whose unscaled gradients
+            # overflow is the nan policy's, not the scaler's
+            if not self.scaler.unscale_and_update(grads):
+                return self._drop()
+            if nb.has_non_finite(grads):
+                if self.nan_policy is GradNanPolicy.SKIP:
+                    return self._drop()
+                raise TrainError("non-finite gradient")
+            nb.accumulate(self._accum, grads)
+            sumsq = None
+        else:
+            # steps 1-3 in one pass over the gradients; a non-finite micro-batch leaves garbage
+            # in the buffer, which is dropped with it
+            ok, sumsq = nb.unscale_accumulate(self._accum, grads, scaler=self.scaler,
+                                              check_finite=self.nan_policy is not None)
+            if not ok:
+                if self.scaler is None and self.nan_policy is GradNanPolicy.STOP:
+                    raise TrainError("non-finite gradient")
+                return self._drop()
         self._accum_count += 1
         if self._accum_count < self.state.grad_accum:
             return False
         self._set_lr()
         # clip_grad_norm, step and the re-zeroing of the buffer (:274-290)
-        self.optimizer.fused_step(self.params, self._accum, scaler=None, max_norm=self.grad_clip or 0.0,
-                                  zero_grads=True)
+        if sumsq is None:
+            self.optimizer.fused_step(self.params, self._accum, scaler=None, max_norm=self.grad_clip or 0.0,
+                                      zero_grads=True)
+        else:
+            self.optimizer.fused_step_norm(self.params, self._accum, sumsq, max_norm=self.grad_clip or 0.0,
+                                           zero_grads=True)
         self._accum_count = 0
         self.state.step += 1
         return True

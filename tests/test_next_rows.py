@@ -239,6 +239,105 @@ def test_accumulate_matches_add(gpu):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16", "f64"])
+def test_unscale_accumulate_is_unscale_then_accumulate_in_one_pass(gpu, dtype):
+    """nbo_unscale_accumulate against nbo_scaler_unscale_and_update + nbo_accumulate and against
+    the oracle's unscale / add: same buffer, same gradients written back, same decision and
+    loss-scale sequence, and a sum of squares that is the clip's norm squared."""
+    from tests import helpers as H
+
+    shapes = [(1, 5), (3, 2741), (1, 8193), (0, 4), (2, 8192), (1, 16391)]
+    np_t = {"f32": np.float32, "f64": np.float64}.get(dtype)
+
+    def conv(arrs):
+        return H.narrow_list(arrs, dtype) if np_t is None else [a.astype(np_t) for a in arrs]
+
+    scale0 = 3.0 * 512.0  # T(1 / scale) is inexact
+    fused_scaler, plain_scaler = nb.GradScaler.new(), nb.GradScaler.new()
+    for sc in (fused_scaler, plain_scaler):
+        sc.load_state(nb.GradScalerState(scale0, 2.0, 0.5, 2, 0))
+    ref_scaler = O.ScalerState(scale0, 2.0, 0.5, 2, 0)
+    buf0 = conv(H.randn_list(shapes, 40, 0.5))
+    fused_buf, plain_buf, ref_buf = H.dev_list(buf0, shapes), H.dev_list(buf0, shapes), H.copy_list(buf0)
+    for k in range(5):
+        g = conv([a * np.float32(ref_scaler.scale) for a in H.randn_list(shapes, 50 + k, 1e-2)])
+        if k == 2:
+            g[4].reshape(-1).view(np.uint16 if g[4].itemsize == 2 else g[4].dtype)[9000] = \
+                {2: 0x7F80 if dtype == "bf16" else 0x7C00}.get(g[4].itemsize, np.inf)
+        fused_g, plain_g = H.dev_list(g, shapes), H.dev_list(g, shapes)
+        ok, sumsq = nb.unscale_accumulate(fused_buf, fused_g, scaler=fused_scaler, write_grads=True)
+        plain_ok = plain_scaler.unscale_and_update(plain_g)
+        ref_g = H.copy_list(g)
+        assert ok == plain_ok == O.scaler_unscale_and_update(ref_scaler, ref_g), k
+        assert fused_scaler.state().scale == plain_scaler.state().scale == ref_scaler.scale, k
+        H.assert_bits_equal(H.host_list(fused_g), ref_g, f"gradients written back, micro-batch {k}")
+        H.assert_bits_equal(H.host_list(plain_g), ref_g, f"in-place unscale, micro-batch {k}")
+        if not ok:  # the Trainer drops the accumulation: start again from the same buffer
+            fused_buf = H.dev_list(ref_buf, shapes)
+            continue
+        nb.accumulate(plain_buf, plain_g)
+        ref_buf = [O.add(b, x) for b, x in zip(ref_buf, ref_g)]
+        H.assert_bits_equal(H.host_list(fused_buf), ref_buf, f"buffer, micro-batch {k}")
+        H.assert_bits_equal(H.host_list(plain_buf), ref_buf, f"two-pass buffer, micro-batch {k}")
+        norm = O.clip_grad_norm(H.copy_list(ref_buf), 1e30)  # far above the norm: nothing is scaled
+        assert abs(np.sqrt(sumsq) - norm) <= 1e-13 * norm, k
+    # without write_grads the gradients stay as they were; without a scaler nothing is unscaled
+    g = conv(H.randn_list(shapes, 70, 1e-2))
+    g_dev = H.dev_list(g, shapes)
+    ok, _ = nb.unscale_accumulate(fused_buf, g_dev)
+    assert ok
+    H.assert_bits_equal(H.host_list(g_dev), g, "gradients untouched")
+    H.assert_bits_equal(H.host_list(fused_buf), [O.add(b, x) for b, x in zip(ref_buf, g)], "plain accumulation")
+    g[1][5] = np.nan if g[1].itemsize != 2 or dtype == "f16" else 0x7FC0
+    assert nb.unscale_accumulate(fused_buf, H.dev_list(g, shapes))[0]            # nobody asked
+    assert not nb.unscale_accumulate(fused_buf, H.dev_list(g, shapes), check_finite=True)[0]
+    with pytest.raises(nb.NablaPanic):
+        nb.unscale_accumulate(fused_buf, g_dev[:2])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["f32", "mixed", "bf16"])
+def test_fused_step_with_a_known_norm_equals_the_fused_step(gpu, mode):
+    """nbo_fused_step_norm fed with the sum of squares nbo_unscale_accumulate returned for the
+    buffer: same parameters, moments, step record and zeroed buffer as nbo_fused_step, which
+    runs the norm pass itself."""
+    import torch
+
+    from tests import helpers as H
+
+    shapes = [(3, 5), (1, 9001), (129, 257), (1, 8192)]
+    half = {"mixed": "bf16", "bf16": "bf16"}.get(mode)
+    conv = (lambda arrs: H.narrow_list(arrs, half)) if half else (lambda arrs: arrs)
+    p0, g = conv(H.randn_list(shapes, 90, 0.02)), conv(H.randn_list(shapes, 91, 1e-2))
+
+    def fresh():
+        o = nb.AdamW.new(1e-3, shapes, master=mode == "mixed", dtype="bf16" if mode == "bf16" else "f32") \
+            .beta2(0.95).weight_decay(0.1)
+        p = H.dev_list(p0, shapes)
+        if mode == "mixed":
+            o.master_from_params(p)
+        return o, p
+
+    (o1, p1), (o2, p2) = fresh(), fresh()
+    for step in range(3):
+        buf1 = [torch.zeros_like(t) for t in H.dev_list(g, shapes)]
+        ok, sumsq = nb.unscale_accumulate(buf1, H.dev_list(g, shapes))
+        assert ok
+        buf2 = [b.clone() for b in buf1]
+        o1.fused_step_norm(p1, buf1, sumsq, max_norm=0.05, zero_grads=True)
+        o2.fused_step(p2, buf2, max_norm=0.05, zero_grads=True)
+        a, b = o1.last_step(), o2.last_step()
+        assert (a.norm, a.clipped, a.step_count, a.found_inf) == (b.norm, b.clipped, b.step_count, b.found_inf)
+        assert a.clipped == 1 and a.step_count == step + 1
+        assert not any(t.any() for t in H.host_list(buf1))
+    H.assert_bits_equal(H.host_list(p1), H.host_list(p2), "params")
+    for x, y in zip(o1.moments(), o2.moments()):
+        H.assert_bits_equal(H.host_list(x), H.host_list(y), "moments")
+    with pytest.raises(Exception, match="negative or NaN"):
+        o1.fused_step_norm(p1, buf1, float("nan"), max_norm=0.05)
+
+
+@pytest.mark.gpu
 def test_checkpoint_round_trip_restores_bit_identical_training(gpu, tmp_path):
     """Train 3 steps, save, restore into fresh objects, train 2 more on both: identical bits."""
     from tests import helpers as H
