@@ -15,6 +15,8 @@
 //   nbo_cast_*      bf16 / f16 <-> f32 casts (common/scalar/mod.rs:338-344), casts between lists
 //   nbo_ew_*        the Backend primitives as single passes (nabla-core/src/cpu/mod.rs:211-272)
 //   nbo_accum_*     gradient accumulation buf += g (trainer.rs:253-267)
+//   nbo_accnorm_*   a whole micro-batch of the accumulating Trainer in one pass: finite scan,
+//                   unscale, accumulate, first stage of the buffer's sum of squares (trainer.rs:230-267)
 //
 // Numerics contract: every arithmetic operation of the reference is one IEEE
 // round-to-nearest operation here, in the same order, never contracted into an
