@@ -162,6 +162,21 @@ public:
                                     scaler ? scaler->handle() : nullptr, all_grads_->handle(), max_norm,
                                     zero_grads ? NBO_STEP_ZERO_GRADS : 0u));
     }
+    // the same over gradients whose sum of squares is already known (nbo_unscale_accumulate)
+    void fused_step_norm(const std::vector<Tensor> &params, const std::vector<Tensor> &grads, double sumsq,
+                         double max_norm, bool zero_grads = false)
+    {
+        bind(params, grads);
+        std::vector<nbo_optim *> opts;
+        std::vector<nbo_list *> pl, gl;
+        for (Entry &g : groups_) {
+            opts.push_back(g.optimizer->handle());
+            pl.push_back(g.params->handle());
+            gl.push_back(g.grads->handle());
+        }
+        check(nbo_fused_step_groups_norm(groups_.size(), opts.data(), pl.data(), gl.data(), max_norm, sumsq,
+                                         zero_grads ? NBO_STEP_ZERO_GRADS : 0u));
+    }
     void reset()
     {
         for (Entry &g : groups_) g.optimizer->reset();

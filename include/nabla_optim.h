@@ -236,6 +236,10 @@ int nbo_unscale_accumulate(nbo_scaler *scaler, nbo_list *accum, nbo_list *grads,
  * finite check: both belong to the micro-batches.  Asynchronous. */
 int nbo_fused_step_norm(nbo_optim *opt, nbo_list *params, nbo_list *grads, double max_norm, double sumsq,
                         uint32_t flags);
+/* The same for GroupOptimizer (optim/groups.rs:269-293): `sumsq` is that of all the groups'
+ * gradients together.  Asynchronous. */
+int nbo_fused_step_groups_norm(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,
+                               nbo_list *const *grads, double max_norm, double sumsq, uint32_t flags);
 /* ---- Backend primitives on tensor lists ------------------------------------------------
  * The single passes the reference's optimizers are chains of, as multi-tensor launches:
  * BackendCore::{scale, axpy_inplace, add, zeros, clone_storage}

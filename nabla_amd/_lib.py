@@ -113,6 +113,8 @@ SYMBOLS = {
     "nbo_accumulate": (C.c_int, [_P, _P, C.c_int]),
     "nbo_unscale_accumulate": (C.c_int, [_P, _P, _P, C.c_uint32, C.POINTER(C.c_int), C.POINTER(C.c_double)]),
     "nbo_fused_step_norm": (C.c_int, [_P, _P, _P, C.c_double, C.c_double, C.c_uint32]),
+    "nbo_fused_step_groups_norm": (C.c_int, [C.c_uint64, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P),
+                                             C.c_double, C.c_double, C.c_uint32]),
     "nbo_backend_apply": (C.c_int, [C.c_int, _P, _P, _P, C.c_double]),
     "nbo_backend_cast": (C.c_int, [_P, _P]),
     "nbo_optim_last_step": (C.c_int, [_P, C.POINTER(StepInfo)]),

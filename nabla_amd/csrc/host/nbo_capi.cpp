@@ -762,23 +762,49 @@ int nbo_fused_step(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, nbo_lis
     });
 }
 
+// Argument checks shared by the two group entry points; returns how many tensors the groups cover.
+static uint64_t check_group_args(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,
+                                 nbo_list *const *grads, int grads_dtype)
+{
+    require(n_groups == 0 || (opts && params && grads), NBO_ERR_ARG, "null group arrays");
+    uint64_t covered = 0;
+    for (uint64_t g = 0; g < n_groups; g++) {
+        check_step_args(opts[g], params[g], grads[g]);
+        require(grads[g]->dtype == grads_dtype, NBO_ERR_DTYPE,
+                "group gradients differ in element type from the whole list");
+        require(pure_half(opts[g]) == pure_half(opts[0]), NBO_ERR_DTYPE,
+                "groups mix bf16 and f32 optimizer state");
+        covered += grads[g]->layout.nt();
+    }
+    return covered;
+}
+
+// Each group's scalars and update from the one decision in the runtime's scratch.
+static void launch_group_updates(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,
+                                 nbo_list *const *grads, nbo_scaler *scaler, uint32_t flags)
+{
+    Runtime &rt = Runtime::get();
+    for (uint64_t g = 0; g < n_groups; g++) {
+        NboPrepArgs p = {};
+        p.opt = opts[g]->dev;
+        p.gf = rt.gf_scratch();
+        p.scaler = scaler ? scaler->dev : nullptr;
+        p.trace = opts[g]->trace;
+        p.hyper = hyper_of(opts[g]);
+        rt.launch(K_PREP, 1, 64, p);
+        const NboUpdateArgs a = update_args(opts[g], params[g], grads[g], true,
+                                            (flags & NBO_STEP_ZERO_GRADS) != 0, rt.gf_scratch());
+        rt.launch(update_kernel(opts[g], params[g]), opts[g]->layout.nchunks, NBO_BLOCK, a);
+    }
+}
+
 int nbo_fused_step_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,
                           nbo_list *const *grads, nbo_scaler *scaler, nbo_list *all_grads,
                           double max_norm, uint32_t flags)
 {
     return guarded([&] {
-        require(n_groups == 0 || (opts && params && grads), NBO_ERR_ARG, "null group arrays");
         require(all_grads != nullptr, NBO_ERR_ARG, "null gradient list");
-        uint64_t covered = 0;
-        for (uint64_t g = 0; g < n_groups; g++) {
-            check_step_args(opts[g], params[g], grads[g]);
-            require(grads[g]->dtype == all_grads->dtype, NBO_ERR_DTYPE,
-                    "group gradients differ in element type from the whole list");
-            require(pure_half(opts[g]) == pure_half(opts[0]), NBO_ERR_DTYPE,
-                    "groups mix bf16 and f32 optimizer state");
-            covered += grads[g]->layout.nt();
-        }
-        if (covered != all_grads->layout.nt())
+        if (check_group_args(n_groups, opts, params, grads, all_grads->dtype) != all_grads->layout.nt())
             fail(NBO_ERR_COUNT_MISMATCH, "nabla-train: GroupOptimizer param count mismatch");
         Runtime &rt = Runtime::get();
         // one decision for all groups: the reference unscales and clips the whole
@@ -792,18 +818,27 @@ int nbo_fused_step_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *c
         f.gf = rt.gf_scratch();
         f.max_norm = max_norm;
         rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
-        for (uint64_t g = 0; g < n_groups; g++) {
-            NboPrepArgs p = {};
-            p.opt = opts[g]->dev;
-            p.gf = rt.gf_scratch();
-            p.scaler = scaler ? scaler->dev : nullptr;
-            p.trace = opts[g]->trace;
-            p.hyper = hyper_of(opts[g]);
-            rt.launch(K_PREP, 1, 64, p);
-            const NboUpdateArgs a = update_args(opts[g], params[g], grads[g], true,
-                                                (flags & NBO_STEP_ZERO_GRADS) != 0, rt.gf_scratch());
-            rt.launch(update_kernel(opts[g], params[g]), opts[g]->layout.nchunks, NBO_BLOCK, a);
-        }
+        launch_group_updates(n_groups, opts, params, grads, scaler, flags);
+    });
+}
+
+int nbo_fused_step_groups_norm(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,
+                               nbo_list *const *grads, double max_norm, double sumsq, uint32_t flags)
+{
+    return guarded([&] {
+        require(sumsq >= 0.0, NBO_ERR_ARG, "the sum of squares is negative or NaN");
+        check_group_args(n_groups, opts, params, grads, n_groups ? grads[0]->dtype : (int)NBO_DT_F32);
+        Runtime &rt = Runtime::get();
+        NboFinalizeArgs f = {};
+        f.partial_sumsq = rt.partial_sumsq();
+        f.partial_flag = rt.partial_flag();
+        f.grid = 0; // nothing to reduce: the sum of squares comes with the call
+        f.use_sumsq_in = 1;
+        f.sumsq_in = sumsq;
+        f.gf = rt.gf_scratch();
+        f.max_norm = max_norm;
+        rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
+        launch_group_updates(n_groups, opts, params, grads, nullptr, flags);
     });
 }
 

@@ -217,6 +217,21 @@ class GroupOptimizer:
         _call(_lib.load().nbo_fused_step_groups(n, opts, pl, gl, scaler._handle() if scaler else None,
                                                 self._all_grads._h, float(max_norm), flags))
 
+    def fused_step_norm(self, params, grads, sumsq: float, max_norm: float = 0.0,
+                        zero_grads: bool = False) -> None:
+        """clip + every group's step (+ zeroing) over gradients whose sum of squares is known."""
+        self._check(params, grads)
+        n = len(self._groups)
+        opts = (C.c_void_p * n)(*[g.optimizer._handle() for g in self._groups])
+        pl = (C.c_void_p * n)(*[self._lists(g, "p", params)._h for g in self._groups])
+        gl = (C.c_void_p * n)(*[self._lists(g, "g", grads)._h for g in self._groups])
+        _call(_lib.load().nbo_fused_step_groups_norm(n, opts, pl, gl, float(max_norm), float(sumsq),
+                                                     _lib.STEP_ZERO_GRADS if zero_grads else 0))
+
+    def last_step(self):
+        """Outcome of the most recent fused step (one decision for all groups)."""
+        return self._groups[0].optimizer.last_step()
+
     def reset(self) -> None:
         for g in self._groups:
             g.optimizer.reset()

@@ -165,3 +165,61 @@ def test_reference_checkpoint_roundtrip_with_schedule(gpu, tmp_path):
     assert schedule2 is not None and schedule2.base_lr == 0.1 and schedule2.schedule == Step(1, 0.9)
     assert [k for k, _ in params] == ["w", "b"] and float(params[0][1].reshape(-1)[0]) == 1.5
     assert scaler2.state().scale == 65536.0 and opt2.meta().lr == 0.1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("use_scaler", [False, True])
+def test_trainer_tail_drives_a_group_optimizer_with_accumulation(gpu, use_scaler):
+    """TrainerTail over a GroupOptimizer (no-decay group for biases and norms) with
+    grad_accum = 2: the one-pass micro-batch and the known-norm group step against the
+    separate entry points -- unscale, accumulate, then the grouped fused step, which is itself
+    checked against the oracle in test_next_rows -- on a second copy of everything."""
+    import torch
+
+    from nabla_amd import groups as G
+
+    names = ["embed", "l0.w", "l0.bias", "l0.norm", "l1.w", "head"]
+    shapes = [(50, 16), (16, 16), (1, 16), (1, 16), (16, 9000), (16, 50)]
+    p0 = H.randn_list(shapes, 4200, 0.02)
+    scale0 = 2048.0 if use_scaler else 1.0
+
+    def fresh():
+        p = H.dev_list(p0, shapes)
+        opt = G.GroupOptimizer.adamw_with_decay_exclusions(list(zip(names, p)), 1e-3, 0.1, ["bias", "norm"])
+        sc = None
+        if use_scaler:
+            sc = nb.GradScaler.new()
+            sc.load_state(nb.GradScalerState(scale0, 2.0, 0.5, 3, 0))
+        return p, opt, sc
+
+    p1, o1, s1 = fresh()
+    p2, o2, s2 = fresh()
+    tail = TrainerTail(o1, p1).with_grad_accum(2).with_grad_clip(0.05)
+    if use_scaler:
+        tail.with_grad_scaler(s1)
+    buf, count, steps = None, 0, 0
+    for k in range(9):
+        scale = s2.scale_factor() if use_scaler else 1.0
+        g = [a * np.float32(scale) for a in H.randn_list(shapes, 4300 + k, 1e-3)]
+        if use_scaler and k == 3:
+            g[4][77] = np.inf
+        stepped = tail.after_backward(H.dev_list(g, shapes))
+        g2 = H.dev_list(g, shapes)
+        if use_scaler and not s2.unscale_and_update(g2):
+            buf, count = None, 0
+            assert not stepped
+            continue
+        if buf is None:
+            buf = [torch.zeros_like(t) for t in g2]
+        nb.accumulate(buf, g2)
+        count += 1
+        if count == 2:
+            o2.fused_step(p2, buf, max_norm=0.05, zero_grads=True)
+            count, steps = 0, steps + 1
+        assert stepped == (count == 0), k
+    assert steps == (3 if use_scaler else 4) and tail.state.step == steps
+    H.assert_bits_equal(H.host_list(p1), H.host_list(p2), "params")
+    for (n1, t1), (n2, t2) in zip(o1.state_tensors(), o2.state_tensors()):
+        assert n1 == n2
+        H.assert_bits_equal([H.to_host(t1)], [H.to_host(t2)], n1)
+    assert o1.last_step().step_count == o2.last_step().step_count == steps
