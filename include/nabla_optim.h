@@ -94,7 +94,9 @@ typedef struct nbo_scaler nbo_scaler; /* GradScaler */
  * entry point calls it implicitly). */
 int nbo_init(void);
 /* Use `hip_stream` (a hipStream_t) for all subsequent work; NULL = the null stream,
- * which is what the reference's HIP backend launches on (hip/backend.rs:337). */
+ * which is what the reference's HIP backend launches on (hip/backend.rs:337).  Waits for
+ * what is already enqueued on the previous stream (the two share the library's scratch and
+ * the optimizers' state), so call it outside stream capture. */
 int nbo_set_stream(void *hip_stream);
 /* B::sync (common/backend/mod.rs:82-216): wait for all enqueued work. */
 int nbo_sync(void);

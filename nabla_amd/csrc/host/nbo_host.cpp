@@ -91,6 +91,16 @@ Runtime::Runtime()
 
 void Runtime::sync() { hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize"); }
 
+void Runtime::set_stream(hipStream_t s)
+{
+    if (s == stream_) return;
+    // What is already enqueued on the previous stream shares the reduction scratch, the
+    // staging buffer and the optimizers' state with what follows on the new one, and nothing
+    // orders two streams: finish it first.
+    hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize (previous stream)");
+    stream_ = s;
+}
+
 void Runtime::launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct)
 {
     if (grid == 0) return;

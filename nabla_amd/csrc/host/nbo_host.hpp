@@ -66,7 +66,7 @@ class Runtime {
 public:
     static Runtime &get(); // creates on first use; throws Error on failure
     hipStream_t stream() const { return stream_; }
-    void set_stream(hipStream_t s) { stream_ = s; }
+    void set_stream(hipStream_t s);
     void sync();
 
     template <typename Args> void launch(int kernel, uint32_t grid, uint32_t block, const Args &args)

@@ -682,3 +682,38 @@ def test_two_host_threads_drive_two_optimizers(gpu):
             assert c["opt"].step_count() == 25
     finally:
         O.set_pow_mode(O.POW_LIBM)
+
+
+def test_switching_streams_keeps_the_steps_in_order(gpu):
+    """nbo_set_stream waits for what is enqueued on the previous stream, so steps issued
+    alternately on two non-blocking streams and the null stream run in call order: the result
+    is the oracle's for the same sequence."""
+    import torch
+
+    from nabla_amd import _lib
+
+    shapes = [(1, 70001), (64, 130), (1, 5)]
+    p0 = H.randn_list(shapes, 800, 0.05)
+    grads = [H.randn_list(shapes, 810 + s, 1e-2) for s in range(12)]
+    p_dev, g_dev = H.dev_list(p0, shapes), [H.dev_list(g, shapes) for g in grads]
+    torch.cuda.synchronize()
+    opt = nb.AdamW.new(1e-3, shapes)
+    lib = _lib.load()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream(), None]
+    try:
+        for s, g in enumerate(g_dev):
+            st = streams[s % 3]
+            _lib.check(lib.nbo_set_stream(st.cuda_stream if st is not None else None))
+            opt.fused_step(p_dev, g, max_norm=0.5)
+    finally:
+        _lib.check(lib.nbo_set_stream(None))
+    nb.sync()
+    pr, m, v, meta = H.copy_list(p0), H.zeros_like_list(p0), H.zeros_like_list(p0), O.adamw_meta(1e-3)
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        for g in grads:
+            O.f32_step(meta, None, 0.5, pr, H.copy_list(g), m, v)
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+    H.assert_bits_equal(H.host_list(p_dev), pr, "params")
+    H.assert_bits_equal(H.host_list(opt.moments()[1]), v, "v")
