@@ -588,8 +588,9 @@ public:
         } else {
             dirty_ = true; // a non-finite micro-batch leaves garbage in the buffer
             if (!unscale_accumulate(accum_, grads, scaler_, &sumsq, has_policy_)) {
+                drop();
                 if (!scaler_ && policy_ == GradNanPolicy::Stop) throw TrainError("non-finite gradient");
-                return drop();
+                return false;
             }
         }
         accum_count_ += 1;

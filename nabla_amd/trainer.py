@@ -120,8 +120,7 @@ class TrainerTail:
         import torch
 
         tensors = grads.tensors if isinstance(grads, nb.TensorList) else grads
-        fresh = self._accum is None
-        if fresh:
+        if self._accum is None:
             self._accum = [torch.zeros_like(g) for g in tensors]
         if self.scaler is not None and self.nan_policy is not None:
             # both decisions, in the reference's order: a micro-batch whose unscaled gradients
@@ -140,9 +139,10 @@ class TrainerTail:
             ok, sumsq = nb.unscale_accumulate(self._accum, grads, scaler=self.scaler,
                                               check_finite=self.nan_policy is not None)
             if not ok:
+                self._drop()
                 if self.scaler is None and self.nan_policy is GradNanPolicy.STOP:
                     raise TrainError("non-finite gradient")
-                return self._drop()
+                return False
         self._accum_count += 1
         if self._accum_count < self.state.grad_accum:
             return False
