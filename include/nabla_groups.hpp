@@ -79,6 +79,17 @@ struct ParamGroupConfig {
     }
 };
 
+// groups.rs:134-150
+enum class ParamExclusionPreset { Bias, Norm, Embedding };
+inline std::vector<std::string> preset_patterns(ParamExclusionPreset p)
+{
+    switch (p) {
+    case ParamExclusionPreset::Bias: return {"bias"};
+    case ParamExclusionPreset::Norm: return {"norm", "bn", "ln"};
+    default: return {"embed", "embedding"};
+    }
+}
+
 class GroupOptimizer {
 public:
     // groups.rs:168-226; throws StateError("nabla-train: group assignment incomplete")
@@ -120,7 +131,8 @@ public:
     // groups.rs:228-242
     static GroupOptimizer adamw_with_decay_exclusions(const std::vector<std::pair<std::string, Tensor>> &named,
                                                       double lr, double weight_decay,
-                                                      const std::vector<std::string> &exclude)
+                                                      const std::vector<std::string> &exclude,
+                                                      nbo_dtype state_dtype = NBO_DT_F32, bool master = false)
     {
         std::vector<ParamMatch> m;
         for (const std::string &s : exclude) {
@@ -129,7 +141,19 @@ public:
         }
         const ParamGroupConfig no_decay = ParamGroupConfig::adamw("no_decay", ParamSelector::Any(m), lr, 0.0);
         const ParamGroupConfig decay = ParamGroupConfig::adamw("decay", ParamSelector::All(), lr, weight_decay);
-        return from_named_params(named, {no_decay}, &decay);
+        return from_named_params(named, {no_decay}, &decay, state_dtype, master);
+    }
+
+    // groups.rs:244-261
+    static GroupOptimizer adamw_with_decay_presets(const std::vector<std::pair<std::string, Tensor>> &named, double lr,
+                                                   double weight_decay,
+                                                   const std::vector<ParamExclusionPreset> &presets,
+                                                   nbo_dtype state_dtype = NBO_DT_F32, bool master = false)
+    {
+        std::vector<std::string> patterns;
+        for (ParamExclusionPreset p : presets)
+            for (const std::string &s : preset_patterns(p)) patterns.push_back(s);
+        return adamw_with_decay_exclusions(named, lr, weight_decay, patterns, state_dtype, master);
     }
 
     size_t groups() const { return groups_.size(); }

@@ -335,6 +335,27 @@ static void panics_and_errors()  // alg.rs:110-119, 531-545; tensor/ops.rs:638-6
     EXPECT(p.get() == 1.0);  // nothing ran
 }
 
+static void decay_presets_and_known_norm_group_step()  // groups.rs:134-150, 244-261
+{
+    Mat e({1.0}), w({2.0}), b({3.0}), ln({4.0}), ge({0.0}), gw({3.0}), gb({4.0}), gl({0.0});
+    const std::vector<std::pair<std::string, Tensor>> named = {
+        {"embed.table", e.tensor()}, {"l0.weight", w.tensor()}, {"l0.bias", b.tensor()}, {"l0.ln", ln.tensor()}};
+    GroupOptimizer opt = GroupOptimizer::adamw_with_decay_presets(
+        named, 0.1, 0.5, {ParamExclusionPreset::Bias, ParamExclusionPreset::Norm, ParamExclusionPreset::Embedding},
+        NBO_DT_F64);
+    EXPECT(opt.groups() == 2 && (opt.group_indices(0) == std::vector<size_t>{0, 2, 3}) &&
+           (opt.group_indices(1) == std::vector<size_t>{1}));
+    // gradients (0, 3, 4, 0): norm 5, clipped to 2.5 -> (1.5, 2); first AdamW step moves by lr * sign(g)
+    const std::vector<Tensor> params = {e.tensor(), w.tensor(), b.tensor(), ln.tensor()};
+    const std::vector<Tensor> grads = {ge.tensor(), gw.tensor(), gb.tensor(), gl.tensor()};
+    opt.fused_step_norm(params, grads, 25.0, 2.5);
+    EXPECT(e.get() == 1.0 && ln.get() == 4.0);                    // no gradient, no decay
+    EXPECT(std::fabs(b.get() - (3.0 - 0.1)) < 1e-6);              // no decay
+    EXPECT(std::fabs(w.get() - (2.0 * (1.0 - 0.05) - 0.1)) < 1e-6);  // decayed by lr * wd
+    const nbo_step_info info = opt.group_optimizer(0).last_step();
+    EXPECT(info.norm == 5.0 && info.clipped == 1 && info.step_count == 1);
+}
+
 static void constructors_and_set_state()  // alg.rs:41-45, 90-105, 244-250, 374-378; core.rs:12-16
 {
     Mat p({1.0, 2.0}), g({1.0, 1.0});
@@ -405,7 +426,8 @@ int main(int argc, char **argv)
                  {"backend_axpy_is_multiply_then_add", backend_axpy_is_multiply_then_add},
                  {"checkpoint_roundtrip_with_schedule", checkpoint_roundtrip_with_schedule},
                  {"panics_and_errors", panics_and_errors},
-                 {"constructors_and_set_state", constructors_and_set_state}};
+                 {"constructors_and_set_state", constructors_and_set_state},
+                 {"decay_presets_and_known_norm_group_step", decay_presets_and_known_norm_group_step}};
     try {
         check(nbo_init());
         for (auto &t : tests) {

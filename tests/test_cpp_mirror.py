@@ -40,7 +40,7 @@ def test_cpp_replay_of_reference_tests(gpu, tmp_path):
     r = subprocess.run([BIN, str(tmp_path)], capture_output=True, text=True, timeout=120)
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count("ok    ") == 15 and "0 failure(s)" in r.stdout
+    assert r.stdout.count("ok    ") == 16 and "0 failure(s)" in r.stdout
 
     # the checkpoint the C++ side left behind is the one the Python mirror writes and reads
     from nabla_amd import checkpoint as ck
