@@ -201,6 +201,9 @@ public:
         check(nbo_fused_step_groups_norm(groups_.size(), opts.data(), pl.data(), gl.data(), max_norm, sumsq,
                                          zero_grads ? NBO_STEP_ZERO_GRADS : 0u));
     }
+    // optim.nbla of a checkpoint with the keys of groups.rs:320-350 ("g{gi}.m{i}", "g{gi}.v{i}")
+    void save_state(const std::string &path) { check(nbo_optim_save_state_groups(groups_.size(), handles().data(), path.c_str())); }
+    void load_state(const std::string &path) { check(nbo_optim_load_state_groups(groups_.size(), handles().data(), path.c_str())); }
     void reset()
     {
         for (Entry &g : groups_) g.optimizer->reset();
@@ -235,6 +238,12 @@ private:
         auto o = std::make_shared<Sgd>(c.lr, shapes, dt, master);
         o->momentum(c.momentum).weight_decay(c.weight_decay);
         return o;
+    }
+    std::vector<nbo_optim *> handles()
+    {
+        std::vector<nbo_optim *> h;
+        for (Entry &g : groups_) h.push_back(g.optimizer->handle());
+        return h;
     }
     static std::vector<const void *> key_of(const std::vector<Tensor> &t)
     {

@@ -301,6 +301,12 @@ int nbo_optim_save_state(nbo_optim *opt, const char *path);
  * "bad tensor key: k", "m index out of range: i", "missing m{i}" / "missing v{i}"; other
  * prefixes are ignored.  Nothing is written unless the whole file checks out. */
 int nbo_optim_load_state(nbo_optim *opt, const char *path);
+/* The same for GroupOptimizer's OptimState (optim/groups.rs:320-350): group gi's tensors
+ * carry the keys "g{gi}.m{i}" / "g{gi}.v{i}"; loading refuses any other key ("bad group tensor
+ * key: k", "bad group index: x", "group index out of range: gi") and then applies each
+ * group's own checks.  Nothing is written unless the whole file checks out. */
+int nbo_optim_save_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path);
+int nbo_optim_load_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path);
 
 /* ---- measurement helpers --------------------------------------------------------------- */
 

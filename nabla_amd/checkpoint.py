@@ -231,19 +231,35 @@ def load_params_native(path: str, named_tensors: Sequence[Tuple[str, object]]) -
     _native(_lib.load().nbo_nbla_load_list, path.encode(), lst._h, _name_array([n for n, _ in named_tensors]))
 
 
+def _group_handles(optimizer):
+    import ctypes as C
+
+    subs = optimizer.group_optimizers()
+    return len(subs), (C.c_void_p * len(subs))(*[o._handle() for o in subs])
+
+
 def save_optim_native(path: str, optimizer) -> None:
-    """optim.nbla from the optimizer's device state (nbo_optim_save_state)."""
+    """optim.nbla from the optimizer's device state (nbo_optim_save_state; for a
+    GroupOptimizer nbo_optim_save_state_groups, keys "g{gi}.m{i}")."""
     from . import _lib
 
-    _native(_lib.load().nbo_optim_save_state, optimizer._handle(), path.encode())
+    if hasattr(optimizer, "group_optimizers"):
+        n, handles = _group_handles(optimizer)
+        _native(_lib.load().nbo_optim_save_state_groups, n, handles, path.encode())
+    else:
+        _native(_lib.load().nbo_optim_save_state, optimizer._handle(), path.encode())
 
 
 def load_optim_native(path: str, optimizer) -> None:
     """load_tensors + load_state_tensors into the optimizer's device state
-    (nbo_optim_load_state)."""
+    (nbo_optim_load_state / nbo_optim_load_state_groups)."""
     from . import _lib
 
-    _native(_lib.load().nbo_optim_load_state, optimizer._handle(), path.encode())
+    if hasattr(optimizer, "group_optimizers"):
+        n, handles = _group_handles(optimizer)
+        _native(_lib.load().nbo_optim_load_state_groups, n, handles, path.encode())
+    else:
+        _native(_lib.load().nbo_optim_load_state, optimizer._handle(), path.encode())
 
 
 def save_checkpoint(directory: str, params: Sequence[Tuple[str, object]], optimizer,

@@ -1068,6 +1068,29 @@ int nbo_optim_load_state(nbo_optim *opt, const char *path)
     });
 }
 
+static void require_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path)
+{
+    require(path != nullptr, NBO_ERR_ARG, "null path");
+    require(n_groups == 0 || opts != nullptr, NBO_ERR_ARG, "null group array");
+    for (uint64_t g = 0; g < n_groups; g++) require(opts[g] != nullptr, NBO_ERR_ARG, "null optimizer");
+}
+
+int nbo_optim_save_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path)
+{
+    return guarded([&] {
+        require_groups(n_groups, opts, path);
+        optim_save_state_groups(n_groups, opts, path);
+    });
+}
+
+int nbo_optim_load_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path)
+{
+    return guarded([&] {
+        require_groups(n_groups, opts, path);
+        optim_load_state_groups(n_groups, opts, path);
+    });
+}
+
 int nbo_copy_bytes(const void *src_dev, void *dst_dev, uint64_t bytes)
 {
     return guarded([&] {

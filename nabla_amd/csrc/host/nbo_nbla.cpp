@@ -277,75 +277,164 @@ void nbla_load_list(const char *path, nbo_list *list, const char *const *names)
     }
 }
 
-// OptimState::state_tensors (alg.rs:476-485, 553-562, 623-629) written by save_tensors:
-// m0.., then v0.. (Sgd: v0.. = velocity).
-void optim_save_state(const nbo_optim *opt, const char *path)
+namespace {
+
+// One optimizer's state tensors in state_tensors() order -- m0.., then v0.. (Sgd: v0.. =
+// velocity) -- each name behind `prefix` (alg.rs:476-485, 553-562, 623-629).
+void write_optim_entries(std::FILE *f, const nbo_optim *opt, const std::string &prefix, Buffers &b)
 {
     const uint64_t nt = opt->layout.nt();
     const bool adam_like = opt->meta.kind != NBO_KIND_SGD;
-    Runtime::get().sync();
-    FilePtr f = open_file(path, "wb");
-    Buffers b;
-    write_all(f.get(), "NBLA", 4);
-    write_u32(f.get(), (uint32_t)(nt * (adam_like ? 2 : 1)));
     const size_t eb = opt->elem_bytes();
     for (int which = 0; which < (adam_like ? 2 : 1); which++) {
-        const char prefix = adam_like && which == 0 ? 'm' : 'v';
+        const char letter = adam_like && which == 0 ? 'm' : 'v';
         const uint32_t part = which == 0 ? 0u : opt->arena.part_v;
         for (uint64_t t = 0; t < nt; t++) {
-            write_header(f.get(), prefix + std::to_string(t), opt->layout.rows[t], opt->layout.cols[t]);
+            write_header(f, prefix + letter + std::to_string(t), opt->layout.rows[t], opt->layout.cols[t]);
             const char *dev = (const char *)opt->arena.part[part] + (size_t)opt->layout.soff[t] * eb;
-            stream_out(f.get(), dev, opt->state_dtype, opt->layout.n[t], b);
+            stream_out(f, dev, opt->state_dtype, opt->layout.n[t], b);
         }
     }
-    if (std::fflush(f.get()) != 0) fail(NBO_ERR_IO, std::string("write failed: ") + std::strerror(errno));
 }
 
-// OptimState::load_state_tensors (alg.rs:487-516, 564-593, 631-648) over load_tensors:
-// other prefixes are ignored, every expected tensor must be present; nothing is written
-// unless the whole file checks out.
-void optim_load_state(nbo_optim *opt, const char *path)
+uint64_t optim_entry_count(const nbo_optim *opt)
+{
+    return opt->layout.nt() * (opt->meta.kind != NBO_KIND_SGD ? 2u : 1u);
+}
+
+// Where in the file each state tensor of one optimizer is.
+struct LoadPlan {
+    std::vector<long> m_at, v_at;
+};
+
+// OptimState::load_state_tensors (alg.rs:487-516, 564-593, 631-648) up to the point where it
+// would start writing: other prefixes are ignored, every expected tensor must be present.
+// `names[k]` is entry k's key as this optimizer sees it (a group prefix already taken off).
+LoadPlan plan_optim_load(const nbo_optim *opt, const std::vector<const Entry *> &entries,
+                         const std::vector<std::string> &names)
 {
     const uint64_t nt = opt->layout.nt();
     const bool adam_like = opt->meta.kind != NBO_KIND_SGD;
-    FilePtr f = open_file(path, "rb");
-    const std::vector<Entry> index = read_index(f.get());
-    std::vector<long> m_at(nt, -1), v_at(nt, -1);
-    for (const Entry &e : index) {
-        const char c = e.name.empty() ? '\0' : e.name[0];
+    LoadPlan plan;
+    plan.m_at.assign(nt, -1);
+    plan.v_at.assign(nt, -1);
+    for (size_t k = 0; k < entries.size(); k++) {
+        const Entry &e = *entries[k];
+        const std::string &name = names[k];
+        const char c = name.empty() ? '\0' : name[0];
         if (!(c == 'v' || (c == 'm' && adam_like))) continue;
         // what Rust's str::parse::<usize> accepts: an optional '+', then decimal digits
-        const char *p = e.name.c_str() + 1;
+        const char *p = name.c_str() + 1;
         if (*p == '+') p++;
-        if (*p == '\0') fail(NBO_ERR_STATE_KEY, "bad tensor key: " + e.name);
+        if (*p == '\0') fail(NBO_ERR_STATE_KEY, "bad tensor key: " + name);
         uint64_t idx = 0;
         for (; *p; p++) {
             if (*p < '0' || *p > '9' || idx > (UINT64_MAX - (uint64_t)(*p - '0')) / 10)
-                fail(NBO_ERR_STATE_KEY, "bad tensor key: " + e.name);
+                fail(NBO_ERR_STATE_KEY, "bad tensor key: " + name);
             idx = idx * 10 + (uint64_t)(*p - '0');
         }
         if (idx >= nt) fail(NBO_ERR_STATE_INDEX, std::string(1, c) + " index out of range: " + std::to_string(idx));
         if (e.rows * e.cols != opt->layout.n[idx])
-            fail(NBO_ERR_SHAPE, "state tensor " + e.name + " has " + std::to_string(opt->layout.n[idx]) +
+            fail(NBO_ERR_SHAPE, "state tensor " + name + " has " + std::to_string(opt->layout.n[idx]) +
                                     " elements, file has " + std::to_string(e.rows * e.cols));
-        (c == 'm' ? m_at : v_at)[idx] = e.data_offset; // a later duplicate wins, as in the reference
+        (c == 'm' ? plan.m_at : plan.v_at)[idx] = e.data_offset; // a later duplicate wins, as in the reference
     }
     if (adam_like)
         for (uint64_t t = 0; t < nt; t++)
-            if (m_at[t] < 0) fail(NBO_ERR_STATE_KEY, "missing m" + std::to_string(t));
+            if (plan.m_at[t] < 0) fail(NBO_ERR_STATE_KEY, "missing m" + std::to_string(t));
     for (uint64_t t = 0; t < nt; t++)
-        if (v_at[t] < 0) fail(NBO_ERR_STATE_KEY, "missing v" + std::to_string(t));
-    Buffers b;
+        if (plan.v_at[t] < 0) fail(NBO_ERR_STATE_KEY, "missing v" + std::to_string(t));
+    return plan;
+}
+
+void apply_optim_load(std::FILE *f, nbo_optim *opt, const LoadPlan &plan, Buffers &b)
+{
+    const uint64_t nt = opt->layout.nt();
+    const bool adam_like = opt->meta.kind != NBO_KIND_SGD;
     const size_t eb = opt->elem_bytes();
     for (int which = 0; which < (adam_like ? 2 : 1); which++) {
-        const std::vector<long> &at = adam_like && which == 0 ? m_at : v_at;
+        const std::vector<long> &at = adam_like && which == 0 ? plan.m_at : plan.v_at;
         const uint32_t part = which == 0 ? 0u : opt->arena.part_v;
         for (uint64_t t = 0; t < nt; t++) {
-            seek_to(f.get(), at[t]);
+            seek_to(f, at[t]);
             char *dev = (char *)opt->arena.part[part] + (size_t)opt->layout.soff[t] * eb;
-            stream_in(f.get(), dev, opt->state_dtype, opt->layout.n[t], b);
+            stream_in(f, dev, opt->state_dtype, opt->layout.n[t], b);
         }
     }
+}
+
+} // namespace
+
+// optim.nbla of a checkpoint: OptimState::state_tensors written by save_tensors
+// (checkpoint.rs:59-62).
+void optim_save_state(const nbo_optim *opt, const char *path)
+{
+    Runtime::get().sync();
+    FilePtr f = open_file(path, "wb");
+    Buffers b;
+    write_all(f.get(), "NBLA", 4);
+    write_u32(f.get(), (uint32_t)optim_entry_count(opt));
+    write_optim_entries(f.get(), opt, "", b);
+    if (std::fflush(f.get()) != 0) fail(NBO_ERR_IO, std::string("write failed: ") + std::strerror(errno));
+}
+
+// load_tensors into OptimState::load_state_tensors (checkpoint.rs:92-95); nothing is written
+// unless the whole file checks out.
+void optim_load_state(nbo_optim *opt, const char *path)
+{
+    FilePtr f = open_file(path, "rb");
+    const std::vector<Entry> index = read_index(f.get());
+    std::vector<const Entry *> entries;
+    std::vector<std::string> names;
+    for (const Entry &e : index) entries.push_back(&e), names.push_back(e.name);
+    const LoadPlan plan = plan_optim_load(opt, entries, names);
+    Buffers b;
+    apply_optim_load(f.get(), opt, plan, b);
+}
+
+// GroupOptimizer's OptimState (groups.rs:320-373): every group's tensors behind "g{gi}.".
+void optim_save_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path)
+{
+    uint64_t total = 0;
+    for (uint64_t g = 0; g < n_groups; g++) total += optim_entry_count(opts[g]);
+    if (total > 0xFFFFFFFFull) fail(NBO_ERR_TOO_LARGE, "too many tensors for the file format");
+    Runtime::get().sync();
+    FilePtr f = open_file(path, "wb");
+    Buffers b;
+    write_all(f.get(), "NBLA", 4);
+    write_u32(f.get(), (uint32_t)total);
+    for (uint64_t g = 0; g < n_groups; g++)
+        write_optim_entries(f.get(), opts[g], "g" + std::to_string(g) + ".", b);
+    if (std::fflush(f.get()) != 0) fail(NBO_ERR_IO, std::string("write failed: ") + std::strerror(errno));
+}
+
+void optim_load_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path)
+{
+    FilePtr f = open_file(path, "rb");
+    const std::vector<Entry> index = read_index(f.get());
+    std::vector<std::vector<const Entry *>> entries(n_groups);
+    std::vector<std::vector<std::string>> names(n_groups);
+    for (const Entry &e : index) { // groups.rs:339-361: "g{gi}.{key}", every tensor of the file
+        const size_t dot = e.name.find('.');
+        if (dot == std::string::npos || e.name[0] != 'g') fail(NBO_ERR_STATE_KEY, "bad group tensor key: " + e.name);
+        const std::string idx = e.name.substr(1, dot - 1);
+        const char *p = idx.c_str();
+        if (*p == '+') p++;
+        if (*p == '\0') fail(NBO_ERR_STATE_KEY, "bad group index: " + idx);
+        uint64_t gi = 0;
+        for (; *p; p++) {
+            if (*p < '0' || *p > '9' || gi > (UINT64_MAX - (uint64_t)(*p - '0')) / 10)
+                fail(NBO_ERR_STATE_KEY, "bad group index: " + idx);
+            gi = gi * 10 + (uint64_t)(*p - '0');
+        }
+        if (gi >= n_groups) fail(NBO_ERR_STATE_INDEX, "group index out of range: " + std::to_string(gi));
+        entries[gi].push_back(&e);
+        names[gi].push_back(e.name.substr(dot + 1));
+    }
+    std::vector<LoadPlan> plans;
+    for (uint64_t g = 0; g < n_groups; g++) plans.push_back(plan_optim_load(opts[g], entries[g], names[g]));
+    Buffers b;
+    for (uint64_t g = 0; g < n_groups; g++) apply_optim_load(f.get(), opts[g], plans[g], b);
 }
 
 } // namespace nbo

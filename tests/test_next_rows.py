@@ -510,6 +510,53 @@ def test_native_nbla_reader_round_trip_and_errors(gpu, tmp_path):
 
 
 @pytest.mark.gpu
+def test_native_group_optimizer_state_file(gpu, tmp_path):
+    """nbo_optim_{save,load}_state_groups: the file is the Python writer's over
+    GroupOptimizer.state_tensors() byte for byte (keys g{gi}.m{i} / g{gi}.v{i}, groups.rs:320-329),
+    loads back into a fresh GroupOptimizer, and refuses what the reference refuses."""
+    import torch
+
+    names = ["embed", "l0.w", "l0.bias", "l0.norm", "head"]
+    shapes = [(50, 16), (16, 300), (1, 16), (1, 16), (16, 50)]
+    torch.manual_seed(12)
+    params = [torch.randn(s, device=gpu) * 0.1 for s in shapes]
+
+    def make():
+        sgd = G.ParamGroupConfig.sgd("plain", G.ParamSelector.Any([G.Prefix("embed")]), 0.1, 0.9, 0.0)
+        nod = G.ParamGroupConfig.adamw("no_decay", G.ParamSelector.Any([G.Suffix("bias"), G.Contains("norm")]), 1e-3, 0.0)
+        dec = G.ParamGroupConfig.adamw("decay", G.ParamSelector.All(), 1e-3, 0.1)
+        return G.GroupOptimizer.from_named_params(list(zip(names, params)), [sgd, nod], dec)
+
+    opt = make()
+    for k in range(2):
+        opt.step(params, [torch.randn(s, device=gpu) * 1e-2 for s in shapes])
+    ck.save_tensors(opt.state_tensors(), str(tmp_path / "py.nbla"))
+    ck.save_optim_native(str(tmp_path / "native.nbla"), opt)
+    assert _file_bytes(tmp_path / "native.nbla") == _file_bytes(tmp_path / "py.nbla")
+    keys = [n for n, _ in ck.load_tensors(str(tmp_path / "native.nbla"))]
+    assert keys == ["g0.v0", "g1.m0", "g1.m1", "g1.v0", "g1.v1", "g2.m0", "g2.m1", "g2.v0", "g2.v1"]
+    other = make()
+    ck.load_optim_native(str(tmp_path / "native.nbla"), other)
+    for (n1, t1), (n2, t2) in zip(opt.state_tensors(), other.state_tensors()):
+        assert n1 == n2 and torch.equal(t1, t2), n1
+    tensors = ck.load_tensors(str(tmp_path / "native.nbla"))
+    bad = str(tmp_path / "bad.nbla")
+    for extra, message in ((("m0", np.zeros((1, 1))), "bad group tensor key: m0"),
+                           (("x1.m0", np.zeros((1, 1))), "bad group tensor key: x1.m0"),
+                           (("gx.m0", np.zeros((1, 1))), "bad group index: x"),
+                           (("g7.m0", np.zeros((1, 1))), "group index out of range: 7"),
+                           (("g1.m9", np.zeros((1, 1))), "m index out of range: 9")):
+        ck.save_tensors(tensors + [extra], bad)
+        with pytest.raises(ck.CheckpointError, match=message):
+            ck.load_optim_native(bad, other)
+    ck.save_tensors([t for t in tensors if t[0] != "g2.v1"], bad)
+    with pytest.raises(ck.CheckpointError, match="missing v1"):
+        ck.load_optim_native(bad, other)
+    for (n1, t1), (n2, t2) in zip(opt.state_tensors(), other.state_tensors()):
+        assert torch.equal(t1, t2), f"{n1} changed by a refused load"
+
+
+@pytest.mark.gpu
 def test_native_checkpoint_resumes_bit_identical_training(gpu, tmp_path):
     """save_checkpoint(native=True) after two steps, load_checkpoint(into=...) into a fresh
     optimizer and fresh tensors, two more steps on both: identical bits, and the files are
