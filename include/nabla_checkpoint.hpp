@@ -21,7 +21,7 @@
 #include <utility>
 #include <vector>
 
-#include "nabla_optim.hpp"
+#include "nabla_groups.hpp"
 
 namespace nabla {
 namespace optim {
@@ -180,9 +180,46 @@ inline std::optional<ScheduleState> parse_schedule_state(const MetaMap &m)
     throw StateError("bad schedule.kind: " + kind);
 }
 
+// OptimState::meta_pairs / load_meta_pairs: the defaults (core.rs:71-78) for Sgd / Adam /
+// AdamW, GroupOptimizer's own (groups.rs:368-420)
+inline Pairs meta_pairs_of(Optimizer &o) { return optim_meta_pairs(o.meta()); }
+inline void load_meta_pairs_into(Optimizer &o, const MetaMap &m) { o.load_meta(parse_optim_meta(m)); }
+inline Pairs meta_pairs_of(GroupOptimizer &o)
+{
+    Pairs out = {{"optim.group.count", std::to_string(o.groups())}};
+    for (size_t gi = 0; gi < o.groups(); gi++) {
+        const std::string p = "optim.group." + std::to_string(gi) + ".";
+        out.push_back({p + "name", o.group_name(gi)});
+        for (const auto &kv : optim_meta_pairs(o.group_optimizer(gi).meta()))
+            out.push_back({p + kv.first.substr(6), kv.second}); // "optim.lr" -> "optim.group.{gi}.lr"
+    }
+    return out;
+}
+inline void load_meta_pairs_into(GroupOptimizer &o, const MetaMap &m)
+{
+    if (detail::parse_usize(m, "optim.group.count") != o.groups()) throw StateError("optim.group.count mismatch");
+    for (size_t gi = 0; gi < o.groups(); gi++) {
+        const std::string p = "optim.group." + std::to_string(gi) + ".";
+        if (detail::get(m, p + "name") != o.group_name(gi))
+            throw StateError("optim.group." + std::to_string(gi) + ".name mismatch");
+        const std::string &kind = detail::get(m, p + "kind");
+        OptimKind k;
+        if (kind == "adamw") k = OptimKind::AdamW;
+        else if (kind == "adam") k = OptimKind::Adam;
+        else if (kind == "sgd") k = OptimKind::Sgd;
+        else throw StateError("bad optim.kind: " + kind);
+        o.group_optimizer(gi).load_meta({k, detail::parse_f64(m, p + "lr"), detail::parse_f64(m, p + "beta1"),
+                                         detail::parse_f64(m, p + "beta2"), detail::parse_f64(m, p + "eps"),
+                                         detail::parse_f64(m, p + "weight_decay"), detail::parse_f64(m, p + "momentum"),
+                                         detail::parse_usize(m, p + "step_count")});
+    }
+    o.refresh_base_lr();
+}
+
 // checkpoint.rs:107-150
-inline void write_meta(const std::string &path, Optimizer &optimizer, GradScaler *scaler,
-                       const ScheduleState *schedule, const TrainState &state)
+template <typename Opt>
+void write_meta(const std::string &path, Opt &optimizer, GradScaler *scaler, const ScheduleState *schedule,
+                const TrainState &state)
 {
     std::ofstream f(path, std::ios::binary | std::ios::trunc);
     if (!f) throw CheckpointError("Io", path + ": cannot create");
@@ -191,7 +228,7 @@ inline void write_meta(const std::string &path, Optimizer &optimizer, GradScaler
       << "step=" << state.step << "\n"
       << "grad_accum=" << state.grad_accum << "\n";
     if (state.rng_state) f << "rng.state=" << *state.rng_state << "\n";
-    for (const auto &kv : optim_meta_pairs(optimizer.meta())) f << kv.first << "=" << kv.second << "\n";
+    for (const auto &kv : meta_pairs_of(optimizer)) f << kv.first << "=" << kv.second << "\n";
     if (schedule)
         for (const auto &kv : schedule_pairs(*schedule)) f << kv.first << "=" << kv.second << "\n";
     if (scaler) {
@@ -215,7 +252,7 @@ struct MetaContents {
 };
 
 // checkpoint.rs:152-212; the optimizer's hyper-parameters and step_count are loaded into it
-inline MetaContents read_meta(const std::string &path, Optimizer &optimizer)
+template <typename Opt> MetaContents read_meta(const std::string &path, Opt &optimizer)
 {
     std::ifstream f(path, std::ios::binary);
     if (!f) throw CheckpointError("Io", path + ": cannot open");
@@ -240,7 +277,7 @@ inline MetaContents read_meta(const std::string &path, Optimizer &optimizer)
     out.state.step = parse(detail::parse_usize, "step");
     out.state.grad_accum = parse(detail::parse_usize, "grad_accum");
     try {
-        optimizer.load_meta(parse_optim_meta(m)); // load_meta_pairs, core.rs:75-78
+        load_meta_pairs_into(optimizer, m);
     } catch (const StateError &e) {
         throw CheckpointError("Optim", e.what());
     }
@@ -284,9 +321,9 @@ template <typename F> void tensor_file(const char *kind, F &&call)
 
 // checkpoint.rs:38-69.  `params` / `names` are the module's state_dict (for a
 // mixed-precision optimizer: its f32 master weights).
-inline void save_checkpoint(const std::string &dir, TensorList &params, const std::vector<std::string> &names,
-                            Optimizer &optimizer, GradScaler *scaler, const ScheduleState *schedule,
-                            const TrainState &state)
+template <typename Opt>
+void save_checkpoint(const std::string &dir, TensorList &params, const std::vector<std::string> &names, Opt &optimizer,
+                     GradScaler *scaler, const ScheduleState *schedule, const TrainState &state)
 {
     ::mkdir(dir.c_str(), 0777); // fs::create_dir_all for the last component; an existing directory is fine
     detail::tensor_file("State", [&] { save_tensors(dir + "/params.nbla", params, names); });
@@ -296,9 +333,9 @@ inline void save_checkpoint(const std::string &dir, TensorList &params, const st
 
 // checkpoint.rs:71-105: parameters into `params` (load_state_dict), moments and meta into
 // `optimizer`, the scaler's state into `scaler` if both are there.
-inline void load_checkpoint(const std::string &dir, TensorList &params, const std::vector<std::string> &names,
-                            Optimizer &optimizer, GradScaler *scaler, std::optional<ScheduleState> &schedule,
-                            TrainState &state)
+template <typename Opt>
+void load_checkpoint(const std::string &dir, TensorList &params, const std::vector<std::string> &names, Opt &optimizer,
+                     GradScaler *scaler, std::optional<ScheduleState> &schedule, TrainState &state)
 {
     detail::tensor_file("State", [&] { load_state_dict(dir + "/params.nbla", params, names); });
     detail::tensor_file("Optim", [&] { optimizer.load_state(dir + "/optim.nbla"); });

@@ -159,6 +159,12 @@ public:
     size_t groups() const { return groups_.size(); }
     const std::vector<size_t> &group_indices(size_t g) const { return groups_[g].indices; }
     Optimizer &group_optimizer(size_t g) { return *groups_[g].optimizer; }
+    const std::string &group_name(size_t g) const { return groups_[g].name; }
+    // groups.rs:416-418: after the groups' metas were loaded, the base lr is the first group's
+    void refresh_base_lr()
+    {
+        if (!groups_.empty()) base_lr_ = groups_.front().optimizer->meta().lr;
+    }
 
     // trait Optimizer, groups.rs:268-313
     void step(const std::vector<Tensor> &params, const std::vector<Tensor> &grads)

@@ -356,6 +356,56 @@ static void decay_presets_and_known_norm_group_step()  // groups.rs:134-150, 244
     EXPECT(info.norm == 5.0 && info.clipped == 1 && info.step_count == 1);
 }
 
+static void group_checkpoint_roundtrip()  // checkpoint.rs:38-105 with groups.rs:320-420 as the OptimState
+{
+    if (g_checkpoint_dir.empty()) return;
+    const std::string dir = g_checkpoint_dir + "/groups";
+    Mat w({2.0, -1.0}), b({3.0}), gw({0.5, 0.25}), gb({1.0});
+    const std::vector<std::pair<std::string, Tensor>> named = {{"l.weight", w.tensor()}, {"l.bias", b.tensor()}};
+    const std::vector<std::string> names = {"l.weight", "l.bias"};
+    auto make = [&](const std::vector<std::pair<std::string, Tensor>> &n) {
+        const ParamGroupConfig plain =
+            ParamGroupConfig::sgd("plain", ParamSelector::Any({{ParamMatch::Suffix, "bias"}}), 0.5, 0.9, 0.0);
+        const ParamGroupConfig decay = ParamGroupConfig::adamw("decay", ParamSelector::All(), 0.01, 0.1);
+        return GroupOptimizer::from_named_params(n, {plain}, &decay, NBO_DT_F64);
+    };
+    GroupOptimizer opt = make(named);
+    opt.step({w.tensor(), b.tensor()}, {gw.tensor(), gb.tensor()});
+    opt.step({w.tensor(), b.tensor()}, {gw.tensor(), gb.tensor()});
+    TensorList module({w.tensor(), b.tensor()});
+    const ScheduleState sched{0.5, LrSchedule::cosine(1, 10, 0.0)};
+    save_checkpoint(dir, module, names, opt, nullptr, &sched, TrainState{1, 2, 1, std::nullopt});
+
+    Mat w2({0.0, 0.0}), b2({0.0});
+    GroupOptimizer opt2 = make({{"l.weight", w2.tensor()}, {"l.bias", b2.tensor()}});
+    TensorList module2({w2.tensor(), b2.tensor()});
+    std::optional<ScheduleState> schedule2;
+    TrainState state2;
+    load_checkpoint(dir, module2, names, opt2, nullptr, schedule2, state2);
+    EXPECT(w2.get(0) == w.get(0) && w2.get(1) == w.get(1) && b2.get() == b.get());
+    EXPECT(state2.epoch == 1 && state2.step == 2 && !state2.rng_state && schedule2 && schedule2->base_lr == 0.5);
+    EXPECT(opt2.group_optimizer(1).step_count() == 2 && opt2.group_optimizer(0).meta().momentum == 0.9);
+    double m1[2] = {0, 0}, m2[2] = {0, 0}, v1 = 0, v2 = 0;
+    opt.group_optimizer(1).state_read("m0", m1, 2, false), opt2.group_optimizer(1).state_read("m0", m2, 2, false);
+    opt.group_optimizer(0).state_read("v0", &v1, 1, false), opt2.group_optimizer(0).state_read("v0", &v2, 1, false);
+    EXPECT(m1[0] == m2[0] && m1[1] == m2[1] && m1[1] != 0.0 && v1 == v2 && v1 != 0.0);
+    // one more step on both: the same parameters
+    opt.step({w.tensor(), b.tensor()}, {gw.tensor(), gb.tensor()});
+    opt2.step({w2.tensor(), b2.tensor()}, {gw.tensor(), gb.tensor()});
+    EXPECT(w2.get(0) == w.get(0) && w2.get(1) == w.get(1) && b2.get() == b.get());
+    // a checkpoint with another group layout is refused with the reference's error
+    const ParamGroupConfig all = ParamGroupConfig::adamw("decay", ParamSelector::All(), 0.01, 0.1);
+    GroupOptimizer one = GroupOptimizer::from_named_params({{"l.weight", w2.tensor()}, {"l.bias", b2.tensor()}}, {}, &all,
+                                                           NBO_DT_F64);
+    std::string what;
+    try {
+        load_checkpoint(dir, module2, names, one, nullptr, schedule2, state2);
+    } catch (const CheckpointError &e) {
+        what = e.what();
+    }
+    EXPECT(what.find("group index out of range: 1") != std::string::npos);
+}
+
 static void constructors_and_set_state()  // alg.rs:41-45, 90-105, 244-250, 374-378; core.rs:12-16
 {
     Mat p({1.0, 2.0}), g({1.0, 1.0});
@@ -426,6 +476,7 @@ int main(int argc, char **argv)
                  {"backend_axpy_is_multiply_then_add", backend_axpy_is_multiply_then_add},
                  {"checkpoint_roundtrip_with_schedule", checkpoint_roundtrip_with_schedule},
                  {"panics_and_errors", panics_and_errors},
+                 {"group_checkpoint_roundtrip", group_checkpoint_roundtrip},
                  {"constructors_and_set_state", constructors_and_set_state},
                  {"decay_presets_and_known_norm_group_step", decay_presets_and_known_norm_group_step}};
     try {

@@ -40,7 +40,7 @@ def test_cpp_replay_of_reference_tests(gpu, tmp_path):
     r = subprocess.run([BIN, str(tmp_path)], capture_output=True, text=True, timeout=120)
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count("ok    ") == 16 and "0 failure(s)" in r.stdout
+    assert r.stdout.count("ok    ") == 17 and "0 failure(s)" in r.stdout
 
     # the checkpoint the C++ side left behind is the one the Python mirror writes and reads
     from nabla_amd import checkpoint as ck
@@ -48,7 +48,7 @@ def test_cpp_replay_of_reference_tests(gpu, tmp_path):
     from nabla_amd.schedule import ScheduleState, Step
     from tests import helpers as H
 
-    assert sorted(os.listdir(tmp_path)) == ["meta.txt", "optim.nbla", "params.nbla"]
+    assert sorted(os.listdir(tmp_path)) == ["groups", "meta.txt", "optim.nbla", "params.nbla"]
     shapes = [(1, 1), (1, 1)]
     opt = nb.Sgd.new(0.7, shapes, dtype="f64")
     scaler = nb.GradScaler.new()
@@ -64,3 +64,26 @@ def test_cpp_replay_of_reference_tests(gpu, tmp_path):
                        ck.TrainState(epoch=2, step=3, grad_accum=1, rng_state=42))
     for name in ("meta.txt", "params.nbla", "optim.nbla"):
         assert (other / name).read_bytes() == (tmp_path / name).read_bytes(), name
+
+    # and the GroupOptimizer checkpoint: meta.txt with the optim.group.* keys, optim.nbla with g{gi}. keys
+    from nabla_amd import groups as G
+    from nabla_amd.schedule import Cosine
+
+    gdir = tmp_path / "groups"
+    meta = (gdir / "meta.txt").read_text().splitlines()
+    assert meta[:4] == ["version=1", "epoch=1", "step=2", "grad_accum=1"]
+    assert meta[4:8] == ["optim.group.count=2", "optim.group.0.name=plain", "optim.group.0.kind=sgd", "optim.group.0.lr=0.5"]
+    assert "optim.group.0.momentum=0.9" in meta and "optim.group.1.step_count=2" in meta and meta[-1] == "scaler.enabled=0"
+    assert [n for n, _ in ck.load_tensors(str(gdir / "optim.nbla"))] == ["g0.v0", "g1.m0", "g1.v0"]
+    w, b = H.to_dev(np.zeros(2), (1, 2)), H.to_dev(np.zeros(1), (1, 1))
+    plain = G.ParamGroupConfig.sgd("plain", G.ParamSelector.Any([G.Suffix("bias")]), 0.5, 0.9, 0.0)
+    decay = G.ParamGroupConfig.adamw("decay", G.ParamSelector.All(), 0.01, 0.1)
+    gopt = G.GroupOptimizer.from_named_params([("l.weight", w), ("l.bias", b)], [plain], decay, dtype="f64")
+    params, state, schedule = ck.load_checkpoint(str(gdir), gopt, None, into=[("l.weight", w), ("l.bias", b)])
+    assert (state.epoch, state.step) == (1, 2) and schedule == ScheduleState(0.5, Cosine(1, 10, 0.0))
+    assert gopt.group_optimizers()[1].step_count() == 2
+    again = tmp_path / "groups_py"
+    ck.save_checkpoint(str(again), [("l.weight", w), ("l.bias", b)], gopt, None, schedule,
+                       ck.TrainState(epoch=1, step=2, grad_accum=1, rng_state=None), native=True)
+    for name in ("meta.txt", "params.nbla", "optim.nbla"):
+        assert (again / name).read_bytes() == (gdir / name).read_bytes(), name
