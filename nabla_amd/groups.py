@@ -9,7 +9,7 @@ from dataclasses import dataclass, field, replace
 from typing import Dict, List, Optional, Sequence, Tuple
 
 from . import _lib
-from .optim import (Adam, AdamW, GradScaler, NablaPanic, OptimMeta, OptimStateError, Sgd, TensorList,
+from .optim import (Adam, AdamW, GradScaler, NablaPanic, OptimMeta, OptimStateError, Sgd, TensorList, _ListCache,
                     _call, _shape2, rust_f64_str)
 
 
@@ -115,7 +115,7 @@ class _GroupEntry:
     name: str
     base_lr: float
     optimizer: object
-    lists: Dict[str, TensorList] = field(default_factory=dict)
+    lists: _ListCache = field(default_factory=_ListCache)  # this group's param / grad descriptors
 
 
 class GroupOptimizer:
@@ -125,7 +125,7 @@ class GroupOptimizer:
         self._groups = groups
         self._param_count = param_count
         self._base_lr = base_lr
-        self._all_grads: Optional[TensorList] = None
+        self._all_grads = _ListCache()
 
     @classmethod
     def from_named_params(cls, named: Sequence[Tuple[str, object]], groups: Sequence[ParamGroupConfig],
@@ -190,12 +190,7 @@ class GroupOptimizer:
             raise NablaPanic("nabla-train: GroupOptimizer param count mismatch")
 
     def _lists(self, group: _GroupEntry, slot: str, tensors) -> TensorList:
-        sub = [tensors[i] for i in group.indices]
-        cur = group.lists.get(slot)
-        if cur is None or any(a.data_ptr() != b.data_ptr() for a, b in zip(cur.tensors, sub)):
-            cur = TensorList(sub)
-            group.lists[slot] = cur
-        return cur
+        return group.lists.get(slot, [tensors[i] for i in group.indices])
 
     def step(self, params, grads) -> None:
         self._check(params, grads)
@@ -206,16 +201,14 @@ class GroupOptimizer:
                    zero_grads: bool = False, skip_nonfinite: bool = False) -> None:
         """The Trainer tail with one unscale / clip decision over all gradients."""
         self._check(params, grads)
-        if self._all_grads is None or any(a.data_ptr() != b.data_ptr()
-                                          for a, b in zip(self._all_grads.tensors, grads)):
-            self._all_grads = TensorList(list(grads))
+        all_grads = self._all_grads.get("g", list(grads))
         n = len(self._groups)
         opts = (C.c_void_p * n)(*[g.optimizer._handle() for g in self._groups])
         pl = (C.c_void_p * n)(*[self._lists(g, "p", params)._h for g in self._groups])
         gl = (C.c_void_p * n)(*[self._lists(g, "g", grads)._h for g in self._groups])
         flags = (_lib.STEP_ZERO_GRADS if zero_grads else 0) | (_lib.STEP_SKIP_NONFINITE if skip_nonfinite else 0)
         _call(_lib.load().nbo_fused_step_groups(n, opts, pl, gl, scaler._handle() if scaler else None,
-                                                self._all_grads._h, float(max_norm), flags))
+                                                all_grads._h, float(max_norm), flags))
 
     def fused_step_norm(self, params, grads, sumsq: float, max_norm: float = 0.0,
                         zero_grads: bool = False) -> None:

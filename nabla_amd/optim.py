@@ -95,7 +95,8 @@ class TensorList:
         n = len(self.tensors)
         rows = _u64_array([s[0] for s in self.shapes])
         cols = _u64_array([s[1] for s in self.shapes])
-        ptrs = (C.c_void_p * max(n, 1))(*[t.data_ptr() for t in self.tensors])
+        self.ptrs = [t.data_ptr() for t in self.tensors]  # as described to the device
+        ptrs = (C.c_void_p * max(n, 1))(*self.ptrs)
         self._h = C.c_void_p()
         _call(_lib.load().nbo_list_create(n, rows, cols, dtype, ptrs, C.byref(self._h)))
 
@@ -111,9 +112,10 @@ class TensorList:
         for t in tensors:
             if hasattr(t, "is_contiguous") and not t.is_contiguous():
                 raise ValueError("tensors must be contiguous (row-major, as in the reference)")
-        ptrs = (C.c_void_p * max(len(tensors), 1))(*[t.data_ptr() for t in tensors])
+        new_ptrs = [t.data_ptr() for t in tensors]
+        ptrs = (C.c_void_p * max(len(tensors), 1))(*new_ptrs)
         _call(_lib.load().nbo_list_set_ptrs(self._h, ptrs))
-        self.tensors = tensors
+        self.tensors, self.ptrs = tensors, new_ptrs
 
     def __len__(self):
         return len(self.tensors)
@@ -138,13 +140,12 @@ class _ListCache:
             return tensors
         tensors = list(tensors)
         cur = self._last.get(slot)
+        # compared with what the list was built from, not with its tensor objects as they are
+        # now: the same object may have been resized or given other storage since
         if cur is not None and len(cur) == len(tensors) and all(
-                a is b or (a.data_ptr() == b.data_ptr() and _shape2(a) == _shape2(b)
-                           and a.dtype == b.dtype)
-                for a, b in zip(cur.tensors, tensors)):
-            return cur
-        if cur is not None and len(cur) == len(tensors) and all(
-                _shape2(a) == _shape2(b) and a.dtype == b.dtype for a, b in zip(cur.tensors, tensors)):
+                s == _shape2(b) and _dtype_code(b) == cur.dtype for s, b in zip(cur.shapes, tensors)):
+            if all(p == b.data_ptr() for p, b in zip(cur.ptrs, tensors)):
+                return cur
             cur.rebind(tensors)  # same layout, new addresses (fresh gradient tensors every step)
             return cur
         cur = TensorList(tensors)

@@ -642,6 +642,37 @@ def test_list_rebind_follows_moved_tensors(gpu):
         plist.rebind(H.dev_list([p0[0]], [shapes[0]]))
 
 
+def test_a_tensor_object_given_other_storage_is_followed(gpu):
+    """Tensors passed as plain sequences are described to the device once and the description
+    reused; reuse is decided by the addresses and shapes the description was built from, so
+    the same tensor object pointing at other storage (`t.data = ...`) is picked up -- for a
+    plain optimizer and for a GroupOptimizer's per-group lists."""
+    import torch
+
+    from nabla_amd import groups as G
+
+    shapes = [(2, 3), (1, 9000)]
+    p0, g0 = H.randn_list(shapes, 95, 0.05), H.randn_list(shapes, 96, 1e-2)
+    for grouped in (False, True):
+        params, grads = H.dev_list(p0, shapes), H.dev_list(g0, shapes)
+        if grouped:
+            cfg = G.ParamGroupConfig.sgd("all", G.ParamSelector.All(), 0.1, 0.0, 0.0)
+            opt = G.GroupOptimizer.from_named_params(list(zip(["a", "b"], params)), [], cfg)
+        else:
+            opt = nb.Sgd.new(0.1, shapes)
+        opt.step(params, grads)
+        first = [t.clone() for t in params]
+        old_storage = [t.data for t in params]
+        for t, a in zip(params, p0):  # same objects, other memory, the start values again
+            t.data = H.to_dev(a, tuple(t.shape))
+        assert all(t.data_ptr() != o.data_ptr() for t, o in zip(params, old_storage))
+        opt.step(params, grads)
+        want = H.copy_list(p0)
+        O.sgd_step(O.sgd_meta(0.1), want, g0, H.zeros_like_list(p0))
+        H.assert_bits_equal(H.host_list(params), want, f"new storage stepped once (grouped={grouped})")
+        assert all(torch.equal(a, b) for a, b in zip(old_storage, first)), "old storage left alone"
+
+
 def test_two_host_threads_drive_two_optimizers(gpu):
     """Entry points may be called from several threads (ctypes drops the GIL around each
     call, so the calls do overlap in time); the library runs them one at a time and each
