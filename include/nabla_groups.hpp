@@ -227,7 +227,7 @@ private:
         double base_lr;
         std::shared_ptr<Optimizer> optimizer;
         std::shared_ptr<TensorList> params, grads;
-        std::vector<const void *> pkey, gkey;
+        std::vector<uint64_t> pkey, gkey;
     };
     static std::shared_ptr<Optimizer> make(const ParamGroupConfig &c, const Shapes &shapes, nbo_dtype dt, bool master)
     {
@@ -251,10 +251,16 @@ private:
         for (Entry &g : groups_) h.push_back(g.optimizer->handle());
         return h;
     }
-    static std::vector<const void *> key_of(const std::vector<Tensor> &t)
+    // what a list was built from: address, shape and element type of every tensor
+    static std::vector<uint64_t> key_of(const std::vector<Tensor> &t)
     {
-        std::vector<const void *> k;
-        for (const Tensor &x : t) k.push_back(x.data);
+        std::vector<uint64_t> k;
+        for (const Tensor &x : t) {
+            k.push_back((uint64_t)(uintptr_t)x.data);
+            k.push_back(x.rows);
+            k.push_back(x.cols);
+            k.push_back((uint64_t)x.dtype);
+        }
         return k;
     }
     void bind(const std::vector<Tensor> &params, const std::vector<Tensor> &grads)
@@ -272,7 +278,7 @@ private:
     size_t param_count_ = 0;
     double base_lr_ = 1.0;
     std::shared_ptr<TensorList> all_grads_;
-    std::vector<const void *> all_key_;
+    std::vector<uint64_t> all_key_;
 };
 
 } // namespace optim
