@@ -110,7 +110,11 @@ const char *nbo_version(void);
 /* `dev_ptrs[i]` is the device address of tensor i (RtcStorage buffer of the HIP
  * backend, common/rtc.rs:34-37), rows[i] x cols[i] elements of `dtype`.  The
  * packed descriptor is built and uploaded once; nbo_list_set_ptrs re-uploads the
- * addresses when the caller's tensors have moved. */
+ * addresses when the caller's tensors have moved.  Both check every address against
+ * what the HIP runtime knows about it -- device-accessible memory, the tensor ending
+ * inside its allocation -- and return NBO_ERR_ARG otherwise (a host pointer or an
+ * oversized shape would fault the GPU); NBO_CHECK_POINTERS=0 in the environment skips
+ * that.  The same holds for the device buffers of nbo_optim_state_read / _write. */
 int nbo_list_create(uint64_t n_tensors, const uint64_t *rows, const uint64_t *cols, int dtype,
                     const void *const *dev_ptrs, nbo_list **out);
 int nbo_list_set_ptrs(nbo_list *list, const void *const *dev_ptrs);

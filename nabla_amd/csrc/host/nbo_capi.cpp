@@ -1,4 +1,5 @@
 // extern "C" entry points of include/nabla_optim.h.
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -198,6 +199,43 @@ uint32_t state_part_index(const nbo_optim *opt, char which)
     return which == 'm' ? 0 : opt->arena.part_v;
 }
 
+// A kernel that is handed a host address, or a shape larger than the allocation behind the
+// address, faults the GPU -- which can take the whole machine's GPUs down with it -- so every
+// tensor is checked against what the HIP runtime knows about its address before a list is
+// (re)bound: the address must be device-accessible memory the runtime has allocated or
+// registered, and the tensor must end inside that allocation.  (An allocator that hands out
+// pieces of a larger block is only checked against the block.)  NBO_CHECK_POINTERS=0 in the
+// environment skips the check.
+bool pointer_checks_enabled()
+{
+    static const bool on = [] {
+        const char *v = std::getenv("NBO_CHECK_POINTERS");
+        return !(v && v[0] == '0' && v[1] == '\0');
+    }();
+    return on;
+}
+
+void check_tensor_address(const void *ptr, uint64_t bytes, uint64_t t)
+{
+    char where[64];
+    std::snprintf(where, sizeof(where), "tensor %llu at %p", (unsigned long long)t, ptr);
+    hipPointerAttribute_t attr;
+    const hipError_t e = hipPointerGetAttributes(&attr, ptr);
+    if (e != hipSuccess) (void)hipGetLastError();
+    if (e != hipSuccess || attr.type == hipMemoryTypeUnregistered)
+        fail(NBO_ERR_ARG, std::string(where) + ": not memory the HIP runtime knows (a host pointer?)");
+    hipDeviceptr_t base = nullptr;
+    size_t size = 0;
+    if (hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)ptr) != hipSuccess) {
+        (void)hipGetLastError(); // not every kind of memory has a range to ask for: nothing to compare with
+        return;
+    }
+    const uintptr_t end = (uintptr_t)base + size, p = (uintptr_t)ptr;
+    if (p < (uintptr_t)base || bytes > end - p)
+        fail(NBO_ERR_ARG, std::string(where) + ": " + std::to_string(bytes) + " bytes do not fit the allocation (" +
+                              std::to_string(end - p) + " bytes from there to its end)");
+}
+
 // Copies the n elements of tensor i's part `part` between the arena and a dense
 // buffer.
 void part_copy(nbo_optim *opt, uint64_t i, uint32_t part, void *buf, bool on_device, bool to_engine)
@@ -207,6 +245,7 @@ void part_copy(nbo_optim *opt, uint64_t i, uint32_t part, void *buf, bool on_dev
     const size_t bytes = (size_t)opt->layout.n[i] * eb;
     if (bytes == 0) return;
     char *dev = (char *)opt->arena.part[part] + (size_t)opt->layout.soff[i] * eb;
+    if (on_device && pointer_checks_enabled()) check_tensor_address(buf, bytes, i);
     if (on_device)
         hip_check(hipMemcpyAsync(to_engine ? (void *)dev : buf, to_engine ? buf : (void *)dev, bytes,
                                  hipMemcpyDeviceToDevice, rt.stream()),
@@ -310,10 +349,13 @@ static void list_upload_ptrs(nbo_list *list, const void *const *dev_ptrs)
 {
     const uint64_t nt = list->layout.nt();
     require(nt == 0 || dev_ptrs != nullptr, NBO_ERR_ARG, "null pointer array");
+    const uint64_t eb = list->dtype == NBO_DT_F64 ? 8 : is_half(list->dtype) ? 2 : 4;
     std::vector<uint64_t> ptrs(nt);
     for (uint64_t t = 0; t < nt; t++) {
         require(dev_ptrs[t] != nullptr || list->layout.n[t] == 0, NBO_ERR_ARG,
                 "null device address for a non-empty tensor");
+        if (list->layout.n[t] && pointer_checks_enabled())
+            check_tensor_address(dev_ptrs[t], list->layout.n[t] * eb, t);
         ptrs[t] = (uint64_t)(uintptr_t)dev_ptrs[t];
     }
     if (nt) Runtime::get().upload(list->ptrs_dev, ptrs.data(), nt * 8);

@@ -333,6 +333,23 @@ static void panics_and_errors()  // alg.rs:110-119, 531-545; tensor/ops.rs:638-6
     }
     EXPECT(what == "bad tensor key: mx");
     EXPECT(p.get() == 1.0);  // nothing ran
+    // addresses are checked against what the HIP runtime knows before any kernel sees them
+    double on_host = 0.0;
+    what.clear();
+    try {
+        TensorList bad({Tensor{&on_host, 1, 1, NBO_DT_F64}});
+    } catch (const RuntimeError &e) {
+        what = e.what();
+    }
+    EXPECT(what.find("not memory the HIP runtime knows") != std::string::npos);
+    what.clear();
+    try {
+        TensorList bad({Tensor{g2.d, 1, 3, NBO_DT_F64}});  // a 2-element allocation described as 3 elements
+    } catch (const RuntimeError &e) {
+        what = e.what();
+    }
+    EXPECT(what.find("do not fit the allocation") != std::string::npos);
+    TensorList fits({Tensor{g2.d + 1, 1, 1, NBO_DT_F64}});  // an interior address that ends inside
 }
 
 static void decay_presets_and_known_norm_group_step()  // groups.rs:134-150, 244-261

@@ -673,6 +673,31 @@ def test_a_tensor_object_given_other_storage_is_followed(gpu):
         assert all(torch.equal(a, b) for a, b in zip(old_storage, first)), "old storage left alone"
 
 
+def test_host_tensors_and_short_allocations_are_refused_before_any_launch(gpu):
+    """A list is checked against what the HIP runtime knows about each address when it is
+    bound: a CPU tensor and a state buffer in host memory passed as a device buffer are
+    errors, not GPU faults."""
+    import torch
+
+    shapes = [(2, 3)]
+    cpu = [torch.zeros(s) for s in shapes]
+    with pytest.raises(Exception, match="not memory the HIP runtime knows"):
+        nb.TensorList(cpu)
+    good = nb.TensorList([torch.zeros(s, device="cuda:0") for s in shapes])
+    with pytest.raises(Exception, match="not memory the HIP runtime knows"):
+        good.rebind(cpu)
+    opt = nb.Adam.new(1e-3, shapes)
+    from nabla_amd import _lib
+
+    host = torch.zeros(6)
+    rc = _lib.load().nbo_optim_state_write(opt._handle(), b"m0", host.data_ptr(), 6, 1)
+    assert rc == _lib.ERR_ARG and b"not memory the HIP runtime knows" in _lib.load().nbo_last_error()
+    # pinned host memory is device-accessible and passes
+    pinned = torch.zeros(6, pin_memory=True)
+    assert _lib.load().nbo_optim_state_write(opt._handle(), b"m0", pinned.data_ptr(), 6, 1) == 0
+    nb.sync()
+
+
 def test_two_host_threads_drive_two_optimizers(gpu):
     """Entry points may be called from several threads (ctypes drops the GIL around each
     call, so the calls do overlap in time); the library runs them one at a time and each
