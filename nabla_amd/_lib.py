@@ -153,6 +153,15 @@ def load() -> C.CDLL:
             f"{LIB_PATH} is missing: build it with `make -C nabla_amd/csrc` "
             "(or `python -c 'import __graft_entry__ as g; g.build()'`). "
             "There is no fallback path.")
+    # A process must hold one HIP runtime.  PyTorch's ROCm wheels carry their own copy of it,
+    # and if this library pulls in the system's copy first, torch finds no GPU afterwards; with
+    # torch loaded first the library binds to the copy torch brought.  So where torch is
+    # installed it is imported before the library is opened (callers that never use torch are
+    # not affected: without it the system's runtime is the only one).
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = C.CDLL(LIB_PATH)
     for name, (restype, argtypes) in SYMBOLS.items():
         fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
