@@ -61,22 +61,23 @@ def adam_case(kind):
     return out
 
 
-def mixed_case():
-    """bf16 params/grads, f32 master/m/v, scaler (growth every 2 clean steps), clip 1.0,
-    6 steps, +inf injected at step 3."""
+def mixed_case(half="bf16"):
+    """bf16 (uint16 patterns) or f16 (float16) params/grads, f32 master/m/v, scaler (growth
+    every 2 clean steps), clip 1.0, 6 steps, +inf injected at step 3."""
+    narrow = O.bf16_from_f32 if half == "bf16" else (lambda a: O.cast(a, np.float16))
     master = {m: [O.randn_f32(r * c, 500 + i, 0.02) for i, (r, c) in enumerate(SHAPES)] for m in (0, 1)}
     out = {f"w0_{i}": a.copy() for i, a in enumerate(master[0])}
-    pb = {m: [O.bf16_from_f32(a) for a in master[m]] for m in (0, 1)}
+    pb = {m: [narrow(a) for a in master[m]] for m in (0, 1)}
     st = {m: ([np.zeros_like(a) for a in master[m]], [np.zeros_like(a) for a in master[m]]) for m in (0, 1)}
     metas = {m: O.adamw_meta(2e-4, 0.9, 0.95, 1e-8, 0.1) for m in (0, 1)}
     scal = {m: O.ScalerState(65536.0, 2.0, 0.5, 2, 0) for m in (0, 1)}
     trace = []
     for step in range(6):
         scale = scal[0].scale
-        g = [O.bf16_from_f32(O.randn_f32(r * c, 600 + 10 * step + i, 1e-3 * scale))
+        g = [narrow(O.randn_f32(r * c, 600 + 10 * step + i, 1e-3 * scale))
              for i, (r, c) in enumerate(SHAPES)]
         if step == 3:
-            g[2][77] = 0x7F80
+            g[2][77] = 0x7F80 if half == "bf16" else np.inf
         for i, a in enumerate(g):
             out[f"g{step}_{i}"] = a
         for mode in (0, 1):
@@ -98,6 +99,7 @@ def main():
     np.savez_compressed(os.path.join(HERE, "adam_f32.npz"), **adam_case("adam"))
     np.savez_compressed(os.path.join(HERE, "adamw_f32.npz"), **adam_case("adamw"))
     np.savez_compressed(os.path.join(HERE, "mixed_adamw_bf16.npz"), **mixed_case())
+    np.savez_compressed(os.path.join(HERE, "mixed_adamw_f16.npz"), **mixed_case("f16"))
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

@@ -59,10 +59,15 @@ def test_oracle_reproduces_adam_fixture(kind):
                 assert O.ulp_distance_f32(p[i], d[f"{key}_{i}"]).max() <= 2
 
 
-def test_oracle_reproduces_mixed_fixture():
-    d = _load("mixed_adamw_bf16.npz")
+def _narrow(a, half):
+    return O.bf16_from_f32(a) if half == "bf16" else O.cast(a, np.float16)
+
+
+@pytest.mark.parametrize("half", ["bf16", "f16"])
+def test_oracle_reproduces_mixed_fixture(half):
+    d = _load(f"mixed_adamw_{half}.npz")
     w = [d[f"w0_{i}"].copy() for i in range(N)]
-    p = [O.bf16_from_f32(a) for a in w]
+    p = [_narrow(a, half) for a in w]
     m, v = [np.zeros_like(a) for a in w], [np.zeros_like(a) for a in w]
     meta, s = O.adamw_meta(2e-4, 0.9, 0.95, 1e-8, 0.1), O.ScalerState(65536.0, 2.0, 0.5, 2, 0)
     O.set_pow_mode(O.POW_SQRT)
@@ -78,8 +83,12 @@ def test_oracle_reproduces_mixed_fixture():
     for i in range(N):
         assert _bits_equal(p[i], d[f"p_sqrt_{i}"]) and _bits_equal(w[i], d[f"w_sqrt_{i}"])
         assert _bits_equal(m[i], d[f"m_{i}"]) and _bits_equal(v[i], d[f"v_{i}"])
-        assert O.ulp_distance_bf16(d[f"p_libm_{i}"], d[f"p_sqrt_{i}"]).max() <= 1
-        assert O.ulp_distance_f32(d[f"w_libm_{i}"], d[f"w_sqrt_{i}"]).max() <= 2
+        assert O.ulp_distance_bf16(d[f"p_libm_{i}"].view(np.uint16), d[f"p_sqrt_{i}"].view(np.uint16)).max() <= 1
+        # the two lowerings of powf differ by an ulp of the update; where decay and update nearly
+        # cancel that is more than 2 ulp of the small result, and bounded by steps * 8 * lr * 2^-23
+        far = O.ulp_distance_f32(d[f"w_libm_{i}"], d[f"w_sqrt_{i}"]) > 2
+        assert np.abs(d[f"w_libm_{i}"][far].astype(np.float64) - d[f"w_sqrt_{i}"][far]).max(initial=0.0) \
+            <= 6 * 8 * 2e-4 * 2.0 ** -23
 
 
 # ---- GPU: HIP engine vs fixture ------------------------------------------------------------------
@@ -118,13 +127,14 @@ def test_device_matches_adam_fixture(gpu, kind):
 
 
 @pytest.mark.gpu
-def test_device_matches_mixed_fixture(gpu):
+@pytest.mark.parametrize("half", ["bf16", "f16"])
+def test_device_matches_mixed_fixture(gpu, half):
     from nabla_amd import optim as nb
     from tests import helpers as H
 
-    d = _load("mixed_adamw_bf16.npz")
+    d = _load(f"mixed_adamw_{half}.npz")
     w0 = [d[f"w0_{i}"] for i in range(N)]
-    p = H.dev_list([O.bf16_from_f32(a) for a in w0], SHAPES)
+    p = H.dev_list([_narrow(a, half) for a in w0], SHAPES)
     opt = nb.AdamW.new(2e-4, SHAPES, master=True).beta2(0.95).weight_decay(0.1)
     for i in range(N):
         opt.write_state(f"w{i}", H.to_dev(w0[i], SHAPES[i]))
@@ -139,10 +149,10 @@ def test_device_matches_mixed_fixture(gpu):
     assert [t.step_count for t in tr] == [int(x) for x in d["trace"][:, 2]]
     for t, ref in zip(tr, d["trace"][:, 3]):
         assert t.norm == pytest.approx(ref, rel=1e-12)
-    H.assert_bits_equal(H.host_list(p), [d[f"p_sqrt_{i}"] for i in range(N)], "bf16 params")
+    H.assert_bits_equal(H.host_list(p), [d[f"p_sqrt_{i}"] for i in range(N)], "16-bit params")
     H.assert_bits_equal(H.host_list([opt.read_state(f"w{i}") for i in range(N)]),
                         [d[f"w_sqrt_{i}"] for i in range(N)], "master")
     m, v = opt.moments()
     H.assert_bits_equal(H.host_list(m), [d[f"m_{i}"] for i in range(N)], "m")
     H.assert_bits_equal(H.host_list(v), [d[f"v_{i}"] for i in range(N)], "v")
-    assert H.max_ulp_bf16(H.host_list(p), [d[f"p_libm_{i}"] for i in range(N)]) <= 1
+    assert H.max_ulp_half(H.host_list(p), [d[f"p_libm_{i}"] for i in range(N)]) <= 1
