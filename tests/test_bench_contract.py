@@ -1,8 +1,11 @@
-"""bench.py contract checks that need no GPU."""
+"""bench.py contract checks: the ones that need no GPU, and two real runs of the measurement
+scripts on their smallest inputs."""
 import json
 import os
 import subprocess
 import sys
+
+import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -39,3 +42,35 @@ def test_traffic_file_is_consistent_with_the_profile_summary():
     assert 0.99 < total / algorithmic < 1.02
     d = t["_detail"]["per_launch_bytes"]["nbo_update_bf16_adamw"]
     assert d["fetch_bytes"] + d["write_bytes"] == total
+
+
+@pytest.mark.gpu
+def test_small_mlp_bench_line_has_the_contract_fields(gpu):
+    """One real `bench.py` run on the smallest workload: one JSON line with the fields the
+    driver reads, the roofline block and the CPU baseline."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--workload", "mlp-sgd-f32", "--steps", "20",
+                        "--warmup", "3", "--cpu-seconds", "1"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [x for x in r.stdout.splitlines() if x.strip()]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in d, key
+    assert d["n_gpus"] == 1 and d["steps"] == 20 and d["warmup"] == 3 and d["config"]["workload"] == "mlp-sgd-f32"
+    assert d["roofline"]["bound"] == "hbm" and d["roofline"]["peak"] == 8000.0 and d["roofline"]["kernel"] == "nbo_update_f32_sgd"
+    assert abs(d["roofline"]["frac"] - d["roofline"]["achieved"] / d["roofline"]["peak"]) < 1e-3
+    assert d["cpu_baseline"]["kind"] == "port" and d["cpu_baseline"]["cores"] >= 1 and d["value"] > 0
+
+
+@pytest.mark.gpu
+def test_kernel_bench_prints_a_row_for_every_measurement(gpu):
+    """`python -m nabla_amd.kernel_bench` on one tensor: every row has a positive time."""
+    r = subprocess.run([sys.executable, "-m", "nabla_amd.kernel_bench", "--elements", "1e6", "--reps", "1"],
+                       capture_output=True, text=True, timeout=300, cwd=ROOT)
+    assert r.returncode == 0, r.stderr[-2000:]
+    rows = [x for x in r.stdout.splitlines() if x.startswith("| ") and "`nbo_" in x]
+    assert len(rows) >= 45
+    for row in rows:
+        cells = [c.strip() for c in row.strip("|").split("|")]
+        assert float(cells[2]) > 0.0 and float(cells[4]) > 0.0, row
