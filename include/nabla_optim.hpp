@@ -507,13 +507,15 @@ inline double lr_at_step(const LrSchedule &s, double base_lr, uint64_t step)
         return base_lr * (p > 0.0 ? p : 0.0);
     }
     case LrSchedule::OneCycle: {
-        const uint64_t up = (uint64_t)((double)s.total_steps * s.pct_start);
+        // Rust's `as usize`: truncation toward zero, saturating at both ends, NaN -> 0
+        const double upf = (double)s.total_steps * s.pct_start;
+        const uint64_t up = !(upf > 0.0) ? 0 : upf >= 18446744073709551616.0 ? UINT64_MAX : (uint64_t)upf;
         if (step < up) return base_lr + (s.max_lr - base_lr) * (double)step / (double)(up > 1 ? up : 1);
         return cosine_decay(s.max_lr, base_lr, decay_progress(step, up, s.total_steps));
     }
     default: {
         const uint64_t sz = s.step_size > 1 ? s.step_size : 1;
-        return base_lr * powi(s.gamma, (int)(step / sz));
+        return base_lr * powi(s.gamma, (int32_t)(uint32_t)(step / sz)); // `k as i32`: the low 32 bits
     }
     }
 }

@@ -62,12 +62,32 @@ class ScheduleState:
     schedule: object
 
 
+_USIZE_MASK = (1 << 64) - 1
+
+
+def _f64_as_usize(x: float) -> int:
+    """Rust's `x as usize`: truncation toward zero, saturating at both ends, NaN -> 0."""
+    if x != x or x <= 0.0:
+        return 0
+    if x >= 18446744073709551616.0:
+        return _USIZE_MASK
+    return int(x)
+
+
+def _as_i32(k: int) -> int:
+    """Rust's `k as i32` for a usize k: the low 32 bits, reinterpreted as signed."""
+    k &= 0xFFFFFFFF
+    return k - (1 << 32) if k & 0x80000000 else k
+
+
 def _warmup_lr(base_lr, step, warmup_steps):  # core.rs:81-84
     return base_lr * float(step) / float(max(warmup_steps, 1))
 
 
 def _decay_progress(step, start, total):  # core.rs:86-89
-    return float(step - start) / float(max(total - start, 1))
+    # usize subtractions: where total < start (a schedule shorter than its warm-up) the
+    # reference's release build wraps around instead of going negative, and so does this
+    return float((step - start) & _USIZE_MASK) / float(max((total - start) & _USIZE_MASK, 1))
 
 
 def _cosine_decay(high, low, progress):  # core.rs:96-99
@@ -87,14 +107,14 @@ def lr_at_step(schedule, base_lr: float, step: int) -> float:
         progress = _decay_progress(step, schedule.warmup_steps, schedule.total_steps)
         return base_lr * max(1.0 - progress, 0.0)
     if isinstance(schedule, OneCycle):
-        up_steps = int(float(schedule.total_steps) * schedule.pct_start)
+        up_steps = _f64_as_usize(float(schedule.total_steps) * schedule.pct_start)
         if step < up_steps:
             return base_lr + (schedule.max_lr - base_lr) * float(step) / float(max(up_steps, 1))
         return _cosine_decay(schedule.max_lr, base_lr,
                              _decay_progress(step, up_steps, schedule.total_steps))
     if isinstance(schedule, Step):
         k = step // max(schedule.step_size, 1)
-        return base_lr * powi(schedule.gamma, k)
+        return base_lr * powi(schedule.gamma, _as_i32(k))
     raise TypeError(f"not an LrSchedule: {schedule!r}")
 
 

@@ -196,6 +196,14 @@ static double decay_progress(uint64_t step, uint64_t start, uint64_t total)
     return (double)(step - start) / (double)d;
 }
 
+/* Rust's `x as usize` (core.rs:161): truncation toward zero, saturating, NaN -> 0 */
+static uint64_t f64_as_usize(double x)
+{
+    if (!(x > 0.0)) return 0;
+    if (x >= 18446744073709551616.0) return UINT64_MAX;
+    return (uint64_t)x;
+}
+
 static double cosine_decay(double high, double low, double progress)
 {
     return low + 0.5 * (high - low) * (1.0 + cos(3.14159265358979323846264338327950288 * progress));
@@ -213,7 +221,7 @@ double orc_lr_at_step(const orc_schedule *s, double base_lr, uint64_t step)
         return base_lr * (p > 0.0 ? p : 0.0);
     }
     case 2: { /* OneCycle :155-167 */
-        uint64_t up = (uint64_t)((double)s->total_steps * s->b);
+        uint64_t up = f64_as_usize((double)s->total_steps * s->b);
         if (step < up) {
             uint64_t t = up > 1 ? up : 1;
             return base_lr + (s->a - base_lr) * (double)step / (double)t;
@@ -222,7 +230,7 @@ double orc_lr_at_step(const orc_schedule *s, double base_lr, uint64_t step)
     }
     default: { /* Step :168-171 */
         uint64_t sz = s->warmup_steps > 1 ? s->warmup_steps : 1;
-        return base_lr * orc_powi(s->a, (int)(step / sz));
+        return base_lr * orc_powi(s->a, (int32_t)(uint32_t)(step / sz)); /* `k as i32`: low 32 bits */
     }
     }
 }

@@ -29,12 +29,48 @@ def test_lr_schedules_match_oracle_bit_for_bit():
         (S.OneCycle(3e-3, 1000, 0.3), O.Schedule(2, 0, 1000, 3e-3, 0.3), 3e-4),
         (S.Step(2, 0.1), O.Schedule(3, 2, 0, 0.1, 0.0), 1.0),
         (S.Step(0, 0.5), O.Schedule(3, 0, 0, 0.5, 0.0), 1.0),
+        # a schedule shorter than its warm-up: `total - start` is a usize subtraction that wraps
+        # in the reference's release build (core.rs:87-89)
+        (S.Cosine(10, 5, 0.1), O.Schedule(0, 10, 5, 0.1, 0.0), 1.0),
+        (S.Linear(10, 5), O.Schedule(1, 10, 5, 0.0, 0.0), 1.0),
+        (S.Cosine(7, 7, 0.1), O.Schedule(0, 7, 7, 0.1, 0.0), 1.0),  # total == warm-up: max(0, 1)
+        # pct_start beyond 1, zero, negative and NaN: `(total as f64 * pct) as usize` saturates
+        (S.OneCycle(1.0, 10, 1.5), O.Schedule(2, 0, 10, 1.0, 1.5), 0.1),
+        (S.OneCycle(1.0, 10, 0.0), O.Schedule(2, 0, 10, 1.0, 0.0), 0.1),
+        (S.OneCycle(1.0, 10, -0.5), O.Schedule(2, 0, 10, 1.0, -0.5), 0.1),
+        (S.OneCycle(1.0, 10, float("nan")), O.Schedule(2, 0, 10, 1.0, float("nan")), 0.1),
+        (S.OneCycle(1.0, 10, 1e30), O.Schedule(2, 0, 10, 1.0, 1e30), 0.1),
     ]
     for sched, osched, base in cases:
         total = getattr(sched, "total_steps", 40)
-        for step in list(range(0, min(total, 60) + 1)) + [total]:
+        warm = getattr(sched, "warmup_steps", 0)
+        steps = set(range(0, min(total, 60) + 1)) | {total, max(warm - 1, 0), warm, warm + 1, 11, 25}
+        for step in sorted(steps):
             a, b = S.lr_at_step(sched, base, step), O.lr_at_step(osched, base, step)
             assert np.float64(a).tobytes() == np.float64(b).tobytes(), (sched, step, a, b)
+
+
+def test_lr_schedule_edges_in_closed_form():
+    """What the wrapped subtraction and the saturating cast must give, derived by hand and
+    not from either mirror: with total < warm-up the decay's denominator is 2^64 - (warm-up -
+    total), the progress is ~1e-19, cos(pi * progress) is exactly 1 in f64 and the cosine
+    decay returns low + 0.5 * (high - low) * 2; the linear decay gives base * (1 - ~1e-19)
+    = base.  pct_start = 1.5 ramps for 15 of 10 steps; pct_start <= 0 or NaN ramps for
+    none."""
+    for lr_fn in (S.lr_at_step, lambda s, b, k: O.lr_at_step(
+            O.Schedule({S.Cosine: 0, S.Linear: 1, S.OneCycle: 2}[type(s)], getattr(s, "warmup_steps", 0),
+                       s.total_steps, getattr(s, "min_lr", getattr(s, "max_lr", 0.0)),
+                       getattr(s, "pct_start", 0.0)), b, k)):
+        assert lr_fn(S.Cosine(10, 5, 0.1), 1.0, 11) == 0.1 + 0.5 * (1.0 - 0.1) * 2.0
+        assert lr_fn(S.Cosine(10, 5, 0.1), 1.0, 9) == 1.0 * 9.0 / 10.0
+        assert lr_fn(S.Linear(10, 5), 0.5, 12) == 0.5
+        assert lr_fn(S.Cosine(7, 7, 0.25), 1.0, 7) == 0.25 + 0.5 * 0.75 * 2.0  # progress 0 / 1
+        assert lr_fn(S.OneCycle(1.0, 10, 1.5), 0.1, 12) == 0.1 + (1.0 - 0.1) * 12.0 / 15.0
+        for pct in (0.0, -0.5, float("nan")):
+            assert lr_fn(S.OneCycle(1.0, 10, pct), 0.1, 0) == 1.0  # no ramp: cosine from max_lr at progress 0
+        # k as i32 keeps the low 32 bits: step 2^32 with step_size 1 is gamma^0
+    assert S.lr_at_step(S.Step(1, 0.5), 1.0, 1 << 32) == 1.0
+    assert O.lr_at_step(O.Schedule(3, 1, 0, 0.5, 0.0), 1.0, 1 << 32) == 1.0
 
 
 def test_lr_schedule_reference_points():
