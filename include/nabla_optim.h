@@ -211,6 +211,22 @@ int nbo_scale_grad(nbo_list *grads, double factor);
  * is taken on the device; nothing is read back.  Asynchronous. */
 int nbo_fused_step(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, nbo_list *grads,
                    double max_norm, uint32_t flags);
+/* nbo_fused_step for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in
+ * the reference.  Same arguments, same three launches and bit-identical results; the only
+ * difference is where the norm pass keeps its per-workgroup partial results: not in the
+ * buffer nbo_init allocated but in a 32 KiB array that is part of the library's device image
+ * (one copy per GPU, held until the process ends).  The call itself makes no hipMalloc /
+ * hipFree and creates no events (nbo_profile_enable does not time its launches); the handles
+ * it takes were created, with their allocations, beforehand.
+ * Limit: the norm pass may use at most NBO_NOALLOC_MAX_PARTIALS (2048) workgroups, which is
+ * also the grid cap of the ordinary entry point, so every list the library accepts fits;
+ * a library rebuilt with a larger cap returns NBO_ERR_TOO_LARGE here instead of overrunning
+ * the array.  All calls on one GPU share the array: it keeps the previous call's contents
+ * (every slot a call reads is first written by that call, so nothing needs clearing), and two
+ * calls that overlap on one GPU -- different streams or threads -- race on it.  Asynchronous. */
+int nbo_fused_step_noalloc(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, nbo_list *grads,
+                           double max_norm, uint32_t flags);
 /* The same tail for GroupOptimizer (optim/groups.rs:269-293): one unscale / found-inf /
  * clip decision over `all_grads` (every gradient, in the module's order), then each
  * group's update with its own hyper-parameters.  params[g] / grads[g] are the lists of

@@ -108,6 +108,7 @@ SYMBOLS = {
     "nbo_zero_grad": (C.c_int, [_P]),
     "nbo_scale_grad": (C.c_int, [_P, C.c_double]),
     "nbo_fused_step": (C.c_int, [_P, _P, _P, _P, C.c_double, C.c_uint32]),
+    "nbo_fused_step_noalloc": (C.c_int, [_P, _P, _P, _P, C.c_double, C.c_uint32]),
     "nbo_fused_step_groups": (C.c_int, [C.c_uint64, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), _P, _P,
                                         C.c_double, C.c_uint32]),
     "nbo_accumulate": (C.c_int, [_P, _P, C.c_int]),

@@ -6,6 +6,7 @@
 #include <new>
 
 #include "nbo_host.hpp"
+#include "nbo_noalloc.hpp"
 
 using namespace nbo;
 
@@ -135,15 +136,24 @@ uint32_t norm_grid(const Layout &L)
 
 // First stage of the norm / found_inf pass over `grads`; partials land in the
 // runtime's scratch.  Returns the grid used (0 for an empty list).
-uint32_t launch_norm(nbo_list *grads, const NboScalerDev *scaler, bool half_arithmetic = false)
+// Where a norm pass leaves its per-workgroup partial results for the finalize launch.
+struct NormScratch {
+    double *partial_sumsq;  // [NBO_NORM_GRID_MAX]
+    uint32_t *partial_flag; // [NBO_NORM_GRID_MAX]
+    bool may_time;          // launches may be bracketed by timing events
+};
+
+NormScratch runtime_scratch(Runtime &rt) { return NormScratch{rt.partial_sumsq(), rt.partial_flag(), true}; }
+
+uint32_t launch_norm(nbo_list *grads, const NboScalerDev *scaler, bool half_arithmetic, const NormScratch &ws)
 {
     Runtime &rt = Runtime::get();
     NboNormArgs a = {};
     a.L = grads->layout.dev;
     a.g_ptrs = grads->ptrs_dev;
     a.scaler = scaler;
-    a.partial_sumsq = rt.partial_sumsq();
-    a.partial_flag = rt.partial_flag();
+    a.partial_sumsq = ws.partial_sumsq;
+    a.partial_flag = ws.partial_flag;
     a.grid = norm_grid(grads->layout);
     // bf16 / f16 gradients are unscaled in f32 when they feed f32 state (the mixed-precision
     // composition) and in their own type when the optimizer itself is of that type or they are
@@ -151,8 +161,37 @@ uint32_t launch_norm(nbo_list *grads, const NboScalerDev *scaler, bool half_arit
     int k = kernel_for(K_NORM_BASE, K_NORM_F16, grads->dtype);
     if (half_arithmetic && grads->dtype == NBO_DT_BF16) k = K_NORM_PBF16;
     if (half_arithmetic && grads->dtype == NBO_DT_F16) k = K_NORM_PF16;
-    rt.launch(k, a.grid, NBO_BLOCK, a);
+    rt.launch_raw(k, a.grid, NBO_BLOCK, &a, ws.may_time);
     return a.grid;
+}
+
+uint32_t launch_norm(nbo_list *grads, const NboScalerDev *scaler, bool half_arithmetic = false)
+{
+    return launch_norm(grads, scaler, half_arithmetic, runtime_scratch(Runtime::get()));
+}
+
+// The three launches of one fused Trainer tail; `ws` is where the norm pass's partial results
+// travel from the first launch to the second.
+void fused_step_launches(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, nbo_list *grads, double max_norm,
+                         uint32_t flags, const NormScratch &ws)
+{
+    Runtime &rt = Runtime::get();
+    NboFinalizeArgs f = {};
+    f.partial_sumsq = ws.partial_sumsq;
+    f.partial_flag = ws.partial_flag;
+    // without scaler, clipping and nan policy the pass has nothing to decide, but
+    // it still runs so that the trace records every step
+    f.grid = launch_norm(grads, scaler ? scaler->dev : nullptr, pure_half(opt), ws);
+    f.check_finite = (scaler || (flags & NBO_STEP_SKIP_NONFINITE)) ? 1u : 0u;
+    f.scaler = scaler ? scaler->dev : nullptr;
+    f.gf = opt->gf;
+    f.opt = opt->dev;
+    f.trace = opt->trace;
+    f.max_norm = max_norm;
+    f.hyper = hyper_of(opt);
+    rt.launch_raw(K_FINALIZE, 1, NBO_BLOCK, &f, ws.may_time);
+    NboUpdateArgs a = update_args(opt, params, grads, true, (flags & NBO_STEP_ZERO_GRADS) != 0);
+    rt.launch_raw(update_kernel(opt, params), opt->layout.nchunks, NBO_BLOCK, &a, ws.may_time);
 }
 
 void launch_scale(nbo_list *grads, const NboGradFactors *gf, double factor, uint32_t mode)
@@ -783,24 +822,35 @@ int nbo_fused_step(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, nbo_lis
 {
     return guarded([&] {
         check_step_args(opt, params, grads);
-        Runtime &rt = Runtime::get();
-        NboFinalizeArgs f = {};
-        f.partial_sumsq = rt.partial_sumsq();
-        f.partial_flag = rt.partial_flag();
-        // without scaler, clipping and nan policy the pass has nothing to decide, but
-        // it still runs so that the trace records every step
-        f.grid = launch_norm(grads, scaler ? scaler->dev : nullptr, pure_half(opt));
-        f.check_finite = (scaler || (flags & NBO_STEP_SKIP_NONFINITE)) ? 1u : 0u;
-        f.scaler = scaler ? scaler->dev : nullptr;
-        f.gf = opt->gf;
-        f.opt = opt->dev;
-        f.trace = opt->trace;
-        f.max_norm = max_norm;
-        f.hyper = hyper_of(opt);
-        rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
-        const NboUpdateArgs a =
-            update_args(opt, params, grads, true, (flags & NBO_STEP_ZERO_GRADS) != 0);
-        rt.launch(update_kernel(opt, params), opt->layout.nchunks, NBO_BLOCK, a);
+        fused_step_launches(opt, scaler, params, grads, max_norm, flags, runtime_scratch(Runtime::get()));
+    });
+}
+
+int nbo_fused_step_noalloc(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, nbo_list *grads,
+                           double max_norm, uint32_t flags)
+{
+    return guarded([&] {
+        check_step_args(opt, params, grads);
+        // the handles were created through the runtime, so it exists; nothing is created here
+        Runtime *rt = Runtime::existing();
+        require(rt != nullptr, NBO_ERR_ARG, "nbo_fused_step_noalloc: the runtime does not exist (call nbo_init first)");
+        if (rt->static_scratch_status() != hipSuccess)
+            fail(NBO_ERR_HIP + (int)rt->static_scratch_status(),
+                 std::string("nbo_fused_step_noalloc: the address of the library's static device scratch could "
+                             "not be looked up at nbo_init: ") +
+                     hipGetErrorString(rt->static_scratch_status()));
+        char *ws = (char *)noalloc_scratch(rt->device());
+        require(ws != nullptr, NBO_ERR_ARG, "nbo_fused_step_noalloc: no static device scratch on this device");
+        // one partial sum and one flag per workgroup of the norm grid have to fit the array
+        const uint32_t need = norm_grid(grads->layout);
+        if (need > NBO_NOALLOC_MAX_PARTIALS)
+            fail(NBO_ERR_TOO_LARGE, "nbo_fused_step_noalloc: the norm pass over this gradient list needs " +
+                                        std::to_string(need) + " partial results, the static scratch holds " +
+                                        std::to_string(NBO_NOALLOC_MAX_PARTIALS));
+        // Every slot the finalize launch reads ([0, grid)) is written by this call's norm launch
+        // first, so nothing left behind by an earlier call needs clearing.
+        const NormScratch w = {(double *)ws, (uint32_t *)(ws + NBO_NOALLOC_FLAGS_OFFSET), false};
+        fused_step_launches(opt, scaler, params, grads, max_norm, flags, w);
     });
 }
 

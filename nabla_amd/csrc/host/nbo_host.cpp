@@ -1,6 +1,7 @@
 // Runtime, module loading, launches and descriptor building for the fused
 // optimizer-step engine.
 #include "nbo_host.hpp"
+#include "nbo_noalloc.hpp"
 
 #include <algorithm>
 #include <cstdio>
@@ -48,13 +49,20 @@ static const char *const kKernelNames[K_COUNT] = {
     "nbo_accnorm_bf16",      "nbo_accnorm_f64",      "nbo_accnorm_f16",
 };
 
+static std::mutex g_runtime_mu;
+static Runtime *g_runtime = nullptr;
+
 Runtime &Runtime::get()
 {
-    static std::mutex mu;
-    static Runtime *inst = nullptr;
-    std::lock_guard<std::mutex> lock(mu);
-    if (!inst) inst = new Runtime(); // throws Error; retried on the next call
-    return *inst;
+    std::lock_guard<std::mutex> lock(g_runtime_mu);
+    if (!g_runtime) g_runtime = new Runtime(); // throws Error; retried on the next call
+    return *g_runtime;
+}
+
+Runtime *Runtime::existing()
+{
+    std::lock_guard<std::mutex> lock(g_runtime_mu);
+    return g_runtime;
 }
 
 Runtime::Runtime()
@@ -87,6 +95,11 @@ Runtime::Runtime()
     partial_sumsq_ = (double *)dmalloc(NBO_NORM_GRID_MAX * sizeof(double));
     partial_flag_ = (uint32_t *)dmalloc(NBO_NORM_GRID_MAX * sizeof(uint32_t));
     gf_scratch_ = (NboGradFactors *)dmalloc(sizeof(NboGradFactors));
+    // The statically allocated scratch of the allocation-free entry point: its device address
+    // is looked up here, once, with the device current.  A failure is kept for that entry point
+    // to report; nothing else depends on it.
+    static_scratch_status_ = noalloc_setup(&device_);
+    if (static_scratch_status_ != hipSuccess) (void)hipGetLastError();
 }
 
 void Runtime::sync() { hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize"); }
@@ -101,19 +114,20 @@ void Runtime::set_stream(hipStream_t s)
     stream_ = s;
 }
 
-void Runtime::launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct)
+void Runtime::launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct, bool may_time)
 {
     if (grid == 0) return;
     void *args[1] = {arg_struct};
     ProfRec rec = {kernel, nullptr, nullptr};
-    if (profiling_) {
+    const bool timed = profiling_ && may_time; // timing creates two events per launch
+    if (timed) {
         hip_check(hipEventCreate(&rec.begin), "hipEventCreate");
         hip_check(hipEventCreate(&rec.end), "hipEventCreate");
         hip_check(hipEventRecord(rec.begin, stream_), "hipEventRecord");
     }
     hip_check(hipModuleLaunchKernel(fn_[kernel], grid, 1, 1, block, 1, 1, 0, stream_, args, nullptr),
               kKernelNames[kernel]);
-    if (profiling_) {
+    if (timed) {
         hip_check(hipEventRecord(rec.end, stream_), "hipEventRecord");
         prof_.push_back(rec);
     }

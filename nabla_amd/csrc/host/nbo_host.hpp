@@ -65,6 +65,7 @@ enum KernelId {
 class Runtime {
 public:
     static Runtime &get(); // creates on first use; throws Error on failure
+    static Runtime *existing(); // the runtime if it has been created, else null; creates nothing
     hipStream_t stream() const { return stream_; }
     void set_stream(hipStream_t s);
     void sync();
@@ -73,7 +74,9 @@ public:
     {
         launch_raw(kernel, grid, block, const_cast<Args *>(&args));
     }
-    void launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct);
+    // may_time = false: never bracket the launch with timing events, whatever profile_enable
+    // says (creating events allocates host memory)
+    void launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct, bool may_time = true);
     void launch_copy(const void *src, void *dst, uint64_t nvec);
     // Bandwidth (GB/s, best of three) of reading and rewriting `bytes` bytes at a and at
     // b together: the probe StatePlacement classifies HBM regions with.  Synchronous.
@@ -95,6 +98,10 @@ public:
     double *partial_sumsq() const { return partial_sumsq_; }
     uint32_t *partial_flag() const { return partial_flag_; }
     NboGradFactors *gf_scratch() const { return gf_scratch_; }
+    // the device this runtime lives on, and how the look-up of the statically allocated
+    // scratch's address went there
+    int device() const { return device_; }
+    hipError_t static_scratch_status() const { return static_scratch_status_; }
 
 private:
     Runtime();
@@ -108,6 +115,8 @@ private:
     double *partial_sumsq_ = nullptr;
     uint32_t *partial_flag_ = nullptr;
     NboGradFactors *gf_scratch_ = nullptr;
+    int device_ = 0;
+    hipError_t static_scratch_status_ = hipSuccess;
     struct ProfRec {
         int kernel;
         hipEvent_t begin, end;

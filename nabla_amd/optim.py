@@ -353,12 +353,16 @@ class _Optimizer:
     # -- the fused Trainer tail (trainer.rs:230-291) --------------------------------------
     def fused_step(self, params, grads, scaler: Optional["GradScaler"] = None,
                    max_norm: float = 0.0, zero_grads: bool = False,
-                   skip_nonfinite: bool = False) -> None:
+                   skip_nonfinite: bool = False, no_alloc: bool = False) -> None:
+        """`no_alloc=True` goes through nbo_fused_step_noalloc: same results, the norm pass's
+        scratch comes from the library's statically allocated device array (pass TensorLists,
+        or the same tensors as in an earlier call, so that no descriptor is built either)."""
         p = self._cache.get("p", params)
         g = self._cache.get("g", grads)
         flags = (STEP_ZERO_GRADS if zero_grads else 0) | (STEP_SKIP_NONFINITE if skip_nonfinite else 0)
-        _call(_lib.load().nbo_fused_step(self._handle(), scaler._handle() if scaler else None,
-                                         p._h, g._h, float(max_norm), flags))
+        lib = _lib.load()
+        fn = lib.nbo_fused_step_noalloc if no_alloc else lib.nbo_fused_step
+        _call(fn(self._handle(), scaler._handle() if scaler else None, p._h, g._h, float(max_norm), flags))
 
     def fused_step_norm(self, params, grads, sumsq: float, max_norm: float = 0.0,
                         zero_grads: bool = False) -> None:
