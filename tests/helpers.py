@@ -122,3 +122,50 @@ def count_beyond_ulp_f32(a_list, b_list, tol):
             n_bad += int((O.ulp_distance_f32(a, b) > tol).sum())
             total += a.size
     return n_bad, total
+
+
+# ---- the 2-ulp bar for parameters and its one documented escape ------------------------------
+
+# No test may leave more than this many elements per 10^9 element-steps beyond 2 ulp (each of
+# them inside the cancellation bound).  The mechanism: the reference's powf(x, 0.5) and the
+# correctly rounded sqrt differ by 1 ulp for 0.06 % of inputs, which moves the update by 1 ulp;
+# where p * (1 - wd * lr) and the update nearly cancel, that is more than 2 ulp of the tiny
+# result.  Measured on this suite: 0.3 to 3 elements per 10^6 element-steps (the printed reports
+# give each test's count), so the cap below leaves a factor of three.
+ESCAPES_PER_1E9_ELEMENT_STEPS = 10000
+
+
+def tolerance_report(dev_list, ref_list, lr, steps, what, element_steps=None):
+    """f32 parameters against the libm-powf oracle: every element must be within 2 ulp or,
+    failing that, within |delta| <= steps * 8 * lr * 2^-23 (a 1-ulp change of the update
+    against a result that nearly cancelled).  Counts, prints and returns how often the second
+    clause was needed: (n_beyond_2ulp, n_total, worst_ulp, worst_abs, first locations)."""
+    n_total = n_beyond = worst_ulp = 0
+    worst_abs = 0.0
+    first = []
+    bound = steps * 8 * lr * 2.0 ** -23
+    for i, (a, b) in enumerate(zip(dev_list, ref_list)):
+        if not a.size:
+            continue
+        ulp = O.ulp_distance_f32(a, b)
+        absd = np.abs(a.astype(np.float64) - b.astype(np.float64))
+        beyond = ulp > 2
+        n_total += a.size
+        worst_ulp = max(worst_ulp, int(ulp.max()))
+        if beyond.any():
+            idx = np.nonzero(beyond)[0]
+            n_beyond += idx.size
+            worst_abs = max(worst_abs, float(absd[idx].max()))
+            for e in idx[:max(0, 5 - len(first))]:
+                first.append((i, int(e), float(a[e]), float(b[e]), int(ulp[e])))
+            outside = beyond & ~(absd <= bound)
+            assert not outside.any(), (
+                f"{what}: tensor {i}: {int(outside.sum())} params beyond 2 ulp and beyond the cancellation "
+                f"bound {bound:.3e}; worst ulp {int(ulp.max())}, worst |d| {absd.max():.3e}")
+    es = element_steps if element_steps is not None else n_total * steps
+    print(f"[tolerance] {what}: {n_beyond} of {n_total} elements ({es} element-steps) beyond 2 ulp of the "
+          f"libm-powf oracle, all within |d| <= {bound:.3e}; worst {worst_ulp} ulp, worst |d| {worst_abs:.3e}; "
+          f"first (tensor, index, device, oracle, ulp): {first}", flush=True)
+    ceiling = max(5, int(ESCAPES_PER_1E9_ELEMENT_STEPS * es / 1e9))
+    assert n_beyond <= ceiling, f"{what}: {n_beyond} elements beyond 2 ulp, more than the ceiling of {ceiling}"
+    return n_beyond, n_total, worst_ulp, worst_abs, first

@@ -27,15 +27,9 @@ RAGGED = [(1, 1), (1, 3), (3, 5), (1, 4095), (1, 4097), (64, 130), (7, 1171), (1
 
 
 def _param_close(p_dev, p_ref, lr, steps, what):
-    for i, (a, b) in enumerate(zip(p_dev, p_ref)):
-        if not a.size:
-            continue
-        ulp = O.ulp_distance_f32(a, b)
-        absd = np.abs(a.astype(np.float64) - b.astype(np.float64))
-        bad = (ulp > 2) & ~(absd <= steps * 8 * lr * 2.0 ** -23)
-        assert not bad.any(), (
-            f"{what}: tensor {i}: {int(bad.sum())} params beyond 2 ulp and beyond the cancellation "
-            f"bound; worst ulp {int(ulp.max())}, worst |d| {absd.max():.3e}")
+    """2 ulp, or the documented cancellation bound; how often the bound was needed is counted,
+    printed (pytest -s shows it) and capped."""
+    return H.tolerance_report(p_dev, p_ref, lr, steps, what)
 
 
 # ---- config 1: plain SGD on the README MLP parameter set, 100 steps ---------------------
