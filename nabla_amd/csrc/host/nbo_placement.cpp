@@ -6,6 +6,7 @@
 #include <cstdlib>
 
 #include "nbo_host.hpp"
+#include "nbo_placement_plan.hpp"
 
 namespace nbo {
 
@@ -13,9 +14,8 @@ namespace {
 
 constexpr size_t kGiB = (size_t)1 << 30;
 constexpr size_t kMapGranule = (size_t)2 << 20;
-// Two buffers of 1-2 GiB read-modify-written together run at 5.0-5.9 TB/s when both
-// lie in the same 96 GiB region of MI355X's HBM and at 6.3-6.5 TB/s when they do not.
-constexpr double kSameRegionBelowGBps = 6100.0;
+// Memory left alone while chunks are being created.
+constexpr size_t kReserveBytes = (size_t)2 << 30;
 // Below this size per part the step is too short for placement to matter.
 constexpr size_t kMinPlacedBytes = (size_t)128 << 20;
 
@@ -63,13 +63,27 @@ void StatePlacement::release()
     regions_used_ = 0;
 }
 
+namespace {
+std::string fmt(const char *f, double a = 0, double b = 0, double c = 0, double d = 0)
+{
+    char buf[256];
+    std::snprintf(buf, sizeof(buf), f, a, b, c, d);
+    return buf;
+}
+} // namespace
+
 void StatePlacement::allocate(uint32_t nparts, size_t bytes, void **out)
 {
     release();
+    note_.clear();
     for (uint32_t k = 0; k < 3; k++) out[k] = nullptr;
     const char *env = std::getenv("NBO_STATE_SPREAD");
     const bool spread = !(env && env[0] == '0');
-    if (spread && nparts > 1 && bytes >= kMinPlacedBytes && try_placed(nparts, bytes, out)) return;
+    if (!spread) note_ = "plain allocations: NBO_STATE_SPREAD=0";
+    else if (nparts < 2) note_ = "plain allocation: a single state array has nothing to be spread against";
+    else if (bytes < kMinPlacedBytes) note_ = "plain allocations: less than 128 MiB per state array";
+    else if (try_placed(nparts, bytes, out)) return;
+    if (std::getenv("NBO_PLACEMENT_DEBUG")) std::fprintf(stderr, "[nbo placement] %s\n", note_.c_str());
     Runtime &rt = Runtime::get();
     try {
         for (uint32_t k = 0; k < nparts; k++) {
@@ -85,20 +99,31 @@ void StatePlacement::allocate(uint32_t nparts, size_t bytes, void **out)
 bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
 {
     Runtime &rt = Runtime::get();
-    const size_t chunk = bytes >= 16 * kGiB ? 2 * kGiB : kGiB;
-    const size_t window = chunk; // probe size: whole chunks against each other
+    // 1 GiB: large enough for a steady probe, small enough that a chunk the driver pieced
+    // together from scattered physical memory rarely straddles two regions
+    const size_t chunk = kGiB;
     // a part smaller than one chunk still gets a whole chunk of its own (regions can
     // only be told apart at this granularity); larger parts are whole chunks plus a tail
     const size_t full = bytes < chunk ? 1 : bytes / chunk;
     const size_t tail = bytes < chunk ? 0 : round_up(bytes - full * chunk, kMapGranule);
     const size_t part_va = full * chunk + tail;
     const size_t total_full = full * nparts;
+    auto give_up = [&](const std::string &why) {
+        note_ = "plain allocations: " + why;
+        return false;
+    };
     size_t free_b = 0, total_b = 0;
-    if (!ok(hipMemGetInfo(&free_b, &total_b))) return false;
-    const size_t reserve = 2 * kGiB;
-    if (free_b < reserve + nparts * part_va) return false; // let hipMalloc report the shortage
-    const size_t budget = (free_b - reserve - nparts * tail) / chunk;
-    if (budget < total_full) return false;
+    if (!ok(hipMemGetInfo(&free_b, &total_b))) return give_up("hipMemGetInfo failed");
+    if (free_b < kReserveBytes + nparts * part_va) return give_up("not enough free memory to choose chunks from");
+    // The search creates at most `cap` chunks: what the arrays need twice over plus a few,
+    // NBO_PLACEMENT_MAX_GIB if set, never more than what is free minus a reserve.
+    size_t user_cap = 0;
+    if (const char *e = std::getenv("NBO_PLACEMENT_MAX_GIB")) {
+        const double gib = std::atof(e);
+        if (gib > 0.0) user_cap = (size_t)(gib * (double)kGiB / (double)chunk);
+    }
+    const size_t cap = plan::chunk_cap(total_full, (free_b - kReserveBytes - nparts * tail) / chunk, user_cap);
+    if (cap < total_full) return give_up("the chunk limit is below what the state arrays need");
 
     const char *dbg = std::getenv("NBO_PLACEMENT_DEBUG");
     const int debug = dbg ? std::atoi(dbg) : 0;
@@ -111,7 +136,7 @@ bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
     };
     std::vector<Chunk> chunks;
     void *staging = nullptr;
-    const size_t staging_size = budget * chunk;
+    const size_t staging_size = cap * chunk;
     struct PartRange {
         void *va;
         size_t mapped; // bytes mapped so far, from the start of the range
@@ -135,139 +160,122 @@ bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
         }
         (void)hipGetLastError();
     };
+    auto fail_with = [&](const std::string &why) {
+        cleanup();
+        return give_up(why);
+    };
 
     try {
         if (!ok(hipMemAddressReserve(&staging, staging_size, 0, nullptr, 0))) {
             staging = nullptr;
-            cleanup();
-            return false;
+            return fail_with("no virtual address range for the search");
         }
-        std::vector<std::vector<size_t>> region_chunks; // chunk indices per region
-        std::vector<char *> region_rep;                 // one mapped chunk per region
-        // Which regions the parts will use.  Three parts rotate over all three regions.
-        // Two parts use the two regions found last: the first region found is where this
-        // process's most recent allocations went, and the caller's parameters and
-        // gradients -- read and written in the same kernel -- are most likely there.
-        const size_t first_used = nparts == 2 ? 1 : 0;
-        const size_t need_each = (total_full + (3 - first_used) - 1) / (3 - first_used);
-        auto enough = [&]() {
-            if (region_chunks.size() < 3) return false;
-            for (size_t r = first_used; r < 3; r++)
-                if (region_chunks[r].size() < need_each) return false;
+        auto chunk_va = [&](size_t i) { return (char *)staging + i * chunk; };
+        // creates and maps chunks until `target` exist; false when the driver refuses one
+        auto create_until = [&](size_t target) {
+            while (chunks.size() < target) {
+                Chunk c = {};
+                if (!ok(hipMemCreate(&c.h, chunk, &prop, 0))) return false;
+                const size_t idx = chunks.size();
+                chunks.push_back(c);
+                if (!ok(hipMemMap(chunk_va(idx), chunk, 0, c.h, 0))) return false;
+                chunks[idx].mapped_in_staging = true;
+                if (!set_rw(chunk_va(idx), chunk)) return false;
+            }
             return true;
         };
-        while (chunks.size() < budget && !enough()) {
-            Chunk c = {};
-            if (!ok(hipMemCreate(&c.h, chunk, &prop, 0))) break;
-            const size_t idx = chunks.size();
-            char *p = (char *)staging + idx * chunk;
-            chunks.push_back(c);
-            if (!ok(hipMemMap(p, chunk, 0, c.h, 0))) break;
-            chunks[idx].mapped_in_staging = true;
-            if (!set_rw(p, chunk)) break;
-            if (idx == 0) {
-                // the two halves of one chunk certainly share a region: the probe must
-                // call that pair "same", or it cannot tell anything on this system
-                if (rt.probe_pair_gbps(p, p + chunk / 2, chunk / 2) >= kSameRegionBelowGBps) {
-                    cleanup();
-                    return false;
-                }
-            }
-            int region = -1;
-            for (size_t r = 0; r < region_rep.size() && region < 0; r++) {
-                const double g = rt.probe_pair_gbps(region_rep[r], p, window);
-                if (debug > 1) std::fprintf(stderr, "[nbo placement] chunk %zu vs region %zu: %.0f GB/s\n", idx, r, g);
-                if (g < kSameRegionBelowGBps) region = (int)r;
-            }
-            if (region < 0) {
-                if (region_rep.size() == 3) {
-                    // a fourth "region" is measurement noise on this part: count the chunk
-                    // to the smallest region rather than trusting it
-                    region = 0;
-                    for (size_t r = 1; r < 3; r++)
-                        if (region_chunks[r].size() < region_chunks[region].size()) region = (int)r;
-                } else {
-                    region_rep.push_back(p);
-                    region_chunks.emplace_back();
-                    region = (int)region_rep.size() - 1;
-                }
-            }
-            region_chunks[region].push_back(idx);
+        plan::RegionFinder finder;
+        auto probe = [&](size_t a, size_t b) {
+            const double g = rt.probe_pair_gbps(chunk_va(a), chunk_va(b), chunk);
+            if (debug > 1) std::fprintf(stderr, "[nbo placement] chunk %zu with chunk %zu: %.0f GB/s\n", a, b, g);
+            return g;
+        };
+        // the two halves of one chunk certainly share a region: what "same" measures on this GPU now
+        auto halves = [&](size_t a) {
+            const double g = rt.probe_pair_gbps(chunk_va(a), chunk_va(a) + chunk / 2, chunk / 2);
+            if (debug > 1) std::fprintf(stderr, "[nbo placement] chunk %zu, its two halves: %.0f GB/s\n", a, g);
+            return g;
+        };
+        auto counts = [&]() {
+            std::vector<size_t> n;
+            for (const auto &r : finder.chunks_per_region()) n.push_back(r.size());
+            return n;
+        };
+        size_t target = std::min(cap, total_full + 2);
+        for (;;) {
+            const bool created = create_until(target);
+            size_t usable = chunks.size();
+            if (!created && usable && !chunks.back().mapped_in_staging) usable--; // created but not mapped
+            finder.add_chunks(usable, probe, halves);
+            if (plan::enough(counts(), nparts, full)) break;
+            if (!created || chunks.size() >= cap) break;
+            target = std::min(cap, chunks.size() + std::max<size_t>(2, total_full / 4));
         }
-        size_t have = 0;
-        for (const auto &r : region_chunks) have += r.size();
-        if (have < total_full) { // ran out of memory before collecting enough chunks
-            cleanup();
-            return false;
-        }
+        std::vector<std::vector<size_t>> region_chunks = finder.chunks_per_region();
         if (debug) {
-            std::fprintf(stderr, "[nbo placement] %zu chunks of %zu MiB created; per region:", chunks.size(), chunk >> 20);
+            std::fprintf(stderr, "[nbo placement] %zu chunks of %zu MiB created (limit %zu), %zu probes, threshold %.0f GB/s; per region:",
+                         chunks.size(), chunk >> 20, cap, finder.probes(), finder.threshold());
             for (const auto &r : region_chunks) std::fprintf(stderr, " %zu", r.size());
             std::fprintf(stderr, "; %zu needed\n", total_full);
         }
-        // chunk i of part j prefers the ((i + j) mod U)-th of the U regions in use; when
-        // that one has run dry, whichever region still has most chunks
-        const size_t R = region_chunks.size();
-        std::vector<size_t> use;
-        for (size_t r = (R == 3 ? first_used : 0); r < R; r++) use.push_back(r);
-        size_t in_use = 0;
-        for (size_t r : use) in_use += region_chunks[r].size();
-        if (in_use < total_full) { // not enough there: every region is fair game
-            use.clear();
-            for (size_t r = 0; r < R; r++) use.push_back(r);
-        }
+        if (region_chunks.size() < 2)
+            return fail_with(fmt("%.0f chunks created and probed, all read as one region (two halves of a chunk: %.0f GB/s)",
+                                 (double)chunks.size(), finder.same_pair()));
+        const std::vector<std::vector<int>> pick_region = plan::assign(counts(), nparts, full);
+        if (pick_region.empty()) return fail_with("ran out of memory before enough chunks were collected");
         std::vector<std::vector<size_t>> pick(nparts);
-        for (size_t i = 0; i < full; i++)
-            for (uint32_t j = 0; j < nparts; j++) {
-                size_t r = use[(i + j) % use.size()];
-                if (region_chunks[r].empty())
-                    for (size_t q : use)
-                        if (region_chunks[q].size() > region_chunks[r].size()) r = q;
-                pick[j].push_back(region_chunks[r].back());
-                region_chunks[r].pop_back();
+        for (uint32_t j = 0; j < nparts; j++)
+            for (size_t i = 0; i < full; i++) {
+                std::vector<size_t> &pool = region_chunks[(size_t)pick_region[j][i]];
+                pick[j].push_back(pool.back());
+                pool.pop_back();
             }
         // move the chosen chunks from the staging range into the parts' own ranges
         for (uint32_t j = 0; j < nparts; j++) {
             void *va = nullptr;
-            if (!ok(hipMemAddressReserve(&va, part_va, 0, nullptr, 0))) {
-                cleanup();
-                return false;
-            }
+            if (!ok(hipMemAddressReserve(&va, part_va, 0, nullptr, 0))) return fail_with("no virtual address range for a state array");
             part_ranges.push_back({va, 0});
             for (size_t i = 0; i < full; i++) {
                 const size_t idx = pick[j][i];
-                if (!ok(hipMemUnmap((char *)staging + idx * chunk, chunk))) {
-                    cleanup();
-                    return false;
-                }
+                if (!ok(hipMemUnmap(chunk_va(idx), chunk))) return fail_with("hipMemUnmap failed");
                 chunks[idx].mapped_in_staging = false;
-                if (!ok(hipMemMap((char *)va + i * chunk, chunk, 0, chunks[idx].h, 0))) {
-                    cleanup();
-                    return false;
-                }
+                if (!ok(hipMemMap((char *)va + i * chunk, chunk, 0, chunks[idx].h, 0))) return fail_with("hipMemMap failed");
                 part_ranges.back().mapped = (i + 1) * chunk;
                 chunks[idx].keep = true;
             }
             if (tail) {
                 hipMemGenericAllocationHandle_t th;
-                if (!ok(hipMemCreate(&th, tail, &prop, 0))) {
-                    cleanup();
-                    return false;
-                }
+                if (!ok(hipMemCreate(&th, tail, &prop, 0))) return fail_with("the tail of a state array could not be created");
                 tails.push_back(th);
-                if (!ok(hipMemMap((char *)va + full * chunk, tail, 0, th, 0))) {
-                    cleanup();
-                    return false;
-                }
+                if (!ok(hipMemMap((char *)va + full * chunk, tail, 0, th, 0))) return fail_with("hipMemMap failed");
                 part_ranges.back().mapped = part_va;
             }
-            if (!set_rw(va, part_va)) {
-                cleanup();
-                return false;
-            }
+            if (!set_rw(va, part_va)) return fail_with("hipMemSetAccess failed");
         }
+        // Check the finished layout: wherever the plan put two arrays into different regions at
+        // the first position, the probe over those two mapped chunks must read "different" again.
+        size_t checked = 0;
+        for (uint32_t j = 0; j < nparts; j++)
+            for (uint32_t k = j + 1; k < nparts; k++) {
+                if (pick_region[j][0] == pick_region[k][0]) continue;
+                const double g = rt.probe_pair_gbps(part_ranges[j].va, part_ranges[k].va, chunk);
+                if (debug > 1) std::fprintf(stderr, "[nbo placement] check, arrays %u and %u: %.0f GB/s\n", j, k, g);
+                if (!(g >= finder.threshold()))
+                    return fail_with(fmt("the finished layout did not check out: arrays %.0f and %.0f read %.0f GB/s together, "
+                                         "below the threshold of %.0f",
+                                         (double)j, (double)k, g, finder.threshold()));
+                checked++;
+            }
         success = true;
-        regions_used_ = (int)use.size();
+        std::vector<int> distinct;
+        for (const auto &p : pick_region)
+            for (int r : p)
+                if (std::find(distinct.begin(), distinct.end(), r) == distinct.end()) distinct.push_back(r);
+        regions_used_ = (int)distinct.size();
+        note_ = fmt("%.0f regions, chunks of %.0f MiB", (double)regions_used_, (double)(chunk >> 20)) +
+                fmt("; %.0f chunks created, %.0f probes", (double)chunks.size(), (double)finder.probes()) +
+                fmt("; same region %.0f GB/s, threshold %.0f GB/s, %.0f array pairs checked", finder.same_pair(), finder.threshold(),
+                    (double)checked);
         for (uint32_t j = 0; j < nparts; j++) {
             out[j] = part_ranges[j].va;
             ranges_.push_back({part_ranges[j].va, part_va});
@@ -276,10 +284,11 @@ bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
             if (c.keep) handles_.push_back(c.h);
         for (hipMemGenericAllocationHandle_t h : tails) handles_.push_back(h);
         cleanup(); // releases the chunks that were not chosen and the staging range
+        if (debug) std::fprintf(stderr, "[nbo placement] %s\n", note_.c_str());
         return true;
     } catch (...) {
         cleanup();
-        return false;
+        return give_up("an error while choosing chunks");
     }
 }
 

@@ -246,3 +246,18 @@ def test_null_arguments_are_errors_not_crashes():
         assert lib.nbo_last_error(), f"call {k} left no message"
     # destroying nothing is fine, as free(NULL) is
     assert lib.nbo_list_destroy(null) in (0, _lib.ERR_NO_DEVICE)
+
+
+def test_placement_decisions_on_made_up_measurements(tmp_path):
+    """The region search and the chunk assignment of the state placement are GPU-free functions
+    (nabla_amd/csrc/host/nbo_placement_plan.hpp); tests/cpp/test_placement_plan.cpp drives them
+    with a mocked bandwidth probe: three, two and one region, a noisy fourth kind, a failed
+    probe, regions that run dry, exhaustion, a slower and a faster GPU."""
+    import subprocess
+
+    src = os.path.join(ROOT, "tests", "cpp", "test_placement_plan.cpp")
+    exe = str(tmp_path / "test_placement_plan")
+    subprocess.run(["g++", "-O1", "-std=c++17", "-Wall", "-Wextra", "-o", exe, src], check=True)
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "all checks passed" in r.stdout
