@@ -33,6 +33,8 @@ def parse_args():
                     choices=["llama3-8b", "llama-1.1b", "gpt2-small-f32", "mlp-sgd-f32", "ragged-4096",
                              "llama-1.1b-bf16", "llama-1.1b-f16", "llama-1.1b-f16-mixed"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-ceiling", action="store_true",
+                    help="skip the micro-kernel measurement of the memory system's read-modify-write ceiling")
     ap.add_argument("--zero-grads", choices=["off", "fused", "separate"], default="off",
                     help="also clear the gradients every step (trainer.rs:285-290): inside the update "
                          "kernel, or as a separate pass; +2 B/param of writes, reported in the config")
@@ -42,6 +44,9 @@ def parse_args():
                     help="instead of the benchmark, run the library's plain copy kernel over "
                          "this many GiB (--steps times); a transfer of known size against which "
                          "rocprofv3's FETCH_SIZE / WRITE_SIZE counters are scaled")
+    ap.add_argument("--settle-seconds", type=float, default=2.0,
+                    help="idle time between setup and the warm-up steps, for the driver's background clearing of "
+                         "the device memory that setup freed to finish")
     ap.add_argument("--cpu-seconds", type=float, default=20.0,
                     help="rough budget for the CPU baseline sample")
     return ap.parse_args()
@@ -161,7 +166,24 @@ def cpu_baseline(cfg, budget_s):
     }
 
 
-def measure(name, steps, warmup, zero_grads="off"):
+def measured_ceiling(achieved_gbps):
+    """What this GPU's memory system gives an in-place read-modify-write over three streams
+    placed across the HBM's regions like optimizer state, and the update's own stream shape
+    (1 read, 3 in place, 1 written), measured now with the library's probe kernels
+    (`nbo_hbm_ceiling`; `python -m nabla_amd.kernel_bench --ceilings` has the whole table):
+    the yardstick next to the nominal 8 TB/s."""
+    from nabla_amd import kernel_bench as KB
+
+    rows = KB.measure_ceilings(gib=2.0, reps=10, patterns=(6, 7, 9), spreads=(1,))
+    name, spread, best, mean, regions, rw = max(rows, key=lambda r: r[3])
+    return {"ceiling_measured": round(mean, 1),
+            "ceiling_kernel": f"nbo_hbm_ceiling: {name}, 2 GiB per stream, "
+                              f"{'placed across ' + str(regions) + ' HBM regions' if spread else 'one plain allocation'}, "
+                              "mean of 10 launches",
+            "frac_of_ceiling_measured": round(achieved_gbps / mean, 4) if mean > 0 else None}
+
+
+def measure(name, steps, warmup, zero_grads="off", settle_s=2.0):
     """Builds the workload on the device, runs `warmup` + `steps` steps, returns the
     result record (without the CPU baseline)."""
     import ctypes as C
@@ -225,6 +247,13 @@ def measure(name, steps, warmup, zero_grads="off"):
     # launch, so small workloads take their kernel durations from a second, untimed pass.
     events_in_timed_region = n >= 10_000_000
 
+    # Setup has just freed tens of GiB (the placement search's spare chunks, torch's temporaries),
+    # and the driver clears freed device memory in the background: for about a second that
+    # competes with the step for HBM bandwidth (measured: 37.9 instead of 37.3 ms per step on the
+    # 8B set).  It is the benchmark's own setup, not the step, so it is given time to finish.
+    torch.cuda.synchronize()
+    _lib.check(L.nbo_sync())
+    time.sleep(settle_s)
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -255,11 +284,19 @@ def measure(name, steps, warmup, zero_grads="off"):
     dom_gbps = n * dom_b / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
     info = opt.last_step() if fused else None
 
-    traffic = None
+    # HBM bytes per launch by rocprofv3's counters: they cannot be read from inside this process,
+    # so the figure is the one a counter run of this same command left in profiles/traffic.json
+    # (see nabla_amd/profile_summary.py) and the line says so
+    traffic, traffic_source = None, None
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
-            traffic = json.load(f).get(f"{name}:{dom}")
+            table = json.load(f)
+        traffic = table.get(f"{name}:{dom}")
+        det = table.get("_detail", {}).get(name, {})
+        if traffic is not None:
+            traffic_source = (f"profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command at "
+                              f"commit {det.get('commit', '?')} on {det.get('date', '?')}; not measured in this run)")
 
     out = {
         "metric": "AdamW step HBM GB/s (% of peak) + params/s, bf16-mixed, whole step "
@@ -284,7 +321,7 @@ def measure(name, steps, warmup, zero_grads="off"):
                    "bytes_per_param_step": upd_b + nrm_b + zero_b, "zero_grads": zero_grads,
                    "optimizer": cfg["kind"],
                    "loss_scale": scale if cfg["scaler"] else None, "clip_max_norm": cfg["clip"] or None,
-                   "state_hbm_regions": opt.state_regions()},
+                   "state_hbm_regions": opt.state_regions(), "settle_s_after_setup": settle_s},
         "roofline": {
             "kernel": dom,
             "bound": "hbm",
@@ -293,6 +330,7 @@ def measure(name, steps, warmup, zero_grads="off"):
             "unit": "GB/s",
             "frac": round(dom_gbps / HBM_PEAK_GBPS, 4),
             "traffic": traffic,
+            "traffic_source": traffic_source,
             "algorithmic_bytes_per_launch": n * dom_b,
             "avg_launch_ms": round(dom_ms, 4),
             "launches": per_kernel[dom][0],
@@ -340,13 +378,15 @@ def main():
                           "launches": cnt.value, "avg_launch_ms": round(ms.value / max(cnt.value, 1), 4),
                           "GBps": round(2 * nbytes / (ms.value / max(cnt.value, 1)) / 1e6, 1)}))
         return
-    out, cfg = measure(args.workload, args.steps, args.warmup, args.zero_grads)
+    out, cfg = measure(args.workload, args.steps, args.warmup, args.zero_grads, args.settle_seconds)
     if args.workload == "llama3-8b" and not args.primary_only:
         # the metric is quoted on the 1.1B and the 8B shapes: the smaller one rides along
-        small, _ = measure("llama-1.1b", 10, 2)
+        small, _ = measure("llama-1.1b", 10, 2, settle_s=args.settle_seconds)
         out["also"] = {"llama-1.1b": {k: small[k] for k in ("value", "unit", "pct_of_peak", "params_per_s",
                                                             "ms_per_step", "steps", "warmup", "config",
                                                             "roofline", "kernels_ms")}}
+    if not args.no_ceiling and out["roofline"]["achieved"] > 0:
+        out["roofline"].update(measured_ceiling(out["roofline"]["achieved"]))
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_seconds)
         out["cpu_baseline"]["gpu_over_cpu"] = round(out["value"] / max(out["cpu_baseline"]["value"], 1e-9), 1)

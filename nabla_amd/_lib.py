@@ -98,6 +98,7 @@ SYMBOLS = {
     "nbo_optim_master_from_params": (C.c_int, [_P, _P]),
     "nbo_optim_params_from_master": (C.c_int, [_P, _P]),
     "nbo_optim_state_regions": (C.c_int, [_P, C.POINTER(C.c_int)]),
+    "nbo_optim_state_placement_note": (C.c_int, [_P, C.c_char_p, C.c_uint64]),
     "nbo_scaler_create": (C.c_int, [C.POINTER(ScalerState), C.POINTER(_P)]),
     "nbo_scaler_destroy": (C.c_int, [_P]),
     "nbo_scaler_state_get": (C.c_int, [_P, C.POINTER(ScalerState)]),
@@ -127,6 +128,8 @@ SYMBOLS = {
     "nbo_optim_save_state_groups": (C.c_int, [C.c_uint64, C.POINTER(_P), C.c_char_p]),
     "nbo_optim_load_state_groups": (C.c_int, [C.c_uint64, C.POINTER(_P), C.c_char_p]),
     "nbo_copy_bytes": (C.c_int, [_P, _P, C.c_uint64]),
+    "nbo_hbm_ceiling": (C.c_int, [C.c_int, C.c_int, C.c_uint64, C.c_int, C.c_uint32, C.POINTER(C.c_double),
+                                  C.POINTER(C.c_double), C.POINTER(C.c_int)]),
     "nbo_profile_enable": (C.c_int, [C.c_int]),
     "nbo_profile_read": (C.c_int, [C.c_char_p, _U64P, C.POINTER(C.c_double)]),
 }

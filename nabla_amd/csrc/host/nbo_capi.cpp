@@ -659,6 +659,17 @@ int nbo_optim_state_regions(nbo_optim *opt, int *regions)
     });
 }
 
+int nbo_optim_state_placement_note(nbo_optim *opt, char *buf, uint64_t buf_bytes)
+{
+    return guarded([&] {
+        require(opt && buf && buf_bytes > 0, NBO_ERR_ARG, "null optimizer or buffer");
+        const std::string &n = opt->placement.note();
+        const size_t k = n.size() < buf_bytes - 1 ? n.size() : (size_t)(buf_bytes - 1);
+        std::memcpy(buf, n.data(), k);
+        buf[k] = '\0';
+    });
+}
+
 // ---- GradScaler ------------------------------------------------------------------------
 
 int nbo_scaler_create(const nbo_scaler_state *state, nbo_scaler **out)
@@ -1190,6 +1201,63 @@ int nbo_copy_bytes(const void *src_dev, void *dst_dev, uint64_t bytes)
         require(bytes % 16 == 0 && ((uintptr_t)src_dev % 16) == 0 && ((uintptr_t)dst_dev % 16) == 0,
                 NBO_ERR_ARG, "copy needs 16-byte aligned addresses and size");
         Runtime::get().launch_copy(src_dev, dst_dev, bytes / 16);
+    });
+}
+
+int nbo_hbm_ceiling(int pattern, int spread, uint64_t bytes_per_stream, int reps, uint32_t settle_ms,
+                    double *best_gbps, double *mean_gbps, int *regions)
+{
+    return guarded([&] {
+        // streams read, rewritten in place, written
+        static const int kShape[NBO_PROBE_COUNT][3] = {{1, 0, 0}, {3, 0, 0}, {0, 0, 1}, {0, 0, 3}, {1, 0, 1},
+                                                       {0, 1, 0}, {0, 2, 0}, {0, 3, 0}, {0, 6, 0}, {1, 3, 1}};
+        static_assert((int)NBO_PATTERN_READ1 == (int)NBO_PROBE_READ1 && (int)NBO_PATTERN_COPY == (int)NBO_PROBE_COPY &&
+                          (int)NBO_PATTERN_RMW3 == (int)NBO_PROBE_RMW3 &&
+                          (int)NBO_PATTERN_R1_RMW3_W1 == (int)NBO_PROBE_R1_RMW3_W1 &&
+                          (int)NBO_PATTERN_R1_RMW3_W1 + 1 == (int)NBO_PROBE_COUNT,
+                      "public pattern codes and the kernels' must agree");
+        require(pattern >= 0 && pattern < (int)NBO_PROBE_COUNT, NBO_ERR_ARG, "unknown probe pattern");
+        require(best_gbps && mean_gbps, NBO_ERR_ARG, "null output");
+        require(reps >= 1 && reps <= 1000, NBO_ERR_ARG, "1 to 1000 repetitions");
+        require(settle_ms <= 60000, NBO_ERR_ARG, "at most 60 s of untimed launches");
+        const uint64_t window = 8ull * NBO_BLOCK * 16; // bytes of one stream a workgroup covers
+        require(bytes_per_stream >= window && bytes_per_stream % window == 0 &&
+                    bytes_per_stream / window <= 0x7FFFFFFFull,
+                NBO_ERR_ARG, "bytes per stream: a multiple of 32 KiB, at most 2^31 - 1 of them");
+        const int ro = kShape[pattern][0], rmw = kShape[pattern][1], wo = kShape[pattern][2];
+        const uint32_t ns = (uint32_t)(ro + rmw + wo);
+        Runtime &rt = Runtime::get();
+        // Streams are equal slices of up to three arrays.  spread: the arrays come from the
+        // region-aware placement the optimizer state uses, stream s lies in array s mod 3, so
+        // neighbouring streams sit in different HBM regions at every offset.  Otherwise one plain
+        // allocation holds all streams back to back.
+        StatePlacement place;
+        void *part[3] = {nullptr, nullptr, nullptr};
+        const uint32_t nparts = spread ? (ns < 3 ? ns : 3) : 1;
+        const uint32_t per_part = (ns + nparts - 1) / nparts;
+        const size_t part_bytes = (size_t)per_part * bytes_per_stream;
+        if (spread) {
+            place.allocate(nparts, part_bytes, part);
+        } else {
+            part[0] = rt.dmalloc(part_bytes);
+        }
+        try {
+            for (uint32_t k = 0; k < nparts; k++) rt.dzero(part[k], part_bytes);
+            NboStreamProbeArgs a = {};
+            for (uint32_t s = 0; s < ns; s++)
+                a.buf[s] = (char *)part[s % nparts] + (size_t)(s / nparts) * bytes_per_stream;
+            double best_ms = 0.0, mean_ms = 0.0;
+            rt.time_launches(K_STREAM_PROBE_BASE + pattern, (uint32_t)(bytes_per_stream / window), &a, reps, settle_ms, &best_ms, &mean_ms);
+            const double moved = (double)(ro + 2 * rmw + wo) * (double)bytes_per_stream;
+            *best_gbps = best_ms > 0.0 ? moved / best_ms / 1e6 : 0.0;
+            *mean_gbps = mean_ms > 0.0 ? moved / mean_ms / 1e6 : 0.0;
+            if (regions) *regions = spread ? place.regions_used() : 0;
+        } catch (...) {
+            if (!spread) rt.dfree(part[0]);
+            throw;
+        }
+        rt.sync();
+        if (!spread) rt.dfree(part[0]);
     });
 }
 

@@ -4,6 +4,7 @@
 #include "nbo_noalloc.hpp"
 
 #include <algorithm>
+#include <chrono>
 #include <cstdio>
 #include <cstring>
 #include <mutex>
@@ -47,7 +48,12 @@ static const char *const kKernelNames[K_COUNT] = {
     "nbo_norm_f16",          "nbo_norm_pf16",        "nbo_scale_f16",
     "nbo_accum_f16",         "nbo_ew_f16",           "nbo_accnorm_f32",
     "nbo_accnorm_bf16",      "nbo_accnorm_f64",      "nbo_accnorm_f16",
+    "nbo_probe_read1",       "nbo_probe_read3",      "nbo_probe_fill1",
+    "nbo_probe_fill3",       "nbo_probe_copy",       "nbo_probe_rmw1",
+    "nbo_probe_rmw2s",       "nbo_probe_rmw3",       "nbo_probe_rmw6",
+    "nbo_probe_r1_rmw3_w1",
 };
+static_assert(K_STREAM_PROBE_BASE + NBO_PROBE_COUNT == K_COUNT, "one probe kernel per pattern");
 
 static std::mutex g_runtime_mu;
 static Runtime *g_runtime = nullptr;
@@ -208,6 +214,38 @@ double Runtime::probe_pair_gbps(void *a, void *b, size_t bytes)
         if (rep > 0 && (best == 0.0f || ms < best)) best = ms; // first run warms up
     }
     return best > 0.0f ? 4.0 * (double)grid * (double)per_wg * 16 / best / 1e6 : 0.0;
+}
+
+void Runtime::time_launches(int kernel, uint32_t grid, void *arg_struct, int reps, uint32_t settle_ms, double *best_ms,
+                            double *mean_ms)
+{
+    void *args[1] = {arg_struct};
+    const hipEvent_t e0 = probe_ev_[0], e1 = probe_ev_[1];
+    auto one = [&]() {
+        hip_check(hipEventRecord(e0, stream_), "hipEventRecord");
+        hip_check(hipModuleLaunchKernel(fn_[kernel], grid, 1, 1, NBO_BLOCK, 1, 1, 0, stream_, args, nullptr),
+                  kKernelNames[kernel]);
+        hip_check(hipEventRecord(e1, stream_), "hipEventRecord");
+        hip_check(hipEventSynchronize(e1), "hipEventSynchronize");
+        float ms = 0.0f;
+        hip_check(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime");
+        return (double)ms;
+    };
+    // warm-up, and time for the driver's background clearing of memory freed just before (the
+    // placement search's spare chunks, an earlier measurement's buffers) to finish
+    const auto t0 = std::chrono::steady_clock::now();
+    do {
+        (void)one();
+    } while (std::chrono::duration_cast<std::chrono::milliseconds>(std::chrono::steady_clock::now() - t0).count() <
+             (long long)settle_ms);
+    double best = 0.0, sum = 0.0;
+    for (int rep = 0; rep < reps; rep++) {
+        const double ms = one();
+        sum += ms;
+        if (best == 0.0 || ms < best) best = ms;
+    }
+    *best_ms = best;
+    *mean_ms = reps > 0 ? sum / reps : 0.0;
 }
 
 // Both directions run the two halves of the pinned buffer as a pipeline: while the DMA

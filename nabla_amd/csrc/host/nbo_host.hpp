@@ -58,7 +58,8 @@ enum KernelId {
     K_EW_F16 = 42,
     K_ACCNORM_BASE = 43, // + st (f32 / bf16 / f64)
     K_ACCNORM_F16 = 46,
-    K_COUNT = 47
+    K_STREAM_PROBE_BASE = 47, // + NBO_PROBE_* pattern
+    K_COUNT = 57
 };
 
 // Process-wide runtime: device 0, the loaded module, the stream, scratch buffers.
@@ -81,6 +82,10 @@ public:
     // Bandwidth (GB/s, best of three) of reading and rewriting `bytes` bytes at a and at
     // b together: the probe StatePlacement classifies HBM regions with.  Synchronous.
     double probe_pair_gbps(void *a, void *b, size_t bytes);
+    // Untimed launches for `settle_ms` milliseconds (at least one), then `reps` launches each
+    // bracketed by events on the stream: shortest and mean duration in ms.  Synchronous.
+    void time_launches(int kernel, uint32_t grid, void *arg_struct, int reps, uint32_t settle_ms, double *best_ms,
+                       double *mean_ms);
 
     // synchronous transfers through a double-buffered pinned staging buffer
     void read_back(void *host_dst, const void *dev_src, size_t bytes);

@@ -250,4 +250,23 @@ struct NboCastListArgs {
     uint32_t dst_type, src_type; // NBO_F32 / NBO_BF16 / NBO_F64
 };
 
+// Memory-system ceiling probe: which streams are read, rewritten in place or only written.
+enum {
+    NBO_PROBE_READ1 = 0,      // 1 stream read
+    NBO_PROBE_READ3 = 1,      // 3 streams read
+    NBO_PROBE_FILL1 = 2,      // 1 stream written
+    NBO_PROBE_FILL3 = 3,      // 3 streams written
+    NBO_PROBE_COPY = 4,       // stream 0 read, stream 1 written
+    NBO_PROBE_RMW1 = 5,       // N streams read and rewritten in place
+    NBO_PROBE_RMW2 = 6,
+    NBO_PROBE_RMW3 = 7,
+    NBO_PROBE_RMW6 = 8,
+    NBO_PROBE_R1_RMW3_W1 = 9, // the mixed-precision update's shape: 1 read, 3 in place, 1 written
+    NBO_PROBE_COUNT = 10
+};
+
+struct NboStreamProbeArgs {
+    void *buf[8]; // streams in the order read-only, in place, write-only
+};
+
 #endif

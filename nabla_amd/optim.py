@@ -392,6 +392,12 @@ class _Optimizer:
         _call(_lib.load().nbo_optim_state_regions(self._handle(), C.byref(n)))
         return n.value
 
+    def state_placement_note(self) -> str:
+        """What the placement of the state arrays found, or why it fell back to plain allocations."""
+        buf = C.create_string_buffer(512)
+        _call(_lib.load().nbo_optim_state_placement_note(self._handle(), buf, 512))
+        return buf.value.decode("utf-8", "replace")
+
     # -- master weights (mixed precision) -----------------------------------------------
     def master_from_params(self, params) -> None:
         p = self._cache.get("p", params)

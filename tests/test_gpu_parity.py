@@ -767,3 +767,34 @@ def test_switching_streams_keeps_the_steps_in_order(gpu):
         O.set_pow_mode(O.POW_LIBM)
     H.assert_bits_equal(H.host_list(p_dev), pr, "params")
     H.assert_bits_equal(H.host_list(opt.moments()[1]), v, "v")
+
+
+def test_state_placement_says_what_it_found(gpu):
+    """State of 128 MiB per array or more is placed across the HBM's regions when the probe
+    can tell regions apart on this GPU; either way the optimizer reports the outcome and the
+    reason, and steps give the oracle's bits."""
+    shapes = [(4096, 8192 + 8)]  # 33.6 M elements: 134 MB per state array
+    p_ref = H.randn_list(shapes, 4242, 0.02)
+    p_dev = H.dev_list(p_ref, shapes)
+    opt = nb.AdamW.new(1e-3, shapes).weight_decay(0.1)
+    m, v = H.zeros_like_list(p_ref), H.zeros_like_list(p_ref)
+    meta = O.adamw_meta(1e-3, weight_decay=0.1)
+    O.set_pow_mode(O.POW_SQRT)
+    O.set_threads(8)
+    try:
+        for step in range(2):
+            g = H.randn_list(shapes, 4300 + step, 1e-3)
+            opt.step(p_dev, H.dev_list(g, shapes))
+            O.adam_step(meta, p_ref, g, m, v)
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+        O.set_threads(1)
+    regions, note = opt.state_regions(), opt.state_placement_note()
+    print(f"[placement] {regions} regions: {note}")
+    assert note, "the placement always leaves a note"
+    if regions == 0:
+        assert note.startswith("plain allocation")
+    else:
+        assert regions in (2, 3) and note.startswith(f"{regions} regions") and "threshold" in note
+    H.assert_bits_equal(H.host_list(p_dev), p_ref, "params on placed state")
+    H.assert_bits_equal(H.host_list(opt.moments()[1]), v, "v on placed state")
