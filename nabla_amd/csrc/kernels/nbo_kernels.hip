@@ -1323,23 +1323,32 @@ template <int RO, int RMW, int WO> DEV void stream_probe_body(const NboStreamPro
     enum { ROWS = 8, NLOAD = RO + RMW };
     const uint64_t c0 = (uint64_t)blockIdx.x * (ROWS * NBO_BLOCK) + threadIdx.x;
     f32x4 x[NLOAD > 0 ? NLOAD : 1][ROWS];
+    // stream after stream, all rows of a stream back to back: the order the update kernels use
 #pragma unroll
-    for (int u = 0; u < ROWS; u++)
+    for (int s = 0; s < NLOAD; s++)
 #pragma unroll
-        for (int s = 0; s < NLOAD; s++)
+        for (int u = 0; u < ROWS; u++)
             x[s][u] = __builtin_nontemporal_load(GLOBAL_PTR(const f32x4, a.buf[s]) + c0 + u * NBO_BLOCK);
     f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int u = 0; u < ROWS; u++) {
+    for (int s = 0; s < RO; s++)
 #pragma unroll
-        for (int s = 0; s < RO; s++) acc = acc + x[s][u];
+        for (int u = 0; u < ROWS; u++) acc = acc + x[s][u];
 #pragma unroll
-        for (int s = RO; s < NLOAD; s++)
-            __builtin_nontemporal_store(x[s][u] + 1.0f, GLOBAL_PTR(f32x4, a.buf[s]) + c0 + u * NBO_BLOCK);
+    for (int s = RO; s < NLOAD; s++)
 #pragma unroll
-        for (int s = NLOAD; s < NLOAD + WO; s++)
+        for (int u = 0; u < ROWS; u++) x[s][u] = x[s][u] + 1.0f;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = RO; s < NLOAD; s++)
+#pragma unroll
+        for (int u = 0; u < ROWS; u++)
+            __builtin_nontemporal_store(x[s][u], GLOBAL_PTR(f32x4, a.buf[s]) + c0 + u * NBO_BLOCK);
+#pragma unroll
+    for (int s = NLOAD; s < NLOAD + WO; s++)
+#pragma unroll
+        for (int u = 0; u < ROWS; u++)
             __builtin_nontemporal_store(acc, GLOBAL_PTR(f32x4, a.buf[s]) + c0 + u * NBO_BLOCK);
-    }
     // keeps the read-only loads alive without ever storing: the sum of finite inputs is not NaN
     if (RO > 0 && WO == 0 && acc.x != acc.x) *GLOBAL_PTR(float, a.buf[0]) = acc.y + acc.z + acc.w;
 }

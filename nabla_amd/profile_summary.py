@@ -6,9 +6,9 @@
 Expected under DIR, made by these five commands (each from the repository root, after
 `cd /tmp && export TMPDIR=/tmp && cd -`; the program follows `--` directly):
 
-    rocprofv3 --kernel-trace --stats -d DIR/kt -o kt --output-format csv -- python3 bench.py --no-cpu-baseline --primary-only > DIR/kt_bench.json
-    rocprofv3 --pmc FETCH_SIZE -d DIR/fetch -o fetch --output-format csv -- python3 bench.py --no-cpu-baseline --primary-only
-    rocprofv3 --pmc WRITE_SIZE -d DIR/write -o write --output-format csv -- python3 bench.py --no-cpu-baseline --primary-only
+    rocprofv3 --kernel-trace --stats -d DIR/kt -o kt --output-format csv -- python3 bench.py --no-cpu-baseline --primary-only --no-ceiling > DIR/kt_bench.json
+    rocprofv3 --pmc FETCH_SIZE -d DIR/fetch -o fetch --output-format csv -- python3 bench.py --no-cpu-baseline --primary-only --no-ceiling
+    rocprofv3 --pmc WRITE_SIZE -d DIR/write -o write --output-format csv -- python3 bench.py --no-cpu-baseline --primary-only --no-ceiling
     rocprofv3 --pmc FETCH_SIZE -d DIR/cfetch -o cfetch --output-format csv -- python3 bench.py --calibrate-copy 8 --steps 3 > DIR/cfetch.json
     rocprofv3 --pmc WRITE_SIZE -d DIR/cwrite -o cwrite --output-format csv -- python3 bench.py --calibrate-copy 8 --steps 3
 
@@ -91,9 +91,9 @@ def summarize(base: str) -> str:
              "`cd /tmp && export TMPDIR=/tmp && cd -`):\n")
     L.append("```")
     d = base.rstrip("/")
-    L.append(f"rocprofv3 --kernel-trace --stats -d {d}/kt -o kt --output-format csv -- python3 bench.py --no-cpu-baseline --primary-only{flags} > {d}/kt_bench.json")
-    L.append(f"rocprofv3 --pmc FETCH_SIZE -d {d}/fetch -o fetch --output-format csv -- python3 bench.py --no-cpu-baseline --primary-only{flags}")
-    L.append(f"rocprofv3 --pmc WRITE_SIZE -d {d}/write -o write --output-format csv -- python3 bench.py --no-cpu-baseline --primary-only{flags}")
+    L.append(f"rocprofv3 --kernel-trace --stats -d {d}/kt -o kt --output-format csv -- python3 bench.py --no-cpu-baseline --primary-only --no-ceiling{flags} > {d}/kt_bench.json")
+    L.append(f"rocprofv3 --pmc FETCH_SIZE -d {d}/fetch -o fetch --output-format csv -- python3 bench.py --no-cpu-baseline --primary-only --no-ceiling{flags}")
+    L.append(f"rocprofv3 --pmc WRITE_SIZE -d {d}/write -o write --output-format csv -- python3 bench.py --no-cpu-baseline --primary-only --no-ceiling{flags}")
     L.append(f"rocprofv3 --pmc FETCH_SIZE -d {d}/cfetch -o cfetch --output-format csv -- python3 bench.py --calibrate-copy {COPY_GIB} --steps 3 > {d}/cfetch.json")
     L.append(f"rocprofv3 --pmc WRITE_SIZE -d {d}/cwrite -o cwrite --output-format csv -- python3 bench.py --calibrate-copy {COPY_GIB} --steps 3")
     L.append("```\n")
@@ -146,7 +146,7 @@ def summarize(base: str) -> str:
              f"destination both the caller's allocations) moved {copy['GBps']} GB/s in the same session.\n")
     text = "\n".join(L)
     os.makedirs(os.path.join(ROOT, "profiles"), exist_ok=True)
-    md = os.path.join("profiles", f"adamw_fused_step_{workload.replace('-', '_').replace('.', '')}.md")
+    md = os.path.join("profiles", f"adamw_fused_step_{workload.replace('1.1b', '1b').replace('-', '_').replace('.', '_')}.md")
     with open(os.path.join(ROOT, md), "w") as f:
         f.write(text)
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
@@ -167,9 +167,30 @@ def summarize(base: str) -> str:
     return text
 
 
-def main(base: str) -> None:
-    print(summarize(base))
+def counter_table(base: str, kernels=None) -> str:
+    """Markdown table of the per-dispatch averages of every counter of a `rocprofv3 --pmc` run
+    under `base`, one column per kernel of this library (or those named)."""
+    acc = {}
+    with open(_one(os.path.join(base, "**", "*counter_collection.csv*"))) as f:
+        for r in csv.DictReader(f):
+            k = r["Kernel_Name"]
+            if not k.startswith("nbo_") or (kernels and k not in kernels):
+                continue
+            acc.setdefault(r["Counter_Name"], {}).setdefault(k, []).append(float(r["Counter_Value"]))
+    cols = sorted({k for c in acc.values() for k in c})
+    lines = ["| Counter | " + " | ".join(f"{k} (avg of {len(next(iter(acc.values()))[k])} dispatches)" for k in cols) + " |",
+             "|---|" + "---|" * len(cols)]
+    for c in sorted(acc):
+        lines.append(f"| {c} | " + " | ".join(f"{_mean(acc[c][k]):,.0f}" if k in acc[c] else "-" for k in cols) + " |")
+    return "\n".join(lines)
+
+
+def main(base: str, kernels=None) -> None:
+    if os.path.isdir(os.path.join(base, "kt")):
+        print(summarize(base))
+    else:  # a single --pmc run: just the table
+        print(counter_table(base, kernels))
 
 
 if __name__ == "__main__":
-    main(sys.argv[1] if len(sys.argv) > 1 else "gpurun_out/prof")
+    main(sys.argv[1] if len(sys.argv) > 1 else "gpurun_out/prof", sys.argv[2].split(",") if len(sys.argv) > 2 else None)
