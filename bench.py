@@ -30,7 +30,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="llama3-8b",
-                    choices=["llama3-8b", "llama-1.1b", "gpt2-small-f32", "mlp-sgd-f32", "ragged-4096",
+                    choices=["llama3-8b", "llama-1.1b", "gpt2-small-f32", "mlp-sgd-f32", "ragged-4096", "ragged-4096-packed",
                              "llama-1.1b-bf16", "llama-1.1b-f16", "llama-1.1b-f16-mixed"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-ceiling", action="store_true",
@@ -68,8 +68,8 @@ def workload(name):
     if name == "llama-1.1b-f16-mixed":  # f16 tensors over f32 master weights and moments
         return dict(shapes=W.llama_1b_shapes(), mixed=True, half="f16", kind="adamw", lr=2e-4, wd=0.1,
                     betas=(0.9, 0.95), scaler=True, clip=1.0, p_sigma=0.02, g_sigma=1e-3)
-    if name == "ragged-4096":
-        return dict(shapes=[(1, n) for n in W.ragged_sizes()], mixed=True, kind="adamw", lr=2e-4,
+    if name in ("ragged-4096", "ragged-4096-packed"):  # packed: tensors back to back in two flat buffers
+        return dict(packed=name.endswith("packed"), shapes=[(1, n) for n in W.ragged_sizes()], mixed=True, kind="adamw", lr=2e-4,
                     wd=0.1, betas=(0.9, 0.95), scaler=True, clip=1.0, p_sigma=0.02, g_sigma=1e-3)
     if name == "gpt2-small-f32":
         return dict(shapes=W.gpt2_small_shapes(), mixed=False, kind="adam", lr=3e-4, wd=0.0,
@@ -203,8 +203,17 @@ def measure(name, steps, warmup, zero_grads="off", settle_s=2.0):
     pure, half = bool(cfg.get("pure")), cfg.get("half", "bf16")
     hdt = torch.float16 if half == "f16" else torch.bfloat16
     pdt = hdt if (cfg["mixed"] or pure) else torch.float32
-    params = [torch.empty(s, dtype=pdt, device=dev) for s in shapes]
-    grads = [torch.empty(s, dtype=pdt, device=dev) for s in shapes]
+    if cfg.get("packed"):
+        # most tensors then start at addresses that are only element-aligned
+        flat_p, flat_g = torch.empty(n, dtype=pdt, device=dev), torch.empty(n, dtype=pdt, device=dev)
+        offs = [0]
+        for r, c in shapes:
+            offs.append(offs[-1] + r * c)
+        params = [flat_p[offs[i]:offs[i + 1]].view(shapes[i]) for i in range(len(shapes))]
+        grads = [flat_g[offs[i]:offs[i + 1]].view(shapes[i]) for i in range(len(shapes))]
+    else:
+        params = [torch.empty(s, dtype=pdt, device=dev) for s in shapes]
+        grads = [torch.empty(s, dtype=pdt, device=dev) for s in shapes]
     if cfg["kind"] == "sgd":
         opt = nb.Sgd.new(cfg["lr"], shapes)
     elif cfg["kind"] == "adam":

@@ -136,38 +136,48 @@ uint32_t norm_grid(const Layout &L)
 
 // First stage of the norm / found_inf pass over `grads`; partials land in the
 // runtime's scratch.  Returns the grid used (0 for an empty list).
-// Where a norm pass leaves its per-workgroup partial results for the finalize launch.
+// Where a norm pass leaves its per-workgroup partial results for its second stage.
 struct NormScratch {
     double *partial_sumsq;  // [NBO_NORM_GRID_MAX]
     uint32_t *partial_flag; // [NBO_NORM_GRID_MAX]
     bool may_time;          // launches may be bracketed by timing events
 };
 
-NormScratch runtime_scratch(Runtime &rt) { return NormScratch{rt.partial_sumsq(), rt.partial_flag(), true}; }
+NormScratch runtime_scratch(Runtime &rt)
+{
+    return NormScratch{rt.partial_sumsq(), rt.partial_flag(), true};
+}
 
-uint32_t launch_norm(nbo_list *grads, const NboScalerDev *scaler, bool half_arithmetic, const NormScratch &ws)
+// The norm / found_inf pass over `grads` and its second stage `f` (everything but the partial
+// results and the grid filled in by the caller): two launches; for an empty list, the second
+// stage alone.
+void launch_norm(nbo_list *grads, const NboScalerDev *scaler, bool half_arithmetic, const NormScratch &ws,
+                 NboFinalizeArgs f)
 {
     Runtime &rt = Runtime::get();
+    f.partial_sumsq = ws.partial_sumsq;
+    f.partial_flag = ws.partial_flag;
+    f.grid = norm_grid(grads->layout);
     NboNormArgs a = {};
     a.L = grads->layout.dev;
     a.g_ptrs = grads->ptrs_dev;
     a.scaler = scaler;
     a.partial_sumsq = ws.partial_sumsq;
     a.partial_flag = ws.partial_flag;
-    a.grid = norm_grid(grads->layout);
+    a.grid = f.grid;
     // bf16 / f16 gradients are unscaled in f32 when they feed f32 state (the mixed-precision
     // composition) and in their own type when the optimizer itself is of that type or they are
     // scaled in place
     int k = kernel_for(K_NORM_BASE, K_NORM_F16, grads->dtype);
     if (half_arithmetic && grads->dtype == NBO_DT_BF16) k = K_NORM_PBF16;
     if (half_arithmetic && grads->dtype == NBO_DT_F16) k = K_NORM_PF16;
-    rt.launch_raw(k, a.grid, NBO_BLOCK, &a, ws.may_time);
-    return a.grid;
+    rt.launch_raw(k, a.grid, NBO_BLOCK, &a, ws.may_time); // nothing for an empty list
+    rt.launch_raw(K_FINALIZE, 1, NBO_BLOCK, &f, ws.may_time);
 }
 
-uint32_t launch_norm(nbo_list *grads, const NboScalerDev *scaler, bool half_arithmetic = false)
+void launch_norm(nbo_list *grads, const NboScalerDev *scaler, bool half_arithmetic, const NboFinalizeArgs &f)
 {
-    return launch_norm(grads, scaler, half_arithmetic, runtime_scratch(Runtime::get()));
+    launch_norm(grads, scaler, half_arithmetic, runtime_scratch(Runtime::get()), f);
 }
 
 // The three launches of one fused Trainer tail; `ws` is where the norm pass's partial results
@@ -177,11 +187,8 @@ void fused_step_launches(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, n
 {
     Runtime &rt = Runtime::get();
     NboFinalizeArgs f = {};
-    f.partial_sumsq = ws.partial_sumsq;
-    f.partial_flag = ws.partial_flag;
     // without scaler, clipping and nan policy the pass has nothing to decide, but
     // it still runs so that the trace records every step
-    f.grid = launch_norm(grads, scaler ? scaler->dev : nullptr, pure_half(opt), ws);
     f.check_finite = (scaler || (flags & NBO_STEP_SKIP_NONFINITE)) ? 1u : 0u;
     f.scaler = scaler ? scaler->dev : nullptr;
     f.gf = opt->gf;
@@ -189,7 +196,7 @@ void fused_step_launches(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, n
     f.trace = opt->trace;
     f.max_norm = max_norm;
     f.hyper = hyper_of(opt);
-    rt.launch_raw(K_FINALIZE, 1, NBO_BLOCK, &f, ws.may_time);
+    launch_norm(grads, scaler ? scaler->dev : nullptr, pure_half(opt), ws, f);
     NboUpdateArgs a = update_args(opt, params, grads, true, (flags & NBO_STEP_ZERO_GRADS) != 0);
     rt.launch_raw(update_kernel(opt, params), opt->layout.nchunks, NBO_BLOCK, &a, ws.may_time);
 }
@@ -750,16 +757,10 @@ int nbo_scaler_unscale_and_update(nbo_scaler *s, nbo_list *grads, int *ok)
         require(s && grads && ok, NBO_ERR_ARG, "null scaler, list or output");
         Runtime &rt = Runtime::get();
         NboFinalizeArgs f = {};
-        f.partial_sumsq = rt.partial_sumsq();
-        f.partial_flag = rt.partial_flag();
-        f.grid = launch_norm(grads, s->dev, true);
         f.check_finite = 1;
         f.scaler = s->dev;
         f.gf = rt.gf_scratch();
-        f.opt = nullptr;
-        f.trace = nullptr;
-        f.max_norm = 0.0;
-        rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
+        launch_norm(grads, s->dev, true, f);
         launch_scale(grads, rt.gf_scratch(), 1.0, 0);
         NboGradFactors g;
         rt.read_back(&g, rt.gf_scratch(), sizeof(g));
@@ -777,14 +778,9 @@ int nbo_clip_grad_norm(nbo_list *grads, double max_norm, double *norm)
         if (max_norm <= 0.0) return; // trainer.rs:501-503
         Runtime &rt = Runtime::get();
         NboFinalizeArgs f = {};
-        f.partial_sumsq = rt.partial_sumsq();
-        f.partial_flag = rt.partial_flag();
-        f.grid = launch_norm(grads, nullptr);
-        f.check_finite = 0;
-        f.scaler = nullptr;
         f.gf = rt.gf_scratch();
         f.max_norm = max_norm;
-        rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
+        launch_norm(grads, nullptr, false, f);
         launch_scale(grads, rt.gf_scratch(), 1.0, 1);
         NboGradFactors g;
         rt.read_back(&g, rt.gf_scratch(), sizeof(g));
@@ -798,12 +794,9 @@ int nbo_has_non_finite(nbo_list *grads, int *found)
         require(grads && found, NBO_ERR_ARG, "null list or output");
         Runtime &rt = Runtime::get();
         NboFinalizeArgs f = {};
-        f.partial_sumsq = rt.partial_sumsq();
-        f.partial_flag = rt.partial_flag();
-        f.grid = launch_norm(grads, nullptr);
         f.check_finite = 1;
         f.gf = rt.gf_scratch();
-        rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
+        launch_norm(grads, nullptr, false, f);
         NboGradFactors g;
         rt.read_back(&g, rt.gf_scratch(), sizeof(g));
         *found = g.found_inf ? 1 : 0;
@@ -913,14 +906,11 @@ int nbo_fused_step_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *c
         // one decision for all groups: the reference unscales and clips the whole
         // gradient list before any group's step (trainer.rs:230-283)
         NboFinalizeArgs f = {};
-        f.partial_sumsq = rt.partial_sumsq();
-        f.partial_flag = rt.partial_flag();
-        f.grid = launch_norm(all_grads, scaler ? scaler->dev : nullptr, n_groups > 0 && pure_half(opts[0]));
         f.check_finite = (scaler || (flags & NBO_STEP_SKIP_NONFINITE)) ? 1u : 0u;
         f.scaler = scaler ? scaler->dev : nullptr;
         f.gf = rt.gf_scratch();
         f.max_norm = max_norm;
-        rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
+        launch_norm(all_grads, scaler ? scaler->dev : nullptr, n_groups > 0 && pure_half(opts[0]), f);
         launch_group_updates(n_groups, opts, params, grads, scaler, flags);
     });
 }

@@ -41,6 +41,10 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef double f64x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+// the same 128 bits at an address that is only element-aligned (global memory takes such
+// accesses in one instruction; the type keeps the compiler from assuming more)
+typedef float f32x4_e __attribute__((ext_vector_type(4), aligned(4)));
+typedef double f64x2_e __attribute__((ext_vector_type(2), aligned(8)));
 
 #define DEV static __device__ __forceinline__
 
@@ -211,6 +215,28 @@ DEV void st_state(double *p, const double (&x)[2])
     NBO_STORE(v, GLOBAL_PTR(f64x2, p));
 }
 
+// ... at an address that is a whole number of elements, but not of vectors, into the array
+DEV void ld_state_e(const float *p, float (&x)[4])
+{
+    f32x4_e v = NBO_LOAD(GLOBAL_PTR(const f32x4_e, p));
+    x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+}
+DEV void ld_state_e(const double *p, double (&x)[2])
+{
+    f64x2_e v = NBO_LOAD(GLOBAL_PTR(const f64x2_e, p));
+    x[0] = v.x; x[1] = v.y;
+}
+DEV void st_state_e(float *p, const float (&x)[4])
+{
+    f32x4_e v = {x[0], x[1], x[2], x[3]};
+    NBO_STORE(v, GLOBAL_PTR(f32x4_e, p));
+}
+DEV void st_state_e(double *p, const double (&x)[2])
+{
+    f64x2_e v = {x[0], x[1]};
+    NBO_STORE(v, GLOBAL_PTR(f64x2_e, p));
+}
+
 template <int FMT> DEV void ld_state(const Half16<FMT> *p, Half16<FMT> (&x)[8])
 {
     const u32x4 v = NBO_LOAD(GLOBAL_PTR(const u32x4, p));
@@ -230,6 +256,10 @@ template <int FMT> DEV void st_state(Half16<FMT> *p, const Half16<FMT> (&x)[8])
     v.w = (uint32_t)x[6].bits | ((uint32_t)x[7].bits << 16);
     NBO_STORE(v, GLOBAL_PTR(u32x4, p));
 }
+
+// 16-bit state is only ever accessed at vector alignment (see Peel)
+template <int FMT> DEV void ld_state_e(const Half16<FMT> *p, Half16<FMT> (&x)[8]) { ld_state(p, x); }
+template <int FMT> DEV void st_state_e(Half16<FMT> *p, const Half16<FMT> (&x)[8]) { st_state(p, x); }
 
 // caller tensors: vector of VEC storage elements at byte address p
 template <int ST> struct IO;
@@ -422,6 +452,35 @@ template <typename T> DEV T *state_part(const NboArenaDev &A, const ChunkRef &c,
     return (T *)A.part[part] + c.soff + c.base;
 }
 
+// How a chunk of cnt elements is walked when the caller's tensors need not be vector-aligned:
+// `head` single elements up to the first address at which every tensor involved is aligned to
+// a whole vector of vbytes, then `nvec` whole vectors, then single elements for the rest.
+// That works when all tensors are misaligned by the same whole number of elements (tensors
+// packed back to back into flat parameter and gradient buffers are); otherwise, or when
+// `whole_vectors_only` forbids a shifted start, every element goes singly (head = cnt).
+struct Peel {
+    uint32_t head, nvec;
+};
+DEV Peel peel(uint32_t cnt, uint32_t vec, uint32_t sb, bool whole_vectors_only, uintptr_t a0, uintptr_t a1,
+              uintptr_t a2)
+{
+    const uint32_t vbytes = vec * sb;
+    const uint32_t mis = (uint32_t)a0 & (vbytes - 1);
+    Peel r = {cnt, 0};
+    if ((((uint32_t)a1 & (vbytes - 1)) != mis) || (((uint32_t)a2 & (vbytes - 1)) != mis) || (mis % sb) != 0) return r;
+    if (mis != 0 && whole_vectors_only) return r;
+    const uint32_t head = mis ? (vbytes - mis) / sb : 0;
+    if (head >= cnt) return r;
+    r.head = head;
+    r.nvec = (cnt - head) / vec;
+    return r;
+}
+DEV Peel peel(uint32_t cnt, uint32_t vec, uint32_t sb, bool wvo, uintptr_t a0) { return peel(cnt, vec, sb, wvo, a0, a0, a0); }
+DEV Peel peel(uint32_t cnt, uint32_t vec, uint32_t sb, bool wvo, uintptr_t a0, uintptr_t a1)
+{
+    return peel(cnt, vec, sb, wvo, a0, a1, a0);
+}
+
 // ---------------------------------------------------------------------------------
 // Optimizer update: one workgroup per chunk.
 template <int ST, int KIND, int VARIANT = NBO_UPDATE_VARIANT> DEV void update_body(const NboUpdateArgs &a)
@@ -549,29 +608,34 @@ template <int ST, int KIND, int VARIANT = NBO_UPDATE_VARIANT> DEV void update_bo
         return;
     }
 
-    // ragged chunk: whole vectors while they last (if the caller's pointers allow),
-    // then single elements
-    const uint32_t nvec = vec_ok ? c.cnt / VEC : 0;
-    for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
-        const uint32_t e = q * VEC;
+    // ragged chunk, or caller tensors that are not vector-aligned: single elements up to the
+    // first vector-aligned address of the caller's tensors, whole vectors from there (the state
+    // arrays are then read at element alignment, which needs 32- or 64-bit state), single
+    // elements for the rest
+    const Peel pl = peel(c.cnt, VEC, SB, sizeof(T) < 4, (uintptr_t)pp, (uintptr_t)pg);
+    for (uint32_t q = tid; q < pl.nvec; q += NBO_BLOCK) {
+        const uint32_t e = pl.head + q * VEC;
         T g[VEC], p[VEC], m[VEC] = {}, v[VEC] = {};
         IO<ST>::ldv(pg + (uint64_t)e * SB, g);
-        if (mixed) ld_state(aw + e, p);
+        if (mixed) ld_state_e(aw + e, p);
         else IO<ST>::ldv(pp + (uint64_t)e * SB, p);
-        if (use_m) ld_state(am + e, m);
-        if (has_v) ld_state(av + e, v);
+        if (use_m) ld_state_e(am + e, m);
+        if (has_v) ld_state_e(av + e, v);
 #pragma unroll
         for (int k = 0; k < VEC; k++) step_elem<T, KIND>(p[k], g[k], m[k], v[k], s);
-        if (mixed) st_state(aw + e, p);
+        if (mixed) st_state_e(aw + e, p);
         IO<ST>::stv(pp + (uint64_t)e * SB, p);
-        if (use_m) st_state(am + e, m);
-        if (has_v) st_state(av + e, v);
+        if (use_m) st_state_e(am + e, m);
+        if (has_v) st_state_e(av + e, v);
         if (zero_g) {
             T z[VEC] = {};
             IO<ST>::stv(pg + (uint64_t)e * SB, z);
         }
     }
-    for (uint32_t e = nvec * VEC + tid; e < c.cnt; e += NBO_BLOCK) {
+    // elements [0, head) and [head + nvec * VEC, cnt)
+    const uint32_t n_single = c.cnt - pl.nvec * VEC;
+    for (uint32_t i = tid; i < n_single; i += NBO_BLOCK) {
+        const uint32_t e = i < pl.head ? i : i + pl.nvec * VEC;
         T g = IO<ST>::ld1(pg + (uint64_t)e * SB);
         T p = mixed ? aw[e] : IO<ST>::ld1(pp + (uint64_t)e * SB);
         T m = use_m ? am[e] : (T)0;
@@ -642,121 +706,6 @@ DEV uint32_t block_or(uint32_t x, uint32_t *lds)
     return r;
 }
 
-// First stage of the norm / found_inf pass.  A fixed grid walks the chunks with
-// stride grid, so each block's partial sum depends only on the tensor list.
-//   u = g * inv_scale rounded to T (the unscaled gradient the reference stores),
-//   sumsq += (f64)u * (f64)u   (trainer.rs:509-510)
-// For f32/bf16 inputs the f64 product is exact, so fma(d, d, acc) rounds exactly
-// like the reference's separate multiply and add; for f64 inputs it would not, so
-// that case keeps the two roundings.
-template <int ST> DEV double sq_acc(double acc, typename Traits<ST>::T u)
-{
-    const double d = (double)u;
-    if (ST == NBO_F64) {
-        const double q = d * d;
-        return acc + q;
-    }
-    return __builtin_fma(d, d, acc);
-}
-
-template <int ST> DEV bool nonfinite(typename Traits<ST>::T x);
-template <> __device__ __forceinline__ bool nonfinite<NBO_F32>(float x) { return nonfinite_f32(x); }
-template <> __device__ __forceinline__ bool nonfinite<NBO_BF16>(float x) { return nonfinite_f32(x); }
-template <> __device__ __forceinline__ bool nonfinite<NBO_F64>(double x) { return nonfinite_f64(x); }
-template <> __device__ __forceinline__ bool nonfinite<NBO_PBF16>(BF x) { return x.nonfinite(); }
-template <> __device__ __forceinline__ bool nonfinite<NBO_F16>(float x) { return nonfinite_f32(x); }
-template <> __device__ __forceinline__ bool nonfinite<NBO_PF16>(HF x) { return x.nonfinite(); }
-
-// A 16-bit pattern as the arithmetic type of storage ST (exact).
-template <int ST> DEV typename Traits<ST>::T from_half_bits(uint32_t b);
-template <> __device__ __forceinline__ float from_half_bits<NBO_BF16>(uint32_t b) { return bf16_bits_to_f32(b); }
-template <> __device__ __forceinline__ float from_half_bits<NBO_F16>(uint32_t b) { return f16_bits_to_f32(b); }
-template <> __device__ __forceinline__ BF from_half_bits<NBO_PBF16>(uint32_t b) { return half_from_bits<FMT_BF16>(b); }
-template <> __device__ __forceinline__ HF from_half_bits<NBO_PF16>(uint32_t b) { return half_from_bits<FMT_F16>(b); }
-
-template <int ST> DEV void norm_body(const NboNormArgs &a)
-{
-    typedef typename Traits<ST>::T T;
-    enum { SB = Traits<ST>::SBYTES, VEC = Traits<ST>::VEC };
-    __shared__ double lds_d[NBO_BLOCK / 64];
-    __shared__ uint32_t lds_u[NBO_BLOCK / 64];
-    const uint32_t tid = threadIdx.x;
-    const T inv = a.scaler ? (T)(1.0 / a.scaler->scale) : (T)1; // core.rs:355
-    double acc = 0.0;
-    uint32_t bad = 0;
-
-    for (uint32_t ci = blockIdx.x; ci < a.L.nchunks; ci += a.grid) {
-        const ChunkRef c = chunk_ref(a.L, ci);
-        const char *pg = (const char *)a.g_ptrs[c.t] + c.base * SB;
-        uint32_t done = 0;
-        if constexpr (SB == 2) {
-            // 8 half-width elements per 128-bit load.  Inf / NaN test on both halves of a word
-            // at once: adding the exponent field's lowest bit to the masked exponent carries
-            // into the sign position exactly when the exponent is all ones.
-            constexpr bool is_bf = ST == NBO_BF16 || ST == NBO_PBF16;
-            constexpr uint32_t EXP_MASK = is_bf ? 0x7F807F80u : 0x7C007C00u;
-            constexpr uint32_t EXP_LSB = is_bf ? 0x00800080u : 0x04000400u;
-            if ((((uintptr_t)pg) & 15u) == 0) {
-                const uint32_t nvec = c.cnt / 8;
-                uint32_t carries = 0;
-                for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
-                    const u32x4 w = __builtin_nontemporal_load(GLOBAL_PTR(const u32x4, pg) + q);
-                    const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-                    for (int k = 0; k < 4; k++) {
-                        carries |= (ww[k] & EXP_MASK) + EXP_LSB;
-                        const T lo = from_half_bits<ST>(ww[k] & 0xFFFFu), hi = from_half_bits<ST>(ww[k] >> 16);
-                        acc = sq_acc<ST>(acc, (T)(lo * inv));
-                        acc = sq_acc<ST>(acc, (T)(hi * inv));
-                    }
-                }
-                bad |= (uint32_t)((carries & 0x80008000u) != 0);
-                done = nvec * 8;
-            }
-        } else {
-            if ((((uintptr_t)pg) & 15u) == 0) {
-                const uint32_t nvec = c.cnt / VEC;
-                for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
-                    T x[VEC];
-                    IO<ST>::ldv(pg + (uint64_t)q * VEC * SB, x);
-#pragma unroll
-                    for (int k = 0; k < VEC; k++) {
-                        bad |= (uint32_t)nonfinite<ST>(x[k]);
-                        acc = sq_acc<ST>(acc, x[k] * inv);
-                    }
-                }
-                done = nvec * VEC;
-            }
-        }
-        for (uint32_t e = done + tid; e < c.cnt; e += NBO_BLOCK) {
-            const T x = IO<ST>::ld1(pg + (uint64_t)e * SB);
-            bad |= (uint32_t)nonfinite<ST>(x);
-            acc = sq_acc<ST>(acc, x * inv);
-        }
-    }
-    const double bs = block_sum(acc, lds_d);
-    const uint32_t bo = block_or(bad, lds_u);
-    if (tid == 0) {
-        a.partial_sumsq[blockIdx.x] = bs;
-        a.partial_flag[blockIdx.x] = bo;
-    }
-}
-
-#define NBO_NORM_KERNEL(name, ST)                                                           \
-    extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboNormArgs a)       \
-    {                                                                                       \
-        norm_body<ST>(a);                                                                   \
-    }
-NBO_NORM_KERNEL(nbo_norm_f32, NBO_F32)
-NBO_NORM_KERNEL(nbo_norm_bf16, NBO_BF16)
-NBO_NORM_KERNEL(nbo_norm_f64, NBO_F64)
-// bf16 gradients of a bf16 optimizer: the unscaled gradient is itself a bf16 value
-// (g * bf16(1/scale), rounded to bf16) before it is squared.
-NBO_NORM_KERNEL(nbo_norm_pbf16, NBO_PBF16)
-NBO_NORM_KERNEL(nbo_norm_f16, NBO_F16)
-NBO_NORM_KERNEL(nbo_norm_pf16, NBO_PF16)
-
-// ---------------------------------------------------------------------------------
 // Per-step scalars (alg.rs:120-135 AdamW, 265-277 Adam, 393-395 Sgd).  A skipped
 // step leaves step_count alone, because the reference never calls step() then.
 DEV void prep_step(NboOptimDev *o, const NboHyper &h, const NboGradFactors *f)
@@ -834,11 +783,11 @@ extern "C" __global__ __launch_bounds__(64) void nbo_prep(const NboPrepArgs a)
 
 // Second stage: reduce the per-block partials in a fixed order, then the scalar
 // logic of GradScaler::unscale_and_update (core.rs:369-385) and clip_grad_norm
-// (trainer.rs:501-517).  Single workgroup.
-extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_finalize(const NboFinalizeArgs a)
+// (trainer.rs:501-517).  Run by one whole workgroup.  (Letting the norm pass's last workgroup
+// do this instead of a launch of its own was tried and is slower: the device-wide ticket
+// counter that finds the last workgroup costs the pass more than the launch it saves.)
+DEV void finalize_body(const NboFinalizeArgs &a, double *lds_d, uint32_t *lds_u)
 {
-    __shared__ double lds_d[NBO_BLOCK / 64];
-    __shared__ uint32_t lds_u[NBO_BLOCK / 64];
     const uint32_t tid = threadIdx.x;
     double acc = 0.0;
     uint32_t bad = 0;
@@ -894,6 +843,128 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_finalize(const NboFi
     if (a.trace) trace_step(a.trace, &f, a.opt, scale_after);
 }
 
+extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_finalize(const NboFinalizeArgs a)
+{
+    __shared__ double lds_d[NBO_BLOCK / 64];
+    __shared__ uint32_t lds_u[NBO_BLOCK / 64];
+    finalize_body(a, lds_d, lds_u);
+}
+
+// First stage of the norm / found_inf pass.  A fixed grid walks the chunks with
+// stride grid, so each block's partial sum depends only on the tensor list.
+//   u = g * inv_scale rounded to T (the unscaled gradient the reference stores),
+//   sumsq += (f64)u * (f64)u   (trainer.rs:509-510)
+// For f32/bf16 inputs the f64 product is exact, so fma(d, d, acc) rounds exactly
+// like the reference's separate multiply and add; for f64 inputs it would not, so
+// that case keeps the two roundings.
+template <int ST> DEV double sq_acc(double acc, typename Traits<ST>::T u)
+{
+    const double d = (double)u;
+    if (ST == NBO_F64) {
+        const double q = d * d;
+        return acc + q;
+    }
+    return __builtin_fma(d, d, acc);
+}
+
+template <int ST> DEV bool nonfinite(typename Traits<ST>::T x);
+template <> __device__ __forceinline__ bool nonfinite<NBO_F32>(float x) { return nonfinite_f32(x); }
+template <> __device__ __forceinline__ bool nonfinite<NBO_BF16>(float x) { return nonfinite_f32(x); }
+template <> __device__ __forceinline__ bool nonfinite<NBO_F64>(double x) { return nonfinite_f64(x); }
+template <> __device__ __forceinline__ bool nonfinite<NBO_PBF16>(BF x) { return x.nonfinite(); }
+template <> __device__ __forceinline__ bool nonfinite<NBO_F16>(float x) { return nonfinite_f32(x); }
+template <> __device__ __forceinline__ bool nonfinite<NBO_PF16>(HF x) { return x.nonfinite(); }
+
+// A 16-bit pattern as the arithmetic type of storage ST (exact).
+template <int ST> DEV typename Traits<ST>::T from_half_bits(uint32_t b);
+template <> __device__ __forceinline__ float from_half_bits<NBO_BF16>(uint32_t b) { return bf16_bits_to_f32(b); }
+template <> __device__ __forceinline__ float from_half_bits<NBO_F16>(uint32_t b) { return f16_bits_to_f32(b); }
+template <> __device__ __forceinline__ BF from_half_bits<NBO_PBF16>(uint32_t b) { return half_from_bits<FMT_BF16>(b); }
+template <> __device__ __forceinline__ HF from_half_bits<NBO_PF16>(uint32_t b) { return half_from_bits<FMT_F16>(b); }
+
+template <int ST> DEV void norm_body(const NboNormArgs &a)
+{
+    typedef typename Traits<ST>::T T;
+    enum { SB = Traits<ST>::SBYTES, VEC = Traits<ST>::VEC };
+    __shared__ double lds_d[NBO_BLOCK / 64];
+    __shared__ uint32_t lds_u[NBO_BLOCK / 64];
+    const uint32_t tid = threadIdx.x;
+    const T inv = a.scaler ? (T)(1.0 / a.scaler->scale) : (T)1; // core.rs:355
+    double acc = 0.0;
+    uint32_t bad = 0;
+
+    for (uint32_t ci = blockIdx.x; ci < a.L.nchunks; ci += a.grid) {
+        const ChunkRef c = chunk_ref(a.L, ci);
+        const char *pg = (const char *)a.g_ptrs[c.t] + c.base * SB;
+        // single elements up to the first 16-byte boundary, whole 128-bit vectors, single
+        // elements for the rest; every thread adds its elements in this order
+        constexpr uint32_t EPV = 16 / SB; // elements per 128-bit vector
+        const Peel pl = peel(c.cnt, EPV, SB, false, (uintptr_t)pg);
+        for (uint32_t e = tid; e < pl.head; e += NBO_BLOCK) {
+            const T x = IO<ST>::ld1(pg + (uint64_t)e * SB);
+            bad |= (uint32_t)nonfinite<ST>(x);
+            acc = sq_acc<ST>(acc, x * inv);
+        }
+        const char *pv = pg + (uint64_t)pl.head * SB;
+        if constexpr (SB == 2) {
+            // 8 half-width elements per 128-bit load.  Inf / NaN test on both halves of a word
+            // at once: adding the exponent field's lowest bit to the masked exponent carries
+            // into the sign position exactly when the exponent is all ones.
+            constexpr bool is_bf = ST == NBO_BF16 || ST == NBO_PBF16;
+            constexpr uint32_t EXP_MASK = is_bf ? 0x7F807F80u : 0x7C007C00u;
+            constexpr uint32_t EXP_LSB = is_bf ? 0x00800080u : 0x04000400u;
+            uint32_t carries = 0;
+            for (uint32_t q = tid; q < pl.nvec; q += NBO_BLOCK) {
+                const u32x4 w = __builtin_nontemporal_load(GLOBAL_PTR(const u32x4, pv) + q);
+                const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    carries |= (ww[k] & EXP_MASK) + EXP_LSB;
+                    const T lo = from_half_bits<ST>(ww[k] & 0xFFFFu), hi = from_half_bits<ST>(ww[k] >> 16);
+                    acc = sq_acc<ST>(acc, (T)(lo * inv));
+                    acc = sq_acc<ST>(acc, (T)(hi * inv));
+                }
+            }
+            bad |= (uint32_t)((carries & 0x80008000u) != 0);
+        } else {
+            for (uint32_t q = tid; q < pl.nvec; q += NBO_BLOCK) {
+                T x[VEC];
+                IO<ST>::ldv(pv + (uint64_t)q * VEC * SB, x);
+#pragma unroll
+                for (int k = 0; k < VEC; k++) {
+                    bad |= (uint32_t)nonfinite<ST>(x[k]);
+                    acc = sq_acc<ST>(acc, x[k] * inv);
+                }
+            }
+        }
+        for (uint32_t e = pl.head + pl.nvec * EPV + tid; e < c.cnt; e += NBO_BLOCK) {
+            const T x = IO<ST>::ld1(pg + (uint64_t)e * SB);
+            bad |= (uint32_t)nonfinite<ST>(x);
+            acc = sq_acc<ST>(acc, x * inv);
+        }
+    }
+    const double bs = block_sum(acc, lds_d);
+    const uint32_t bo = block_or(bad, lds_u);
+    if (tid == 0) {
+        a.partial_sumsq[blockIdx.x] = bs;
+        a.partial_flag[blockIdx.x] = bo;
+    }
+}
+
+#define NBO_NORM_KERNEL(name, ST)                                                           \
+    extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboNormArgs a)       \
+    {                                                                                       \
+        norm_body<ST>(a);                                                                   \
+    }
+NBO_NORM_KERNEL(nbo_norm_f32, NBO_F32)
+NBO_NORM_KERNEL(nbo_norm_bf16, NBO_BF16)
+NBO_NORM_KERNEL(nbo_norm_f64, NBO_F64)
+// bf16 gradients of a bf16 optimizer: the unscaled gradient is itself a bf16 value
+// (g * bf16(1/scale), rounded to bf16) before it is squared.
+NBO_NORM_KERNEL(nbo_norm_pbf16, NBO_PBF16)
+NBO_NORM_KERNEL(nbo_norm_f16, NBO_F16)
+NBO_NORM_KERNEL(nbo_norm_pf16, NBO_PF16)
+
 // ---------------------------------------------------------------------------------
 // In-place gradient passes of the unfused API: multiply by a factor, or zero.
 template <int ST> DEV void scale_body(const NboScaleArgs &a)
@@ -917,11 +988,10 @@ template <int ST> DEV void scale_body(const NboScaleArgs &a)
             zero = true;
         }
     }
-    const bool vec_ok = (((uintptr_t)pg) & (VEC * SB - 1)) == 0;
-    const uint32_t nvec = vec_ok ? c.cnt / VEC : 0;
-    for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
+    const Peel pl = peel(c.cnt, VEC, SB, false, (uintptr_t)pg);
+    for (uint32_t q = tid; q < pl.nvec; q += NBO_BLOCK) {
         T x[VEC] = {};
-        char *p = pg + (uint64_t)q * VEC * SB;
+        char *p = pg + ((uint64_t)pl.head + (uint64_t)q * VEC) * SB;
         if (!zero) {
             IO<ST>::ldv(p, x);
 #pragma unroll
@@ -929,7 +999,9 @@ template <int ST> DEV void scale_body(const NboScaleArgs &a)
         }
         IO<ST>::stv(p, x);
     }
-    for (uint32_t e = nvec * VEC + tid; e < c.cnt; e += NBO_BLOCK) {
+    const uint32_t n_single = c.cnt - pl.nvec * VEC; // elements [0, head) and [head + nvec * VEC, cnt)
+    for (uint32_t i = tid; i < n_single; i += NBO_BLOCK) {
+        const uint32_t e = i < pl.head ? i : i + pl.nvec * VEC;
         char *p = pg + (uint64_t)e * SB;
         const T x = zero ? (T)0 : IO<ST>::ld1(p) * f;
         IO<ST>::st1(p, x);
@@ -959,24 +1031,26 @@ template <int ST> DEV void accum_body(const NboAccumArgs &a)
     const ChunkRef c = chunk_ref(a.L, blockIdx.x);
     char *pa = (char *)a.a_ptrs[c.t] + c.base * SB;
     char *pb = (char *)a.b_ptrs[c.t] + c.base * SB;
-    const bool vec_ok = ((((uintptr_t)pa) | ((uintptr_t)pb)) & (VEC * SB - 1)) == 0;
-    const uint32_t nvec = vec_ok ? c.cnt / VEC : 0;
-    for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
+    const Peel pl = peel(c.cnt, VEC, SB, false, (uintptr_t)pa, (uintptr_t)pb);
+    for (uint32_t q = tid; q < pl.nvec; q += NBO_BLOCK) {
+        const uint64_t off = ((uint64_t)pl.head + (uint64_t)q * VEC) * SB;
         T x[VEC], y[VEC];
-        IO<ST>::ldv(pa + (uint64_t)q * VEC * SB, x);
-        IO<ST>::ldv(pb + (uint64_t)q * VEC * SB, y);
+        IO<ST>::ldv(pa + off, x);
+        IO<ST>::ldv(pb + off, y);
 #pragma unroll
         for (int k = 0; k < VEC; k++) x[k] = x[k] + y[k];
-        IO<ST>::stv(pa + (uint64_t)q * VEC * SB, x);
+        IO<ST>::stv(pa + off, x);
         if (a.zero_b) {
             T z[VEC] = {};
-            IO<ST>::stv(pb + (uint64_t)q * VEC * SB, z);
+            IO<ST>::stv(pb + off, z);
         }
     }
-    for (uint32_t e = nvec * VEC + tid; e < c.cnt; e += NBO_BLOCK) {
-        const T x = IO<ST>::ld1(pa + (uint64_t)e * SB) + IO<ST>::ld1(pb + (uint64_t)e * SB);
-        IO<ST>::st1(pa + (uint64_t)e * SB, x);
-        if (a.zero_b) IO<ST>::st1(pb + (uint64_t)e * SB, (T)0);
+    const uint32_t n_single = c.cnt - pl.nvec * VEC; // elements [0, head) and [head + nvec * VEC, cnt)
+    for (uint32_t i = tid; i < n_single; i += NBO_BLOCK) {
+        const uint64_t off = (uint64_t)(i < pl.head ? i : i + pl.nvec * VEC) * SB;
+        const T x = IO<ST>::ld1(pa + off) + IO<ST>::ld1(pb + off);
+        IO<ST>::st1(pa + off, x);
+        if (a.zero_b) IO<ST>::st1(pb + off, (T)0);
     }
 }
 
@@ -1012,10 +1086,22 @@ template <int ST> DEV void accnorm_body(const NboAccNormArgs &a)
         const ChunkRef c = chunk_ref(a.L, ci);
         char *pa = (char *)a.acc_ptrs[c.t] + c.base * SB;
         char *pg = (char *)a.g_ptrs[c.t] + c.base * SB;
-        const bool vec_ok = ((((uintptr_t)pa) | ((uintptr_t)pg)) & 15u) == 0;
-        const uint32_t nvec = vec_ok ? c.cnt / VEC : 0;
-        for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
-            const uint64_t off = (uint64_t)q * VEC * SB;
+        // the norm pass's walk: single elements up to the first 16-byte boundary, whole vectors,
+        // single elements for the rest (buffer and gradients misaligned alike, else all single)
+        const Peel pl = peel(c.cnt, VEC, SB, false, (uintptr_t)pa, (uintptr_t)pg);
+        auto single = [&](uint32_t e) {
+            const uint64_t off = (uint64_t)e * SB;
+            const T g = IO<ST>::ld1(pg + off);
+            bad |= (uint32_t)nonfinite<ST>(g);
+            const T u = g * inv;
+            const T b = IO<ST>::ld1(pa + off) + u;
+            acc = sq_acc<ST>(acc, b);
+            IO<ST>::st1(pa + off, b);
+            if (write_g) IO<ST>::st1(pg + off, u);
+        };
+        for (uint32_t e = tid; e < pl.head; e += NBO_BLOCK) single(e);
+        for (uint32_t q = tid; q < pl.nvec; q += NBO_BLOCK) {
+            const uint64_t off = ((uint64_t)pl.head + (uint64_t)q * VEC) * SB;
             T g[VEC], b[VEC];
             IO<ST>::ldv(pg + off, g);
             IO<ST>::ldv(pa + off, b);
@@ -1029,16 +1115,7 @@ template <int ST> DEV void accnorm_body(const NboAccNormArgs &a)
             IO<ST>::stv(pa + off, b);
             if (write_g) IO<ST>::stv(pg + off, g);
         }
-        for (uint32_t e = nvec * VEC + tid; e < c.cnt; e += NBO_BLOCK) {
-            const uint64_t off = (uint64_t)e * SB;
-            const T g = IO<ST>::ld1(pg + off);
-            bad |= (uint32_t)nonfinite<ST>(g);
-            const T u = g * inv;
-            const T b = IO<ST>::ld1(pa + off) + u;
-            acc = sq_acc<ST>(acc, b);
-            IO<ST>::st1(pa + off, b);
-            if (write_g) IO<ST>::st1(pg + off, u);
-        }
+        for (uint32_t e = pl.head + pl.nvec * VEC + tid; e < c.cnt; e += NBO_BLOCK) single(e);
     }
     const double bs = block_sum(acc, lds_d);
     const uint32_t bo = block_or(bad, lds_u);
@@ -1098,6 +1175,41 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_cast_master(const Nb
 // operation is one IEEE operation in the arithmetic type, rounded to the element type:
 // for bf16 that is the f32 operation followed by bf16::from_f32
 // (common/scalar/mod.rs:253-351), including the product inside axpy.
+// Vector accesses of the element-wise passes: 128 bits wide for every element type, i.e. 8
+// elements of a 16-bit tensor computed in f32 (the update kernels take those 4 at a time, in
+// step with their 128-bit f32 state vectors).
+template <int ST> struct EwIO {
+    typedef typename Traits<ST>::T T;
+    enum { EV = Traits<ST>::VEC };
+    DEV void ld(const char *p, T (&x)[EV]) { IO<ST>::ldv(p, x); }
+    DEV void st(char *p, const T (&x)[EV]) { IO<ST>::stv(p, x); }
+};
+template <int ST> struct EwIOHalfWide {
+    enum { EV = 8 };
+    DEV void ld(const char *p, float (&x)[8])
+    {
+        const u32x4 v = NBO_LOAD(GLOBAL_PTR(const u32x4, p));
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            x[2 * k] = from_half_bits<ST>(w[k] & 0xFFFFu);
+            x[2 * k + 1] = from_half_bits<ST>(w[k] >> 16);
+        }
+    }
+    DEV void st(char *p, const float (&x)[8])
+    {
+        uint32_t w[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+            w[k] = ST == NBO_BF16 ? f32_to_bf16_bits(x[2 * k]) | (f32_to_bf16_bits(x[2 * k + 1]) << 16)
+                                  : f32_to_f16_bits(x[2 * k]) | (f32_to_f16_bits(x[2 * k + 1]) << 16);
+        const u32x4 v = {w[0], w[1], w[2], w[3]};
+        NBO_STORE(v, GLOBAL_PTR(u32x4, p));
+    }
+};
+template <> struct EwIO<NBO_BF16> : EwIOHalfWide<NBO_BF16> {};
+template <> struct EwIO<NBO_F16> : EwIOHalfWide<NBO_F16> {};
+
 template <int ST> DEV typename Traits<ST>::T to_storage_precision(typename Traits<ST>::T x) { return x; }
 template <> __device__ __forceinline__ float to_storage_precision<NBO_BF16>(float x)
 {
@@ -1140,7 +1252,7 @@ template <int ST, typename T> DEV T ew_elem(uint32_t op, T o, T a, T b, T s)
 template <int ST> DEV void ew_body(const NboEwArgs &a)
 {
     typedef typename Traits<ST>::T T;
-    enum { SB = Traits<ST>::SBYTES, VEC = Traits<ST>::VEC };
+    enum { SB = Traits<ST>::SBYTES, VEC = EwIO<ST>::EV };
     const uint32_t tid = threadIdx.x;
     const ChunkRef c = chunk_ref(a.L, blockIdx.x);
     const uint32_t op = a.op;
@@ -1151,20 +1263,20 @@ template <int ST> DEV void ew_body(const NboEwArgs &a)
     const char *pa = use_a ? (const char *)a.a_ptrs[c.t] + c.base * SB : po;
     const char *pb = use_b ? (const char *)a.b_ptrs[c.t] + c.base * SB : po;
     const T s = to_storage_precision<ST>((T)a.s);
-    const bool vec_ok = ((((uintptr_t)po) | ((uintptr_t)pa) | ((uintptr_t)pb)) & (VEC * SB - 1)) == 0;
-    const uint32_t nvec = vec_ok ? c.cnt / VEC : 0;
-    for (uint32_t q = tid; q < nvec; q += NBO_BLOCK) {
-        const uint64_t off = (uint64_t)q * VEC * SB;
+    const Peel pl = peel(c.cnt, VEC, SB, false, (uintptr_t)po, (uintptr_t)pa, (uintptr_t)pb);
+    for (uint32_t q = tid; q < pl.nvec; q += NBO_BLOCK) {
+        const uint64_t off = ((uint64_t)pl.head + (uint64_t)q * VEC) * SB;
         T o[VEC] = {}, x[VEC] = {}, y[VEC] = {};
-        if (use_a) IO<ST>::ldv(pa + off, x);
-        if (use_b) IO<ST>::ldv(pb + off, y);
-        if (use_o) IO<ST>::ldv(po + off, o);
+        if (use_a) EwIO<ST>::ld(pa + off, x);
+        if (use_b) EwIO<ST>::ld(pb + off, y);
+        if (use_o) EwIO<ST>::ld(po + off, o);
 #pragma unroll
         for (int k = 0; k < VEC; k++) o[k] = ew_elem<ST, T>(op, o[k], x[k], y[k], s);
-        IO<ST>::stv(po + off, o);
+        EwIO<ST>::st(po + off, o);
     }
-    for (uint32_t e = nvec * VEC + tid; e < c.cnt; e += NBO_BLOCK) {
-        const uint64_t off = (uint64_t)e * SB;
+    const uint32_t n_single = c.cnt - pl.nvec * VEC; // elements [0, head) and [head + nvec * VEC, cnt)
+    for (uint32_t i = tid; i < n_single; i += NBO_BLOCK) {
+        const uint64_t off = (uint64_t)(i < pl.head ? i : i + pl.nvec * VEC) * SB;
         const T x = use_a ? IO<ST>::ld1(pa + off) : (T)0;
         const T y = use_b ? IO<ST>::ld1(pb + off) : (T)0;
         const T o = use_o ? IO<ST>::ld1(po + off) : (T)0;

@@ -136,16 +136,6 @@ struct NboUpdateArgs {
     double sgd_lr, sgd_momentum, sgd_weight_decay;
 };
 
-struct NboNormArgs {
-    NboLayoutDev L;
-    const uint64_t *g_ptrs;
-    const NboScalerDev *scaler; // null: no unscale, inv_scale = 1
-    double *partial_sumsq;      // [grid]
-    uint32_t *partial_flag;     // [grid]
-    uint32_t grid;
-    uint32_t pad;
-};
-
 struct NboFinalizeArgs {
     const double *partial_sumsq;
     const uint32_t *partial_flag;
@@ -161,6 +151,17 @@ struct NboFinalizeArgs {
     uint32_t use_sumsq_in;
     uint32_t pad;
 };
+
+struct NboNormArgs {
+    NboLayoutDev L;
+    const uint64_t *g_ptrs;
+    const NboScalerDev *scaler; // null: no unscale, inv_scale = 1
+    double *partial_sumsq;      // [grid]
+    uint32_t *partial_flag;     // [grid]
+    uint32_t grid;
+    uint32_t pad;
+};
+
 
 struct NboPrepArgs {
     NboOptimDev *opt;
