@@ -17,6 +17,7 @@
 #include <optional>
 #include <sstream>
 #include <string>
+#include <type_traits>
 #include <sys/stat.h>
 #include <utility>
 #include <vector>
@@ -319,14 +320,22 @@ template <typename F> void tensor_file(const char *kind, F &&call)
 }
 } // namespace detail
 
-// checkpoint.rs:38-69.  `params` / `names` are the module's state_dict (for a
-// mixed-precision optimizer: its f32 master weights).
+// checkpoint.rs:38-69.  `params` / `names` are the module's state_dict.  A mixed-precision
+// optimizer's checkpoint keeps its f32 master weights as the parameters, under the parameters'
+// names: the 16-bit tensors are derived from them and could not restore them.
 template <typename Opt>
 void save_checkpoint(const std::string &dir, TensorList &params, const std::vector<std::string> &names, Opt &optimizer,
                      GradScaler *scaler, const ScheduleState *schedule, const TrainState &state)
 {
     ::mkdir(dir.c_str(), 0777); // fs::create_dir_all for the last component; an existing directory is fine
-    detail::tensor_file("State", [&] { save_tensors(dir + "/params.nbla", params, names); });
+    bool from_master = false;
+    if constexpr (std::is_base_of_v<Optimizer, Opt>) {
+        if (optimizer.keeps_master()) {
+            detail::tensor_file("State", [&] { optimizer.save_master(dir + "/params.nbla", names); });
+            from_master = true;
+        }
+    }
+    if (!from_master) detail::tensor_file("State", [&] { save_tensors(dir + "/params.nbla", params, names); });
     detail::tensor_file("Optim", [&] { optimizer.save_state(dir + "/optim.nbla"); });
     write_meta(dir + "/meta.txt", optimizer, scaler, schedule, state);
 }
@@ -337,7 +346,17 @@ template <typename Opt>
 void load_checkpoint(const std::string &dir, TensorList &params, const std::vector<std::string> &names, Opt &optimizer,
                      GradScaler *scaler, std::optional<ScheduleState> &schedule, TrainState &state)
 {
-    detail::tensor_file("State", [&] { load_state_dict(dir + "/params.nbla", params, names); });
+    bool into_master = false;
+    if constexpr (std::is_base_of_v<Optimizer, Opt>) {
+        if (optimizer.keeps_master()) { // master weights into the optimizer, the 16-bit `params` narrowed from them
+            detail::tensor_file("State", [&] {
+                optimizer.load_master(dir + "/params.nbla", names);
+                optimizer.params_from_master(params);
+            });
+            into_master = true;
+        }
+    }
+    if (!into_master) detail::tensor_file("State", [&] { load_state_dict(dir + "/params.nbla", params, names); });
     detail::tensor_file("Optim", [&] { optimizer.load_state(dir + "/optim.nbla"); });
     MetaContents meta = read_meta(dir + "/meta.txt", optimizer);
     if (scaler && meta.scaler) scaler->load_state(*meta.scaler);

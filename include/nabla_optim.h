@@ -326,6 +326,15 @@ int nbo_optim_save_state(nbo_optim *opt, const char *path);
  * "bad tensor key: k", "m index out of range: i", "missing m{i}" / "missing v{i}"; other
  * prefixes are ignored.  Nothing is written unless the whole file checks out. */
 int nbo_optim_load_state(nbo_optim *opt, const char *path);
+/* params.nbla of a mixed-precision optimizer (one created with keep_master): its f32 master
+ * weights under names[i], in the place of the module's state_dict (checkpoint.rs:54-58) -- the
+ * 16-bit parameters are derived from them and would not restore them.  nbo_optim_load_master is
+ * load_tensors + Module::load_state_dict (module/core.rs:281-304) into the master weights, with
+ * load_state_dict's errors plus "missing parameter key: k" (every master tensor must be in the
+ * file); afterwards the master weights count as set, and nbo_optim_params_from_master gives the
+ * 16-bit parameters.  Nothing is written unless the file checks out. */
+int nbo_optim_save_master(nbo_optim *opt, const char *path, const char *const *names);
+int nbo_optim_load_master(nbo_optim *opt, const char *path, const char *const *names);
 /* The same for GroupOptimizer's OptimState (optim/groups.rs:320-350): group gi's tensors
  * carry the keys "g{gi}.m{i}" / "g{gi}.v{i}"; loading refuses any other key ("bad group tensor
  * key: k", "bad group index: x", "group index out of range: gi") and then applies each

@@ -268,6 +268,20 @@ public:
     // save_tensors, load_tensors into load_state_tensors; errors as StateError / RuntimeError
     void save_state(const std::string &path) { check(nbo_optim_save_state(handle(), path.c_str())); }
     void load_state(const std::string &path) { check(nbo_optim_load_state(handle(), path.c_str())); }
+    bool keeps_master() const { return master_; }
+    // params.nbla of a mixed-precision optimizer: its f32 master weights under the parameters' names
+    void save_master(const std::string &path, const std::vector<std::string> &names)
+    {
+        std::vector<const char *> raw;
+        for (const std::string &n : names) raw.push_back(n.c_str());
+        check(nbo_optim_save_master(handle(), path.c_str(), raw.data()));
+    }
+    void load_master(const std::string &path, const std::vector<std::string> &names)
+    {
+        std::vector<const char *> raw;
+        for (const std::string &n : names) raw.push_back(n.c_str());
+        check(nbo_optim_load_master(handle(), path.c_str(), raw.data()));
+    }
     void master_from_params(TensorList &params_half) { check(nbo_optim_master_from_params(handle(), params_half.handle())); }
     void params_from_master(TensorList &params_half) { check(nbo_optim_params_from_master(handle(), params_half.handle())); }
     // names of state_tensors() in their order (alg.rs:476-485, 553-562, 623-629)

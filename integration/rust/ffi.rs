@@ -91,6 +91,9 @@ extern "C" {
     pub fn nbo_nbla_load_list(path: *const c_char, list: *mut NboList, names: *const *const c_char) -> c_int;
     pub fn nbo_optim_save_state(opt: *mut NboOptim, path: *const c_char) -> c_int;
     pub fn nbo_optim_load_state(opt: *mut NboOptim, path: *const c_char) -> c_int;
+    // params.nbla of a mixed-precision optimizer: its f32 master weights (no counterpart in the reference)
+    pub fn nbo_optim_save_master(opt: *mut NboOptim, path: *const c_char, names: *const *const c_char) -> c_int;
+    pub fn nbo_optim_load_master(opt: *mut NboOptim, path: *const c_char, names: *const *const c_char) -> c_int;
     // groups.rs:320-350 (GroupOptimizer's state keys "g{gi}.m{i}" / "g{gi}.v{i}")
     pub fn nbo_optim_save_state_groups(n_groups: u64, opts: *const *mut NboOptim, path: *const c_char) -> c_int;
     pub fn nbo_optim_load_state_groups(n_groups: u64, opts: *const *mut NboOptim, path: *const c_char) -> c_int;

@@ -125,6 +125,8 @@ SYMBOLS = {
     "nbo_nbla_load_list": (C.c_int, [C.c_char_p, _P, C.POINTER(C.c_char_p)]),
     "nbo_optim_save_state": (C.c_int, [_P, C.c_char_p]),
     "nbo_optim_load_state": (C.c_int, [_P, C.c_char_p]),
+    "nbo_optim_save_master": (C.c_int, [_P, C.c_char_p, C.POINTER(C.c_char_p)]),
+    "nbo_optim_load_master": (C.c_int, [_P, C.c_char_p, C.POINTER(C.c_char_p)]),
     "nbo_optim_save_state_groups": (C.c_int, [C.c_uint64, C.POINTER(_P), C.c_char_p]),
     "nbo_optim_load_state_groups": (C.c_int, [C.c_uint64, C.POINTER(_P), C.c_char_p]),
     "nbo_copy_bytes": (C.c_int, [_P, _P, C.c_uint64]),

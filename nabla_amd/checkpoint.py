@@ -262,13 +262,39 @@ def load_optim_native(path: str, optimizer) -> None:
         _native(_lib.load().nbo_optim_load_state, optimizer._handle(), path.encode())
 
 
+def _keeps_master(optimizer) -> bool:
+    return bool(getattr(optimizer, "_master", False))
+
+
+def _groups_keep_master(optimizer) -> bool:
+    return hasattr(optimizer, "group_optimizers") and any(_keeps_master(o) for o in optimizer.group_optimizers())
+
+
 def save_checkpoint(directory: str, params: Sequence[Tuple[str, object]], optimizer,
                     scaler: Optional[GradScaler], schedule: Optional[ScheduleState],
                     state: TrainState, native: bool = False) -> None:
-    """checkpoint.rs:38-69.  `params` is the module's state_dict: (name, tensor) pairs;
-    for a mixed-precision optimizer pass its f32 master weights.  With `native` the two
-    tensor files are written by the library straight from device memory."""
+    """checkpoint.rs:38-69.  `params` is the module's state_dict: (name, tensor) pairs.  With
+    `native` the two tensor files are written by the library straight from device memory.
+    For a mixed-precision optimizer (16-bit parameters over f32 master weights) params.nbla
+    holds the master weights, under the parameters' names: the 16-bit tensors are derived from
+    them and could not restore them; both files then come straight from device memory."""
     os.makedirs(directory, exist_ok=True)
+    if _keeps_master(optimizer):
+        from . import _lib
+
+        _native(_lib.load().nbo_optim_save_master, optimizer._handle(), os.path.join(directory, PARAMS_FILE).encode(),
+                _name_array([n for n, _ in params]))
+        save_optim_native(os.path.join(directory, OPTIM_FILE), optimizer)
+        write_meta(os.path.join(directory, META_FILE), optimizer, scaler, schedule, state)
+        return
+    if _groups_keep_master(optimizer):
+        # the groups' master weights, put back into the module's order under the parameters' names
+        masters = [t for _, t in params]
+        for idxs, o in zip(optimizer.group_indices(), optimizer.group_optimizers()):
+            if _keeps_master(o):
+                for k, i in enumerate(idxs):
+                    masters[i] = o.read_state(f"w{k}")
+        params = [(n, m) for (n, _), m in zip(params, masters)]
     if native:
         save_params_native(os.path.join(directory, PARAMS_FILE), params)
         save_optim_native(os.path.join(directory, OPTIM_FILE), optimizer)
@@ -284,8 +310,45 @@ def load_checkpoint(directory: str, optimizer, scaler: Optional[GradScaler] = No
     tensors and meta are loaded into `optimizer`, the scaler state into `scaler`; the
     parameters are returned for the caller's module to take (load_state_dict) -- or, with
     `into` = the module's named device tensors, read into those by the library itself
-    (then `params` is None)."""
-    if into is not None:
+    (then `params` is None).  For a mixed-precision optimizer params.nbla holds its f32 master
+    weights: they go into the optimizer, and `into` (the module's named 16-bit tensors, needed
+    for their names) receives the parameters narrowed from them."""
+    if _keeps_master(optimizer):
+        from . import _lib
+        from .optim import TensorList
+
+        if into is None:
+            raise ValueError("a mixed-precision optimizer's checkpoint is loaded with into=[(name, 16-bit tensor), ...]: "
+                             "params.nbla holds its master weights under the parameters' names")
+        _native(_lib.load().nbo_optim_load_master, optimizer._handle(), os.path.join(directory, PARAMS_FILE).encode(),
+                _name_array([n for n, _ in into]))
+        optimizer.params_from_master(TensorList([t for _, t in into]))
+        load_optim_native(os.path.join(directory, OPTIM_FILE), optimizer)
+        params = None
+    elif _groups_keep_master(optimizer):
+        import torch
+
+        from .optim import TensorList
+
+        if into is None:
+            raise ValueError("a mixed-precision optimizer's checkpoint is loaded with into=[(name, 16-bit tensor), ...]: "
+                             "params.nbla holds its master weights under the parameters' names")
+        loaded = dict(load_tensors(os.path.join(directory, PARAMS_FILE)))
+        for idxs, o in zip(optimizer.group_indices(), optimizer.group_optimizers()):
+            tensors = [into[i][1] for i in idxs]
+            if not _keeps_master(o):
+                load_params_native(os.path.join(directory, PARAMS_FILE), [into[i] for i in idxs])
+                continue
+            for k, i in enumerate(idxs):
+                name = into[i][0]
+                if name not in loaded:
+                    raise CheckpointError("State", f"missing parameter key: {name}")
+                o.write_state(f"w{k}", torch.from_numpy(loaded[name].astype("float32")).to(tensors[k].device)
+                              .reshape(tensors[k].shape))
+            o.params_from_master(TensorList(tensors))
+        load_optim_native(os.path.join(directory, OPTIM_FILE), optimizer)
+        params = None
+    elif into is not None:
         load_params_native(os.path.join(directory, PARAMS_FILE), into)
         load_optim_native(os.path.join(directory, OPTIM_FILE), optimizer)
         params = None

@@ -1161,6 +1161,22 @@ int nbo_optim_load_state(nbo_optim *opt, const char *path)
     });
 }
 
+int nbo_optim_save_master(nbo_optim *opt, const char *path, const char *const *names)
+{
+    return guarded([&] {
+        require(opt != nullptr && path != nullptr, NBO_ERR_ARG, "null optimizer or path");
+        optim_save_master(opt, path, names);
+    });
+}
+
+int nbo_optim_load_master(nbo_optim *opt, const char *path, const char *const *names)
+{
+    return guarded([&] {
+        require(opt != nullptr && path != nullptr, NBO_ERR_ARG, "null optimizer or path");
+        optim_load_master(opt, path, names);
+    });
+}
+
 static void require_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path)
 {
     require(path != nullptr, NBO_ERR_ARG, "null path");

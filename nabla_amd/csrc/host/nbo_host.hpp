@@ -176,6 +176,8 @@ void nbla_save_list(const char *path, const nbo_list *list, const char *const *n
 void nbla_load_list(const char *path, nbo_list *list, const char *const *names);
 void optim_save_state(const nbo_optim *opt, const char *path);
 void optim_load_state(nbo_optim *opt, const char *path);
+void optim_save_master(const nbo_optim *opt, const char *path, const char *const *names);
+void optim_load_master(nbo_optim *opt, const char *path, const char *const *names);
 void optim_save_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path);
 void optim_load_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path);
 } // namespace nbo

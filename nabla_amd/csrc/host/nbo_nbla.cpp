@@ -392,6 +392,62 @@ void optim_load_state(nbo_optim *opt, const char *path)
     apply_optim_load(f.get(), opt, plan, b);
 }
 
+// params.nbla of a mixed-precision optimizer: the reference has no such optimizer, but what its
+// checkpoint holds as parameters (checkpoint.rs:54-58: the module's state_dict through
+// save_tensors) is here the f32 master weights -- the 16-bit parameters are derived from them.
+void optim_save_master(const nbo_optim *opt, const char *path, const char *const *names)
+{
+    const uint64_t nt = opt->layout.nt();
+    if (!opt->keep_master) fail(NBO_ERR_DTYPE, "optimizer was created without master weights");
+    if (!opt->master_valid) fail(NBO_ERR_NO_MASTER, "master weights not set");
+    if (nt && !names) fail(NBO_ERR_ARG, "null name array");
+    if (nt > 0xFFFFFFFFull) fail(NBO_ERR_TOO_LARGE, "too many tensors for the file format");
+    Runtime::get().sync();
+    FilePtr f = open_file(path, "wb");
+    Buffers b;
+    write_all(f.get(), "NBLA", 4);
+    write_u32(f.get(), (uint32_t)nt);
+    for (uint64_t t = 0; t < nt; t++) {
+        if (!names[t]) fail(NBO_ERR_ARG, "null tensor name");
+        write_header(f.get(), names[t], opt->layout.rows[t], opt->layout.cols[t]);
+        const char *dev = (const char *)opt->arena.part[opt->arena.part_w] + (size_t)opt->layout.soff[t] * 4;
+        stream_out(f.get(), dev, NBO_DT_F32, opt->layout.n[t], b);
+    }
+    if (std::fflush(f.get()) != 0) fail(NBO_ERR_IO, std::string("write failed: ") + std::strerror(errno));
+}
+
+// load_tensors + Module::load_state_dict (module/core.rs:281-304) into the master weights: the
+// same checks as nbla_load_list, and every master tensor must be in the file -- a master weight
+// that kept its old value would silently diverge from its 16-bit parameter.
+void optim_load_master(nbo_optim *opt, const char *path, const char *const *names)
+{
+    const uint64_t nt = opt->layout.nt();
+    if (!opt->keep_master) fail(NBO_ERR_DTYPE, "optimizer was created without master weights");
+    if (nt && !names) fail(NBO_ERR_ARG, "null name array");
+    FilePtr f = open_file(path, "rb");
+    const std::vector<Entry> index = read_index(f.get());
+    std::vector<long> at(nt, -1);
+    for (const Entry &e : index) {
+        uint64_t t = 0;
+        while (t < nt && e.name != names[t]) t++;
+        if (t == nt) fail(NBO_ERR_STATE_KEY, "unknown parameter key: " + e.name);
+        if (e.rows != opt->layout.rows[t] || e.cols != opt->layout.cols[t])
+            fail(NBO_ERR_SHAPE, "shape mismatch for '" + e.name + "': expected (" + std::to_string(opt->layout.rows[t]) +
+                                    ", " + std::to_string(opt->layout.cols[t]) + "), got (" + std::to_string(e.rows) +
+                                    ", " + std::to_string(e.cols) + ")");
+        at[t] = e.data_offset;
+    }
+    for (uint64_t t = 0; t < nt; t++)
+        if (at[t] < 0) fail(NBO_ERR_STATE_KEY, std::string("missing parameter key: ") + names[t]);
+    Buffers b;
+    for (uint64_t t = 0; t < nt; t++) {
+        seek_to(f.get(), at[t]);
+        char *dev = (char *)opt->arena.part[opt->arena.part_w] + (size_t)opt->layout.soff[t] * 4;
+        stream_in(f.get(), dev, NBO_DT_F32, opt->layout.n[t], b);
+    }
+    opt->master_valid = true;
+}
+
 // GroupOptimizer's OptimState (groups.rs:320-373): every group's tensors behind "g{gi}.".
 void optim_save_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path)
 {

@@ -231,6 +231,52 @@ def test_llama3_8b_mixed_adamw_7_steps(gpu):
     _mixed_full(gpu, shapes, 7, seed=5, whole_tensor=len(shapes) - 1)
 
 
+def test_adamw_chain_of_primitives_on_one_full_size_llama3_layer(gpu):
+    """The reference's own formulation of AdamW::step (optim/alg.rs:109-150) -- twelve Backend
+    passes with their temporaries, each a multi-tensor primitive launch here -- against the fused
+    update kernel on one Llama-3-8B layer at its real shapes (218,112,000 parameters, f32): every
+    element of parameters and moments, compared on the device, after each of three steps."""
+    import torch
+
+    from nabla_amd import backend as B
+
+    shapes = W.llama_8b_shapes()[:9]  # q, k, v, o, gate, up, down and the two norm vectors of layer 0
+    assert W.n_params(shapes) == 218_112_000
+    lr, b1, b2, eps, wd = 2e-4, 0.9, 0.95, 1e-8, 0.1
+    torch.manual_seed(11)
+    p = [torch.randn(s, device=gpu) * 0.02 for s in shapes]
+    fused_p = [t.clone() for t in p]
+    opt = nb.AdamW.new(lr, shapes).beta1(b1).beta2(b2).eps(eps).weight_decay(wd)
+    m, v = [torch.zeros_like(t) for t in p], [torch.zeros_like(t) for t in p]
+    t1, t2 = [torch.empty_like(t) for t in p], [torch.empty_like(t) for t in p]
+    lp, lm, lv, l1, l2 = (nb.TensorList(x) for x in (p, m, v, t1, t2))
+    f32 = np.float32
+    for step in range(1, 4):
+        g = [torch.randn(s, device=gpu) * 1e-3 for s in shapes]
+        lg = nb.TensorList(g)
+        opt.step(fused_p, g)
+        bc1, bc2 = 1.0 - O.powi(b1, step), 1.0 - O.powi(b2, step)
+        ss, ibc2, wd_lr = float(f32(lr / bc1)), float(f32(1.0 / bc2)), f32(wd * lr)
+        B.scale(lm, b1, out=lm)                      # m = &m * beta1
+        B.axpy_inplace(lm, 1.0 - b1, lg)             # m.axpy_inplace(1 - beta1, g)
+        B.scale(lv, b2, out=lv)                      # v = &v * beta2
+        B.emul(lg, lg, out=l1)                       # g_sq = g.emul(g)
+        B.axpy_inplace(lv, 1.0 - b2, l1)             # v.axpy_inplace(1 - beta2, &g_sq)
+        B.scale(lv, ibc2, out=l1)                    # v_scaled = &v * inv_bc2
+        B.powf(l1, 0.5, out=l1)                      # .powf(0.5)
+        B.map_add(l1, eps, out=l1)                   # .map(|x| x + eps)
+        B.scale(lm, ss, out=l2)                      # m_scaled = &m * step_size
+        B.ediv(l2, l1, out=l2)                       # update = m_scaled.ediv(&denom)
+        B.scale(lp, float(f32(1.0) - wd_lr), out=lp)  # p = &p * (1 - wd_lr), computed in T
+        B.axpy_inplace(lp, -1.0, l2)                 # p.axpy_inplace(-1, &update)
+        fm, fv = opt.moments()
+        for i in range(len(shapes)):
+            assert torch.equal(p[i].view(torch.int32), fused_p[i].view(torch.int32)), f"params {i}, step {step}"
+            assert torch.equal(m[i].view(torch.int32), fm[i].view(torch.int32)), f"m {i}, step {step}"
+            assert torch.equal(v[i].view(torch.int32), fv[i].view(torch.int32)), f"v {i}, step {step}"
+        del fm, fv, g, lg
+
+
 def test_ragged_4096_dynamic_scale_64_steps(gpu):
     """Config 4 in full: 4096 tensors, sizes log-uniform in [1, 65536], packed back to
     back (so most tensor addresses are only 2-byte aligned), growth interval 4, inf/NaN

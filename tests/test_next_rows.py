@@ -395,20 +395,34 @@ def test_checkpoint_round_trip_restores_bit_identical_training(gpu, tmp_path):
     for k in range(3):
         o1.fused_step(p1, grads[k], scaler=s1, max_norm=1.0)
     sched = S.ScheduleState(2e-4, S.Cosine(2, 10, 1e-5))
-    master = [(f"p{i}", o1.read_state(f"w{i}")) for i in range(len(shapes))]
-    ck.save_checkpoint(str(tmp_path), master, o1, s1, sched, ck.TrainState(1, 3, 1, 7))
+    # nothing but save_checkpoint and load_checkpoint: the module's (16-bit) named parameters go in,
+    # the f32 master weights are what params.nbla holds
+    named1 = [(f"p{i}", p1[i]) for i in range(len(shapes))]
+    ck.save_checkpoint(str(tmp_path), named1, o1, s1, sched, ck.TrainState(1, 3, 1, 7))
     assert sorted(os.listdir(tmp_path)) == ["meta.txt", "optim.nbla", "params.nbla"]
     names = [n for n, _ in ck.load_tensors(os.path.join(tmp_path, "optim.nbla"))]
     assert names == ["m0", "m1", "m2", "v0", "v1", "v2"]
+    saved = ck.load_tensors(os.path.join(tmp_path, "params.nbla"))
+    assert [n for n, _ in saved] == ["p0", "p1", "p2"]
+    for i, (_, a) in enumerate(saved):
+        w = H.to_host(o1.read_state(f"w{i}"))
+        assert np.array_equal(a.reshape(-1), w.astype(np.float64)), "params.nbla holds the f32 master weights, exactly"
+
+    assert not np.array_equal(saved[1][1].reshape(-1), O.bf16_to_f32(H.to_host(p1[1])).astype(np.float64)), \
+        "the 16-bit parameters themselves would have lost the low bits"
 
     o2, s2 = fresh()
-    params, st, sched2 = ck.load_checkpoint(str(tmp_path), o2, s2)
+    p2 = H.dev_list([np.zeros(r * c, np.uint16) for r, c in shapes], shapes)
+    with pytest.raises(ValueError, match="into="):
+        ck.load_checkpoint(str(tmp_path), o2, s2)
+    params, st, sched2 = ck.load_checkpoint(str(tmp_path), o2, s2, into=[(f"p{i}", p2[i]) for i in range(len(shapes))])
+    assert params is None
     assert (st.epoch, st.step, st.rng_state) == (1, 3, 7) and sched2 == sched
     assert o2.step_count() == 3 and o2.meta() == o1.meta()
     assert vars(s2.state()) == vars(s1.state())
-    p2 = H.dev_list([O.bf16_from_f32(a.astype(np.float32).reshape(-1)) for _, a in params], shapes)
-    for i, (_, a) in enumerate(params):
-        o2.write_state(f"w{i}", H.to_dev(a.astype(np.float32).reshape(-1), shapes[i]))
+    H.assert_bits_equal(H.host_list(p2), H.host_list(p1), "16-bit params derived from the restored master weights")
+    with pytest.raises(ck.CheckpointError, match="unknown parameter key: p0"):
+        ck.load_checkpoint(str(tmp_path), o2, s2, into=[(f"q{i}", p2[i]) for i in range(len(shapes))])
     for k in range(3, 5):
         o1.fused_step(p1, grads[k], scaler=s1, max_norm=1.0)
         o2.fused_step(p2, grads[k], scaler=s2, max_norm=1.0)
