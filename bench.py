@@ -44,6 +44,9 @@ def parse_args():
                     help="instead of the benchmark, run the library's plain copy kernel over "
                          "this many GiB (--steps times); a transfer of known size against which "
                          "rocprofv3's FETCH_SIZE / WRITE_SIZE counters are scaled")
+    ap.add_argument("--table", action="store_true",
+                    help="instead of one JSON line, measure every workload (--steps / --warmup each, --cpu-seconds of "
+                         "CPU baseline each) and print a markdown table")
     ap.add_argument("--settle-seconds", type=float, default=2.0,
                     help="idle time between setup and the warm-up steps, for the driver's background clearing of "
                          "the device memory that setup freed to finish")
@@ -386,6 +389,24 @@ def main():
         print(json.dumps({"calibrate": "nbo_copy_f32x4", "bytes_read": nbytes, "bytes_written": nbytes,
                           "launches": cnt.value, "avg_launch_ms": round(ms.value / max(cnt.value, 1), 4),
                           "GBps": round(2 * nbytes / (ms.value / max(cnt.value, 1)) / 1e6, 1)}))
+        return
+    if args.table:
+        names = ["mlp-sgd-f32", "gpt2-small-f32", "llama-1.1b", "llama-1.1b-bf16", "llama-1.1b-f16", "llama-1.1b-f16-mixed",
+                 "ragged-4096", "ragged-4096-packed", "llama3-8b"]
+        print(f"`python bench.py --table --steps {args.steps} --warmup {args.warmup} --cpu-seconds {args.cpu_seconds}` on one "
+              "MI355X: `value` is whole-step algorithmic HBM throughput, `kernel` the dominant kernel's (HIP events on the "
+              "launch stream), `CPU` the oracle in reference-faithful form on the host's cores on a sample of the same "
+              "workload.\n")
+        print("| workload | params | ms/step | value GB/s | % of 8 TB/s | params/s | dominant kernel GB/s | HBM regions "
+              "of state | CPU params/s (cores) | GPU/CPU |")
+        print("|---|---|---|---|---|---|---|---|---|---|")
+        for name in names:
+            d, cfg = measure(name, args.steps, args.warmup, "off", args.settle_seconds)
+            c = cpu_baseline(cfg, args.cpu_seconds)
+            print(f"| {name} | {d['config']['params']:,} | {d['ms_per_step']} | {d['value']} | {d['pct_of_peak']} | "
+                  f"{d['params_per_s']:.3e} | {d['roofline']['achieved']} ({d['roofline']['kernel']}) | "
+                  f"{d['config']['state_hbm_regions']} | {c['params_per_s']:.3e} ({c['cores']}) | "
+                  f"{d['params_per_s'] / c['params_per_s']:.0f}x |", flush=True)
         return
     out, cfg = measure(args.workload, args.steps, args.warmup, args.zero_grads, args.settle_seconds)
     if args.workload == "llama3-8b" and not args.primary_only:

@@ -115,14 +115,15 @@ bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
     size_t free_b = 0, total_b = 0;
     if (!ok(hipMemGetInfo(&free_b, &total_b))) return give_up("hipMemGetInfo failed");
     if (free_b < kReserveBytes + nparts * part_va) return give_up("not enough free memory to choose chunks from");
-    // The search creates at most `cap` chunks: what the arrays need twice over plus a few,
-    // NBO_PLACEMENT_MAX_GIB if set, never more than what is free minus a reserve.
+    // The search creates at most `cap` chunks (plan::chunk_cap): enough to walk past one region
+    // boundary, within half of what is free; NBO_PLACEMENT_MAX_GIB if set.
     size_t user_cap = 0;
     if (const char *e = std::getenv("NBO_PLACEMENT_MAX_GIB")) {
         const double gib = std::atof(e);
         if (gib > 0.0) user_cap = (size_t)(gib * (double)kGiB / (double)chunk);
     }
-    const size_t cap = plan::chunk_cap(total_full, (free_b - kReserveBytes - nparts * tail) / chunk, user_cap);
+    const size_t reach = (size_t)104 * kGiB / chunk; // one 96 GiB region and a bit
+    const size_t cap = plan::chunk_cap(total_full, (free_b - kReserveBytes - nparts * tail) / chunk, user_cap, reach);
     if (cap < total_full) return give_up("the chunk limit is below what the state arrays need");
 
     const char *dbg = std::getenv("NBO_PLACEMENT_DEBUG");
@@ -209,7 +210,7 @@ bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
             finder.add_chunks(usable, probe, halves);
             if (plan::enough(counts(), nparts, full)) break;
             if (!created || chunks.size() >= cap) break;
-            target = std::min(cap, chunks.size() + std::max<size_t>(2, total_full / 4));
+            target = std::min(cap, chunks.size() + std::max<size_t>({2, total_full / 4, chunks.size() / 4}));
         }
         std::vector<std::vector<size_t>> region_chunks = finder.chunks_per_region();
         if (debug) {

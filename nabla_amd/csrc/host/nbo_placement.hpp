@@ -26,9 +26,12 @@ namespace nbo {
 // together than two of different regions): every chunk is probed against the first one, the
 // threshold between "same" and "different" is the middle of the widest gap among those
 // measurements (no absolute bandwidth enters), and chunks that differ from the first are probed
-// against the first chunk of each further region.  Creation stops once every region to be used
-// holds its share of the chunks needed, or at a limit of twice the chunks needed plus eight
-// (NBO_PLACEMENT_MAX_GIB overrides it).  Chunk i of part j then comes from the
+// against the first chunk of each further region.  Creation stops once two or three regions
+// hold their share of the chunks needed, or at a limit: twice the chunks needed plus eight, or
+// 104 GiB if that is more (regions are runs of up to 96 GiB of consecutively created chunks, and
+// a search that is to find a second one must be allowed to walk that far) but then never more
+// than half of the free memory; NBO_PLACEMENT_MAX_GIB overrides the limit.  Until the search is
+// done it holds what it has created.  Chunk i of part j then comes from the
 // ((i + j) mod U)-th of the U regions in use, so that at every position of the update's walk
 // the parts sit in different regions and each region serves an equal share of the traffic.
 // Three parts use all regions found; two parts (Adam / AdamW without master weights) use the

@@ -20,30 +20,46 @@ namespace plan {
 
 constexpr size_t kMaxRegions = 3;
 // Two chunks of one region read and rewritten together run 10-20 % slower than two chunks of
-// different regions, and values of one kind scatter by a few per cent.  A gap between
-// neighbouring sorted measurements is taken for the gap between the two kinds only if it is at
-// least this wide.
-constexpr double kMinGapRatio = 1.06;
+// different regions.  Values of one kind scatter by a few per cent -- mostly downwards: a probe
+// that is disturbed is slower, never faster -- and a chunk the driver pieced together from two
+// regions measures half-way.  The measurements are therefore split into a low and a high class
+// where that separates them best (largest between-class variance), and the split is taken for
+// "same" against "different" only if the class means are at least kMinClassRatio apart and the
+// threshold lies between 3 and 30 % above what the anchor chunk measures against itself
+// (`same_pair`, its two halves, certainly of the low kind).  Anything else is scatter.
+constexpr double kMinClassRatio = 1.08;
+constexpr double kMinAboveSame = 1.03, kMaxAboveSame = 1.30;
 
 // Threshold between "same region" and "different region" from measurements that all involve
-// one fixed chunk: the geometric middle of the widest relative gap between neighbouring sorted
-// values, or +infinity when no gap is wide enough (every value then reads "same").  No absolute
-// bandwidth enters, so a faster, slower or busier GPU moves both kinds together.
-inline double gap_threshold(std::vector<double> samples)
+// one fixed chunk: the geometric mean of the two class means, or +infinity when the values do
+// not fall into two such classes (every value then reads "same").  No absolute bandwidth
+// enters, so a faster, slower or busier GPU moves both kinds together.
+inline double gap_threshold(std::vector<double> samples, double same_pair)
 {
     const double inf = std::numeric_limits<double>::infinity();
+    if (!(same_pair > 0.0)) return inf;
+    samples.push_back(same_pair);
     samples.erase(std::remove_if(samples.begin(), samples.end(), [](double v) { return !(v > 0.0); }), samples.end());
-    if (samples.size() < 2) return inf;
     std::sort(samples.begin(), samples.end());
-    double best = 1.0, thr = inf;
-    for (size_t k = 0; k + 1 < samples.size(); k++) {
-        const double r = samples[k + 1] / samples[k];
-        if (r > best) {
-            best = r;
-            thr = std::sqrt(samples[k] * samples[k + 1]);
+    const size_t n = samples.size();
+    if (n < 2) return inf;
+    double total = 0.0;
+    for (double v : samples) total += v;
+    double best = -1.0, lo_mean = 0.0, hi_mean = 0.0, lo_sum = 0.0;
+    for (size_t k = 0; k + 1 < n; k++) { // low class: samples[0..k]
+        lo_sum += samples[k];
+        const double m0 = lo_sum / (double)(k + 1), m1 = (total - lo_sum) / (double)(n - k - 1);
+        const double between = (double)(k + 1) * (double)(n - k - 1) * (m1 - m0) * (m1 - m0);
+        if (between > best) {
+            best = between;
+            lo_mean = m0;
+            hi_mean = m1;
         }
     }
-    return best >= kMinGapRatio ? thr : inf;
+    if (!(hi_mean >= lo_mean * kMinClassRatio)) return inf;
+    const double thr = std::sqrt(lo_mean * hi_mean);
+    if (thr < same_pair * kMinAboveSame || thr > same_pair * kMaxAboveSame) return inf;
+    return thr;
 }
 
 // Sorts chunks into at most three regions.  Chunks arrive in rounds (add_chunks).  One chunk is
@@ -71,10 +87,10 @@ public:
         anchor_ = 0;
         if (total_ == 0) return;
         for (size_t a = 0; a < kMaxAnchors && a < total_; a++) {
-            std::vector<double> v{base_of(a, halves)};
+            std::vector<double> v;
             for (size_t i = 0; i < total_; i++)
                 if (i != a) v.push_back(measure(a, i, probe));
-            const double t = gap_threshold(v);
+            const double t = gap_threshold(v, base_of(a, halves));
             if (std::isfinite(t)) {
                 threshold_ = t;
                 anchor_ = a;
@@ -216,13 +232,17 @@ inline std::vector<std::vector<int>> assign(std::vector<size_t> avail, uint32_t 
     return pick;
 }
 
-// How many chunks the search may create before it settles for what it has: twice what the
-// arrays need plus a few, within what is free.  On the GPUs measured, regions change every few
-// GiB of consecutively created chunks, and a search that needs more than this is not worth
-// holding more memory for.
-inline size_t chunk_cap(size_t needed, size_t free_chunks, size_t user_cap_chunks)
+// How many chunks the search may create (and hold until it is done) before it settles for what
+// it has.  Regions are runs of consecutively created chunks, up to 96 GiB long, so a search that
+// is to find a second region must be allowed to walk that far: twice what the arrays need plus
+// eight chunks, or `reach_chunks` (what covers one region and a bit) if that is more -- but
+// for the sake of whoever else allocates meanwhile never beyond half of what is free, unless the
+// arrays themselves need more.  A user's limit replaces all of that.
+inline size_t chunk_cap(size_t needed, size_t free_chunks, size_t user_cap_chunks, size_t reach_chunks)
 {
     size_t cap = 2 * needed + 8;
+    const size_t reach = std::min(reach_chunks, free_chunks / 2);
+    if (reach > cap) cap = reach;
     if (user_cap_chunks) cap = user_cap_chunks;
     return std::min(cap, free_chunks);
 }

@@ -65,14 +65,22 @@ static bool matches_truth(const RegionFinder &f, const std::vector<int> &truth)
 
 int main()
 {
-    // gap_threshold: the middle of the widest gap, nothing when the values are of one kind
-    CHECK(std::isinf(gap_threshold({5400, 5450, 5300, 5500})));
+    // gap_threshold: the middle of the widest gap above the anchor's own measure, nothing when
+    // the values are of one kind
+    CHECK(std::isinf(gap_threshold({5400, 5450, 5300, 5500}, 5400)));
     {
-        const double t = gap_threshold({5395, 5481, 5466, 5215, 5359, 6402, 6398, 6397});
+        const double t = gap_threshold({5481, 5466, 5215, 5359, 6402, 6398, 6397}, 5395);
         CHECK(t > 5481 && t < 6397);
     }
-    CHECK(std::isinf(gap_threshold({5400})));
-    CHECK(std::isinf(gap_threshold({0.0, -1.0, 5400})));
+    CHECK(std::isinf(gap_threshold({}, 5400)));
+    CHECK(std::isinf(gap_threshold({0.0, -1.0}, 5400)));
+    CHECK(std::isinf(gap_threshold({6400, 6390}, 0.0))); // no measure of "same": nothing can be told
+    // measured on one GPU: every chunk in the anchor's region, two disturbed (slow) probes; the
+    // gap below the cluster is scatter, not a second region
+    CHECK(std::isinf(gap_threshold({5590, 5566, 5656, 5613, 5622, 5616, 5618, 5614, 5654, 5050, 5075, 5517, 5567, 5424}, 5453)));
+    // a single early sample a little above the anchor's own measure is no gap either
+    CHECK(std::isinf(gap_threshold({5726}, 5385)));
+    CHECK(std::isfinite(gap_threshold({5726, 6337}, 5385)));
 
     // three regions in runs, as measured on one MI355X (5.2-5.7 vs 6.3-6.5 TB/s)
     {
@@ -223,10 +231,14 @@ int main()
         for (size_t i = 0; i < 3; i++) CHECK(!(pick[0][i] == pick[1][i] && pick[1][i] == pick[2][i]));
     }
 
-    // the creation limit: twice the need plus eight, a user's limit, never more than is free
-    CHECK(chunk_cap(12, 250, 0) == 32);
-    CHECK(chunk_cap(42, 60, 0) == 60);
-    CHECK(chunk_cap(12, 250, 20) == 20);
+    // the creation limit: twice the need plus eight or far enough to cross a region boundary
+    // (within half of what is free), a user's limit instead, never more than is free
+    CHECK(chunk_cap(12, 250, 0, 104) == 104);
+    CHECK(chunk_cap(12, 100, 0, 104) == 50);
+    CHECK(chunk_cap(12, 40, 0, 104) == 32);
+    CHECK(chunk_cap(87, 250, 0, 104) == 182);
+    CHECK(chunk_cap(42, 60, 0, 104) == 60);
+    CHECK(chunk_cap(12, 250, 20, 104) == 20);
     std::puts("placement plan: all checks passed");
     return 0;
 }
