@@ -133,6 +133,7 @@ bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
     struct Chunk {
         hipMemGenericAllocationHandle_t h;
         bool mapped_in_staging;
+        bool ready; // mapped and accessible: may be handed to the probe
         bool keep;
     };
     std::vector<Chunk> chunks;
@@ -182,6 +183,7 @@ bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
                 if (!ok(hipMemMap(chunk_va(idx), chunk, 0, c.h, 0))) return false;
                 chunks[idx].mapped_in_staging = true;
                 if (!set_rw(chunk_va(idx), chunk)) return false;
+                chunks[idx].ready = true;
             }
             return true;
         };
@@ -206,7 +208,7 @@ bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
         for (;;) {
             const bool created = create_until(target);
             size_t usable = chunks.size();
-            if (!created && usable && !chunks.back().mapped_in_staging) usable--; // created but not mapped
+            if (usable && !chunks.back().ready) usable--; // the driver refused to map it or to open it for access
             finder.add_chunks(usable, probe, halves);
             if (plan::enough(counts(), nparts, full)) break;
             if (!created || chunks.size() >= cap) break;

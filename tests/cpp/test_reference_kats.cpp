@@ -285,6 +285,104 @@ static void checkpoint_roundtrip_with_schedule()  // trainer.rs tests :249-304
     EXPECT(what.find("missing m0") != std::string::npos || what.find("optim kind mismatch") != std::string::npos);
 }
 
+// A bf16 tensor on the device, filled from floats (rounded to nearest even by the library's cast).
+struct HalfVec {
+    uint16_t *d = nullptr;
+    uint64_t n;
+    explicit HalfVec(uint64_t n_) : n(n_)
+    {
+        if (hipMalloc((void **)&d, n * sizeof(uint16_t)) != hipSuccess) std::abort();
+        if (hipMemset(d, 0, n * sizeof(uint16_t)) != hipSuccess) std::abort();
+    }
+    ~HalfVec() { (void)hipFree(d); }
+    Tensor tensor() const { return Tensor{d, 1, n, NBO_DT_BF16}; }
+    void put(const std::vector<uint16_t> &bits)
+    {
+        if (hipMemcpy(d, bits.data(), n * sizeof(uint16_t), hipMemcpyHostToDevice) != hipSuccess) std::abort();
+    }
+    std::vector<uint16_t> get() const
+    {
+        sync();
+        std::vector<uint16_t> v(n);
+        if (hipMemcpy(v.data(), d, n * sizeof(uint16_t), hipMemcpyDeviceToHost) != hipSuccess) std::abort();
+        return v;
+    }
+};
+
+// Checkpoint of a mixed-precision optimizer (bf16 tensors over f32 master weights; the
+// reference has no such optimizer, the file formats are checkpoint.rs:38-150's): the master
+// weights travel as an f32 params.nbla, and training resumed from the files continues with the
+// bits of the run that was never interrupted.
+static void mixed_precision_checkpoint_resumes_bit_for_bit()
+{
+    std::string dir = g_checkpoint_dir;
+    if (dir.empty()) {
+        char tmpl[] = "/tmp/nbo_ckpt_XXXXXX";
+        const char *made = mkdtemp(tmpl);
+        EXPECT(made != nullptr);
+        dir = made ? made : "/tmp";
+    }
+    dir += "/mixed";
+    const uint64_t n0 = 8192 + 37, n1 = 300;
+    const Shapes shapes = {{1, n0}, {1, n1}};
+    const std::vector<std::string> names = {"layer.w", "layer.b"};
+    auto fill = [](uint64_t n, uint32_t seed, uint16_t exp_bits) { // bf16 bit patterns of moderate size, both signs
+        std::vector<uint16_t> v(n);
+        uint32_t x = seed;
+        for (auto &e : v) {
+            x = x * 1664525u + 1013904223u;
+            e = (uint16_t)(((x >> 16) & 0x807f) | exp_bits);
+        }
+        return v;
+    };
+    HalfVec p0(n0), p1(n1), g0(n0), g1(n1);
+    p0.put(fill(n0, 1, 0x3c00)), p1.put(fill(n1, 2, 0x3c00));
+    TensorList params({p0.tensor(), p1.tensor()}), grads({g0.tensor(), g1.tensor()});
+    AdamW opt(2e-4, shapes, NBO_DT_F32, /*master=*/true);
+    opt.beta2(0.95).weight_decay(0.1);
+    opt.master_from_params(params);
+    GradScaler scaler;
+    auto step = [&](AdamW &o, GradScaler &sc, TensorList &p, uint32_t k) {
+        g0.put(fill(n0, 100 + k, 0x4300)), g1.put(fill(n1, 200 + k, 0x4300)); // about 128..256: times 1/65536 after unscale
+        o.fused_step(p, grads, &sc, 1.0);
+    };
+    for (uint32_t k = 0; k < 3; k++) step(opt, scaler, params, k);
+    TrainState state;
+    state.epoch = 0, state.step = 3, state.grad_accum = 1;
+    save_checkpoint(dir, params, names, opt, &scaler, nullptr, state);
+
+    HalfVec q0(n0), q1(n1);
+    TensorList params2({q0.tensor(), q1.tensor()});
+    AdamW opt2(1.0, shapes, NBO_DT_F32, /*master=*/true);
+    GradScaler scaler2;
+    TrainState state2;
+    std::optional<ScheduleState> schedule2;
+    load_checkpoint(dir, params2, names, opt2, &scaler2, schedule2, state2);
+    EXPECT(state2.step == 3 && !schedule2.has_value());
+    EXPECT(q0.get() == p0.get() && q1.get() == p1.get()); // narrowed from the restored master weights
+    for (uint32_t k = 3; k < 5; k++) {
+        step(opt, scaler, params, k);
+        step(opt2, scaler2, params2, k);
+    }
+    EXPECT(q0.get() == p0.get() && q1.get() == p1.get());
+    for (const char *key : {"w0", "m0", "v0", "w1", "m1", "v1"}) {
+        const uint64_t n = key[1] == '0' ? n0 : n1;
+        std::vector<float> a(n), b(n);
+        opt.state_read(key, a.data(), n, false);
+        opt2.state_read(key, b.data(), n, false);
+        EXPECT(std::memcmp(a.data(), b.data(), n * sizeof(float)) == 0);
+    }
+    EXPECT(opt.last_step().step_count == 5 && opt2.last_step().step_count == 5);
+    // a file key the module does not have is load_state_dict's error (module/core.rs:42, 286-290)
+    std::string what;
+    try {
+        load_checkpoint(dir, params2, {"layer.w", "other.b"}, opt2, &scaler2, schedule2, state2);
+    } catch (const std::exception &e) {
+        what = e.what();
+    }
+    EXPECT(what.find("unknown parameter key: layer.b") != std::string::npos);
+}
+
 static void panics_and_errors()  // alg.rs:110-119, 531-545; tensor/ops.rs:638-646
 {
     Mat p({1.0}), g({1.0}), g2({1.0, 2.0});
@@ -460,7 +558,11 @@ static int print_lr_grid()
     const LrSchedule scheds[] = {LrSchedule::cosine(10, 110, 1e-5), LrSchedule::cosine(0, 7, 0.0),
                                  LrSchedule::linear(5, 50),         LrSchedule::linear(0, 1),
                                  LrSchedule::one_cycle(1e-2, 100, 0.3), LrSchedule::one_cycle(0.5, 9, 0.0),
-                                 LrSchedule::step(3, 0.7),          LrSchedule::step(0, 0.5)};
+                                 LrSchedule::step(3, 0.7),          LrSchedule::step(0, 0.5),
+                                 // the reference's usize arithmetic at its edges (core.rs:86-89, 121-123, 165-167):
+                                 // total_steps below warmup_steps, pct_start above 1, a decay exponent past i32
+                                 LrSchedule::cosine(10, 5, 0.1),    LrSchedule::one_cycle(1e-2, 10, 1.5),
+                                 LrSchedule::linear(40, 12)};
     for (size_t k = 0; k < sizeof(scheds) / sizeof(scheds[0]); k++)
         for (uint64_t step = 0; step <= 120; step += (step < 12 ? 1 : 9)) {
             const double lr = lr_at_step(scheds[k], 3e-4, step);
@@ -492,6 +594,7 @@ int main(int argc, char **argv)
                  {"trainer_accumulates_then_clips_and_steps", trainer_accumulates_then_clips_and_steps},
                  {"backend_axpy_is_multiply_then_add", backend_axpy_is_multiply_then_add},
                  {"checkpoint_roundtrip_with_schedule", checkpoint_roundtrip_with_schedule},
+                 {"mixed_precision_checkpoint_resumes_bit_for_bit", mixed_precision_checkpoint_resumes_bit_for_bit},
                  {"panics_and_errors", panics_and_errors},
                  {"group_checkpoint_roundtrip", group_checkpoint_roundtrip},
                  {"constructors_and_set_state", constructors_and_set_state},

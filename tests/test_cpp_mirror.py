@@ -26,9 +26,10 @@ def test_cpp_lr_at_step_matches_the_oracle_bit_for_bit():
     assert r.returncode == 0, r.stderr
     scheds = [O.Schedule(0, 10, 110, 1e-5, 0.0), O.Schedule(0, 0, 7, 0.0, 0.0), O.Schedule(1, 5, 50, 0.0, 0.0),
               O.Schedule(1, 0, 1, 0.0, 0.0), O.Schedule(2, 0, 100, 1e-2, 0.3), O.Schedule(2, 0, 9, 0.5, 0.0),
-              O.Schedule(3, 3, 0, 0.7, 0.0), O.Schedule(3, 0, 0, 0.5, 0.0)]
+              O.Schedule(3, 3, 0, 0.7, 0.0), O.Schedule(3, 0, 0, 0.5, 0.0),
+              O.Schedule(0, 10, 5, 0.1, 0.0), O.Schedule(2, 0, 10, 1e-2, 1.5), O.Schedule(1, 40, 12, 0.0, 0.0)]
     lines = r.stdout.split("\n")[:-1]
-    assert len(lines) == 8 * 25
+    assert len(lines) == len(scheds) * 25
     for line in lines:
         k, step, bits = line.split()
         want = O.lr_at_step(scheds[int(k)], 3e-4, int(step))
@@ -40,15 +41,16 @@ def test_cpp_replay_of_reference_tests(gpu, tmp_path):
     r = subprocess.run([BIN, str(tmp_path)], capture_output=True, text=True, timeout=120)
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count("ok    ") == 17 and "0 failure(s)" in r.stdout
+    assert r.stdout.count("ok    ") == 18 and "0 failure(s)" in r.stdout
 
     # the checkpoint the C++ side left behind is the one the Python mirror writes and reads
     from nabla_amd import checkpoint as ck
     from nabla_amd import optim as nb
     from nabla_amd.schedule import ScheduleState, Step
+    import oracle as O
     from tests import helpers as H
 
-    assert sorted(os.listdir(tmp_path)) == ["groups", "meta.txt", "optim.nbla", "params.nbla"]
+    assert sorted(os.listdir(tmp_path)) == ["groups", "meta.txt", "mixed", "optim.nbla", "params.nbla"]
     shapes = [(1, 1), (1, 1)]
     opt = nb.Sgd.new(0.7, shapes, dtype="f64")
     scaler = nb.GradScaler.new()
@@ -87,3 +89,25 @@ def test_cpp_replay_of_reference_tests(gpu, tmp_path):
                        ck.TrainState(epoch=1, step=2, grad_accum=1, rng_state=None), native=True)
     for name in ("meta.txt", "params.nbla", "optim.nbla"):
         assert (again / name).read_bytes() == (gdir / name).read_bytes(), name
+
+    # and the mixed-precision checkpoint (f32 master weights as params.nbla): read by the Python
+    # mirror, written again, the same bytes
+    mdir = tmp_path / "mixed"
+    mshapes = [(1, 8192 + 37), (1, 300)]
+    mopt = nb.AdamW.new(1.0, mshapes, master=True)
+    mscaler = nb.GradScaler.new()
+    named = [("layer.w", H.dev_list([np.zeros(8192 + 37, np.uint16)], mshapes[:1])[0]),
+             ("layer.b", H.dev_list([np.zeros(300, np.uint16)], mshapes[1:])[0])]
+    _, mstate, msched = ck.load_checkpoint(str(mdir), mopt, mscaler, into=named)
+    assert (mstate.step, msched) == (3, None) and mopt.step_count() == 3
+    m = mopt.meta()
+    assert (m.lr, m.beta2, m.weight_decay) == (2e-4, 0.95, 0.1)
+    saved = dict(ck.load_tensors(str(mdir / "params.nbla")))
+    for i, (name, p16) in enumerate(named):
+        master = H.to_host(mopt.read_state(f"w{i}"))
+        assert np.array_equal(saved[name].reshape(-1), master.astype(np.float64))
+        H.assert_bits_equal([H.to_host(p16).reshape(-1)], [O.bf16_from_f32(master.reshape(-1))], "params narrowed from the master weights")
+    mixed_again = tmp_path / "mixed_py"
+    ck.save_checkpoint(str(mixed_again), named, mopt, mscaler, None, mstate)
+    for name in ("meta.txt", "params.nbla", "optim.nbla"):
+        assert (mixed_again / name).read_bytes() == (mdir / name).read_bytes(), name
