@@ -125,3 +125,57 @@ def test_the_shim_has_the_references_interface():
     declared = set(_rust_decls())
     for name in set(re.findall(r"ffi::(nbo_[a-z0-9_]+)", src)):
         assert name in declared, name
+
+
+def _strip_rust(text: str) -> str:
+    """Rust source with comments, string and char literals blanked (lifetimes are left alone)."""
+    text = re.sub(r"//[^\n]*", "", text)
+    text = re.sub(r'"(?:\\.|[^"\\])*"', '""', text)
+    return re.sub(r"'(?:\\.|[^'\\])'", "' '", text)
+
+
+def _call_args(text: str, open_paren: int):
+    """Top-level arguments of the call whose '(' is at `open_paren`."""
+    depth, args, start = 0, [], open_paren + 1
+    for i in range(open_paren, len(text)):
+        ch = text[i]
+        if ch in "([{":
+            depth += 1
+        elif ch in ")]}":
+            depth -= 1
+            if depth == 0:
+                last = text[start:i].strip()
+                return args + ([last] if last else [])
+        elif ch == "," and depth == 1:
+            args.append(text[start:i].strip())
+            start = i + 1
+    raise AssertionError("unbalanced call")
+
+
+def test_every_call_into_the_ffi_block_passes_the_declared_number_of_arguments():
+    """What a compiler would have said first: a call site in mod.rs whose argument count differs
+    from the declaration in ffi.rs, a symbol that is not declared, or delimiters that do not
+    balance."""
+    decls = _rust_decls()
+    for path in (FFI, MOD):
+        text = _strip_rust(open(path).read())
+        stack = []
+        for ch in text:
+            if ch in "([{":
+                stack.append(ch)
+            elif ch in ")]}":
+                assert stack and stack.pop() == {")": "(", "]": "[", "}": "{"}[ch], f"{os.path.basename(path)}: unbalanced {ch}"
+        assert not stack, f"{os.path.basename(path)}: unclosed {stack[-1]}"
+    text = _strip_rust(open(MOD).read())
+    calls = [(m.group(1), m.end() - 1) for m in re.finditer(r"ffi::(nbo_[a-z0-9_]+)\s*\(", text)]
+    assert len(calls) >= 25
+    for name, at in calls:
+        assert name in decls, f"mod.rs calls ffi::{name}, which ffi.rs does not declare"
+        got = len(_call_args(text, at))
+        assert got == len(decls[name][1]), f"ffi::{name}: {got} arguments at the call site, {len(decls[name][1])} declared"
+    # every entry point a drop-in needs is actually used by the shim
+    used = {name for name, _ in calls}
+    for name in ("nbo_optim_step", "nbo_optim_reset", "nbo_optim_set_lr", "nbo_optim_state_read", "nbo_optim_state_write",
+                 "nbo_optim_get_meta", "nbo_optim_load_meta", "nbo_scaler_unscale_and_update", "nbo_clip_grad_norm",
+                 "nbo_zero_grad", "nbo_fused_step"):
+        assert name in used, name
