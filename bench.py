@@ -15,6 +15,7 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -22,6 +23,29 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 BYTES_UPDATE = 28       # per param: R g2 + master4 + m4 + v4, W master4 + m4 + v4 + p2
 BYTES_NORM = 2          # per param: R g2
 ROOT = os.path.dirname(os.path.abspath(__file__))
+
+# The driver clears device memory that has been freed, in the background, and that competes with
+# the step for HBM bandwidth until it is done (measured: the 1.1B set runs 5.20 instead of 5.13 ms
+# per step for 3.7 s after its placement search released 91 GiB; the free-memory figure does not
+# show it).  The benchmark therefore keeps count of what it -- and the state placement on its
+# behalf -- has released, and idles in proportion before it times anything.
+CLEARING_GIB_PER_S = 20.0  # cautious: 24-25 GiB/s was observed, with the GPU busy or idle
+_released_gib = 0.0
+
+
+def note_released(gib):
+    global _released_gib
+    _released_gib += max(0.0, gib)
+
+
+def wait_for_clearing(base_s):
+    """Idles base_s plus the time the driver needs for what has been released so far; returns
+    the seconds waited."""
+    global _released_gib
+    wait = base_s + (_released_gib / CLEARING_GIB_PER_S if base_s > 0 else 0.0)
+    _released_gib = 0.0
+    time.sleep(wait)
+    return round(wait, 2)
 
 
 def parse_args():
@@ -49,7 +73,8 @@ def parse_args():
                          "CPU baseline each) and print a markdown table")
     ap.add_argument("--settle-seconds", type=float, default=2.0,
                     help="idle time between setup and the warm-up steps, for the driver's background clearing of "
-                         "the device memory that setup freed to finish")
+                         "the device memory that setup freed to finish; one second per 20 GiB released is added "
+                         "(0: no waiting at all)")
     ap.add_argument("--cpu-seconds", type=float, default=20.0,
                     help="rough budget for the CPU baseline sample")
     return ap.parse_args()
@@ -177,6 +202,7 @@ def measured_ceiling(achieved_gbps):
     the yardstick next to the nominal 8 TB/s."""
     from nabla_amd import kernel_bench as KB
 
+    wait_for_clearing(1.0)  # the workloads measured before have just been torn down
     rows = KB.measure_ceilings(gib=2.0, reps=10, patterns=(6, 7, 9), spreads=(1,))
     name, spread, best, mean, regions, rw = max(rows, key=lambda r: r[3])
     return {"ceiling_measured": round(mean, 1),
@@ -217,6 +243,7 @@ def measure(name, steps, warmup, zero_grads="off", settle_s=2.0):
     else:
         params = [torch.empty(s, dtype=pdt, device=dev) for s in shapes]
         grads = [torch.empty(s, dtype=pdt, device=dev) for s in shapes]
+    free_before_state = torch.cuda.mem_get_info()[0]
     if cfg["kind"] == "sgd":
         opt = nb.Sgd.new(cfg["lr"], shapes)
     elif cfg["kind"] == "adam":
@@ -224,6 +251,11 @@ def measure(name, steps, warmup, zero_grads="off", settle_s=2.0):
     else:
         opt = nb.AdamW.new(cfg["lr"], shapes, master=cfg["mixed"], dtype=half if pure else "f32") \
             .beta1(cfg["betas"][0]).beta2(cfg["betas"][1]).eps(cfg.get("eps", 1e-8)).weight_decay(cfg["wd"])
+    # what the placement search created beyond what the state keeps has been released again
+    searched = re.search(r"chunks of (\d+) MiB; (\d+) chunks created", opt.state_placement_note())
+    if searched:
+        kept_gib = (free_before_state - torch.cuda.mem_get_info()[0]) / 2**30
+        note_released(int(searched.group(1)) * int(searched.group(2)) / 1024 - kept_gib)
     scale = 65536.0 if cfg["scaler"] else 1.0
     for i, s in enumerate(shapes):  # synthetic, random-init
         w = torch.randn(s, dtype=torch.float32, device=dev) * cfg["p_sigma"]
@@ -237,7 +269,9 @@ def measure(name, steps, warmup, zero_grads="off", settle_s=2.0):
     if cfg["mixed"]:
         opt.params_from_master(plist)
     scaler = nb.GradScaler.new() if cfg["scaler"] else None
+    reserved = torch.cuda.memory_reserved()
     torch.cuda.empty_cache()
+    note_released((reserved - torch.cuda.memory_reserved()) / 2**30)  # the temporaries of the fill above
 
     fused = cfg["scaler"] or cfg["clip"] > 0
 
@@ -259,13 +293,13 @@ def measure(name, steps, warmup, zero_grads="off", settle_s=2.0):
     # launch, so small workloads take their kernel durations from a second, untimed pass.
     events_in_timed_region = n >= 10_000_000
 
-    # Setup has just freed tens of GiB (the placement search's spare chunks, torch's temporaries),
-    # and the driver clears freed device memory in the background: for about a second that
-    # competes with the step for HBM bandwidth (measured: 37.9 instead of 37.3 ms per step on the
-    # 8B set).  It is the benchmark's own setup, not the step, so it is given time to finish.
+    # Setup has just freed tens of GiB (the placement search's spare chunks, torch's temporaries,
+    # the previous workload), and the driver clears freed device memory in the background
+    # (measured: 37.9 instead of 37.3 ms per step on the 8B set while it does).  It is the
+    # benchmark's own setup, not the step, so it is given time to finish.
     torch.cuda.synchronize()
     _lib.check(L.nbo_sync())
-    time.sleep(settle_s)
+    settled_s = wait_for_clearing(settle_s)
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -333,7 +367,8 @@ def measure(name, steps, warmup, zero_grads="off", settle_s=2.0):
                    "bytes_per_param_step": upd_b + nrm_b + zero_b, "zero_grads": zero_grads,
                    "optimizer": cfg["kind"],
                    "loss_scale": scale if cfg["scaler"] else None, "clip_max_norm": cfg["clip"] or None,
-                   "state_hbm_regions": opt.state_regions(), "settle_s_after_setup": settle_s},
+                   "state_hbm_regions": opt.state_regions(), "state_placement": opt.state_placement_note(),
+                   "settle_s_after_setup": settled_s},
         "roofline": {
             "kernel": dom,
             "bound": "hbm",
@@ -352,8 +387,10 @@ def measure(name, steps, warmup, zero_grads="off", settle_s=2.0):
     if info is not None:
         out["last_step"] = {"found_inf": info.found_inf, "clipped": info.clipped,
                             "norm": info.norm, "scale": info.scale, "step_count": info.step_count}
+    free_before_teardown = torch.cuda.mem_get_info()[0]
     del opt, plist, glist, params, grads
     torch.cuda.empty_cache()
+    note_released((torch.cuda.mem_get_info()[0] - free_before_teardown) / 2**30)
     return out, cfg
 
 
@@ -411,7 +448,8 @@ def main():
     out, cfg = measure(args.workload, args.steps, args.warmup, args.zero_grads, args.settle_seconds)
     if args.workload == "llama3-8b" and not args.primary_only:
         # the metric is quoted on the 1.1B and the 8B shapes: the smaller one rides along
-        small, _ = measure("llama-1.1b", 10, 2, settle_s=args.settle_seconds)
+        # (ten warm-up steps: after the idle wait the GPU takes some 20 ms of work to clock up again)
+        small, _ = measure("llama-1.1b", 20, 10, settle_s=args.settle_seconds)
         out["also"] = {"llama-1.1b": {k: small[k] for k in ("value", "unit", "pct_of_peak", "params_per_s",
                                                             "ms_per_step", "steps", "warmup", "config",
                                                             "roofline", "kernels_ms")}}
