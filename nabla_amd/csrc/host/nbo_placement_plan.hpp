@@ -118,15 +118,28 @@ public:
     const std::vector<int> &region_of() const { return region_of_; }
     const std::vector<size_t> &leaders() const { return leaders_; }
     size_t probes() const { return cache_.size() + bases_.size(); }
+    // The chunks of every region, the ones that measured slowest together with their region's
+    // leader -- the ones most surely all of that region; a chunk the driver pieced together
+    // from several regions measures higher -- at the back, where they are taken from first.
     std::vector<std::vector<size_t>> chunks_per_region() const
     {
         std::vector<std::vector<size_t>> out(leaders_.size());
         for (size_t i = 0; i < region_of_.size(); i++)
             if (region_of_[i] >= 0) out[(size_t)region_of_[i]].push_back(i);
+        for (size_t k = 0; k < out.size(); k++)
+            std::stable_sort(out[k].begin(), out[k].end(), [&](size_t x, size_t y) {
+                return with_leader(k, x) > with_leader(k, y);
+            });
         return out;
     }
 
 private:
+    double with_leader(size_t k, size_t i) const // what chunk i measured together with region k's leader
+    {
+        if (leaders_[k] == i) return 0.0;
+        auto it = cache_.find(std::pair<size_t, size_t>(std::min(leaders_[k], i), std::max(leaders_[k], i)));
+        return it == cache_.end() ? 0.0 : it->second;
+    }
     template <typename Halves> double base_of(size_t a, Halves &&halves)
     {
         auto it = bases_.find(a);
@@ -171,7 +184,6 @@ inline std::vector<size_t> choose_regions(const std::vector<size_t> &avail, uint
         return true;
     };
     std::vector<std::vector<size_t>> candidates;
-    if (R >= 3 && nparts >= 3) candidates.push_back({0, 1, 2});
     std::vector<std::vector<size_t>> pairs;
     if (R >= 3) pairs = {{1, 2}, {0, 2}, {0, 1}};
     else if (R == 2) pairs = {{0, 1}};
@@ -180,6 +192,7 @@ inline std::vector<size_t> choose_regions(const std::vector<size_t> &avail, uint
             return avail[x[0]] + avail[x[1]] > avail[y[0]] + avail[y[1]];
         });
     candidates.insert(candidates.end(), pairs.begin(), pairs.end());
+    if (R >= 3 && nparts >= 3) candidates.push_back({0, 1, 2});
     for (const auto &set : candidates)
         if (holds(set)) return set;
     return {};

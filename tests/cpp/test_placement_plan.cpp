@@ -196,6 +196,29 @@ int main()
         }
         CHECK((used == std::vector<size_t>{4, 4, 4}));
     }
+    // three arrays, three regions that each hold plenty: two of them are used, not three (two regions
+    // measured 35.0-35.2 ms per update of the 8B set, three 35.4)
+    {
+        CHECK(choose_regions({10, 10, 10}, 3, 4).size() == 2);
+        const auto pick = assign({10, 10, 10}, 3, 4);
+        std::vector<size_t> used(3, 0);
+        for (size_t i = 0; i < 4; i++)
+            for (int j = 0; j < 3; j++) used[pick[j][i]]++;
+        CHECK(std::count(used.begin(), used.end(), (size_t)0) == 1 && std::count(used.begin(), used.end(), (size_t)6) == 2);
+    }
+    // within a region the chunks that measured lowest with its leader (surest to be all of that region)
+    // are handed out first
+    {
+        const std::vector<int> truth{0, 0, 0, 1, 1, 1, 0, 1};
+        const std::vector<double> wobble{0, 120, 10, 0, 90, 20, 60, 5}; // how far from its own kind a chunk measures
+        auto probe = [&](size_t a, size_t b) { return (truth[a] == truth[b] ? 5450.0 : 6400.0) + wobble[a] + wobble[b]; };
+        auto halves = [&](size_t) { return 5440.0; };
+        RegionFinder f;
+        f.add_chunks(8, probe, halves);
+        const auto pools = f.chunks_per_region();
+        CHECK(pools.size() == 2);
+        CHECK((pools[0] == std::vector<size_t>{1, 6, 2, 0}) && (pools[1] == std::vector<size_t>{4, 5, 7, 3}));
+    }
     // two arrays and three regions: the first region is left to the caller's tensors
     {
         const auto pick = assign({6, 3, 3}, 2, 3);
