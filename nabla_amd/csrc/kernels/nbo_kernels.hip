@@ -59,21 +59,6 @@ typedef double f64x2_e __attribute__((ext_vector_type(2), aligned(8)));
 #ifndef NBO_NT_STORES
 #define NBO_NT_STORES 1
 #endif
-// Update kernels, order of the memory instructions of a chunk.  Bit 0: stores grouped by stream
-// after all rows are computed (instead of row by row).  Bit 1: loads grouped by stream
-// (instead of row by row).  Both together measured 1.3 % faster than neither on the 8B set
-// (35.0 against 35.5 ms, alternating launches inside one process); either alone, next to nothing.
-#ifndef NBO_UPDATE_VARIANT
-#define NBO_UPDATE_VARIANT 3
-#endif
-#ifndef NBO_UPDATE_WAVES_PER_EU
-#define NBO_UPDATE_WAVES_PER_EU 0 // update kernels: cap on resident waves per SIMD (0: compiler's choice)
-#endif
-#if NBO_UPDATE_WAVES_PER_EU
-#define NBO_UPDATE_OCCUPANCY __attribute__((amdgpu_waves_per_eu(1, NBO_UPDATE_WAVES_PER_EU)))
-#else
-#define NBO_UPDATE_OCCUPANCY
-#endif
 #if NBO_NT_LOADS
 #define NBO_LOAD(p) __builtin_nontemporal_load(p)
 #else
@@ -483,9 +468,8 @@ DEV Peel peel(uint32_t cnt, uint32_t vec, uint32_t sb, bool wvo, uintptr_t a0, u
 
 // ---------------------------------------------------------------------------------
 // Optimizer update: one workgroup per chunk.
-template <int ST, int KIND, int VARIANT = NBO_UPDATE_VARIANT> DEV void update_body(const NboUpdateArgs &a)
+template <int ST, int KIND> DEV void update_body(const NboUpdateArgs &a)
 {
-    constexpr bool store_batch = (VARIANT & 1) != 0, stream_major = (VARIANT & 2) != 0, wave_rows = (VARIANT & 4) != 0;
     typedef typename Traits<ST>::T T;
     enum {
         VEC = Traits<ST>::VEC,
@@ -524,86 +508,58 @@ template <int ST, int KIND, int VARIANT = NBO_UPDATE_VARIANT> DEV void update_bo
 
     if (c.cnt == NBO_CHUNK && vec_ok) {
         for (int it = 0; it < ITERS; it++) {
-            // rows of the workgroup (each wave takes a quarter of every 4 KiB row), or, with
-            // wave_rows, rows of the wave (each wave walks a contiguous U KiB of every stream)
-            constexpr uint32_t RS = wave_rows ? 64 * VEC : ROW;
-            const uint32_t e0 = it * (U * ROW) + (wave_rows ? (tid >> 6) * (U * 64 * VEC) + (tid & 63u) * VEC : tid * VEC);
+            // U rows of the workgroup at once.  The memory instructions are issued stream by
+            // stream -- every row's gradient load, then every row's master load, ... and after
+            // all rows are computed every row's master store, ... -- not row by row: the memory
+            // then sees longer runs per stream, which measured 1.3 % faster on the 8B set (35.0
+            // against 35.5 ms in alternating launches inside one process; loads or stores alone
+            // in this order: next to nothing).
+            const uint32_t e0 = it * (U * ROW) + tid * VEC;
             T g[U][VEC], p[U][VEC], m[U][VEC] = {}, v[U][VEC] = {};
-            if constexpr (stream_major) {
-                // all rows of one stream back to back, stream after stream
 #pragma unroll
-                for (int u = 0; u < U; u++) IO<ST>::ldv(pg + (uint64_t)(e0 + u * RS) * SB, g[u]);
+            for (int u = 0; u < U; u++) IO<ST>::ldv(pg + (uint64_t)(e0 + u * ROW) * SB, g[u]);
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                if (mixed) ld_state(aw + e0 + u * ROW, p[u]);
+                else IO<ST>::ldv(pp + (uint64_t)(e0 + u * ROW) * SB, p[u]);
+            }
+            if (use_m) {
+#pragma unroll
+                for (int u = 0; u < U; u++) ld_state(am + e0 + u * ROW, m[u]);
+            }
+            if (has_v) {
+#pragma unroll
+                for (int u = 0; u < U; u++) ld_state(av + e0 + u * ROW, v[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++)
+#pragma unroll
+                for (int k = 0; k < VEC; k++) step_elem<T, KIND>(p[u][k], g[u][k], m[u][k], v[u][k], s);
+            // the scheduling barriers keep the compiler from interleaving the stores with the
+            // arithmetic again
+            __builtin_amdgcn_sched_barrier(0);
+            if (mixed) {
+#pragma unroll
+                for (int u = 0; u < U; u++) st_state(aw + e0 + u * ROW, p[u]);
+            }
+            if (use_m) {
+#pragma unroll
+                for (int u = 0; u < U; u++) st_state(am + e0 + u * ROW, m[u]);
+            }
+            if (has_v) {
+#pragma unroll
+                for (int u = 0; u < U; u++) st_state(av + e0 + u * ROW, v[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) IO<ST>::stv(pp + (uint64_t)(e0 + u * ROW) * SB, p[u]);
+            if (zero_g) {
 #pragma unroll
                 for (int u = 0; u < U; u++) {
-                    if (mixed) ld_state(aw + e0 + u * RS, p[u]);
-                    else IO<ST>::ldv(pp + (uint64_t)(e0 + u * RS) * SB, p[u]);
-                }
-                if (use_m) {
-#pragma unroll
-                    for (int u = 0; u < U; u++) ld_state(am + e0 + u * RS, m[u]);
-                }
-                if (has_v) {
-#pragma unroll
-                    for (int u = 0; u < U; u++) ld_state(av + e0 + u * RS, v[u]);
-                }
-            } else {
-#pragma unroll
-                for (int u = 0; u < U; u++) {
-                    const uint32_t e = e0 + u * RS;
-                    IO<ST>::ldv(pg + (uint64_t)e * SB, g[u]);
-                    if (mixed) ld_state(aw + e, p[u]);
-                    else IO<ST>::ldv(pp + (uint64_t)e * SB, p[u]);
-                    if (use_m) ld_state(am + e, m[u]);
-                    if (has_v) ld_state(av + e, v[u]);
+                    T z[VEC] = {};
+                    IO<ST>::stv(pg + (uint64_t)(e0 + u * ROW) * SB, z);
                 }
             }
-            if constexpr (store_batch) {
-                // every row computed first, then the stores of one stream back to back, stream
-                // after stream; the scheduling barriers keep the compiler from interleaving
-                // them with the arithmetic again
-#pragma unroll
-                for (int u = 0; u < U; u++)
-#pragma unroll
-                    for (int k = 0; k < VEC; k++) step_elem<T, KIND>(p[u][k], g[u][k], m[u][k], v[u][k], s);
-                __builtin_amdgcn_sched_barrier(0);
-                if (mixed) {
-#pragma unroll
-                    for (int u = 0; u < U; u++) st_state(aw + e0 + u * RS, p[u]);
-                }
-                if (use_m) {
-#pragma unroll
-                    for (int u = 0; u < U; u++) st_state(am + e0 + u * RS, m[u]);
-                }
-                if (has_v) {
-#pragma unroll
-                    for (int u = 0; u < U; u++) st_state(av + e0 + u * RS, v[u]);
-                }
-#pragma unroll
-                for (int u = 0; u < U; u++) IO<ST>::stv(pp + (uint64_t)(e0 + u * RS) * SB, p[u]);
-                if (zero_g) {
-#pragma unroll
-                    for (int u = 0; u < U; u++) {
-                        T z[VEC] = {};
-                        IO<ST>::stv(pg + (uint64_t)(e0 + u * RS) * SB, z);
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            } else {
-#pragma unroll
-                for (int u = 0; u < U; u++) {
-                    const uint32_t e = e0 + u * RS;
-#pragma unroll
-                    for (int k = 0; k < VEC; k++) step_elem<T, KIND>(p[u][k], g[u][k], m[u][k], v[u][k], s);
-                    if (mixed) st_state(aw + e, p[u]);
-                    IO<ST>::stv(pp + (uint64_t)e * SB, p[u]);
-                    if (use_m) st_state(am + e, m[u]);
-                    if (has_v) st_state(av + e, v[u]);
-                    if (zero_g) {
-                        T z[VEC] = {};
-                        IO<ST>::stv(pg + (uint64_t)e * SB, z);
-                    }
-                }
-            }
+            __builtin_amdgcn_sched_barrier(0);
         }
         return;
     }
@@ -650,7 +606,7 @@ template <int ST, int KIND, int VARIANT = NBO_UPDATE_VARIANT> DEV void update_bo
 }
 
 #define NBO_UPDATE_KERNEL(name, ST, KIND)                                                   \
-    extern "C" __global__ __launch_bounds__(NBO_BLOCK) NBO_UPDATE_OCCUPANCY void name(const NboUpdateArgs a) \
+    extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboUpdateArgs a) \
     {                                                                                       \
         update_body<ST, KIND>(a);                                                           \
     }
