@@ -1,7 +1,7 @@
 """Turns raw rocprofv3 output of the benchmark into the short summaries kept under profiles/.
 
-    python -m nabla_amd.kernel_bench --summarize gpurun_out/prof [--workload llama3-8b]
-    (or: python -m nabla_amd.profile_summary gpurun_out/prof)
+    python -m nabla_amd.kernel_bench --summarize DIR [--workload llama3-8b]
+    (or: python -m nabla_amd.profile_summary DIR)
 
 Expected under DIR, made by these five commands (each from the repository root, after
 `cd /tmp && export TMPDIR=/tmp && cd -`; the program follows `--` directly):
@@ -193,4 +193,6 @@ def main(base: str, kernels=None) -> None:
 
 
 if __name__ == "__main__":
-    main(sys.argv[1] if len(sys.argv) > 1 else "gpurun_out/prof", sys.argv[2].split(",") if len(sys.argv) > 2 else None)
+    if len(sys.argv) < 2:
+        sys.exit("usage: python -m nabla_amd.profile_summary DIR [kernel,kernel,...]")
+    main(sys.argv[1], sys.argv[2].split(",") if len(sys.argv) > 2 else None)
