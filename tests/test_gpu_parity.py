@@ -798,3 +798,21 @@ def test_state_placement_says_what_it_found(gpu):
         assert regions in (2, 3) and note.startswith(f"{regions} regions") and "threshold" in note
     H.assert_bits_equal(H.host_list(p_dev), p_ref, "params on placed state")
     H.assert_bits_equal(H.host_list(opt.moments()[1]), v, "v on placed state")
+
+
+def test_state_placement_switches(gpu, monkeypatch):
+    """NBO_STATE_SPREAD=0 and a chunk limit below what the state needs both end in plain
+    allocations, say so, and the optimizer steps as usual."""
+    shapes = [(4096, 8192 + 8)]  # 134 MB per state array: placed by default
+    for env, reason in ((("NBO_STATE_SPREAD", "0"), "NBO_STATE_SPREAD=0"),
+                        (("NBO_PLACEMENT_MAX_GIB", "1"), "chunk limit")):
+        monkeypatch.setenv(*env)
+        opt = nb.Adam.new(1e-3, shapes)
+        regions, note = opt.state_regions(), opt.state_placement_note()  # the first call creates the state
+        monkeypatch.delenv(env[0])
+        assert regions == 0
+        assert note.startswith("plain allocation") and reason in note, note
+        p = H.dev_list(H.randn_list(shapes, 1, 0.02), shapes)
+        g = H.dev_list(H.randn_list(shapes, 2, 1e-3), shapes)
+        opt.step(p, g)
+        assert opt.step_count() == 1
