@@ -240,6 +240,7 @@ impl<T: Scalar> Engine<T> {
 
     /// One cloned state tensor, as `state_tensors()` returns them (`alg.rs:476-485`).
     fn read_state(&mut self, name: &str, shape: (usize, usize)) -> Tensor<T, Hip> {
+        self.state_is_t();
         let h = self.handle();
         let t = Tensor::<T, Hip>::zeros(shape.0, shape.1);
         let key = CString::new(name).expect("state names hold no NUL");
@@ -250,6 +251,38 @@ impl<T: Scalar> Engine<T> {
     }
 
     fn write_state(&mut self, name: &str, t: &Tensor<T, Hip>) -> Result<(), String> {
+        self.state_is_t();
+        let h = self.handle();
+        let key = CString::new(name).map_err(|_| format!("bad tensor key: {name}"))?;
+        let (r, c) = t.shape();
+        check_state(unsafe {
+            ffi::nbo_optim_state_write(h, key.as_ptr(), t.device_ptr() as *const c_void, (r * c) as u64, 1)
+        })
+    }
+
+    /// With f32 master weights the state is f32 whatever `T` is: a `Tensor<T, Hip>` cannot hold
+    /// it, and the trait's `state_tensors` / `load_state_tensors` (typed in `T`) do not apply --
+    /// `state_tensors_f32` / `load_state_tensors_f32` do.
+    fn state_is_t(&self) {
+        assert!(
+            !self.keep_master || TypeId::of::<T>() == TypeId::of::<f32>(),
+            "nabla-train: this optimizer keeps f32 state under 16-bit tensors; use state_tensors_f32 / load_state_tensors_f32"
+        );
+    }
+
+    fn read_state_f32(&mut self, name: &str, shape: (usize, usize)) -> Tensor<f32, Hip> {
+        assert!(self.keep_master, "f32 state access is for optimizers with f32 master weights");
+        let h = self.handle();
+        let t = Tensor::<f32, Hip>::zeros(shape.0, shape.1);
+        let key = CString::new(name).expect("state names hold no NUL");
+        check(unsafe {
+            ffi::nbo_optim_state_read(h, key.as_ptr(), t.device_ptr() as *mut c_void, (shape.0 * shape.1) as u64, 1)
+        });
+        t
+    }
+
+    fn write_state_f32(&mut self, name: &str, t: &Tensor<f32, Hip>) -> Result<(), String> {
+        assert!(self.keep_master, "f32 state access is for optimizers with f32 master weights");
         let h = self.handle();
         let key = CString::new(name).map_err(|_| format!("bad tensor key: {name}"))?;
         let (r, c) = t.shape();
@@ -449,6 +482,43 @@ impl<T: Scalar> MiAdamW<T> {
             step_count,
         };
         self.e.get_mut().load_meta(&meta).expect("same kind");
+    }
+
+    /// Moments and master weights of the mixed-precision composition, as f32 tensors under the
+    /// keys `m{i}`, `v{i}`, `w{i}` (what a checkpoint of such an optimizer has to carry; the
+    /// library also writes them to NBLA files itself, `nbo_optim_save_state` /
+    /// `nbo_optim_save_master`).
+    pub fn state_tensors_f32(&mut self) -> Vec<(String, Tensor<f32, Hip>)> {
+        let e = self.e.get_mut();
+        let shapes = e.shapes.clone();
+        let mut out = Vec::with_capacity(3 * shapes.len());
+        for prefix in ["m", "v", "w"] {
+            for (i, &s) in shapes.iter().enumerate() {
+                let name = format!("{prefix}{i}");
+                let t = e.read_state_f32(&name, s);
+                out.push((name, t));
+            }
+        }
+        out
+    }
+
+    /// The reverse: every `m{i}`, `v{i}` and `w{i}` must be there (`missing m{i}` otherwise, as
+    /// `alg.rs:487-516` says it); afterwards the master weights count as set.
+    pub fn load_state_tensors_f32(&mut self, tensors: &[(String, Tensor<f32, Hip>)]) -> Result<(), String> {
+        let e = self.e.get_mut();
+        let n = e.shapes.len();
+        for prefix in ["m", "v", "w"] {
+            for i in 0..n {
+                let key = format!("{prefix}{i}");
+                if !tensors.iter().any(|(name, _)| *name == key) {
+                    return Err(format!("missing {key}"));
+                }
+            }
+        }
+        for (name, t) in tensors {
+            e.write_state_f32(name, t)?; // bad keys and indices come back as the reference's errors
+        }
+        Ok(())
     }
 
     /// master = f32(params), for the mixed-precision composition.
