@@ -653,7 +653,8 @@ int nbo_optim_master_from_params(nbo_optim *opt, nbo_list *params_half)
 int nbo_optim_params_from_master(nbo_optim *opt, nbo_list *params_half)
 {
     return guarded([&] {
-        require(opt && opt->master_valid, NBO_ERR_NO_MASTER, "master weights not set");
+        require(opt != nullptr, NBO_ERR_ARG, "null optimizer");
+        require(opt->master_valid, NBO_ERR_NO_MASTER, "master weights not set");
         cast_master(opt, params_half, 1);
     });
 }

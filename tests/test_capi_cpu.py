@@ -240,6 +240,15 @@ def test_null_arguments_are_errors_not_crashes():
         lambda: lib.nbo_optim_load_state(null, b"/nonexistent/x"),
         lambda: lib.nbo_copy_bytes(null, null, 16),
         lambda: lib.nbo_profile_read(null, null, null),
+        lambda: lib.nbo_fused_step_noalloc(null, null, null, null, 1.0, 0),
+        lambda: lib.nbo_fused_step_norm(null, null, null, 1.0, 1.0, 0),
+        lambda: lib.nbo_unscale_accumulate(null, null, null, 0, null, null),
+        lambda: lib.nbo_optim_state_placement_note(null, null, 0),
+        lambda: lib.nbo_optim_save_master(null, b"/nonexistent/x", null),
+        lambda: lib.nbo_optim_load_master(null, b"/nonexistent/x", null),
+        lambda: lib.nbo_optim_params_from_master(null, null),
+        lambda: lib.nbo_hbm_ceiling(0, 0, 1 << 20, 2, 0, null, null, null),
+        lambda: lib.nbo_hbm_ceiling(99, 0, 1 << 20, 2, 0, null, null, null),
     ]
     for k, call in enumerate(calls):
         assert call() == _lib.ERR_ARG, f"call {k}"
