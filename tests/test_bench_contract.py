@@ -75,3 +75,29 @@ def test_kernel_bench_prints_a_row_for_every_measurement(gpu):
     for row in rows:
         cells = [c.strip() for c in row.strip("|").split("|")]
         assert float(cells[2]) > 0.0 and float(cells[4]) > 0.0, row
+
+
+@pytest.mark.gpu
+def test_every_ceiling_probe_runs_and_reports_a_rate(gpu):
+    """`nbo_hbm_ceiling` for every access pattern, in one plain allocation and across the HBM's
+    regions, on streams of 192 MiB: a positive rate below the nominal peak, best >= mean, and the
+    argument checks of the entry point."""
+    import ctypes as C
+
+    from nabla_amd import _lib
+    from nabla_amd import kernel_bench as KB
+
+    L = _lib.load()
+    nbytes = 192 << 20
+    for pat, (name, ro, rmw, wo) in enumerate(KB.PATTERNS):
+        for spread in (0, 1):
+            best, mean, regions = C.c_double(), C.c_double(), C.c_int(-1)
+            _lib.check(L.nbo_hbm_ceiling(pat, spread, nbytes, 3, 5, C.byref(best), C.byref(mean), C.byref(regions)))
+            assert 500.0 < mean.value <= best.value < 8000.0, (name, spread, best.value, mean.value)
+            assert regions.value in ((0, 2, 3) if spread else (0,)), (name, spread, regions.value)
+    best, mean = C.c_double(), C.c_double()
+    for bad in (lambda: L.nbo_hbm_ceiling(len(KB.PATTERNS), 0, nbytes, 3, 0, C.byref(best), C.byref(mean), None),
+                lambda: L.nbo_hbm_ceiling(0, 0, nbytes + 4096, 3, 0, C.byref(best), C.byref(mean), None),
+                lambda: L.nbo_hbm_ceiling(0, 0, nbytes, 0, 0, C.byref(best), C.byref(mean), None),
+                lambda: L.nbo_hbm_ceiling(0, 0, nbytes, 3, 0, None, C.byref(mean), None)):
+        assert bad() == _lib.ERR_ARG
