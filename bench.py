@@ -6,9 +6,11 @@
 One "step" is one Trainer tail over the whole synthetic parameter set, with
 gradients already resident in HBM: unscale + found-inf check, global-norm clip to
 1.0, mixed-precision AdamW update (bf16 params/grads, f32 master/m/v).  Prints one
-JSON line: whole-step algorithmic HBM throughput (30 B/param/step), the roofline
-figure of the dominant kernel measured with HIP events on its launch stream, and the
-CPU restatement of the reference timed on this host's cores on a bounded sample.
+JSON line: whole-step algorithmic HBM throughput (30 B/param/step) from a timed pass
+that records no events, the spread over the steps and the roofline figure of the
+dominant kernel from two further passes with HIP events on the launch stream, the CPU
+restatement of the reference timed on this host's cores on a bounded sample, and the
+device path's parity with it on that sample.
 """
 from __future__ import annotations
 
@@ -117,6 +119,31 @@ def bytes_per_param(cfg):
     return 28, 0
 
 
+def baseline_sample(cfg):
+    """The tensors the CPU baseline and the parity check run on: the workload's own tensors in
+    list order until the sample holds ~24 M params (a tensor that would take it past 64 M is
+    left out), but at least one tensor."""
+    sample, n = [], 0
+    for s in cfg["shapes"]:
+        if n and n + s[0] * s[1] > 64_000_000:
+            continue
+        sample.append(s)
+        n += s[0] * s[1]
+        if n >= 24_000_000:
+            break
+    return sample, n
+
+
+def _oracle_meta(cfg):
+    import oracle as O
+
+    if cfg["kind"] == "sgd":
+        return O.sgd_meta(cfg["lr"])
+    if cfg["kind"] == "adam":
+        return O.adam_meta(cfg["lr"], *cfg["betas"])
+    return O.adamw_meta(cfg["lr"], *cfg["betas"], eps=cfg.get("eps", 1e-8), weight_decay=cfg["wd"])
+
+
 def cpu_baseline(cfg, budget_s):
     """The oracle ("port" of the reference's CPU backend) on this host: every Backend
     primitive a separate pass with a fresh output, element-parallel passes on all
@@ -128,17 +155,7 @@ def cpu_baseline(cfg, budget_s):
 
     cores = len(os.sched_getaffinity(0))
     O.set_threads(cores)
-    shapes = cfg["shapes"]
-    # take tensors in list order until the sample holds ~24 M params (one pass chain
-    # over that takes seconds), but at least one tensor
-    sample, n = [], 0
-    for s in shapes:
-        if n and n + s[0] * s[1] > 64_000_000:
-            continue
-        sample.append(s)
-        n += s[0] * s[1]
-        if n >= 24_000_000:
-            break
+    sample, n = baseline_sample(cfg)
     rng = np.random.default_rng(0)
     f32 = np.float32
     master = [(rng.standard_normal(r * c, dtype=f32) * f32(cfg["p_sigma"])) for r, c in sample]
@@ -146,12 +163,7 @@ def cpu_baseline(cfg, budget_s):
     v = [np.zeros_like(a) for a in master]
     scale = 65536.0 if cfg["scaler"] else 1.0
     g32 = [(rng.standard_normal(r * c, dtype=f32) * f32(cfg["g_sigma"] * scale)) for r, c in sample]
-    if cfg["kind"] == "sgd":
-        meta = O.sgd_meta(cfg["lr"])
-    elif cfg["kind"] == "adam":
-        meta = O.adam_meta(cfg["lr"], *cfg["betas"])
-    else:
-        meta = O.adamw_meta(cfg["lr"], *cfg["betas"], eps=cfg.get("eps", 1e-8), weight_decay=cfg["wd"])
+    meta = _oracle_meta(cfg)
     scaler = O.default_scaler() if cfg["scaler"] else None
     narrow = (lambda a: O.cast(a, np.float16)) if cfg.get("half") == "f16" else O.bf16_from_f32
     if cfg.get("pure"):
@@ -168,6 +180,8 @@ def cpu_baseline(cfg, budget_s):
         g = [narrow(a) for a in g32]
         p = [narrow(a) for a in master]
         run = lambda: O.mixed_step(meta, scaler, cfg["clip"], p, g, master, m, v)  # noqa: E731
+    elif cfg["kind"] == "sgd":
+        run = lambda: O.sgd_step(meta, master, g32, m)  # noqa: E731
     else:
         def run():
             gg = [a.copy() for a in g32]
@@ -192,6 +206,137 @@ def cpu_baseline(cfg, budget_s):
         "sample": f"first {len(sample)} tensors of the workload ({n} params), {steps} steps; "
                   "reference-faithful pass chain (12 passes/tensor for AdamW, fresh output each), "
                   f"rayon-parallel passes on {cores} threads, map/scan/clip passes serial",
+    }
+
+
+def parity_check(cfg, steps=3):
+    """Part of the CPU-baseline leg: the device path and the oracle on the same seeded inputs
+    (the reference's xorshift64 + Box-Muller generator), `steps` steps over the CPU baseline's
+    sample of the workload, compared after the last step against both variants of the oracle
+    (denominator by correctly rounded sqrt, as the device computes it, and by libm powf as the
+    reference's source reads).  Reports, per state array, the largest distance in units of the
+    last place, the number of elements beyond 2 ulp (f32) / 1 ulp (16-bit), and whether every
+    step's decisions (found_inf, clipped, scale, step_count) agree bit for bit."""
+    import numpy as np
+    import torch
+
+    import oracle as O
+    from nabla_amd import optim as nb
+
+    sample, n = baseline_sample(cfg)
+    pure, half = bool(cfg.get("pure")), cfg.get("half", "bf16")
+    mixed = cfg["mixed"]
+    scale = 65536.0 if cfg["scaler"] else 1.0
+    master0 = [O.randn_f32(r * c, 1000 + i, cfg["p_sigma"]) for i, (r, c) in enumerate(sample)]
+    g32 = [O.randn_f32(r * c, 5000 + i, cfg["g_sigma"] * scale) for i, (r, c) in enumerate(sample)]
+    narrow = (lambda a: O.cast(a, np.float16)) if half == "f16" else O.bf16_from_f32
+    hdt = torch.float16 if half == "f16" else torch.bfloat16
+
+    def dev(a, shape):
+        if a.dtype == np.uint16:
+            return torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16).to("cuda:0").reshape(shape)
+        return torch.from_numpy(a.copy()).to("cuda:0").reshape(shape)
+
+    def host(t):
+        t = t.detach().reshape(-1).cpu()
+        if t.dtype == torch.bfloat16:
+            return t.view(torch.int16).numpy().view(np.uint16).copy()
+        return t.numpy().copy()
+
+    if pure or mixed:
+        p0, g0 = [narrow(a) for a in master0], [narrow(a) for a in g32]
+    else:
+        p0, g0 = [a.copy() for a in master0], g32
+    # ---- device ----
+    if cfg["kind"] == "sgd":
+        opt = nb.Sgd.new(cfg["lr"], sample)
+    elif cfg["kind"] == "adam":
+        opt = nb.Adam.new(cfg["lr"], sample).beta1(cfg["betas"][0]).beta2(cfg["betas"][1])
+    else:
+        opt = nb.AdamW.new(cfg["lr"], sample, master=mixed, dtype=half if pure else "f32") \
+            .beta1(cfg["betas"][0]).beta2(cfg["betas"][1]).eps(cfg.get("eps", 1e-8)).weight_decay(cfg["wd"])
+    p_dev = [dev(a, s) for a, s in zip(p0, sample)]
+    g_dev = [dev(a, s) for a, s in zip(g0, sample)]
+    if mixed:
+        for i, a in enumerate(master0):
+            opt.write_state(f"w{i}", dev(a, sample[i]))
+    scaler_dev = nb.GradScaler.new() if cfg["scaler"] else None
+    fused = cfg["scaler"] or cfg["clip"] > 0
+    dev_decisions = []
+    for _ in range(steps):
+        if fused:
+            opt.fused_step(p_dev, g_dev, scaler=scaler_dev, max_norm=cfg["clip"])
+            i = opt.last_step()
+            dev_decisions.append((i.found_inf, i.clipped, i.scale, i.step_count))
+        else:
+            opt.step(p_dev, g_dev)
+    got = {"params": [host(t) for t in p_dev]}
+    if cfg["kind"] != "sgd":
+        got["m"] = [host(opt.read_state(f"m{i}")) for i in range(len(sample))]
+        got["v"] = [host(opt.read_state(f"v{i}")) for i in range(len(sample))]
+    if mixed:
+        got["master"] = [host(opt.read_state(f"w{i}")) for i in range(len(sample))]
+    del opt, p_dev, g_dev
+
+    # ---- oracle, both variants of the denominator ----
+    def oracle_run(mode):
+        O.set_pow_mode(mode)
+        try:
+            meta = _oracle_meta(cfg)
+            sc = O.default_scaler() if cfg["scaler"] else None
+            p = [a.copy() for a in p0]
+            master = [a.copy() for a in master0]
+            zeros = (lambda: [np.zeros_like(a) for a in p]) if pure else (lambda: [np.zeros_like(a) for a in master0])
+            m, v = zeros(), zeros()
+            decisions = []
+            for _ in range(steps):
+                if pure:
+                    gg = [a.copy() for a in g0]
+                    ok = O.scaler_unscale_and_update(sc, gg)
+                    norm = O.clip_grad_norm(gg, cfg["clip"]) if ok else 0.0
+                    if ok:
+                        O.adam_step(meta, p, gg, m, v)
+                    decisions.append((0 if ok else 1, int(ok and norm > cfg["clip"] > 0), sc.scale, meta.step_count))
+                elif mixed:
+                    ok, norm = O.mixed_step(meta, sc, cfg["clip"], p, g0, master, m, v)
+                    decisions.append((0 if ok else 1, int(ok and norm > cfg["clip"] > 0), sc.scale, meta.step_count))
+                elif cfg["kind"] == "sgd":
+                    O.sgd_step(meta, p, g0, m)
+                else:
+                    gg = [a.copy() for a in g0]
+                    O.f32_step(meta, sc, cfg["clip"], p, gg, m, v)
+            ref = {"params": p}
+            if cfg["kind"] != "sgd":
+                ref["m"], ref["v"] = m, v
+            if mixed:
+                ref["master"] = master
+            return ref, decisions
+        finally:
+            O.set_pow_mode(O.POW_LIBM)
+
+    def compare(ref):
+        out = {}
+        for key, arrs in got.items():
+            sixteen = arrs[0].dtype in (np.uint16, np.float16)
+            worst = beyond = 0
+            for a, b in zip(arrs, ref[key]):
+                if not a.size:
+                    continue
+                d = O.ulp_distance_bf16(a.view(np.uint16), b.view(np.uint16)) if sixteen else O.ulp_distance_f32(a, b)
+                worst = max(worst, int(d.max()))
+                beyond += int((d > (1 if sixteen else 2)).sum())
+            out[key] = {"max_ulp": worst, "beyond_bar": beyond}
+        return out
+
+    ref_sqrt, dec_sqrt = oracle_run(O.POW_SQRT)
+    ref_libm, dec_libm = oracle_run(O.POW_LIBM)
+    return {
+        "sample": f"first {len(sample)} tensors of the workload ({n} params), {steps} steps, inputs from the "
+                  "reference's xorshift64 + Box-Muller generator",
+        "bar": "f32 states within 2 ulp, 16-bit params within 1 ulp, decisions bit-exact",
+        "decisions_bit_exact": (not fused) or (dev_decisions == dec_sqrt == dec_libm),
+        "vs_oracle_sqrt": compare(ref_sqrt),
+        "vs_oracle_libm_powf": compare(ref_libm),
     }
 
 
@@ -287,13 +432,9 @@ def measure(name, steps, warmup, zero_grads="off", settle_s=2.0):
     upd_b, nrm_b = bytes_per_param(cfg)
     zero_b = 0 if zero_grads == "off" else (2 if (cfg["mixed"] or pure) else 4)
     fam = ("pf16" if half == "f16" else "pbf16") if pure else half if cfg["mixed"] else "f32"
-    dom = f"nbo_update_{fam}_{cfg['kind']}"
-    names = [dom] + ([f"nbo_norm_{fam}", "nbo_finalize"] if fused
-                     else ([] if cfg["kind"] == "sgd" else ["nbo_prep"]))
-    # A step of a few microseconds would be dominated by the event records around each
-    # launch, so small workloads take their kernel durations from a second, untimed pass.
-    events_in_timed_region = n >= 10_000_000
-
+    # an unfused Adam / AdamW step is one launch of the kernel that prepares its own scalars
+    dom = f"nbo_update_{fam}_{cfg['kind']}" + ("" if fused or cfg["kind"] == "sgd" else "_self")
+    names = [dom] + ([f"nbo_norm_{fam}", "nbo_finalize"] if fused else [])
     # Setup has just freed tens of GiB (the placement search's spare chunks, torch's temporaries,
     # the previous workload), and the driver clears freed device memory in the background
     # (measured: 37.9 instead of 37.3 ms per step on the 8B set while it does).  It is the
@@ -312,18 +453,28 @@ def measure(name, steps, warmup, zero_grads="off", settle_s=2.0):
         step()
     torch.cuda.synchronize()
     _lib.check(L.nbo_sync())
-    if events_in_timed_region:
-        _lib.check(L.nbo_profile_enable(1))
+    # The timed region holds the steps and nothing else: no event is recorded inside it.
     t0 = time.perf_counter()
     for _ in range(steps):
         step()
     _lib.check(L.nbo_sync())
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    if not events_in_timed_region:
-        _lib.check(L.nbo_profile_enable(1))
-        for _ in range(steps):
-            step()
+    # Second pass, untimed: every step between one pair of events on the stream the library
+    # launches on (the null stream, which is torch's current one), for the spread over the steps.
+    assert torch.cuda.current_stream().cuda_stream == 0, "the library launches on the null stream"
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for e0, e1 in pairs:
+        e0.record()
+        step()
+        e1.record()
+    torch.cuda.synchronize()
+    per_step = sorted(e0.elapsed_time(e1) for e0, e1 in pairs)
+    # Third pass, untimed: the library brackets each of its launches with events on its launch
+    # stream; the dominant kernel's average duration is the roofline figure.
+    _lib.check(L.nbo_profile_enable(1))
+    for _ in range(steps):
+        step()
     per_kernel = {}
     for kname in names:
         cnt, ms = C.c_uint64(0), C.c_double(0.0)
@@ -364,6 +515,11 @@ def measure(name, steps, warmup, zero_grads="off", settle_s=2.0):
         "steps": steps,
         "warmup": warmup,
         "ms_per_step": round(ms_step, 4),
+        "ms_per_step_spread": {"min": round(per_step[0], 4), "median": round(per_step[len(per_step) // 2], 4),
+                               "max": round(per_step[-1], 4),
+                               "how": "a second pass of the same number of steps, each between one pair of HIP "
+                                      "events on the launch stream; `ms_per_step` and `value` are the mean of the "
+                                      "timed pass (wall clock around all steps, no events inside)"},
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -390,6 +546,8 @@ def measure(name, steps, warmup, zero_grads="off", settle_s=2.0):
             "algorithmic_bytes_per_launch": n * dom_b,
             "avg_launch_ms": round(dom_ms, 4),
             "launches": per_kernel[dom][0],
+            "how": "HIP events around each launch on the library's launch stream, in a pass of its own after the "
+                   "timed one",
         },
         "kernels_ms": {k: round(v[1] / max(v[0], 1), 4) for k, v in per_kernel.items()},
     }
@@ -443,16 +601,28 @@ def main():
               "MI355X: `value` is whole-step algorithmic HBM throughput, `kernel` the dominant kernel's (HIP events on the "
               "launch stream), `CPU` the oracle in reference-faithful form on the host's cores on a sample of the same "
               "workload.\n")
-        print("| workload | params | ms/step | value GB/s | % of 8 TB/s | params/s | dominant kernel GB/s | HBM regions "
-              "of state | CPU params/s (cores) | GPU/CPU |")
-        print("|---|---|---|---|---|---|---|---|---|---|")
+        print("| workload | params | ms/step (min / median / max) | value GB/s | % of 8 TB/s | params/s | dominant kernel "
+              "GB/s | HBM regions of state | CPU params/s (cores) | GPU/CPU | parity vs sqrt oracle: max ulp m / v / "
+              "master / params | parity vs libm-powf oracle: max ulp m / v / master / params (elements beyond the bar) | "
+              "decisions |")
+        print("|---|---|---|---|---|---|---|---|---|---|---|---|---|")
+
+        def ulps(cmp):
+            return " / ".join(str(cmp[k]["max_ulp"]) if k in cmp else "-" for k in ("m", "v", "master", "params"))
+
         for name in names:
             d, cfg = measure(name, args.steps, args.warmup, "off", args.settle_seconds)
             c = cpu_baseline(cfg, args.cpu_seconds)
-            print(f"| {name} | {d['config']['params']:,} | {d['ms_per_step']} | {d['value']} | {d['pct_of_peak']} | "
+            par = parity_check(cfg)
+            beyond = sum(x["beyond_bar"] for x in par["vs_oracle_libm_powf"].values())
+            sp = d["ms_per_step_spread"]
+            print(f"| {name} | {d['config']['params']:,} | {d['ms_per_step']} ({sp['min']} / {sp['median']} / {sp['max']}) | "
+                  f"{d['value']} | {d['pct_of_peak']} | "
                   f"{d['params_per_s']:.3e} | {d['roofline']['achieved']} ({d['roofline']['kernel']}) | "
                   f"{d['config']['state_hbm_regions']} | {c['params_per_s']:.3e} ({c['cores']}) | "
-                  f"{d['params_per_s'] / c['params_per_s']:.0f}x |", flush=True)
+                  f"{d['params_per_s'] / c['params_per_s']:.0f}x | {ulps(par['vs_oracle_sqrt'])} | "
+                  f"{ulps(par['vs_oracle_libm_powf'])} ({beyond}) | "
+                  f"{'bit-exact' if par['decisions_bit_exact'] else 'DIFFER'} |", flush=True)
         return
     out, cfg = measure(args.workload, args.steps, args.warmup, args.zero_grads, args.settle_seconds)
     if args.workload == "llama3-8b" and not args.primary_only:
@@ -461,8 +631,8 @@ def main():
         try:
             small, _ = measure("llama-1.1b", 20, 10, settle_s=args.settle_seconds)
             out["also"] = {"llama-1.1b": {k: small[k] for k in ("value", "unit", "pct_of_peak", "params_per_s",
-                                                                "ms_per_step", "steps", "warmup", "config",
-                                                                "roofline", "kernels_ms")}}
+                                                                "ms_per_step", "ms_per_step_spread", "steps", "warmup",
+                                                                "config", "roofline", "kernels_ms")}}
         except Exception as e:  # the ride-along must not cost the headline measurement
             out["also"] = {"llama-1.1b": {"error": str(e)}}
     if not args.no_ceiling and out["roofline"]["achieved"] > 0:
@@ -473,6 +643,10 @@ def main():
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_seconds)
         out["cpu_baseline"]["gpu_over_cpu"] = round(out["value"] / max(out["cpu_baseline"]["value"], 1e-9), 1)
+        try:
+            out["parity"] = parity_check(cfg)
+        except Exception as e:  # the check must not cost the measurement
+            out["parity"] = {"error": f"{type(e).__name__}: {e}"}
     print(json.dumps(out), flush=True)
 
 

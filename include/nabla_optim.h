@@ -342,45 +342,6 @@ int nbo_optim_load_master(nbo_optim *opt, const char *path, const char *const *n
 int nbo_optim_save_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path);
 int nbo_optim_load_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path);
 
-/* ---- measurement helpers --------------------------------------------------------------- */
-
-/* Device-to-device streaming copy of `bytes` (multiple of 16) with the engine's own
- * copy kernel; used to calibrate HBM byte counters against a known transfer. */
-int nbo_copy_bytes(const void *src_dev, void *dst_dev, uint64_t bytes);
-/* What the memory system gives an access pattern, measured with the library's own probe
- * kernel (one workgroup per 32 KiB window of every stream, 128-bit accesses, all loads issued
- * before the first use -- the update kernels' access shape): the yardstick the update kernels'
- * throughput is judged against.  `pattern` names the streams (nbo_probe_pattern).  spread = 0:
- * all streams lie back to back in one plain allocation; spread = 1: they are slices of up to
- * three arrays placed across the HBM's regions exactly as optimizer state is (*regions then
- * receives what nbo_optim_state_regions would report).  Allocates and frees its buffers
- * (bytes_per_stream: a multiple of 32 KiB), launches untimed for settle_ms milliseconds (at
- * least once: the driver clears freed device memory in the background, which competes for
- * bandwidth for about a second after a large free) and then `reps` times, timed;
- * *best_gbps / *mean_gbps are bytes moved per launch (reads + writes) over the shortest /
- * the mean duration.  No counterpart in the reference.  Synchronous. */
-typedef enum nbo_probe_pattern {
-    NBO_PATTERN_READ1 = 0,       /* 1 stream read */
-    NBO_PATTERN_READ3 = 1,       /* 3 streams read */
-    NBO_PATTERN_FILL1 = 2,       /* 1 stream written */
-    NBO_PATTERN_FILL3 = 3,       /* 3 streams written */
-    NBO_PATTERN_COPY = 4,        /* 1 stream read, 1 written */
-    NBO_PATTERN_RMW1 = 5,        /* N streams read and rewritten in place */
-    NBO_PATTERN_RMW2 = 6,
-    NBO_PATTERN_RMW3 = 7,
-    NBO_PATTERN_RMW6 = 8,
-    NBO_PATTERN_R1_RMW3_W1 = 9   /* 1 read, 3 in place, 1 written: the mixed-precision update's streams */
-} nbo_probe_pattern;
-int nbo_hbm_ceiling(int pattern, int spread, uint64_t bytes_per_stream, int reps, uint32_t settle_ms,
-                    double *best_gbps, double *mean_gbps, int *regions);
-/* Per-kernel timing: while enabled, every kernel launch is bracketed by HIP events on
- * the launch stream.  nbo_profile_read synchronises and returns the number of
- * launches of `kernel_name` (e.g. "nbo_update_bf16_adamw") since profiling was
- * enabled and the sum of their durations.  (The reference times its steps with host
- * timers around a stream sync, nabla-train/src/profiler.rs:176-197.) */
-int nbo_profile_enable(int on);
-int nbo_profile_read(const char *kernel_name, uint64_t *launches, double *total_ms);
-
 #pragma GCC visibility pop
 
 #ifdef __cplusplus

@@ -103,10 +103,16 @@ extern "C" {
     pub fn nbo_optim_state_placement_note(opt: *mut NboOptim, buf: *mut c_char, buf_bytes: u64) -> c_int;
     pub fn nbo_status_string(status: c_int) -> *const c_char;
     pub fn nbo_version() -> *const c_char;
-    // measurement helpers (no counterpart in the reference)
+    // measurement helpers of nabla_optim_bench.h (no counterpart in the reference)
     pub fn nbo_copy_bytes(src_dev: *const c_void, dst_dev: *mut c_void, bytes: u64) -> c_int;
     pub fn nbo_hbm_ceiling(pattern: c_int, spread: c_int, bytes_per_stream: u64, reps: c_int, settle_ms: u32,
                            best_gbps: *mut f64, mean_gbps: *mut f64, regions: *mut c_int) -> c_int;
+    pub fn nbo_hbm_ceiling_shape(pattern: c_int, shape: c_int, spread: c_int, bytes_per_stream: u64, reps: c_int,
+                                 settle_ms: u32, best_gbps: *mut f64, mean_gbps: *mut f64, regions: *mut c_int,
+                                 mismatches: *mut u64) -> c_int;
+    pub fn nbo_hbm_ceiling_compare(pattern: c_int, n_shapes: c_int, shapes: *const c_int, iters: *const u32,
+                                   spread: c_int, bytes_per_stream: u64, rounds: c_int, reps: c_int, settle_ms: u32,
+                                   best_gbps: *mut f64, mean_gbps: *mut f64, regions: *mut c_int) -> c_int;
     pub fn nbo_profile_enable(on: c_int) -> c_int;
     pub fn nbo_profile_read(kernel_name: *const c_char, launches: *mut u64, total_ms: *mut f64) -> c_int;
 }

@@ -1,4 +1,5 @@
-"""ctypes binding of libnabla_optim.so (the C ABI of include/nabla_optim.h).
+"""ctypes binding of libnabla_optim.so (the C ABI of include/nabla_optim.h and, for
+measurement, include/nabla_optim_bench.h).
 
 The library is the product; there is no Python or CPU fallback.  If the shared
 object is missing, or no gfx950 device can be initialised, importing is still
@@ -129,9 +130,17 @@ SYMBOLS = {
     "nbo_optim_load_master": (C.c_int, [_P, C.c_char_p, C.POINTER(C.c_char_p)]),
     "nbo_optim_save_state_groups": (C.c_int, [C.c_uint64, C.POINTER(_P), C.c_char_p]),
     "nbo_optim_load_state_groups": (C.c_int, [C.c_uint64, C.POINTER(_P), C.c_char_p]),
+}
+# every symbol include/nabla_optim_bench.h declares (measurement only)
+BENCH_SYMBOLS = {
     "nbo_copy_bytes": (C.c_int, [_P, _P, C.c_uint64]),
     "nbo_hbm_ceiling": (C.c_int, [C.c_int, C.c_int, C.c_uint64, C.c_int, C.c_uint32, C.POINTER(C.c_double),
                                   C.POINTER(C.c_double), C.POINTER(C.c_int)]),
+    "nbo_hbm_ceiling_shape": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_uint64, C.c_int, C.c_uint32,
+                                        C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_int), _U64P]),
+    "nbo_hbm_ceiling_compare": (C.c_int, [C.c_int, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_uint32), C.c_int,
+                                          C.c_uint64, C.c_int, C.c_int, C.c_uint32, C.POINTER(C.c_double),
+                                          C.POINTER(C.c_double), C.POINTER(C.c_int)]),
     "nbo_profile_enable": (C.c_int, [C.c_int]),
     "nbo_profile_read": (C.c_int, [C.c_char_p, _U64P, C.POINTER(C.c_double)]),
 }
@@ -169,7 +178,7 @@ def load() -> C.CDLL:
     except ImportError:
         pass
     lib = C.CDLL(LIB_PATH)
-    for name, (restype, argtypes) in SYMBOLS.items():
+    for name, (restype, argtypes) in list(SYMBOLS.items()) + list(BENCH_SYMBOLS.items()):
         fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
         fn.restype = restype
         fn.argtypes = argtypes

@@ -5,41 +5,21 @@
 #include <mutex>
 #include <new>
 
+#include "nbo_api_guard.hpp"
 #include "nbo_host.hpp"
 #include "nbo_noalloc.hpp"
 
 using namespace nbo;
 
+namespace nbo {
+std::recursive_mutex &api_mutex()
+{
+    static std::recursive_mutex m;
+    return m;
+}
+} // namespace nbo
+
 namespace {
-
-// The runtime's stream, staging buffer and reduction scratch are shared by every
-// handle, so entry points run one at a time; the device work they enqueue is ordered
-// by the one stream.
-std::recursive_mutex g_api_mutex;
-
-// Runs `body`, mapping internal errors to status codes; nothing escapes the C ABI.
-template <typename F> int guarded(F &&body)
-{
-    std::lock_guard<std::recursive_mutex> lock(g_api_mutex);
-    try {
-        body();
-        return NBO_OK;
-    } catch (const Error &e) {
-        set_last_error(e.msg);
-        return e.status;
-    } catch (const std::bad_alloc &) {
-        set_last_error("host allocation failed");
-        return NBO_ERR_ARG;
-    } catch (...) {
-        set_last_error("unexpected internal error");
-        return NBO_ERR_ARG;
-    }
-}
-
-void require(bool cond, int status, const char *msg)
-{
-    if (!cond) fail(status, msg);
-}
 
 const char *kind_name(int kind)
 {
@@ -127,6 +107,29 @@ int update_kernel(const nbo_optim *opt, const nbo_list *params)
     if (opt->state_dtype == NBO_DT_F16) return K_UPDATE_PF16_BASE + kind;
     if (params->dtype == NBO_DT_F16) return K_UPDATE_F16_BASE + kind;
     return K_UPDATE_BASE + params->dtype * 3 + kind;
+}
+
+// ... of the kernels that prepare the step's scalars themselves
+int self_update_kernel(const nbo_optim *opt, const nbo_list *params)
+{
+    const int family = opt->state_dtype == NBO_DT_BF16 ? 4 : opt->state_dtype == NBO_DT_F16 ? 5 :
+                       params->dtype == NBO_DT_F16 ? 3 : params->dtype; // f32 0, bf16 1, f64 2
+    return K_UPDATE_SELF_BASE + family * 3 + opt->meta.kind;
+}
+
+// One launch that prepares its own scalars, advances step_count (unless *gf says the step is
+// skipped) and writes the trace entry.  Not for an empty list: no workgroup would run.
+bool self_update_possible(const nbo_optim *opt) { return opt->layout.nchunks > 0; }
+
+void launch_self_update(nbo_optim *opt, nbo_list *params, nbo_list *grads, const NboGradFactors *gf, bool zero_grads,
+                        NboTraceDev *trace, const NboScalerDev *scaler)
+{
+    NboUpdateArgs a = update_args(opt, params, grads, false, zero_grads, gf);
+    a.hyper = hyper_of(opt);
+    a.opt_rw = opt->dev;
+    a.trace = trace;
+    a.scaler = scaler;
+    Runtime::get().launch(self_update_kernel(opt, params), opt->layout.nchunks, NBO_BLOCK, a);
 }
 
 uint32_t norm_grid(const Layout &L)
@@ -539,6 +542,10 @@ int nbo_optim_step(nbo_optim *opt, nbo_list *params, nbo_list *grads)
             a.sgd_lr = opt->meta.lr;
             a.sgd_momentum = opt->meta.momentum;
             a.sgd_weight_decay = opt->meta.weight_decay;
+        } else if (self_update_possible(opt)) {
+            // Adam::step / AdamW::step is one call (alg.rs:109-150, 254-291): one launch
+            launch_self_update(opt, params, grads, nullptr, false, nullptr, nullptr);
+            return;
         } else {
             NboPrepArgs p = {};
             p.opt = opt->dev;
@@ -876,12 +883,19 @@ static uint64_t check_group_args(uint64_t n_groups, nbo_optim *const *opts, nbo_
     return covered;
 }
 
-// Each group's scalars and update from the one decision in the runtime's scratch.
+// Each group's scalars and update from the one decision in the runtime's scratch: one launch
+// per group (two for an empty group, see self_update_possible).
 static void launch_group_updates(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,
                                  nbo_list *const *grads, nbo_scaler *scaler, uint32_t flags)
 {
     Runtime &rt = Runtime::get();
     for (uint64_t g = 0; g < n_groups; g++) {
+        if (self_update_possible(opts[g])) {
+            // one launch per group: it derives the group's scalars from the shared decision itself
+            launch_self_update(opts[g], params[g], grads[g], rt.gf_scratch(), (flags & NBO_STEP_ZERO_GRADS) != 0,
+                               opts[g]->trace, scaler ? scaler->dev : nullptr);
+            continue;
+        }
         NboPrepArgs p = {};
         p.opt = opts[g]->dev;
         p.gf = rt.gf_scratch();
@@ -1198,86 +1212,6 @@ int nbo_optim_load_state_groups(uint64_t n_groups, nbo_optim *const *opts, const
     return guarded([&] {
         require_groups(n_groups, opts, path);
         optim_load_state_groups(n_groups, opts, path);
-    });
-}
-
-int nbo_copy_bytes(const void *src_dev, void *dst_dev, uint64_t bytes)
-{
-    return guarded([&] {
-        require(src_dev && dst_dev, NBO_ERR_ARG, "null address");
-        require(bytes % 16 == 0 && ((uintptr_t)src_dev % 16) == 0 && ((uintptr_t)dst_dev % 16) == 0,
-                NBO_ERR_ARG, "copy needs 16-byte aligned addresses and size");
-        Runtime::get().launch_copy(src_dev, dst_dev, bytes / 16);
-    });
-}
-
-int nbo_hbm_ceiling(int pattern, int spread, uint64_t bytes_per_stream, int reps, uint32_t settle_ms,
-                    double *best_gbps, double *mean_gbps, int *regions)
-{
-    return guarded([&] {
-        // streams read, rewritten in place, written
-        static const int kShape[NBO_PROBE_COUNT][3] = {{1, 0, 0}, {3, 0, 0}, {0, 0, 1}, {0, 0, 3}, {1, 0, 1},
-                                                       {0, 1, 0}, {0, 2, 0}, {0, 3, 0}, {0, 6, 0}, {1, 3, 1}};
-        static_assert((int)NBO_PATTERN_READ1 == (int)NBO_PROBE_READ1 && (int)NBO_PATTERN_COPY == (int)NBO_PROBE_COPY &&
-                          (int)NBO_PATTERN_RMW3 == (int)NBO_PROBE_RMW3 &&
-                          (int)NBO_PATTERN_R1_RMW3_W1 == (int)NBO_PROBE_R1_RMW3_W1 &&
-                          (int)NBO_PATTERN_R1_RMW3_W1 + 1 == (int)NBO_PROBE_COUNT,
-                      "public pattern codes and the kernels' must agree");
-        require(pattern >= 0 && pattern < (int)NBO_PROBE_COUNT, NBO_ERR_ARG, "unknown probe pattern");
-        require(best_gbps && mean_gbps, NBO_ERR_ARG, "null output");
-        require(reps >= 1 && reps <= 1000, NBO_ERR_ARG, "1 to 1000 repetitions");
-        require(settle_ms <= 60000, NBO_ERR_ARG, "at most 60 s of untimed launches");
-        const uint64_t window = 8ull * NBO_BLOCK * 16; // bytes of one stream a workgroup covers
-        require(bytes_per_stream >= window && bytes_per_stream % window == 0 &&
-                    bytes_per_stream / window <= 0x7FFFFFFFull,
-                NBO_ERR_ARG, "bytes per stream: a multiple of 32 KiB, at most 2^31 - 1 of them");
-        const int ro = kShape[pattern][0], rmw = kShape[pattern][1], wo = kShape[pattern][2];
-        const uint32_t ns = (uint32_t)(ro + rmw + wo);
-        Runtime &rt = Runtime::get();
-        // Streams are equal slices of up to three arrays.  spread: the arrays come from the
-        // region-aware placement the optimizer state uses, stream s lies in array s mod 3, so
-        // neighbouring streams sit in different HBM regions at every offset.  Otherwise one plain
-        // allocation holds all streams back to back.
-        StatePlacement place;
-        void *part[3] = {nullptr, nullptr, nullptr};
-        const uint32_t nparts = spread ? (ns < 3 ? ns : 3) : 1;
-        const uint32_t per_part = (ns + nparts - 1) / nparts;
-        const size_t part_bytes = (size_t)per_part * bytes_per_stream;
-        if (spread) {
-            place.allocate(nparts, part_bytes, part);
-        } else {
-            part[0] = rt.dmalloc(part_bytes);
-        }
-        try {
-            for (uint32_t k = 0; k < nparts; k++) rt.dzero(part[k], part_bytes);
-            NboStreamProbeArgs a = {};
-            for (uint32_t s = 0; s < ns; s++)
-                a.buf[s] = (char *)part[s % nparts] + (size_t)(s / nparts) * bytes_per_stream;
-            double best_ms = 0.0, mean_ms = 0.0;
-            rt.time_launches(K_STREAM_PROBE_BASE + pattern, (uint32_t)(bytes_per_stream / window), &a, reps, settle_ms, &best_ms, &mean_ms);
-            const double moved = (double)(ro + 2 * rmw + wo) * (double)bytes_per_stream;
-            *best_gbps = best_ms > 0.0 ? moved / best_ms / 1e6 : 0.0;
-            *mean_gbps = mean_ms > 0.0 ? moved / mean_ms / 1e6 : 0.0;
-            if (regions) *regions = spread ? place.regions_used() : 0;
-        } catch (...) {
-            if (!spread) rt.dfree(part[0]);
-            throw;
-        }
-        rt.sync();
-        if (!spread) rt.dfree(part[0]);
-    });
-}
-
-int nbo_profile_enable(int on)
-{
-    return guarded([&] { Runtime::get().profile_enable(on != 0); });
-}
-
-int nbo_profile_read(const char *kernel_name, uint64_t *launches, double *total_ms)
-{
-    return guarded([&] {
-        require(kernel_name && launches && total_ms, NBO_ERR_ARG, "null argument");
-        Runtime::get().profile_read(kernel_name, launches, total_ms);
     });
 }
 

@@ -11,7 +11,8 @@
 
 // The gfx950 code object, embedded by nbo_code_object.S.
 extern "C" const unsigned char nbo_code_object[];
-extern "C" const unsigned char nbo_code_object_end[];
+// The measurement kernels' code object, likewise.
+extern "C" const unsigned char nbo_bench_code_object[];
 
 namespace nbo {
 
@@ -38,7 +39,7 @@ static const char *const kKernelNames[K_COUNT] = {
     "nbo_norm_f32",          "nbo_norm_bf16",        "nbo_norm_f64",
     "nbo_scale_f32",         "nbo_scale_bf16",       "nbo_scale_f64",
     "nbo_prep",              "nbo_finalize",         "nbo_cast_master",
-    "nbo_copy_f32x4",        "nbo_probe_rmw2",       "nbo_accum_f32",
+    nullptr,                 "nbo_probe_rmw2",       "nbo_accum_f32",
     "nbo_accum_bf16",        "nbo_accum_f64",        "nbo_fill_zero",
     "nbo_ew_f32",            "nbo_ew_bf16",          "nbo_ew_f64",
     "nbo_cast_list",         "nbo_update_pbf16_adamw", "nbo_update_pbf16_adam",
@@ -48,12 +49,14 @@ static const char *const kKernelNames[K_COUNT] = {
     "nbo_norm_f16",          "nbo_norm_pf16",        "nbo_scale_f16",
     "nbo_accum_f16",         "nbo_ew_f16",           "nbo_accnorm_f32",
     "nbo_accnorm_bf16",      "nbo_accnorm_f64",      "nbo_accnorm_f16",
-    "nbo_probe_read1",       "nbo_probe_read3",      "nbo_probe_fill1",
-    "nbo_probe_fill3",       "nbo_probe_copy",       "nbo_probe_rmw1",
-    "nbo_probe_rmw2s",       "nbo_probe_rmw3",       "nbo_probe_rmw6",
-    "nbo_probe_r1_rmw3_w1",
+    "nbo_update_f32_adamw_self",   "nbo_update_f32_adam_self",   "nbo_update_f32_sgd_self",
+    "nbo_update_bf16_adamw_self",  "nbo_update_bf16_adam_self",  "nbo_update_bf16_sgd_self",
+    "nbo_update_f64_adamw_self",   "nbo_update_f64_adam_self",   "nbo_update_f64_sgd_self",
+    "nbo_update_f16_adamw_self",   "nbo_update_f16_adam_self",   "nbo_update_f16_sgd_self",
+    "nbo_update_pbf16_adamw_self", "nbo_update_pbf16_adam_self", "nbo_update_pbf16_sgd_self",
+    "nbo_update_pf16_adamw_self",  "nbo_update_pf16_adam_self",  "nbo_update_pf16_sgd_self",
 };
-static_assert(K_STREAM_PROBE_BASE + NBO_PROBE_COUNT == K_COUNT, "one probe kernel per pattern");
+static_assert(K_UPDATE_SELF_BASE + 18 == K_COUNT, "six families of three self-preparing update kernels");
 
 static std::mutex g_runtime_mu;
 static Runtime *g_runtime = nullptr;
@@ -93,7 +96,7 @@ Runtime::Runtime()
                  hipGetErrorString(e));
     }
     for (int k = 0; k < K_COUNT; k++)
-        hip_check(hipModuleGetFunction(&fn_[k], module_, kKernelNames[k]), kKernelNames[k]);
+        if (kKernelNames[k]) hip_check(hipModuleGetFunction(&fn_[k], module_, kKernelNames[k]), kKernelNames[k]);
     pinned_bytes_ = 8 << 20; // two halves of 4 MiB
     hip_check(hipHostMalloc(&pinned_, pinned_bytes_, hipHostMallocDefault), "hipHostMalloc");
     for (hipEvent_t &e : staged_) hip_check(hipEventCreateWithFlags(&e, hipEventDisableTiming), "hipEventCreate");
@@ -120,9 +123,45 @@ void Runtime::set_stream(hipStream_t s)
     stream_ = s;
 }
 
+hipFunction_t Runtime::function(int kernel) const
+{
+    if (kernel >= 0 && kernel < K_COUNT && fn_[kernel]) return fn_[kernel];
+    if (kernel >= K_COUNT && (size_t)(kernel - K_COUNT) < bench_fn_.size()) return bench_fn_[kernel - K_COUNT];
+    fail(NBO_ERR_ARG, "internal: unknown kernel id " + std::to_string(kernel));
+}
+
+const char *Runtime::kernel_name(int kernel) const
+{
+    if (kernel >= 0 && kernel < K_COUNT && kKernelNames[kernel]) return kKernelNames[kernel];
+    if (kernel >= K_COUNT && (size_t)(kernel - K_COUNT) < bench_names_.size())
+        return bench_names_[kernel - K_COUNT].c_str();
+    return "?";
+}
+
+int Runtime::bench_kernel(const char *name)
+{
+    for (size_t k = 0; k < bench_names_.size(); k++)
+        if (bench_names_[k] == name) return K_COUNT + (int)k;
+    if (!bench_module_) {
+        const hipError_t e = hipModuleLoadData(&bench_module_, nbo_bench_code_object);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            bench_module_ = nullptr;
+            fail(NBO_ERR_HIP + (int)e, std::string("hipModuleLoadData of the measurement code object failed: ") +
+                                           hipGetErrorString(e));
+        }
+    }
+    hipFunction_t f = nullptr;
+    hip_check(hipModuleGetFunction(&f, bench_module_, name), name);
+    bench_names_.push_back(name);
+    bench_fn_.push_back(f);
+    return K_COUNT + (int)bench_names_.size() - 1;
+}
+
 void Runtime::launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct, bool may_time)
 {
     if (grid == 0) return;
+    const hipFunction_t fn = function(kernel);
     void *args[1] = {arg_struct};
     ProfRec rec = {kernel, nullptr, nullptr};
     const bool timed = profiling_ && may_time; // timing creates two events per launch
@@ -131,8 +170,7 @@ void Runtime::launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_st
         hip_check(hipEventCreate(&rec.end), "hipEventCreate");
         hip_check(hipEventRecord(rec.begin, stream_), "hipEventRecord");
     }
-    hip_check(hipModuleLaunchKernel(fn_[kernel], grid, 1, 1, block, 1, 1, 0, stream_, args, nullptr),
-              kKernelNames[kernel]);
+    hip_check(hipModuleLaunchKernel(fn, grid, 1, 1, block, 1, 1, 0, stream_, args, nullptr), kernel_name(kernel));
     if (timed) {
         hip_check(hipEventRecord(rec.end, stream_), "hipEventRecord");
         prof_.push_back(rec);
@@ -153,8 +191,17 @@ void Runtime::profile_read(const char *kernel_name, uint64_t *launches, double *
 {
     int id = -1;
     for (int k = 0; k < K_COUNT; k++)
-        if (std::strcmp(kernel_name, kKernelNames[k]) == 0) id = k;
-    if (id < 0) fail(NBO_ERR_ARG, std::string("unknown kernel name: ") + kernel_name);
+        if (kKernelNames[k] && std::strcmp(kernel_name, kKernelNames[k]) == 0) id = k;
+    for (size_t k = 0; k < bench_names_.size(); k++)
+        if (bench_names_[k] == kernel_name) id = K_COUNT + (int)k;
+    if (id < 0) {
+        // perhaps a measurement kernel that has not been launched yet
+        try {
+            id = bench_kernel(kernel_name);
+        } catch (const Error &) {
+            fail(NBO_ERR_ARG, std::string("unknown kernel name: ") + kernel_name);
+        }
+    }
     sync();
     uint64_t n = 0;
     double ms = 0.0;
@@ -172,25 +219,36 @@ void Runtime::profile_read(const char *kernel_name, uint64_t *launches, double *
 void Runtime::launch_copy(const void *src, void *dst, uint64_t nvec)
 {
     if (nvec == 0) return;
+    const int k = bench_kernel("nbo_copy_f32x4");
     uint64_t blocks = (nvec + NBO_BLOCK - 1) / NBO_BLOCK;
     // four 128-bit vectors per thread in flight keeps the loop short without
     // starving the memory system
     uint64_t grid = (blocks + 3) / 4;
     if (grid > 0x7FFFFFFFull) grid = 0x7FFFFFFFull;
     void *args[3] = {(void *)&src, (void *)&dst, (void *)&nvec};
-    ProfRec rec = {K_COPY, nullptr, nullptr};
+    ProfRec rec = {k, nullptr, nullptr};
     if (profiling_) {
         hip_check(hipEventCreate(&rec.begin), "hipEventCreate");
         hip_check(hipEventCreate(&rec.end), "hipEventCreate");
         hip_check(hipEventRecord(rec.begin, stream_), "hipEventRecord");
     }
-    hip_check(hipModuleLaunchKernel(fn_[K_COPY], (uint32_t)grid, 1, 1, NBO_BLOCK, 1, 1, 0, stream_,
-                                    args, nullptr),
-              kKernelNames[K_COPY]);
+    hip_check(hipModuleLaunchKernel(function(k), (uint32_t)grid, 1, 1, NBO_BLOCK, 1, 1, 0, stream_, args, nullptr),
+              "nbo_copy_f32x4");
     if (profiling_) {
         hip_check(hipEventRecord(rec.end, stream_), "hipEventRecord");
         prof_.push_back(rec);
     }
+}
+
+void Runtime::launch_fill_index(void *dst, uint64_t nvec)
+{
+    if (nvec == 0) return;
+    const int k = bench_kernel("nbo_probe_fill_index");
+    uint64_t grid = (nvec + NBO_BLOCK - 1) / NBO_BLOCK;
+    if (grid > 65536) grid = 65536;
+    void *args[2] = {(void *)&dst, (void *)&nvec};
+    hip_check(hipModuleLaunchKernel(function(k), (uint32_t)grid, 1, 1, NBO_BLOCK, 1, 1, 0, stream_, args, nullptr),
+              "nbo_probe_fill_index");
 }
 
 double Runtime::probe_pair_gbps(void *a, void *b, size_t bytes)
@@ -216,15 +274,15 @@ double Runtime::probe_pair_gbps(void *a, void *b, size_t bytes)
     return best > 0.0f ? 4.0 * (double)grid * (double)per_wg * 16 / best / 1e6 : 0.0;
 }
 
-void Runtime::time_launches(int kernel, uint32_t grid, void *arg_struct, int reps, uint32_t settle_ms, double *best_ms,
-                            double *mean_ms)
+uint64_t Runtime::time_launches(int kernel, uint32_t grid, uint32_t block, void *arg_struct, int reps,
+                                uint32_t settle_ms, double *best_ms, double *mean_ms)
 {
     void *args[1] = {arg_struct};
+    const hipFunction_t fn = function(kernel);
     const hipEvent_t e0 = probe_ev_[0], e1 = probe_ev_[1];
     auto one = [&]() {
         hip_check(hipEventRecord(e0, stream_), "hipEventRecord");
-        hip_check(hipModuleLaunchKernel(fn_[kernel], grid, 1, 1, NBO_BLOCK, 1, 1, 0, stream_, args, nullptr),
-                  kKernelNames[kernel]);
+        hip_check(hipModuleLaunchKernel(fn, grid, 1, 1, block, 1, 1, 0, stream_, args, nullptr), kernel_name(kernel));
         hip_check(hipEventRecord(e1, stream_), "hipEventRecord");
         hip_check(hipEventSynchronize(e1), "hipEventSynchronize");
         float ms = 0.0f;
@@ -233,9 +291,11 @@ void Runtime::time_launches(int kernel, uint32_t grid, void *arg_struct, int rep
     };
     // warm-up, and time for the driver's background clearing of memory freed just before (the
     // placement search's spare chunks, an earlier measurement's buffers) to finish
+    uint64_t launches = 0;
     const auto t0 = std::chrono::steady_clock::now();
     do {
         (void)one();
+        launches++;
     } while (std::chrono::duration_cast<std::chrono::milliseconds>(std::chrono::steady_clock::now() - t0).count() <
              (long long)settle_ms);
     double best = 0.0, sum = 0.0;
@@ -246,6 +306,7 @@ void Runtime::time_launches(int kernel, uint32_t grid, void *arg_struct, int rep
     }
     *best_ms = best;
     *mean_ms = reps > 0 ? sum / reps : 0.0;
+    return launches + (uint64_t)(reps > 0 ? reps : 0);
 }
 
 // Both directions run the two halves of the pinned buffer as a pipeline: while the DMA

@@ -41,7 +41,7 @@ enum KernelId {
     K_PREP = 15,
     K_FINALIZE = 16,
     K_CAST_MASTER = 17,
-    K_COPY = 18,
+    K_UNUSED_18 = 18, // (was the calibration copy: now in the measurement code object)
     K_PROBE = 19,
     K_ACCUM_BASE = 20, // + st
     K_FILL_ZERO = 23,
@@ -58,8 +58,10 @@ enum KernelId {
     K_EW_F16 = 42,
     K_ACCNORM_BASE = 43, // + st (f32 / bf16 / f64)
     K_ACCNORM_F16 = 46,
-    K_STREAM_PROBE_BASE = 47, // + NBO_PROBE_* pattern
-    K_COUNT = 57
+    // update kernels that prepare their own per-step scalars: + family * 3 + kind, family =
+    // f32, bf16, f64, f16, pbf16, pf16
+    K_UPDATE_SELF_BASE = 47,
+    K_COUNT = 65 // ids from here on are measurement kernels, handed out by Runtime::bench_kernel
 };
 
 // Process-wide runtime: device 0, the loaded module, the stream, scratch buffers.
@@ -78,14 +80,21 @@ public:
     // may_time = false: never bracket the launch with timing events, whatever profile_enable
     // says (creating events allocates host memory)
     void launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct, bool may_time = true);
+    // Id of kernel `name` of the measurement code object (nbo_bench_kernels.hip), which is
+    // loaded when the first such id is asked for; the id works with launch, time_launches and
+    // the per-kernel timing like the ids above.
+    int bench_kernel(const char *name);
     void launch_copy(const void *src, void *dst, uint64_t nvec);
+    // float i of the nvec 128-bit vectors at dst = i mod 1024 (start contents of a checked probe run)
+    void launch_fill_index(void *dst, uint64_t nvec);
     // Bandwidth (GB/s, best of three) of reading and rewriting `bytes` bytes at a and at
     // b together: the probe StatePlacement classifies HBM regions with.  Synchronous.
     double probe_pair_gbps(void *a, void *b, size_t bytes);
     // Untimed launches for `settle_ms` milliseconds (at least one), then `reps` launches each
-    // bracketed by events on the stream: shortest and mean duration in ms.  Synchronous.
-    void time_launches(int kernel, uint32_t grid, void *arg_struct, int reps, uint32_t settle_ms, double *best_ms,
-                       double *mean_ms);
+    // bracketed by events on the stream: shortest and mean duration in ms.  Returns how many
+    // launches were made in all.  Synchronous.
+    uint64_t time_launches(int kernel, uint32_t grid, uint32_t block, void *arg_struct, int reps, uint32_t settle_ms,
+                       double *best_ms, double *mean_ms);
 
     // synchronous transfers through a double-buffered pinned staging buffer
     void read_back(void *host_dst, const void *dev_src, size_t bytes);
@@ -110,8 +119,13 @@ public:
 
 private:
     Runtime();
+    hipFunction_t function(int kernel) const;
+    const char *kernel_name(int kernel) const;
     hipModule_t module_ = nullptr;
     hipFunction_t fn_[K_COUNT] = {};
+    hipModule_t bench_module_ = nullptr; // loaded on first use
+    std::vector<std::string> bench_names_;
+    std::vector<hipFunction_t> bench_fn_;
     hipStream_t stream_ = nullptr;
     void *pinned_ = nullptr;
     size_t pinned_bytes_ = 0;

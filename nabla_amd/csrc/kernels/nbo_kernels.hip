@@ -466,9 +466,41 @@ DEV Peel peel(uint32_t cnt, uint32_t vec, uint32_t sb, bool wvo, uintptr_t a0, u
     return peel(cnt, vec, sb, wvo, a0, a1, a0);
 }
 
+DEV void prep_step(NboOptimDev *o, const NboHyper &h, const NboGradFactors *f);
+DEV void trace_step(NboTraceDev *t, const NboGradFactors *f, const NboOptimDev *o, double scale);
+
+// A per-step scalar that every lane has computed alike, moved to a scalar register (the
+// vector units do all f64 arithmetic; without this the scalars would occupy a vector register each).
+DEV float uniform(float x) { return __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(x))); }
+DEV double uniform(double x)
+{
+    const uint64_t b = (uint64_t)__double_as_longlong(x);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b), hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+    return __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
+}
+// ... for the scalars of a whole step (the fields Scal reads)
+DEV void make_uniform(NboOptimDev &o)
+{
+    o.b1 = uniform(o.b1); o.omb1 = uniform(o.omb1); o.b2 = uniform(o.b2); o.omb2 = uniform(o.omb2);
+    o.eps_t = uniform(o.eps_t); o.ss = uniform(o.ss); o.ibc2 = uniform(o.ibc2); o.omw = uniform(o.omw);
+    o.neg_lr = uniform(o.neg_lr); o.momentum_t = uniform(o.momentum_t); o.wd_t = uniform(o.wd_t);
+    o.wd_lr_t = uniform(o.wd_lr_t);
+    o.d_b1 = uniform(o.d_b1); o.d_omb1 = uniform(o.d_omb1); o.d_b2 = uniform(o.d_b2); o.d_omb2 = uniform(o.d_omb2);
+    o.d_eps = uniform(o.d_eps); o.d_ss = uniform(o.d_ss); o.d_ibc2 = uniform(o.d_ibc2); o.d_omw = uniform(o.d_omw);
+    o.d_neg_lr = uniform(o.d_neg_lr); o.d_momentum = uniform(o.d_momentum); o.d_wd = uniform(o.d_wd);
+}
+
 // ---------------------------------------------------------------------------------
 // Optimizer update: one workgroup per chunk.
-template <int ST, int KIND> DEV void update_body(const NboUpdateArgs &a)
+//
+// SELF: the launch prepares its own per-step scalars instead of reading what a launch before
+// it left in a.opt.  Every workgroup derives them from a.opt->step_count, the hyper-parameters
+// in the argument block and the decision in a.gf (the f64 prologue of alg.rs:120-135, some
+// hundred operations).  step_count has to advance exactly once, and only after every
+// workgroup has read it: each workgroup, once its read has returned, adds one to a counter in
+// device memory, and the workgroup whose addition completes the grid -- nobody waits for
+// anybody -- writes the advanced step_count and the trace entry and clears the counter.
+template <int ST, int KIND> DEV void update_chunk(const NboUpdateArgs &a, const NboOptimDev *o)
 {
     typedef typename Traits<ST>::T T;
     enum {
@@ -496,14 +528,14 @@ template <int ST, int KIND> DEV void update_body(const NboUpdateArgs &a)
     const bool vec_ok = ((((uintptr_t)pp) | ((uintptr_t)pg)) & (vbytes - 1)) == 0;
 
     const bool direct = KIND == NBO_SGD && a.direct != 0;
-    if (!direct && a.opt->skip) {
+    if (!direct && o->skip) {
         // found_inf: parameters, moments and step_count stay untouched
         // (trainer.rs:230-236); the gradients become zeros (core.rs:372-375).
         if (zero_g)
             for (uint32_t i = tid; i < c.cnt; i += NBO_BLOCK) IO<ST>::st1(pg + (uint64_t)i * SB, (T)0);
         return;
     }
-    const Scal<T> s = direct ? Scal<T>(a.sgd_lr, a.sgd_momentum, a.sgd_weight_decay) : Scal<T>(a.opt, a.gf);
+    const Scal<T> s = direct ? Scal<T>(a.sgd_lr, a.sgd_momentum, a.sgd_weight_decay) : Scal<T>(o, a.gf);
     const bool use_m = KIND != NBO_SGD || s.use_mom;
 
     if (c.cnt == NBO_CHUNK && vec_ok) {
@@ -605,6 +637,32 @@ template <int ST, int KIND> DEV void update_body(const NboUpdateArgs &a)
     }
 }
 
+template <int ST, int KIND, bool SELF = false> DEV void update_body(const NboUpdateArgs &a)
+{
+    if (!SELF) {
+        update_chunk<ST, KIND>(a, a.opt);
+        return;
+    }
+    uint32_t sc_lo = (uint32_t)a.opt->step_count, sc_hi = (uint32_t)(a.opt->step_count >> 32);
+    // the value is in registers -- the read has returned -- before anything below is issued
+    asm volatile("" : "+v"(sc_lo), "+v"(sc_hi)::"memory");
+    uint32_t readers_before = 0;
+    if (threadIdx.x == 0)
+        readers_before = __hip_atomic_fetch_add(&a.opt_rw->ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    NboOptimDev own = {};
+    own.step_count = ((uint64_t)sc_hi << 32) | sc_lo;
+    prep_step(&own, a.hyper, a.gf);
+    make_uniform(own);
+    update_chunk<ST, KIND>(a, &own);
+    // the counter's answer is not looked at before the chunk is done: it has long arrived then
+    __builtin_amdgcn_sched_barrier(0);
+    if (threadIdx.x == 0 && readers_before == gridDim.x - 1) {
+        a.opt_rw->step_count = own.step_count;
+        if (a.trace) trace_step(a.trace, a.gf, &own, a.scaler ? a.scaler->scale : 0.0);
+        __hip_atomic_store(&a.opt_rw->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 #define NBO_UPDATE_KERNEL(name, ST, KIND)                                                   \
     extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboUpdateArgs a) \
     {                                                                                       \
@@ -629,6 +687,34 @@ NBO_UPDATE_KERNEL(nbo_update_f16_sgd, NBO_F16, NBO_SGD)
 NBO_UPDATE_KERNEL(nbo_update_pf16_adamw, NBO_PF16, NBO_ADAMW)
 NBO_UPDATE_KERNEL(nbo_update_pf16_adam, NBO_PF16, NBO_ADAM)
 NBO_UPDATE_KERNEL(nbo_update_pf16_sgd, NBO_PF16, NBO_SGD)
+
+// Adam / AdamW launches that prepare their own scalars: the unfused Optimizer::step (one launch
+// per call, as the reference's one call) and every group of a grouped fused step.
+#define NBO_UPDATE_SELF_KERNEL(name, ST, KIND)                                              \
+    extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboUpdateArgs a)     \
+    {                                                                                       \
+        update_body<ST, KIND, true>(a);                                                     \
+    }
+NBO_UPDATE_SELF_KERNEL(nbo_update_f32_adamw_self, NBO_F32, NBO_ADAMW)
+NBO_UPDATE_SELF_KERNEL(nbo_update_f32_adam_self, NBO_F32, NBO_ADAM)
+NBO_UPDATE_SELF_KERNEL(nbo_update_bf16_adamw_self, NBO_BF16, NBO_ADAMW)
+NBO_UPDATE_SELF_KERNEL(nbo_update_bf16_adam_self, NBO_BF16, NBO_ADAM)
+NBO_UPDATE_SELF_KERNEL(nbo_update_f64_adamw_self, NBO_F64, NBO_ADAMW)
+NBO_UPDATE_SELF_KERNEL(nbo_update_f64_adam_self, NBO_F64, NBO_ADAM)
+NBO_UPDATE_SELF_KERNEL(nbo_update_f16_adamw_self, NBO_F16, NBO_ADAMW)
+NBO_UPDATE_SELF_KERNEL(nbo_update_f16_adam_self, NBO_F16, NBO_ADAM)
+NBO_UPDATE_SELF_KERNEL(nbo_update_pbf16_adamw_self, NBO_PBF16, NBO_ADAMW)
+NBO_UPDATE_SELF_KERNEL(nbo_update_pbf16_adam_self, NBO_PBF16, NBO_ADAM)
+NBO_UPDATE_SELF_KERNEL(nbo_update_pf16_adamw_self, NBO_PF16, NBO_ADAMW)
+NBO_UPDATE_SELF_KERNEL(nbo_update_pf16_adam_self, NBO_PF16, NBO_ADAM)
+// SGD has no step_count; inside a grouped fused step its group still needs the skip decision and
+// a trace entry
+NBO_UPDATE_SELF_KERNEL(nbo_update_f32_sgd_self, NBO_F32, NBO_SGD)
+NBO_UPDATE_SELF_KERNEL(nbo_update_bf16_sgd_self, NBO_BF16, NBO_SGD)
+NBO_UPDATE_SELF_KERNEL(nbo_update_f64_sgd_self, NBO_F64, NBO_SGD)
+NBO_UPDATE_SELF_KERNEL(nbo_update_f16_sgd_self, NBO_F16, NBO_SGD)
+NBO_UPDATE_SELF_KERNEL(nbo_update_pbf16_sgd_self, NBO_PBF16, NBO_SGD)
+NBO_UPDATE_SELF_KERNEL(nbo_update_pf16_sgd_self, NBO_PF16, NBO_SGD)
 
 // ---------------------------------------------------------------------------------
 // Deterministic block reduction: xor-butterfly inside each 64-lane wavefront, then
@@ -1324,16 +1410,6 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_cast_list(const NboC
     else cast_from<NBO_F64>(a);
 }
 
-// Plain streaming copy used only to calibrate the HBM byte counters of a profile
-// against a transfer of known size.
-extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_copy_f32x4(const f32x4 *src, f32x4 *dst,
-                                                                      uint64_t nvec)
-{
-    const uint64_t stride = (uint64_t)gridDim.x * NBO_BLOCK;
-    for (uint64_t i = (uint64_t)blockIdx.x * NBO_BLOCK + threadIdx.x; i < nvec; i += stride)
-        __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
-}
-
 // Zero-fill of an arbitrary byte range: single bytes up to the first 16-byte boundary,
 // 128-bit stores for the body, single bytes for the rest.  Takes the place of
 // hipMemsetAsync so that everything the library enqueues is a kernel launch (a caller
@@ -1377,63 +1453,3 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_probe_rmw2(f32x4 *a,
         __builtin_nontemporal_store(vb[u] + 1.0f, b + i);
     }
 }
-
-// ---------------------------------------------------------------------------------
-// Memory-system ceilings.  One workgroup per 32 KiB window of every stream (8 rows of
-// NBO_BLOCK 128-bit vectors, the update kernel's own access shape), over RO read-only streams,
-// RMW streams that are read and rewritten in place, and WO write-only streams; all loads are
-// issued before the first use.  What a pure read, a pure fill, a copy and an N-stream
-// read-modify-write reach on a given placement of the buffers is what the update kernel's
-// throughput is judged against.  The host launches nvec / (8 * NBO_BLOCK) workgroups, so no
-// access leaves [0, nvec) of any stream.
-template <int RO, int RMW, int WO> DEV void stream_probe_body(const NboStreamProbeArgs &a)
-{
-    enum { ROWS = 8, NLOAD = RO + RMW };
-    const uint64_t c0 = (uint64_t)blockIdx.x * (ROWS * NBO_BLOCK) + threadIdx.x;
-    f32x4 x[NLOAD > 0 ? NLOAD : 1][ROWS];
-    // stream after stream, all rows of a stream back to back: the order the update kernels use
-#pragma unroll
-    for (int s = 0; s < NLOAD; s++)
-#pragma unroll
-        for (int u = 0; u < ROWS; u++)
-            x[s][u] = __builtin_nontemporal_load(GLOBAL_PTR(const f32x4, a.buf[s]) + c0 + u * NBO_BLOCK);
-    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-    for (int s = 0; s < RO; s++)
-#pragma unroll
-        for (int u = 0; u < ROWS; u++) acc = acc + x[s][u];
-#pragma unroll
-    for (int s = RO; s < NLOAD; s++)
-#pragma unroll
-        for (int u = 0; u < ROWS; u++) x[s][u] = x[s][u] + 1.0f;
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int s = RO; s < NLOAD; s++)
-#pragma unroll
-        for (int u = 0; u < ROWS; u++)
-            __builtin_nontemporal_store(x[s][u], GLOBAL_PTR(f32x4, a.buf[s]) + c0 + u * NBO_BLOCK);
-#pragma unroll
-    for (int s = NLOAD; s < NLOAD + WO; s++)
-#pragma unroll
-        for (int u = 0; u < ROWS; u++)
-            __builtin_nontemporal_store(acc, GLOBAL_PTR(f32x4, a.buf[s]) + c0 + u * NBO_BLOCK);
-    // keeps the read-only loads alive without ever storing: the sum of finite inputs is not NaN
-    if (RO > 0 && WO == 0 && acc.x != acc.x) *GLOBAL_PTR(float, a.buf[0]) = acc.y + acc.z + acc.w;
-}
-
-// one kernel per pattern, so that each has the register budget (and occupancy) of its own shape
-#define NBO_STREAM_PROBE_KERNEL(name, RO, RMW, WO)                                                     \
-    extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboStreamProbeArgs a)           \
-    {                                                                                                  \
-        stream_probe_body<RO, RMW, WO>(a);                                                             \
-    }
-NBO_STREAM_PROBE_KERNEL(nbo_probe_read1, 1, 0, 0)
-NBO_STREAM_PROBE_KERNEL(nbo_probe_read3, 3, 0, 0)
-NBO_STREAM_PROBE_KERNEL(nbo_probe_fill1, 0, 0, 1)
-NBO_STREAM_PROBE_KERNEL(nbo_probe_fill3, 0, 0, 3)
-NBO_STREAM_PROBE_KERNEL(nbo_probe_copy, 1, 0, 1)
-NBO_STREAM_PROBE_KERNEL(nbo_probe_rmw1, 0, 1, 0)
-NBO_STREAM_PROBE_KERNEL(nbo_probe_rmw2s, 0, 2, 0)
-NBO_STREAM_PROBE_KERNEL(nbo_probe_rmw3, 0, 3, 0)
-NBO_STREAM_PROBE_KERNEL(nbo_probe_rmw6, 0, 6, 0)
-NBO_STREAM_PROBE_KERNEL(nbo_probe_r1_rmw3_w1, 1, 3, 1)

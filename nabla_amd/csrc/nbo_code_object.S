@@ -1,11 +1,10 @@
-/* Embeds the device-only gfx950 code object into the host library, so that the
- * shared object is self-contained: hipModuleLoadData reads it from here. */
+/* Embeds a device-only gfx950 code object into the host library, so that the shared object
+ * is self-contained: hipModuleLoadData reads it from here.  Assembled once per code object
+ * with NBO_CODE_OBJECT_PATH and NBO_CODE_OBJECT_SYMBOL set. */
     .section .rodata
-    .global nbo_code_object
-    .global nbo_code_object_end
+    .global NBO_CODE_OBJECT_SYMBOL
     .balign 4096
-nbo_code_object:
+NBO_CODE_OBJECT_SYMBOL:
     .incbin NBO_CODE_OBJECT_PATH
-nbo_code_object_end:
     .byte 0
     .section .note.GNU-stack,"",@progbits

@@ -80,6 +80,11 @@ struct NboOptimDev {
     float wd_lr_t; // T::from_f64(weight_decay * lr) for T = f32 (bf16 narrows it once more)
     double d_b1, d_omb1, d_b2, d_omb2, d_eps, d_ss, d_ibc2, d_omw;
     double d_neg_lr, d_momentum, d_wd;
+    // Counts the workgroups of a "_self" update launch that have read step_count; the one that
+    // brings it to the grid size knows that all have, advances step_count in place and puts the
+    // counter back to zero.  Zero between launches.
+    uint32_t ticket;
+    uint32_t pad;
 };
 
 // Hyper-parameters as the host holds them; handed to the device with every step so
@@ -134,6 +139,15 @@ struct NboUpdateArgs {
     // here and `opt` is not read, which saves the scalar-preparation launch
     uint32_t direct;
     double sgd_lr, sgd_momentum, sgd_weight_decay;
+    // The "_self" kernels prepare the step's scalars themselves (every workgroup, from
+    // opt->step_count, `hyper` and *gf); the workgroup that is the last to have read
+    // step_count (opt->ticket counts them) writes the advanced step_count back through opt_rw
+    // (= opt) and, if set, a trace entry (with the scaler's scale after its update).  Unused
+    // by the other kernels.
+    NboHyper hyper;
+    NboOptimDev *opt_rw;
+    NboTraceDev *trace;
+    const NboScalerDev *scaler;
 };
 
 struct NboFinalizeArgs {
@@ -267,7 +281,9 @@ enum {
 };
 
 struct NboStreamProbeArgs {
-    void *buf[8]; // streams in the order read-only, in place, write-only
+    void *buf[8];   // streams in the order read-only, in place, write-only
+    uint32_t iters;      // windows per workgroup, for the shapes whose workgroups loop
+    uint32_t contiguous; // those windows are neighbours (1) or a whole grid apart (0)
 };
 
 #endif

@@ -27,10 +27,32 @@ PATTERNS = [  # nbo_probe_pattern: name, streams read, rewritten in place, writt
     ("read-modify-write, 6 streams", 0, 6, 0), ("1 read + 3 read-modify-write + 1 written (update's shape)", 1, 3, 1)]
 
 
+SHAPES = [  # nbo_probe_shape
+    "the update kernels' own: 256 threads per 32 KiB window, 8 rows through registers",
+    "512-thread workgroups, 8 rows through registers (64 KiB windows)",
+    "1024-thread workgroups, 4 rows through registers (64 KiB windows)",
+    "loads straight into LDS (global_load_lds_dwordx4), 64 KiB of LDS per workgroup",
+    "loads straight into LDS, 128-144 KiB of LDS per workgroup",
+    "8 rows through registers + the 64 KiB of LDS rows, together in flight",
+    "512 threads: 4 waves only load (into LDS), 4 waves only store; double-buffered, 8 windows per workgroup",
+    "next window's loads issued before the current window's stores (2 x 4 rows in registers, 8 windows per workgroup)",
+    "shape 0's window, 8 of them per workgroup one after the other (nothing overlapped)",
+    "next window's loads global -> LDS while the current one (LDS -> registers) is stored; 256 threads, <= 64 KiB LDS",
+    "the same with 512 threads and twice the LDS",
+    "the same with 256 threads and twice the rows",
+    "shape 0's eight rows taken from 2 places of every stream at once (windows of 4 rows, a grid apart)",
+    "shape 0's eight rows taken from 4 places of every stream at once (windows of 2 rows)",
+    "shape 0's eight rows taken from 8 places of every stream at once (windows of 1 row)",
+]
+NEIGHBOURS = 0x80000000  # flag on a compare run's window count: the windows of a workgroup are neighbours
+FULL_PATTERNS = (4, 5, 7, 9)  # the 1:1 read/write patterns every shape exists for
+
+
 def measure_ceilings(gib: float = 2.0, reps: int = 10, patterns=None, settle_ms: int = 1500, spreads=(0, 1),
-                     quiet_s: float = 2.0):
+                     quiet_s: float = 2.0, shape: int = 0):
     """[(pattern name, spread, best GB/s, mean GB/s, regions, read:write)] over `patterns`
-    (indices into PATTERNS; default all), each with plain and with region-spread buffers.
+    (indices into PATTERNS; default all), each with plain and with region-spread buffers,
+    moved in access shape `shape` (index into SHAPES).
     Every measurement waits `quiet_s` before it allocates and then launches untimed for
     `settle_ms`: the driver clears freed device memory in the background, each measurement frees
     the previous one's buffers, and the placement search frees its spare chunks."""
@@ -51,10 +73,51 @@ def measure_ceilings(gib: float = 2.0, reps: int = 10, patterns=None, settle_ms:
             # the previous measurement's buffers have just been freed: the driver is still clearing
             # them, which would disturb the placement search's own short probes
             time.sleep(quiet_s)
-            _lib.check(L.nbo_hbm_ceiling(pat, spread, nbytes, reps, settle_ms, C.byref(best), C.byref(mean),
-                                         C.byref(regions)))
+            _lib.check(L.nbo_hbm_ceiling_shape(pat, shape, spread, nbytes, reps, settle_ms, C.byref(best),
+                                               C.byref(mean), C.byref(regions), None))
             out.append((name, spread, best.value, mean.value, regions.value, f"{ro + rmw}:{rmw + wo}"))
     return out
+
+
+def compare_shapes(pattern: int, shapes, iters=None, gib: float = 2.0, rounds: int = 5, reps: int = 5,
+                   settle_ms: int = 1500, spread: int = 1):
+    """Mean and best GB/s of several access shapes over the SAME buffers, measured in turn
+    `rounds` times (`nbo_hbm_ceiling_compare`): [(shape, iters, mean, best)], regions."""
+    from . import _lib
+
+    _lib.init()
+    L = _lib.load()
+    n = len(shapes)
+    iters = list(iters) if iters is not None else [0] * n
+    nbytes = int(gib * (1 << 30)) // 32768 * 32768
+    best, mean, regions = (C.c_double * n)(), (C.c_double * n)(), C.c_int()
+    _lib.check(L.nbo_hbm_ceiling_compare(pattern, n, (C.c_int * n)(*shapes), (C.c_uint32 * n)(*iters), spread, nbytes,
+                                         rounds, reps, settle_ms, best, mean, C.byref(regions)))
+    return [(shapes[k], iters[k], mean[k], best[k]) for k in range(n)], regions.value
+
+
+def compare_main(args) -> None:
+    """Every access shape over the same buffers, for the four 1:1 read/write patterns."""
+    import time
+
+    runs = [(sh, 0) for sh in range(len(SHAPES))] + [(7, 2), (7, 4), (7, 32), (8, 2), (9, 32),
+                                                       (7, 2 | NEIGHBOURS), (7, 8 | NEIGHBOURS), (8, 2 | NEIGHBOURS)]
+    print(f"{args.gib} GiB per stream; per pattern all shapes share one set of buffers (placed across regions; a "
+          f"single stream: one plain allocation) and are measured in turn, {args.rounds} rounds of {args.reps} "
+          "launches each; mean (best) GB/s\n")
+    print("| shape (windows per workgroup) | " + " | ".join(PATTERNS[p][0] for p in FULL_PATTERNS) + " |")
+    print("|---|" + "---|" * len(FULL_PATTERNS))
+    cols = []
+    for pat in FULL_PATTERNS:
+        time.sleep(2.0)
+        single = sum(PATTERNS[pat][1:]) < 2
+        rows, _ = compare_shapes(pat, [r[0] for r in runs], [r[1] for r in runs], args.gib, args.rounds, args.reps,
+                                 spread=0 if single else 1)
+        cols.append(rows)
+    for k, (sh, it) in enumerate(runs):
+        label = f"{sh}: {SHAPES[sh]}" + (f" [{it & ~NEIGHBOURS} windows per workgroup"
+                                         f"{', neighbours' if it & NEIGHBOURS else ''}]" if it else "")
+        print(f"| {label} | " + " | ".join(f"{c[k][2]:.0f} ({c[k][3]:.0f})" for c in cols) + " |", flush=True)
 
 
 def ceilings_main(args) -> None:
@@ -62,14 +125,27 @@ def ceilings_main(args) -> None:
           "written per launch / duration\n")
     print("| pattern | read : written streams | buffers | regions | best GB/s | mean GB/s |")
     print("|---|---|---|---|---|---|")
-    rows = measure_ceilings(args.gib, args.reps)
+    rows = [] if args.shapes_only else measure_ceilings(args.gib, args.reps)
     for name, spread, best, mean, regions, rw in rows:
         where = "across regions" if spread else "one plain allocation"
         print(f"| {name} | {rw} | {where} | {regions if spread else '-'} | {best:.0f} | {mean:.0f} |", flush=True)
     one_to_one = [r for r in rows if r[5] in ("1:1", "2:2", "3:3", "6:6", "4:4")]
-    top = max(one_to_one, key=lambda r: r[3])
-    print(f"\nBest 1:1 read/write rate: {top[3]:.0f} GB/s mean ({top[2]:.0f} best launch), {top[0]}, "
-          f"{'across regions' if top[1] else 'one plain allocation'}.")
+    if one_to_one:
+        top = max(one_to_one, key=lambda r: r[3])
+        print(f"\nBest 1:1 read/write rate: {top[3]:.0f} GB/s mean ({top[2]:.0f} best launch), {top[0]}, "
+              f"{'across regions' if top[1] else 'one plain allocation'}.")
+    print("\nOther access shapes over the 1:1 read/write patterns, streams placed across regions (a single "
+          "stream: one plain allocation):\n")
+    print("| shape | " + " | ".join(PATTERNS[p][0] for p in FULL_PATTERNS) + " |")
+    print("|---|" + "---|" * len(FULL_PATTERNS))
+    for shape in range(len(SHAPES)):
+        cells = []
+        for pat in FULL_PATTERNS:
+            single = sum(PATTERNS[pat][1:]) < 2  # one stream: nothing to spread it against
+            r = measure_ceilings(args.gib, args.reps, patterns=(pat,), spreads=(0,) if single else (1,), shape=shape)[0]
+            cells.append(f"{r[3]:.0f} ({r[2]:.0f})")
+        print(f"| {shape}: {SHAPES[shape]} | " + " | ".join(cells) + " |", flush=True)
+    print("\nmean (best) GB/s")
 
 
 def main() -> None:
@@ -78,6 +154,11 @@ def main() -> None:
     ap.add_argument("--reps", type=int, default=None)
     ap.add_argument("--ceilings", action="store_true", help="measure the memory system's ceilings instead")
     ap.add_argument("--gib", type=float, default=2.0, help="--ceilings: GiB per stream")
+    ap.add_argument("--shapes-only", action="store_true", help="--ceilings: only the table of access shapes")
+    ap.add_argument("--compare", action="store_true",
+                    help="all access shapes over the same buffers, measured in turn (differences of a per cent "
+                         "show here; --ceilings allocates anew for every row)")
+    ap.add_argument("--rounds", type=int, default=5, help="--compare: rounds over all shapes")
     ap.add_argument("--summarize", metavar="DIR", help="turn the rocprofv3 output under DIR into profiles/ summaries "
                                                         "(see nabla_amd/profile_summary.py) instead of measuring")
     args = ap.parse_args()
@@ -85,6 +166,10 @@ def main() -> None:
         from . import profile_summary
 
         profile_summary.main(args.summarize)
+        return
+    if args.compare:
+        args.reps = args.reps or 5
+        compare_main(args)
         return
     if args.ceilings:
         args.reps = args.reps or 10
@@ -173,7 +258,7 @@ def main() -> None:
     timeit("Sgd::step f32, momentum", lambda: sgdm.step(pl, gl), 20, "nbo_update_f32_sgd")
     del sgdm
     adam = nb.Adam.new(1e-3, shapes)
-    timeit("Adam::step f32", lambda: adam.step(pl, gl), 28, "nbo_update_f32_adam")
+    timeit("Adam::step f32", lambda: adam.step(pl, gl), 28, "nbo_update_f32_adam_self")
     del adam, pl, gl, p, g
 
 

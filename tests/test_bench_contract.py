@@ -80,9 +80,11 @@ def test_kernel_bench_prints_a_row_for_every_measurement(gpu):
 @pytest.mark.gpu
 def test_every_ceiling_probe_runs_and_reports_a_rate(gpu):
     """`nbo_hbm_ceiling` for every access pattern, in one plain allocation and across the HBM's
-    regions, on streams of 192 MiB: a positive rate below the nominal peak, best >= mean, and the
-    argument checks of the entry point."""
+    regions, on streams of 192 MiB: a finite positive rate, best >= mean, and the argument checks
+    of the entry point.  (No bounds on the rate itself: 192 MiB fits the last-level cache, and a
+    shared or throttled GPU may be slow; rates are what `kernel_bench --ceilings` reports.)"""
     import ctypes as C
+    import math
 
     from nabla_amd import _lib
     from nabla_amd import kernel_bench as KB
@@ -93,7 +95,7 @@ def test_every_ceiling_probe_runs_and_reports_a_rate(gpu):
         for spread in (0, 1):
             best, mean, regions = C.c_double(), C.c_double(), C.c_int(-1)
             _lib.check(L.nbo_hbm_ceiling(pat, spread, nbytes, 3, 5, C.byref(best), C.byref(mean), C.byref(regions)))
-            assert 500.0 < mean.value <= best.value < 8000.0, (name, spread, best.value, mean.value)
+            assert math.isfinite(best.value) and 0.0 < mean.value <= best.value, (name, spread, best.value, mean.value)
             assert regions.value in ((0, 2, 3) if spread else (0,)), (name, spread, regions.value)
     best, mean = C.c_double(), C.c_double()
     for bad in (lambda: L.nbo_hbm_ceiling(len(KB.PATTERNS), 0, nbytes, 3, 0, C.byref(best), C.byref(mean), None),
@@ -101,3 +103,33 @@ def test_every_ceiling_probe_runs_and_reports_a_rate(gpu):
                 lambda: L.nbo_hbm_ceiling(0, 0, nbytes, 0, 0, C.byref(best), C.byref(mean), None),
                 lambda: L.nbo_hbm_ceiling(0, 0, nbytes, 3, 0, None, C.byref(mean), None)):
         assert bad() == _lib.ERR_ARG
+
+
+@pytest.mark.gpu
+def test_every_probe_shape_touches_each_vector_exactly_once_per_launch(gpu):
+    """`nbo_hbm_ceiling_shape`: every access shape (register rows, LDS-direct loads, both at once,
+    loading and storing waves apart, software-pipelined) over the four 1:1 read/write patterns.
+    The in-place streams start at zero and every launch adds 1.0 to each element, so after the
+    run every element must equal the number of launches: a window that was skipped, done twice
+    or written to the wrong place shows as a mismatch."""
+    import ctypes as C
+    import math
+
+    from nabla_amd import _lib
+    from nabla_amd import kernel_bench as KB
+
+    L = _lib.load()
+    nbytes = 48 << 20
+    for shape in range(len(KB.SHAPES)):
+        for pat in KB.FULL_PATTERNS:
+            print(f"probe shape {shape} pattern {pat}", flush=True)
+            best, mean, regions, bad = C.c_double(), C.c_double(), C.c_int(-1), C.c_uint64(1 << 60)
+            _lib.check(L.nbo_hbm_ceiling_shape(pat, shape, 0, nbytes, 2, 0, C.byref(best), C.byref(mean),
+                                               C.byref(regions), C.byref(bad)))
+            assert bad.value == 0, (shape, pat, bad.value)
+            assert math.isfinite(best.value) and 0.0 < mean.value <= best.value, (shape, pat)
+    best, mean = C.c_double(), C.c_double()
+    for bad_call in (lambda: L.nbo_hbm_ceiling_shape(0, 3, 0, nbytes, 2, 0, C.byref(best), C.byref(mean), None, None),
+                     lambda: L.nbo_hbm_ceiling_shape(9, len(KB.SHAPES), 0, nbytes, 2, 0, C.byref(best), C.byref(mean), None, None),
+                     lambda: L.nbo_hbm_ceiling_shape(9, 6, 0, 32768, 2, 0, C.byref(best), C.byref(mean), None, None)):
+        assert bad_call() == _lib.ERR_ARG

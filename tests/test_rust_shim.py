@@ -8,6 +8,7 @@ import re
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "nabla_optim.h")
+BENCH_HEADER = os.path.join(ROOT, "include", "nabla_optim_bench.h")
 FFI = os.path.join(ROOT, "integration", "rust", "ffi.rs")
 MOD = os.path.join(ROOT, "integration", "rust", "mod.rs")
 
@@ -29,7 +30,7 @@ def _rust_kind(ty: str) -> str:
 
 
 def _header_decls():
-    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read() + open(BENCH_HEADER).read(), flags=re.S)
     out = {}
     for ret, name, args in re.findall(r"\b(int|const char \*)\s*(nbo_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text):
         args = args.strip()
