@@ -174,7 +174,7 @@ public:
     }
     // the Trainer tail with one unscale / found-inf / clip decision over all gradients
     void fused_step(const std::vector<Tensor> &params, const std::vector<Tensor> &grads, GradScaler *scaler,
-                    double max_norm, bool zero_grads = false)
+                    double max_norm, bool zero_grads = false, bool zero_on_skip = false)
     {
         bind(params, grads);
         if (!all_grads_ || all_key_ != key_of(grads)) {
@@ -190,7 +190,7 @@ public:
         }
         check(nbo_fused_step_groups(groups_.size(), opts.data(), pl.data(), gl.data(),
                                     scaler ? scaler->handle() : nullptr, all_grads_->handle(), max_norm,
-                                    zero_grads ? NBO_STEP_ZERO_GRADS : 0u));
+                                    (zero_grads ? NBO_STEP_ZERO_GRADS : 0u) | (zero_on_skip ? NBO_STEP_ZERO_ON_SKIP : 0u)));
     }
     // the same over gradients whose sum of squares is already known (nbo_unscale_accumulate)
     void fused_step_norm(const std::vector<Tensor> &params, const std::vector<Tensor> &grads, double sumsq,

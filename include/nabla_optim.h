@@ -203,6 +203,8 @@ int nbo_scale_grad(nbo_list *grads, double factor);
 
 #define NBO_STEP_ZERO_GRADS 1u     /* trainer.rs:285-290 folded into the update */
 #define NBO_STEP_SKIP_NONFINITE 2u /* GradNanPolicy::Skip (trainer.rs:239-245) without a scaler */
+#define NBO_STEP_ZERO_ON_SKIP 4u   /* a skipped step leaves zeros in the gradients, as unscale_and_update
+                                      does when it finds inf / NaN (optim/core.rs:372-375) */
 
 /* One Trainer iteration after backward (trainer.rs:230-291) in three launches:
  *   scaler.unscale_and_update(grads)  -> found_inf, skip, scale update
@@ -213,7 +215,10 @@ int nbo_scale_grad(nbo_list *grads, double factor);
  * `scaler` may be NULL.  Gradients are not modified (except for the optional
  * zeroing): the two factors are applied inside the update, element by element,
  * with the same roundings as the reference's in-place passes.  The skip decision
- * is taken on the device; nothing is read back.  Asynchronous. */
+ * is taken on the device; nothing is read back.  On a skipped step the reference's
+ * unscale_and_update replaces the gradients by zeros (core.rs:372-375); this call does that
+ * with NBO_STEP_ZERO_ON_SKIP (or NBO_STEP_ZERO_GRADS, which zeroes after every step) and
+ * otherwise leaves them as they are, inf / NaN included.  Asynchronous. */
 int nbo_fused_step(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, nbo_list *grads,
                    double max_norm, uint32_t flags);
 /* nbo_fused_step for callers that cannot allocate device memory: code under HIP graph

@@ -220,11 +220,12 @@ public:
 
     // the Trainer tail (trainer.rs:230-291) in one asynchronous call
     void fused_step(TensorList &params, TensorList &grads, GradScaler *scaler, double max_norm,
-                    bool zero_grads = false, bool skip_nonfinite = false)
+                    bool zero_grads = false, bool skip_nonfinite = false, bool zero_on_skip = false)
     {
         check(nbo_fused_step(handle(), scaler ? scaler->handle() : nullptr, params.handle(), grads.handle(),
                              max_norm,
-                             (zero_grads ? NBO_STEP_ZERO_GRADS : 0u) | (skip_nonfinite ? NBO_STEP_SKIP_NONFINITE : 0u)));
+                             (zero_grads ? NBO_STEP_ZERO_GRADS : 0u) | (skip_nonfinite ? NBO_STEP_SKIP_NONFINITE : 0u) |
+                                 (zero_on_skip ? NBO_STEP_ZERO_ON_SKIP : 0u)));
     }
     // clip + step (+ zeroing) over gradients whose sum of squares is already known
     void fused_step_norm(TensorList &params, TensorList &grads, double sumsq, double max_norm, bool zero_grads = false)

@@ -21,6 +21,7 @@ pub const NBO_DT_F32: c_int = 0; pub const NBO_DT_BF16: c_int = 1; pub const NBO
 pub const NBO_DT_F16: c_int = 3;
 pub const NBO_KIND_ADAMW: i32 = 0; pub const NBO_KIND_ADAM: i32 = 1; pub const NBO_KIND_SGD: i32 = 2;
 pub const NBO_STEP_ZERO_GRADS: u32 = 1; pub const NBO_STEP_SKIP_NONFINITE: u32 = 2;
+pub const NBO_STEP_ZERO_ON_SKIP: u32 = 4;
 pub const NBO_ACC_CHECK_FINITE: u32 = 1; pub const NBO_ACC_WRITE_GRADS: u32 = 2;
 // nbo_status
 pub const NBO_OK: c_int = 0; pub const NBO_ERR_LEN_MISMATCH: c_int = 1; pub const NBO_ERR_COUNT_MISMATCH: c_int = 2;

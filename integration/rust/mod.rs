@@ -532,7 +532,8 @@ impl<T: Scalar> MiAdamW<T> {
     /// The Trainer's tail after backward (`trainer.rs:230-291`) in three launches: unscale +
     /// found-inf + loss-scale update, clip, step, optional zeroing of the gradients; a
     /// non-finite gradient skips the step on the device.  Nothing is read back; `last_step`
-    /// tells what was decided.
+    /// tells what was decided.  A skipped step leaves zeros in the gradients, as
+    /// `GradScaler::unscale_and_update` does (`optim/core.rs:372-375`).
     pub fn fused_step(&mut self, scaler: Option<&mut MiGradScaler>, params: &mut [&mut Tensor<T, Hip>],
                       grads: &[&Tensor<T, Hip>], max_norm: f64, zero_grads: bool) {
         let e = self.e.get_mut();
@@ -541,7 +542,7 @@ impl<T: Scalar> MiAdamW<T> {
         let p = e.params.get(&p_refs);
         let g = e.grads.get(grads);
         let s = scaler.map_or(ptr::null_mut(), |s| s.h);
-        let flags = if zero_grads { ffi::NBO_STEP_ZERO_GRADS } else { 0 };
+        let flags = ffi::NBO_STEP_ZERO_ON_SKIP | if zero_grads { ffi::NBO_STEP_ZERO_GRADS } else { 0 };
         check(unsafe { ffi::nbo_fused_step(h, s, p, g, max_norm, flags) });
     }
 

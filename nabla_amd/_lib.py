@@ -35,6 +35,7 @@ KIND_ADAMW, KIND_ADAM, KIND_SGD = 0, 1, 2
 
 STEP_ZERO_GRADS = 1
 STEP_SKIP_NONFINITE = 2
+STEP_ZERO_ON_SKIP = 4
 ACC_CHECK_FINITE = 1
 ACC_WRITE_GRADS = 2
 

@@ -80,8 +80,14 @@ void check_step_args(const nbo_optim *opt, const nbo_list *params, const nbo_lis
     }
 }
 
+// which of a fused step's flags ask the update kernel to write zeros over the gradients
+uint32_t zero_mode(uint32_t flags)
+{
+    return ((flags & NBO_STEP_ZERO_GRADS) ? 1u : 0u) | ((flags & NBO_STEP_ZERO_ON_SKIP) ? 2u : 0u);
+}
+
 NboUpdateArgs update_args(nbo_optim *opt, nbo_list *params, nbo_list *grads, bool with_gf,
-                          bool zero_grads, const NboGradFactors *shared_gf = nullptr)
+                          uint32_t zero_grads, const NboGradFactors *shared_gf = nullptr)
 {
     NboUpdateArgs a = {};
     a.L = opt->layout.dev;
@@ -90,7 +96,7 @@ NboUpdateArgs update_args(nbo_optim *opt, nbo_list *params, nbo_list *grads, boo
     a.arena = opt->arena;
     a.opt = opt->dev;
     a.gf = shared_gf ? shared_gf : with_gf ? opt->gf : nullptr;
-    a.zero_grads = zero_grads ? 1u : 0u;
+    a.zero_grads = zero_grads;
     return a;
 }
 
@@ -121,7 +127,7 @@ int self_update_kernel(const nbo_optim *opt, const nbo_list *params)
 // skipped) and writes the trace entry.  Not for an empty list: no workgroup would run.
 bool self_update_possible(const nbo_optim *opt) { return opt->layout.nchunks > 0; }
 
-void launch_self_update(nbo_optim *opt, nbo_list *params, nbo_list *grads, const NboGradFactors *gf, bool zero_grads,
+void launch_self_update(nbo_optim *opt, nbo_list *params, nbo_list *grads, const NboGradFactors *gf, uint32_t zero_grads,
                         NboTraceDev *trace, const NboScalerDev *scaler)
 {
     NboUpdateArgs a = update_args(opt, params, grads, false, zero_grads, gf);
@@ -200,7 +206,7 @@ void fused_step_launches(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, n
     f.max_norm = max_norm;
     f.hyper = hyper_of(opt);
     launch_norm(grads, scaler ? scaler->dev : nullptr, pure_half(opt), ws, f);
-    NboUpdateArgs a = update_args(opt, params, grads, true, (flags & NBO_STEP_ZERO_GRADS) != 0);
+    NboUpdateArgs a = update_args(opt, params, grads, true, zero_mode(flags));
     rt.launch_raw(update_kernel(opt, params), opt->layout.nchunks, NBO_BLOCK, &a, ws.may_time);
 }
 
@@ -535,7 +541,7 @@ int nbo_optim_step(nbo_optim *opt, nbo_list *params, nbo_list *grads)
     return guarded([&] {
         check_step_args(opt, params, grads);
         Runtime &rt = Runtime::get();
-        NboUpdateArgs a = update_args(opt, params, grads, false, false);
+        NboUpdateArgs a = update_args(opt, params, grads, false, 0u);
         if (opt->meta.kind == NBO_KIND_SGD) {
             // no step_count, no skip: one launch, scalars in the argument block
             a.direct = 1;
@@ -544,7 +550,7 @@ int nbo_optim_step(nbo_optim *opt, nbo_list *params, nbo_list *grads)
             a.sgd_weight_decay = opt->meta.weight_decay;
         } else if (self_update_possible(opt)) {
             // Adam::step / AdamW::step is one call (alg.rs:109-150, 254-291): one launch
-            launch_self_update(opt, params, grads, nullptr, false, nullptr, nullptr);
+            launch_self_update(opt, params, grads, nullptr, 0u, nullptr, nullptr);
             return;
         } else {
             NboPrepArgs p = {};
@@ -892,7 +898,7 @@ static void launch_group_updates(uint64_t n_groups, nbo_optim *const *opts, nbo_
     for (uint64_t g = 0; g < n_groups; g++) {
         if (self_update_possible(opts[g])) {
             // one launch per group: it derives the group's scalars from the shared decision itself
-            launch_self_update(opts[g], params[g], grads[g], rt.gf_scratch(), (flags & NBO_STEP_ZERO_GRADS) != 0,
+            launch_self_update(opts[g], params[g], grads[g], rt.gf_scratch(), zero_mode(flags),
                                opts[g]->trace, scaler ? scaler->dev : nullptr);
             continue;
         }
@@ -904,7 +910,7 @@ static void launch_group_updates(uint64_t n_groups, nbo_optim *const *opts, nbo_
         p.hyper = hyper_of(opts[g]);
         rt.launch(K_PREP, 1, 64, p);
         const NboUpdateArgs a = update_args(opts[g], params[g], grads[g], true,
-                                            (flags & NBO_STEP_ZERO_GRADS) != 0, rt.gf_scratch());
+                                            zero_mode(flags), rt.gf_scratch());
         rt.launch(update_kernel(opts[g], params[g]), opts[g]->layout.nchunks, NBO_BLOCK, a);
     }
 }
@@ -1029,7 +1035,7 @@ int nbo_fused_step_norm(nbo_optim *opt, nbo_list *params, nbo_list *grads, doubl
         f.hyper = hyper_of(opt);
         rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
         const NboUpdateArgs a =
-            update_args(opt, params, grads, true, (flags & NBO_STEP_ZERO_GRADS) != 0);
+            update_args(opt, params, grads, true, zero_mode(flags));
         rt.launch(update_kernel(opt, params), opt->layout.nchunks, NBO_BLOCK, a);
     });
 }

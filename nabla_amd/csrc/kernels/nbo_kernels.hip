@@ -523,15 +523,16 @@ template <int ST, int KIND> DEV void update_chunk(const NboUpdateArgs &a, const 
     T *am = state_part<T>(a.arena, c, 0);
     T *av = has_v ? state_part<T>(a.arena, c, a.arena.part_v) : nullptr;
     T *aw = mixed ? state_part<T>(a.arena, c, a.arena.part_w) : nullptr;
-    const bool zero_g = a.zero_grads != 0;
+    const bool zero_g = (a.zero_grads & 1u) != 0;
     const uint32_t vbytes = VEC * SB;
     const bool vec_ok = ((((uintptr_t)pp) | ((uintptr_t)pg)) & (vbytes - 1)) == 0;
 
     const bool direct = KIND == NBO_SGD && a.direct != 0;
     if (!direct && o->skip) {
         // found_inf: parameters, moments and step_count stay untouched
-        // (trainer.rs:230-236); the gradients become zeros (core.rs:372-375).
-        if (zero_g)
+        // (trainer.rs:230-236); the gradients become zeros (core.rs:372-375) if the caller
+        // asked for zeroing, after every step or after a skipped one only.
+        if (a.zero_grads != 0)
             for (uint32_t i = tid; i < c.cnt; i += NBO_BLOCK) IO<ST>::st1(pg + (uint64_t)i * SB, (T)0);
         return;
     }

@@ -133,7 +133,8 @@ struct NboUpdateArgs {
     NboArenaDev arena;
     const NboOptimDev *opt;
     const NboGradFactors *gf; // null: gradients are used as they are
-    uint32_t zero_grads;      // write zeros over the gradients after reading them
+    uint32_t zero_grads;      // bit 0: write zeros over the gradients after reading them (and on a skipped
+                              // step); bit 1: on a skipped step only (core.rs:372-375)
     // SGD outside the fused tail needs no device-side state at all (it has no
     // step_count and cannot be skipped): with `direct` set its three scalars come from
     // here and `opt` is not read, which saves the scalar-preparation launch

@@ -198,7 +198,7 @@ class GroupOptimizer:
             g.optimizer.step(self._lists(g, "p", params), self._lists(g, "g", grads))
 
     def fused_step(self, params, grads, scaler: Optional[GradScaler] = None, max_norm: float = 0.0,
-                   zero_grads: bool = False, skip_nonfinite: bool = False) -> None:
+                   zero_grads: bool = False, skip_nonfinite: bool = False, zero_on_skip: bool = False) -> None:
         """The Trainer tail with one unscale / clip decision over all gradients."""
         self._check(params, grads)
         all_grads = self._all_grads.get("g", list(grads))
@@ -206,7 +206,8 @@ class GroupOptimizer:
         opts = (C.c_void_p * n)(*[g.optimizer._handle() for g in self._groups])
         pl = (C.c_void_p * n)(*[self._lists(g, "p", params)._h for g in self._groups])
         gl = (C.c_void_p * n)(*[self._lists(g, "g", grads)._h for g in self._groups])
-        flags = (_lib.STEP_ZERO_GRADS if zero_grads else 0) | (_lib.STEP_SKIP_NONFINITE if skip_nonfinite else 0)
+        flags = ((_lib.STEP_ZERO_GRADS if zero_grads else 0) | (_lib.STEP_SKIP_NONFINITE if skip_nonfinite else 0)
+                 | (_lib.STEP_ZERO_ON_SKIP if zero_on_skip else 0))
         _call(_lib.load().nbo_fused_step_groups(n, opts, pl, gl, scaler._handle() if scaler else None,
                                                 all_grads._h, float(max_norm), flags))
 

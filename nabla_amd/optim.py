@@ -19,7 +19,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 
 from . import _lib
 from ._lib import (DT_BF16, DT_F16, DT_F32, DT_F64, KIND_ADAM, KIND_ADAMW, KIND_SGD, STEP_SKIP_NONFINITE,
-                   STEP_ZERO_GRADS, NablaOptimError)
+                   STEP_ZERO_GRADS, STEP_ZERO_ON_SKIP, NablaOptimError)
 
 
 class NablaPanic(AssertionError):
@@ -353,13 +353,16 @@ class _Optimizer:
     # -- the fused Trainer tail (trainer.rs:230-291) --------------------------------------
     def fused_step(self, params, grads, scaler: Optional["GradScaler"] = None,
                    max_norm: float = 0.0, zero_grads: bool = False,
-                   skip_nonfinite: bool = False, no_alloc: bool = False) -> None:
-        """`no_alloc=True` goes through nbo_fused_step_noalloc: same results, the norm pass's
+                   skip_nonfinite: bool = False, no_alloc: bool = False, zero_on_skip: bool = False) -> None:
+        """`zero_on_skip=True`: a skipped step leaves zeros in the gradients, as the reference's
+        `unscale_and_update` does when it finds inf / NaN (optim/core.rs:372-375).
+        `no_alloc=True` goes through nbo_fused_step_noalloc: same results, the norm pass's
         scratch comes from the library's statically allocated device array (pass TensorLists,
         or the same tensors as in an earlier call, so that no descriptor is built either)."""
         p = self._cache.get("p", params)
         g = self._cache.get("g", grads)
-        flags = (STEP_ZERO_GRADS if zero_grads else 0) | (STEP_SKIP_NONFINITE if skip_nonfinite else 0)
+        flags = ((STEP_ZERO_GRADS if zero_grads else 0) | (STEP_SKIP_NONFINITE if skip_nonfinite else 0)
+                 | (STEP_ZERO_ON_SKIP if zero_on_skip else 0))
         lib = _lib.load()
         fn = lib.nbo_fused_step_noalloc if no_alloc else lib.nbo_fused_step
         _call(fn(self._handle(), scaler._handle() if scaler else None, p._h, g._h, float(max_norm), flags))

@@ -84,7 +84,8 @@ def test_constants_agree_with_the_header():
         c_val = int(re.search(r"\b%s = (\d+)" % name, header).group(1))
         r_val = int(re.search(r"pub const %s: \w+ = (\d+);" % name, ffi).group(1))
         assert c_val == r_val, name
-    for name in ("NBO_STEP_ZERO_GRADS", "NBO_STEP_SKIP_NONFINITE", "NBO_ACC_CHECK_FINITE", "NBO_ACC_WRITE_GRADS"):
+    for name in ("NBO_STEP_ZERO_GRADS", "NBO_STEP_SKIP_NONFINITE", "NBO_STEP_ZERO_ON_SKIP", "NBO_ACC_CHECK_FINITE",
+                 "NBO_ACC_WRITE_GRADS"):
         c_val = int(re.search(r"#define %s (\d+)u" % name, header).group(1))
         r_val = int(re.search(r"pub const %s: u32 = (\d+);" % name, ffi).group(1))
         assert c_val == r_val, name
