@@ -131,6 +131,14 @@ def set_pow_mode(mode: int) -> None:
     lib().orc_set_pow_mode(int(mode))
 
 
+def set_clip_norm_override(norm: float) -> None:
+    """Test hook: norm >= 0 makes clip_grad_norm decide and scale with `norm` (its return value
+    stays the square root of its own serial sum); negative switches it off."""
+    L = lib()
+    L.orc_set_clip_norm_override.argtypes = [C.c_double]
+    L.orc_set_clip_norm_override(float(norm))
+
+
 def set_threads(n: int) -> None:
     lib().orc_set_threads(int(n))
 

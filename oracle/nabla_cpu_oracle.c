@@ -14,12 +14,19 @@
 
 static int g_pow_mode = ORC_POW_LIBM;
 static int g_threads = 1;
+/* Test hook: with a value >= 0, clip_grad_norm takes this as the norm instead of the square root
+ * of its own serial sum (which it still computes, and still returns).  The device adds the
+ * squares in a tree, so its norm can differ from the serial one in the last bits of the f64, and
+ * once in some thousand steps that changes the f32 clip factor; a parity test then repeats the
+ * oracle's step with the device's norm and still demands equal bits. */
+static double g_norm_override = -1.0;
 /* Below this many elements a pass is not worth forking threads for; the result
  * does not depend on it (every pass is element-wise). */
 #define PAR_MIN 32768L
 
 void orc_set_pow_mode(int mode) { g_pow_mode = mode == ORC_POW_SQRT ? ORC_POW_SQRT : ORC_POW_LIBM; }
 int orc_get_pow_mode(void) { return g_pow_mode; }
+void orc_set_clip_norm_override(double norm) { g_norm_override = norm; }
 void orc_set_threads(int n) { g_threads = n < 1 ? 1 : n; }
 int orc_get_threads(void) { return g_threads; }
 

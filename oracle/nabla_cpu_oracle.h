@@ -63,6 +63,10 @@ extern "C" {
 enum { ORC_POW_LIBM = 0, ORC_POW_SQRT = 1 };
 void orc_set_pow_mode(int mode);
 int orc_get_pow_mode(void);
+/* Test hook, not part of the reference: norm >= 0 makes every clip_grad_norm decide and scale
+ * with `norm` in the place of sqrt(its own serial sum); the return value stays its own norm.
+ * A negative value switches the hook off. */
+void orc_set_clip_norm_override(double norm);
 
 /* Worker threads for the passes the reference runs under rayon par_iter
  * (nabla-core/src/cpu/mod.rs:44-64,211-223,264-272).  Passes the reference runs

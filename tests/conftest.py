@@ -22,3 +22,21 @@ def gpu():
 
     _lib.init()
     return torch.device("cuda:0")
+
+
+def pytest_terminal_summary(terminalreporter, exitstatus, config):
+    """The counts the parity tests keep -- elements that needed the tolerance clause of the
+    parameter comparison, oracle steps that had to follow the device's norm -- belong in the
+    log of every run, captured output or not."""
+    try:
+        from tests import helpers as H
+    except Exception:
+        return
+    if not H.REPORT_LINES and not H.NORM_FOLLOWED["steps"]:
+        return
+    tr = terminalreporter
+    tr.section("parity: tolerance clause and norm differences")
+    for line in H.REPORT_LINES:
+        tr.write_line(line)
+    tr.write_line(f"[norm-follow] {H.NORM_FOLLOWED['events']} of {H.NORM_FOLLOWED['steps']} clipped-capable oracle "
+                  "steps had to be repeated with the device's norm")

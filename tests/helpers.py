@@ -124,6 +124,71 @@ def count_beyond_ulp_f32(a_list, b_list, tol):
     return n_bad, total
 
 
+# ---- what the tests report beyond pass / fail ---------------------------------------------------
+
+# Lines for pytest's terminal summary (tests/conftest.py prints them whether or not output is
+# captured): every use of the tolerance clause below, every oracle step that had to follow the
+# device's norm.
+REPORT_LINES = []
+
+
+def report(line):
+    REPORT_LINES.append(line)
+    print(line, flush=True)
+
+
+# ---- the one legitimate difference between the device's norm and the reference's ---------------
+
+NORM_FOLLOWED = {"steps": 0, "events": 0}
+
+
+def oracle_step_with_device_norm(step_fn, state_lists, scalars, max_norm, dev_info, what):
+    """Runs one oracle step, `step_fn() -> (ran, norm)`, next to a device step whose outcome is
+    `dev_info` (nbo_step_info).  The reference adds the squares of the gradients serially, the
+    device in a fixed tree: the two f64 norms agree to ~1e-13 relative but not always in the last
+    bit, and T(max_norm / norm) -- the factor every gradient is multiplied by -- can then differ
+    (about once in 10^4 clipped steps of a long list).  That difference is within the tolerance,
+    but everything after it stops being bit-comparable, so: if the factor (or the decision to
+    clip) differs, the oracle's state is put back and the step repeated with the device's norm in
+    the place of the serial one, and the caller can go on demanding equal bits.  The norms
+    themselves are always held to 1e-12 relative.  `state_lists` are the lists of arrays and
+    `scalars` the ctypes structures (meta, scaler state) the step changes."""
+    import copy
+
+    if max_norm <= 0 or dev_info is None:
+        return step_fn()
+    snap_lists = [[a.copy() for a in lst] for lst in state_lists]
+    snap_scalars = [copy.copy(x) if x is not None else None for x in scalars]
+    ran, norm = step_fn()
+    NORM_FOLLOWED["steps"] += 1
+    if not ran or dev_info.found_inf:
+        return ran, norm
+    assert abs(dev_info.norm - norm) <= 1e-12 * norm, f"{what}: device norm {dev_info.norm!r} vs serial {norm!r}"
+
+    def factor(n):  # None: not clipped (trainer.rs:515)
+        return np.float32(max_norm / n).tobytes() if (n > max_norm and n > 0.0) else None
+
+    if factor(dev_info.norm) != factor(norm):
+        for lst, snap in zip(state_lists, snap_lists):
+            for a, b in zip(lst, snap):
+                a[...] = b
+        for x, sx in zip(scalars, snap_scalars):
+            if x is not None:
+                C = type(x)
+                import ctypes
+
+                ctypes.memmove(ctypes.byref(x), ctypes.byref(sx), ctypes.sizeof(C))
+        O.set_clip_norm_override(dev_info.norm)
+        try:
+            ran, _ = step_fn()
+        finally:
+            O.set_clip_norm_override(-1.0)
+        NORM_FOLLOWED["events"] += 1
+        report(f"[norm-follow] {what}: clip factor from the device's norm {dev_info.norm!r} differs from the serial "
+               f"norm's {norm!r}; the oracle step was repeated with the device's norm")
+    return ran, norm
+
+
 # ---- the 2-ulp bar for parameters and its one documented escape ------------------------------
 
 # No test may leave more than this many elements per 10^9 element-steps beyond 2 ulp (each of
@@ -162,10 +227,16 @@ def tolerance_report(dev_list, ref_list, lr, steps, what, element_steps=None):
             assert not outside.any(), (
                 f"{what}: tensor {i}: {int(outside.sum())} params beyond 2 ulp and beyond the cancellation "
                 f"bound {bound:.3e}; worst ulp {int(ulp.max())}, worst |d| {absd.max():.3e}")
+            # the mechanism itself: a difference of a few ulps of the update can only be many
+            # ulps of the parameter where the parameter is no larger than a few updates
+            big = np.maximum(np.abs(a[idx]), np.abs(b[idx])).astype(np.float64)
+            assert (big < 16.0 * lr * steps).all(), (
+                f"{what}: tensor {i}: an element beyond 2 ulp has magnitude {big.max():.3e}, not below "
+                f"16 * lr * steps = {16.0 * lr * steps:.3e}: this is not the near-cancellation the clause is for")
     es = element_steps if element_steps is not None else n_total * steps
-    print(f"[tolerance] {what}: {n_beyond} of {n_total} elements ({es} element-steps) beyond 2 ulp of the "
-          f"libm-powf oracle, all within |d| <= {bound:.3e}; worst {worst_ulp} ulp, worst |d| {worst_abs:.3e}; "
-          f"first (tensor, index, device, oracle, ulp): {first}", flush=True)
+    report(f"[tolerance] {what}: {n_beyond} of {n_total} elements ({es} element-steps) beyond 2 ulp of the "
+           f"libm-powf oracle, all within |d| <= {bound:.3e} and of magnitude < 16 * lr * steps; worst {worst_ulp} ulp, "
+           f"worst |d| {worst_abs:.3e}; first (tensor, index, device, oracle, ulp): {first}")
     ceiling = max(5, int(ESCAPES_PER_1E9_ELEMENT_STEPS * es / 1e9))
     assert n_beyond <= ceiling, f"{what}: {n_beyond} elements beyond 2 ulp, more than the ceiling of {ceiling}"
     return n_beyond, n_total, worst_ulp, worst_abs, first

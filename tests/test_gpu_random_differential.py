@@ -4,6 +4,8 @@ random optimizer kind / element type / hyper-parameters, and random sequences of
 the device against the same sequence on the oracle (sqrt variant): every bit of params,
 moments, master weights, scaler state and step_count must agree.  The directed tests pin
 each feature; this one pins their combinations."""
+from types import SimpleNamespace
+
 import numpy as np
 import pytest
 
@@ -129,33 +131,45 @@ def _case(seed):
             keep.append(kg)
             fused = is_mixed or rng.random() < 0.6
             zero = fused and rng.random() < 0.3
+            info = None  # what the device decided, where it keeps a record of it
             if fused:
                 opt.fused_step(p_dev, g_dev, scaler=scaler, max_norm=clip, skip_nonfinite=nan_policy, zero_grads=zero)
+                info = opt.last_step()
             else:
                 ok = scaler.unscale_and_update(g_dev) if scaler else True
                 if ok and nan_policy and nb.has_non_finite(g_dev):
                     ok = False
                 if ok:
                     if clip > 0:
-                        nb.clip_grad_norm(g_dev, clip)
+                        info = SimpleNamespace(found_inf=0, norm=nb.clip_grad_norm(g_dev, clip))
                     opt.step(p_dev, g_dev)
             # the reference's order (trainer.rs:230-283) on the oracle
             if is_mixed:
                 skip = nan_policy and ref_scaler is None and any(not np.isfinite(a).all() for a in H.widen_list(g))
                 if not skip:
-                    O.mixed_step(meta, ref_scaler, clip, ref_p, g, ref_w, ref_m, ref_v)
+                    H.oracle_step_with_device_norm(
+                        lambda: O.mixed_step(meta, ref_scaler, clip, ref_p, g, ref_w, ref_m, ref_v),
+                        [ref_p, ref_w, ref_m, ref_v], [meta, ref_scaler], clip, info, what + f": step {step}")
             else:
-                gr = H.copy_list(g)
-                ok = O.scaler_unscale_and_update(ref_scaler, gr) if ref_scaler else True
-                if ok and nan_policy:
-                    vals = H.widen_list(gr) if is_pure else gr
-                    ok = all(np.isfinite(a).all() for a in vals)
-                if ok:
-                    O.clip_grad_norm(gr, clip)
-                    if kind == "sgd":
-                        O.sgd_step(meta, ref_p, gr, ref_m)
-                    else:
-                        O.adam_step(meta, ref_p, gr, ref_m, ref_v)
+                def plain_step():
+                    gr = H.copy_list(g)
+                    ok = O.scaler_unscale_and_update(ref_scaler, gr) if ref_scaler else True
+                    if ok and nan_policy:
+                        vals = H.widen_list(gr) if is_pure else gr
+                        ok = all(np.isfinite(a).all() for a in vals)
+                    norm = 0.0
+                    if ok:
+                        norm = O.clip_grad_norm(gr, clip)
+                        if kind == "sgd":
+                            O.sgd_step(meta, ref_p, gr, ref_m)
+                        else:
+                            O.adam_step(meta, ref_p, gr, ref_m, ref_v)
+                    return ok, norm
+
+                # (info is None for an unfused step that was skipped or does not clip: the oracle's
+                # step then stands as it is)
+                H.oracle_step_with_device_norm(plain_step, [ref_p, ref_m, ref_v], [meta, ref_scaler], clip, info,
+                                               what + f": step {step}")
             if zero:
                 assert not any(t.any() for t in H.host_list(g_dev)), what + f": step {step}: grads not zeroed"
     finally:
