@@ -306,6 +306,14 @@ template <typename Opt> MetaContents read_meta(const std::string &path, Opt &opt
 }
 
 namespace detail {
+// an optimizer that reads and writes the module's params.nbla itself (GroupOptimizer: its groups
+// may hold master weights for some of the parameters)
+template <typename Opt, typename = void> struct has_params_file : std::false_type {};
+template <typename Opt>
+struct has_params_file<Opt, std::void_t<decltype(std::declval<Opt &>().save_params(
+                                std::declval<const std::string &>(), std::declval<const std::vector<Tensor> &>(),
+                                std::declval<const std::vector<std::string> &>()))>> : std::true_type {};
+
 template <typename F> void tensor_file(const char *kind, F &&call)
 {
     try {
@@ -334,6 +342,11 @@ void save_checkpoint(const std::string &dir, TensorList &params, const std::vect
             detail::tensor_file("State", [&] { optimizer.save_master(dir + "/params.nbla", names); });
             from_master = true;
         }
+    } else if constexpr (detail::has_params_file<Opt>::value) {
+        if (optimizer.keeps_master()) {
+            detail::tensor_file("State", [&] { optimizer.save_params(dir + "/params.nbla", params.tensors(), names); });
+            from_master = true;
+        }
     }
     if (!from_master) detail::tensor_file("State", [&] { save_tensors(dir + "/params.nbla", params, names); });
     detail::tensor_file("Optim", [&] { optimizer.save_state(dir + "/optim.nbla"); });
@@ -353,6 +366,11 @@ void load_checkpoint(const std::string &dir, TensorList &params, const std::vect
                 optimizer.load_master(dir + "/params.nbla", names);
                 optimizer.params_from_master(params);
             });
+            into_master = true;
+        }
+    } else if constexpr (detail::has_params_file<Opt>::value) {
+        if (optimizer.keeps_master()) { // each group's master weights, then its 16-bit tensors narrowed from them
+            detail::tensor_file("State", [&] { optimizer.load_params(dir + "/params.nbla", params.tensors(), names); });
             into_master = true;
         }
     }

@@ -210,6 +210,26 @@ public:
     // optim.nbla of a checkpoint with the keys of groups.rs:320-350 ("g{gi}.m{i}", "g{gi}.v{i}")
     void save_state(const std::string &path) { check(nbo_optim_save_state_groups(groups_.size(), handles().data(), path.c_str())); }
     void load_state(const std::string &path) { check(nbo_optim_load_state_groups(groups_.size(), handles().data(), path.c_str())); }
+    // params.nbla of a checkpoint (checkpoint.rs:54-58, 88-90) for the module whose parameters
+    // these groups hold: a group that keeps master weights writes (receives) those under the
+    // parameters' names -- the 16-bit tensors are derived from them and are narrowed from them
+    // again after loading -- the other groups their tensors as they are.
+    bool keeps_master() const
+    {
+        for (const Entry &g : groups_)
+            if (g.optimizer->keeps_master()) return true;
+        return false;
+    }
+    void save_params(const std::string &path, const std::vector<Tensor> &params, const std::vector<std::string> &names)
+    {
+        params_file(nbo_optim_save_params_groups, path, params, names);
+    }
+    void load_params(const std::string &path, const std::vector<Tensor> &params, const std::vector<std::string> &names)
+    {
+        params_file(nbo_optim_load_params_groups, path, params, names);
+        for (Entry &g : groups_)
+            if (g.optimizer->keeps_master()) g.optimizer->params_from_master(*g.params);
+    }
     void reset()
     {
         for (Entry &g : groups_) g.optimizer->reset();
@@ -263,16 +283,42 @@ private:
         }
         return k;
     }
+    void bind_params(const std::vector<Tensor> &params)
+    {
+        if (params.size() != param_count_) throw Panic("nabla-train: GroupOptimizer param count mismatch");
+        for (Entry &g : groups_) {
+            std::vector<Tensor> p;
+            for (size_t i : g.indices) p.push_back(params[i]);
+            if (!g.params || g.pkey != key_of(p)) g.params.reset(new TensorList(p)), g.pkey = key_of(p);
+        }
+    }
     void bind(const std::vector<Tensor> &params, const std::vector<Tensor> &grads)
     {
         if (params.size() != grads.size()) throw Panic("nabla-train: GroupOptimizer params/grads length mismatch");
-        if (params.size() != param_count_) throw Panic("nabla-train: GroupOptimizer param count mismatch");
+        bind_params(params);
         for (Entry &g : groups_) {
-            std::vector<Tensor> p, q;
-            for (size_t i : g.indices) p.push_back(params[i]), q.push_back(grads[i]);
-            if (!g.params || g.pkey != key_of(p)) g.params.reset(new TensorList(p)), g.pkey = key_of(p);
+            std::vector<Tensor> q;
+            for (size_t i : g.indices) q.push_back(grads[i]);
             if (!g.grads || g.gkey != key_of(q)) g.grads.reset(new TensorList(q)), g.gkey = key_of(q);
         }
+    }
+    template <typename Call>
+    void params_file(Call call, const std::string &path, const std::vector<Tensor> &params,
+                     const std::vector<std::string> &names)
+    {
+        if (names.size() != params.size()) throw Panic("nabla-train: GroupOptimizer param count mismatch");
+        bind_params(params);
+        std::vector<uint32_t> group_of(params.size()), index_in(params.size());
+        std::vector<nbo_list *> lists;
+        for (size_t g = 0; g < groups_.size(); g++) {
+            lists.push_back(groups_[g].params->handle());
+            for (size_t k = 0; k < groups_[g].indices.size(); k++)
+                group_of[groups_[g].indices[k]] = (uint32_t)g, index_in[groups_[g].indices[k]] = (uint32_t)k;
+        }
+        std::vector<const char *> raw;
+        for (const std::string &n : names) raw.push_back(n.c_str());
+        check(call(groups_.size(), handles().data(), lists.data(), params.size(), group_of.data(), index_in.data(),
+                   raw.data(), path.c_str()));
     }
     std::vector<Entry> groups_;
     size_t param_count_ = 0;

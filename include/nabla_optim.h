@@ -346,6 +346,22 @@ int nbo_optim_load_master(nbo_optim *opt, const char *path, const char *const *n
  * group's own checks.  Nothing is written unless the whole file checks out. */
 int nbo_optim_save_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path);
 int nbo_optim_load_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path);
+/* params.nbla of a module whose parameters are spread over a GroupOptimizer's groups
+ * (checkpoint.rs:54-58, 88-90; optim/groups.rs:168-226): parameter i of the module, named
+ * names[i], is tensor index_in_group[i] of group group_of[i]; params[g] lists group g's tensors
+ * in the group's order.  What is written for a parameter is its group's f32 master weight if
+ * the group keeps master weights, else the tensor itself.  Loading is load_tensors +
+ * Module::load_state_dict (module/core.rs:281-304) with its errors ("unknown parameter key: k",
+ * "shape mismatch for 'k': ...") plus "missing parameter key: k" for a parameter whose group
+ * keeps master weights; nothing is written unless the whole file checks out, the master
+ * weights then count as set, and nbo_optim_params_from_master per group gives the 16-bit
+ * parameters. */
+int nbo_optim_save_params_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,
+                                 uint64_t n_params, const uint32_t *group_of, const uint32_t *index_in_group,
+                                 const char *const *names, const char *path);
+int nbo_optim_load_params_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,
+                                 uint64_t n_params, const uint32_t *group_of, const uint32_t *index_in_group,
+                                 const char *const *names, const char *path);
 
 #pragma GCC visibility pop
 

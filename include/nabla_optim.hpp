@@ -69,7 +69,7 @@ public:
     explicit TensorList(const std::vector<Tensor> &tensors) { assign(tensors); }
     TensorList(const TensorList &) = delete;
     TensorList &operator=(const TensorList &) = delete;
-    TensorList(TensorList &&o) noexcept : h_(o.h_), n_(o.n_) { o.h_ = nullptr; }
+    TensorList(TensorList &&o) noexcept : h_(o.h_), n_(o.n_), tensors_(std::move(o.tensors_)) { o.h_ = nullptr; }
     ~TensorList() { reset(); }
 
     void assign(const std::vector<Tensor> &tensors)
@@ -86,9 +86,12 @@ public:
         }
         n_ = tensors.size();
         check(nbo_list_create(n_, rows.data(), cols.data(), dt, ptrs.data(), &h_));
+        tensors_ = tensors;
     }
     nbo_list *handle() const { return h_; }
     size_t size() const { return n_; }
+    // what the list was made from
+    const std::vector<Tensor> &tensors() const { return tensors_; }
 
 private:
     void reset()
@@ -98,6 +101,7 @@ private:
     }
     nbo_list *h_ = nullptr;
     size_t n_ = 0;
+    std::vector<Tensor> tensors_;
 };
 
 enum class OptimKind { AdamW = NBO_KIND_ADAMW, Adam = NBO_KIND_ADAM, Sgd = NBO_KIND_SGD };

@@ -98,6 +98,13 @@ extern "C" {
     // groups.rs:320-350 (GroupOptimizer's state keys "g{gi}.m{i}" / "g{gi}.v{i}")
     pub fn nbo_optim_save_state_groups(n_groups: u64, opts: *const *mut NboOptim, path: *const c_char) -> c_int;
     pub fn nbo_optim_load_state_groups(n_groups: u64, opts: *const *mut NboOptim, path: *const c_char) -> c_int;
+    // checkpoint.rs:54-58, 88-90 for a module whose parameters are spread over the groups
+    pub fn nbo_optim_save_params_groups(n_groups: u64, opts: *const *mut NboOptim, params: *const *mut NboList,
+                                        n_params: u64, group_of: *const u32, index_in_group: *const u32,
+                                        names: *const *const c_char, path: *const c_char) -> c_int;
+    pub fn nbo_optim_load_params_groups(n_groups: u64, opts: *const *mut NboOptim, params: *const *mut NboList,
+                                        n_params: u64, group_of: *const u32, index_in_group: *const u32,
+                                        names: *const *const c_char, path: *const c_char) -> c_int;
     pub fn nbo_optim_trace_read(opt: *mut NboOptim, out: *mut NboStepInfo, max_entries: u64,
                                 n_out: *mut u64, total: *mut u64) -> c_int;
     pub fn nbo_optim_state_regions(opt: *mut NboOptim, regions: *mut c_int) -> c_int;

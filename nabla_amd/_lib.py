@@ -131,6 +131,12 @@ SYMBOLS = {
     "nbo_optim_load_master": (C.c_int, [_P, C.c_char_p, C.POINTER(C.c_char_p)]),
     "nbo_optim_save_state_groups": (C.c_int, [C.c_uint64, C.POINTER(_P), C.c_char_p]),
     "nbo_optim_load_state_groups": (C.c_int, [C.c_uint64, C.POINTER(_P), C.c_char_p]),
+    "nbo_optim_save_params_groups": (C.c_int, [C.c_uint64, C.POINTER(_P), C.POINTER(_P), C.c_uint64,
+                                               C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_char_p),
+                                               C.c_char_p]),
+    "nbo_optim_load_params_groups": (C.c_int, [C.c_uint64, C.POINTER(_P), C.POINTER(_P), C.c_uint64,
+                                               C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_char_p),
+                                               C.c_char_p]),
 }
 # every symbol include/nabla_optim_bench.h declares (measurement only)
 BENCH_SYMBOLS = {

@@ -262,6 +262,27 @@ def load_optim_native(path: str, optimizer) -> None:
         _native(_lib.load().nbo_optim_load_state, optimizer._handle(), path.encode())
 
 
+def _group_params_file(call, optimizer, named_tensors: Sequence[Tuple[str, object]], path: str) -> None:
+    """params.nbla of a module whose parameters are spread over a GroupOptimizer's groups
+    (nbo_optim_save_params_groups / nbo_optim_load_params_groups): a group that keeps master
+    weights contributes (or receives) those, the other groups their tensors."""
+    import ctypes as C
+
+    tensors = [t for _, t in named_tensors]
+    groups = optimizer._groups
+    n = len(groups)
+    group_of, index_in = [0] * len(tensors), [0] * len(tensors)
+    for g, entry in enumerate(groups):
+        for k, i in enumerate(entry.indices):
+            group_of[i], index_in[i] = g, k
+    opts = (C.c_void_p * max(n, 1))(*[e.optimizer._handle() for e in groups])
+    lists = [optimizer._lists(e, "p", tensors) for e in groups]
+    pl = (C.c_void_p * max(n, 1))(*[lst._h for lst in lists])
+    m = len(tensors)
+    _native(call, n, opts, pl, m, (C.c_uint32 * max(m, 1))(*group_of), (C.c_uint32 * max(m, 1))(*index_in),
+            _name_array([name for name, _ in named_tensors]), path.encode())
+
+
 def _keeps_master(optimizer) -> bool:
     return bool(getattr(optimizer, "_master", False))
 
@@ -288,13 +309,17 @@ def save_checkpoint(directory: str, params: Sequence[Tuple[str, object]], optimi
         write_meta(os.path.join(directory, META_FILE), optimizer, scaler, schedule, state)
         return
     if _groups_keep_master(optimizer):
-        # the groups' master weights, put back into the module's order under the parameters' names
-        masters = [t for _, t in params]
-        for idxs, o in zip(optimizer.group_indices(), optimizer.group_optimizers()):
-            if _keeps_master(o):
-                for k, i in enumerate(idxs):
-                    masters[i] = o.read_state(f"w{k}")
-        params = [(n, m) for (n, _), m in zip(params, masters)]
+        # the groups' master weights, in the module's order under the parameters' names; the
+        # tensors of a group without master weights as they are
+        from . import _lib
+
+        if len(params) != optimizer._param_count:
+            raise CheckpointError("State", "nabla-train: GroupOptimizer param count mismatch")
+        _group_params_file(_lib.load().nbo_optim_save_params_groups, optimizer, params,
+                           os.path.join(directory, PARAMS_FILE))
+        save_optim_native(os.path.join(directory, OPTIM_FILE), optimizer)
+        write_meta(os.path.join(directory, META_FILE), optimizer, scaler, schedule, state)
+        return
     if native:
         save_params_native(os.path.join(directory, PARAMS_FILE), params)
         save_optim_native(os.path.join(directory, OPTIM_FILE), optimizer)
@@ -326,26 +351,20 @@ def load_checkpoint(directory: str, optimizer, scaler: Optional[GradScaler] = No
         load_optim_native(os.path.join(directory, OPTIM_FILE), optimizer)
         params = None
     elif _groups_keep_master(optimizer):
-        import torch
-
+        from . import _lib
         from .optim import TensorList
 
         if into is None:
             raise ValueError("a mixed-precision optimizer's checkpoint is loaded with into=[(name, 16-bit tensor), ...]: "
                              "params.nbla holds its master weights under the parameters' names")
-        loaded = dict(load_tensors(os.path.join(directory, PARAMS_FILE)))
+        if len(into) != optimizer._param_count:
+            raise CheckpointError("State", "nabla-train: GroupOptimizer param count mismatch")
+        # the whole file is checked against all names and shapes before anything is written
+        _group_params_file(_lib.load().nbo_optim_load_params_groups, optimizer, into,
+                           os.path.join(directory, PARAMS_FILE))
         for idxs, o in zip(optimizer.group_indices(), optimizer.group_optimizers()):
-            tensors = [into[i][1] for i in idxs]
-            if not _keeps_master(o):
-                load_params_native(os.path.join(directory, PARAMS_FILE), [into[i] for i in idxs])
-                continue
-            for k, i in enumerate(idxs):
-                name = into[i][0]
-                if name not in loaded:
-                    raise CheckpointError("State", f"missing parameter key: {name}")
-                o.write_state(f"w{k}", torch.from_numpy(loaded[name].astype("float32")).to(tensors[k].device)
-                              .reshape(tensors[k].shape))
-            o.params_from_master(TensorList(tensors))
+            if _keeps_master(o):
+                o.params_from_master(TensorList([into[i][1] for i in idxs]))
         load_optim_native(os.path.join(directory, OPTIM_FILE), optimizer)
         params = None
     elif into is not None:

@@ -1221,4 +1221,26 @@ int nbo_optim_load_state_groups(uint64_t n_groups, nbo_optim *const *opts, const
     });
 }
 
+int nbo_optim_save_params_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,
+                                 uint64_t n_params, const uint32_t *group_of, const uint32_t *index_in_group,
+                                 const char *const *names, const char *path)
+{
+    return guarded([&] {
+        require_groups(n_groups, opts, path);
+        require(n_groups == 0 || params != nullptr, NBO_ERR_ARG, "null list array");
+        optim_save_params_groups(n_groups, opts, params, n_params, group_of, index_in_group, names, path);
+    });
+}
+
+int nbo_optim_load_params_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,
+                                 uint64_t n_params, const uint32_t *group_of, const uint32_t *index_in_group,
+                                 const char *const *names, const char *path)
+{
+    return guarded([&] {
+        require_groups(n_groups, opts, path);
+        require(n_groups == 0 || params != nullptr, NBO_ERR_ARG, "null list array");
+        optim_load_params_groups(n_groups, opts, params, n_params, group_of, index_in_group, names, path);
+    });
+}
+
 } // extern "C"

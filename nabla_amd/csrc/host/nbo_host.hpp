@@ -194,6 +194,12 @@ void optim_save_master(const nbo_optim *opt, const char *path, const char *const
 void optim_load_master(nbo_optim *opt, const char *path, const char *const *names);
 void optim_save_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path);
 void optim_load_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path);
+void optim_save_params_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params, uint64_t n_params,
+                              const uint32_t *group_of, const uint32_t *index_in_group, const char *const *names,
+                              const char *path);
+void optim_load_params_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params, uint64_t n_params,
+                              const uint32_t *group_of, const uint32_t *index_in_group, const char *const *names,
+                              const char *path);
 } // namespace nbo
 
 #endif

@@ -448,6 +448,113 @@ void optim_load_master(nbo_optim *opt, const char *path, const char *const *name
     opt->master_valid = true;
 }
 
+// params.nbla of a GroupOptimizer (checkpoint.rs:54-58 over the module's state_dict): the module's
+// parameter i is tensor index_in_group[i] of group group_of[i]; what is written under names[i] is
+// that group's f32 master weight if the group keeps master weights, else the caller's tensor itself.
+namespace {
+struct GroupSlot { // where parameter i lives
+    int dtype;
+    uint64_t rows, cols, n;
+    void *dev;
+    bool master;
+};
+
+std::vector<GroupSlot> group_slots(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,
+                                   uint64_t n_params, const uint32_t *group_of, const uint32_t *index_in_group,
+                                   bool saving)
+{
+    if (n_params && (!group_of || !index_in_group)) fail(NBO_ERR_ARG, "null index array");
+    std::vector<GroupSlot> out(n_params);
+    std::vector<std::vector<char>> seen(n_groups);
+    for (uint64_t g = 0; g < n_groups; g++) {
+        if (!opts[g] || !params[g]) fail(NBO_ERR_ARG, "null optimizer or list");
+        if (params[g]->layout.nt() != opts[g]->layout.nt()) fail(NBO_ERR_COUNT_MISMATCH, "params count mismatch");
+        seen[g].assign(opts[g]->layout.nt(), 0);
+    }
+    for (uint64_t i = 0; i < n_params; i++) {
+        const uint32_t g = group_of[i], k = index_in_group[i];
+        if (g >= n_groups || k >= opts[g]->layout.nt() || seen[g][k])
+            fail(NBO_ERR_ARG, "parameter " + std::to_string(i) + ": not a tensor of its group, or named twice");
+        seen[g][k] = 1;
+        const nbo_optim *o = opts[g];
+        GroupSlot &s = out[i];
+        s.master = o->keep_master;
+        s.rows = o->layout.rows[k], s.cols = o->layout.cols[k], s.n = o->layout.n[k];
+        if (params[g]->layout.rows[k] != s.rows || params[g]->layout.cols[k] != s.cols)
+            fail(NBO_ERR_SHAPE, "shapes must match (group " + std::to_string(g) + ", tensor " + std::to_string(k) + ")");
+        if (s.master) {
+            if (saving && !o->master_valid) fail(NBO_ERR_NO_MASTER, "master weights not set");
+            s.dtype = NBO_DT_F32;
+            s.dev = (char *)o->arena.part[o->arena.part_w] + (size_t)o->layout.soff[k] * 4;
+        } else {
+            s.dtype = params[g]->dtype;
+            s.dev = (void *)(uintptr_t)params[g]->ptrs[k];
+        }
+    }
+    for (uint64_t g = 0; g < n_groups; g++)
+        for (char c : seen[g])
+            if (!c) fail(NBO_ERR_COUNT_MISMATCH, "nabla-train: GroupOptimizer param count mismatch");
+    return out;
+}
+} // namespace
+
+void optim_save_params_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params, uint64_t n_params,
+                              const uint32_t *group_of, const uint32_t *index_in_group, const char *const *names,
+                              const char *path)
+{
+    if (n_params && !names) fail(NBO_ERR_ARG, "null name array");
+    if (n_params > 0xFFFFFFFFull) fail(NBO_ERR_TOO_LARGE, "too many tensors for the file format");
+    const std::vector<GroupSlot> slots = group_slots(n_groups, opts, params, n_params, group_of, index_in_group, true);
+    Runtime::get().sync();
+    FilePtr f = open_file(path, "wb");
+    Buffers b;
+    write_all(f.get(), "NBLA", 4);
+    write_u32(f.get(), (uint32_t)n_params);
+    for (uint64_t i = 0; i < n_params; i++) {
+        if (!names[i]) fail(NBO_ERR_ARG, "null tensor name");
+        write_header(f.get(), names[i], slots[i].rows, slots[i].cols);
+        stream_out(f.get(), slots[i].dev, slots[i].dtype, slots[i].n, b);
+    }
+    if (std::fflush(f.get()) != 0) fail(NBO_ERR_IO, std::string("write failed: ") + std::strerror(errno));
+}
+
+// load_tensors + Module::load_state_dict (module/core.rs:281-304) for a GroupOptimizer's module:
+// every tensor of the file must name a parameter and have its shape, and every parameter whose
+// group keeps master weights must be in the file (a master weight that kept its old value would
+// silently diverge from its 16-bit parameter).  Nothing is written unless the whole file checks
+// out.  Afterwards those groups' master weights count as set; the caller derives the 16-bit
+// parameters from them (nbo_optim_params_from_master per group).
+void optim_load_params_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params, uint64_t n_params,
+                              const uint32_t *group_of, const uint32_t *index_in_group, const char *const *names,
+                              const char *path)
+{
+    if (n_params && !names) fail(NBO_ERR_ARG, "null name array");
+    const std::vector<GroupSlot> slots = group_slots(n_groups, opts, params, n_params, group_of, index_in_group, false);
+    FilePtr f = open_file(path, "rb");
+    const std::vector<Entry> index = read_index(f.get());
+    std::vector<long> at(n_params, -1);
+    for (const Entry &e : index) {
+        uint64_t i = 0;
+        while (i < n_params && e.name != names[i]) i++;
+        if (i == n_params) fail(NBO_ERR_STATE_KEY, "unknown parameter key: " + e.name);
+        if (e.rows != slots[i].rows || e.cols != slots[i].cols)
+            fail(NBO_ERR_SHAPE, "shape mismatch for '" + e.name + "': expected (" + std::to_string(slots[i].rows) + ", " +
+                                    std::to_string(slots[i].cols) + "), got (" + std::to_string(e.rows) + ", " +
+                                    std::to_string(e.cols) + ")");
+        at[i] = e.data_offset;
+    }
+    for (uint64_t i = 0; i < n_params; i++)
+        if (at[i] < 0 && slots[i].master) fail(NBO_ERR_STATE_KEY, std::string("missing parameter key: ") + names[i]);
+    Buffers b;
+    for (uint64_t i = 0; i < n_params; i++) {
+        if (at[i] < 0) continue;
+        seek_to(f.get(), at[i]);
+        stream_in(f.get(), slots[i].dev, slots[i].dtype, slots[i].n, b);
+    }
+    for (uint64_t g = 0; g < n_groups; g++)
+        if (opts[g]->keep_master) opts[g]->master_valid = true;
+}
+
 // GroupOptimizer's OptimState (groups.rs:320-373): every group's tensors behind "g{gi}.".
 void optim_save_state_groups(uint64_t n_groups, nbo_optim *const *opts, const char *path)
 {

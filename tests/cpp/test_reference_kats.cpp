@@ -383,6 +383,85 @@ static void mixed_precision_checkpoint_resumes_bit_for_bit()
     EXPECT(what.find("unknown parameter key: layer.b") != std::string::npos);
 }
 
+// The same for a GroupOptimizer whose groups keep master weights: params.nbla holds every group's
+// f32 master weights in the module's order under the parameters' names, the restored groups'
+// 16-bit tensors are narrowed from them, and training goes on with the uninterrupted run's bits.
+static void group_mixed_precision_checkpoint_resumes_bit_for_bit()
+{
+    if (g_checkpoint_dir.empty()) return;
+    const std::string dir = g_checkpoint_dir + "/groups_mixed";
+    const uint64_t nw = 8192 + 37, nb = 300, nn = 64;
+    const std::vector<std::string> names = {"layer.w", "layer.bias", "layer.norm"};
+    auto fill = [](uint64_t n, uint32_t seed, uint16_t exp_bits) {
+        std::vector<uint16_t> v(n);
+        uint32_t x = seed;
+        for (auto &e : v) {
+            x = x * 1664525u + 1013904223u;
+            e = (uint16_t)(((x >> 16) & 0x807f) | exp_bits);
+        }
+        return v;
+    };
+    HalfVec pw(nw), pb(nb), pn(nn), gw(nw), gb(nb), gn(nn);
+    pw.put(fill(nw, 1, 0x3c00)), pb.put(fill(nb, 2, 0x3c00)), pn.put(fill(nn, 3, 0x3c00));
+    auto make = [&](const std::vector<Tensor> &t) {
+        return GroupOptimizer::adamw_with_decay_exclusions({{names[0], t[0]}, {names[1], t[1]}, {names[2], t[2]}}, 2e-4, 0.1,
+                                                           {"bias", "norm"}, NBO_DT_F32, /*master=*/true);
+    };
+    const std::vector<Tensor> params = {pw.tensor(), pb.tensor(), pn.tensor()};
+    const std::vector<Tensor> grads = {gw.tensor(), gb.tensor(), gn.tensor()};
+    GroupOptimizer opt = make(params);
+    EXPECT(opt.groups() == 2 && opt.keeps_master() && (opt.group_indices(0) == std::vector<size_t>{1, 2}));
+    for (size_t g = 0; g < opt.groups(); g++) {
+        std::vector<Tensor> mine;
+        for (size_t i : opt.group_indices(g)) mine.push_back(params[i]);
+        TensorList l(mine);
+        opt.group_optimizer(g).master_from_params(l);
+    }
+    GradScaler scaler;
+    auto step = [&](GroupOptimizer &o, GradScaler &sc, const std::vector<Tensor> &p, uint32_t k) {
+        gw.put(fill(nw, 100 + k, 0x4300)), gb.put(fill(nb, 200 + k, 0x4300)), gn.put(fill(nn, 300 + k, 0x4300));
+        o.fused_step(p, grads, &sc, 1.0);
+    };
+    for (uint32_t k = 0; k < 3; k++) step(opt, scaler, params, k);
+    TensorList module(params);
+    TrainState state;
+    state.epoch = 0, state.step = 3, state.grad_accum = 1;
+    save_checkpoint(dir, module, names, opt, &scaler, nullptr, state);
+
+    HalfVec qw(nw), qb(nb), qn(nn);
+    const std::vector<Tensor> params2 = {qw.tensor(), qb.tensor(), qn.tensor()};
+    GroupOptimizer opt2 = make(params2);
+    TensorList module2(params2);
+    GradScaler scaler2;
+    TrainState state2;
+    std::optional<ScheduleState> schedule2;
+    load_checkpoint(dir, module2, names, opt2, &scaler2, schedule2, state2);
+    EXPECT(state2.step == 3 && !schedule2.has_value());
+    EXPECT(qw.get() == pw.get() && qb.get() == pb.get() && qn.get() == pn.get()); // narrowed from the master weights
+    for (uint32_t k = 3; k < 5; k++) {
+        step(opt, scaler, params, k);
+        step(opt2, scaler2, params2, k);
+    }
+    EXPECT(qw.get() == pw.get() && qb.get() == pb.get() && qn.get() == pn.get());
+    for (size_t g = 0; g < opt.groups(); g++)
+        for (const char *key : {"w0", "m0", "v0"}) {
+            const uint64_t n = g == 0 ? nb : nw;
+            std::vector<float> a(n), b(n);
+            opt.group_optimizer(g).state_read(key, a.data(), n, false);
+            opt2.group_optimizer(g).state_read(key, b.data(), n, false);
+            EXPECT(std::memcmp(a.data(), b.data(), n * sizeof(float)) == 0);
+        }
+    EXPECT(opt.group_optimizer(1).last_step().step_count == 5 && opt2.group_optimizer(1).last_step().step_count == 5);
+    // the file is checked as a whole before anything is written: a key the module does not have
+    std::string what;
+    try {
+        load_checkpoint(dir, module2, {"layer.w", "layer.bias", "other.norm"}, opt2, &scaler2, schedule2, state2);
+    } catch (const std::exception &e) {
+        what = e.what();
+    }
+    EXPECT(what.find("unknown parameter key: layer.norm") != std::string::npos);
+}
+
 static void panics_and_errors()  // alg.rs:110-119, 531-545; tensor/ops.rs:638-646
 {
     Mat p({1.0}), g({1.0}), g2({1.0, 2.0});
@@ -595,6 +674,8 @@ int main(int argc, char **argv)
                  {"backend_axpy_is_multiply_then_add", backend_axpy_is_multiply_then_add},
                  {"checkpoint_roundtrip_with_schedule", checkpoint_roundtrip_with_schedule},
                  {"mixed_precision_checkpoint_resumes_bit_for_bit", mixed_precision_checkpoint_resumes_bit_for_bit},
+                 {"group_mixed_precision_checkpoint_resumes_bit_for_bit",
+                  group_mixed_precision_checkpoint_resumes_bit_for_bit},
                  {"panics_and_errors", panics_and_errors},
                  {"group_checkpoint_roundtrip", group_checkpoint_roundtrip},
                  {"constructors_and_set_state", constructors_and_set_state},

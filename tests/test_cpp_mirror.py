@@ -41,7 +41,7 @@ def test_cpp_replay_of_reference_tests(gpu, tmp_path):
     r = subprocess.run([BIN, str(tmp_path)], capture_output=True, text=True, timeout=120)
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count("ok    ") == 18 and "0 failure(s)" in r.stdout
+    assert r.stdout.count("ok    ") == 19 and "0 failure(s)" in r.stdout
 
     # the checkpoint the C++ side left behind is the one the Python mirror writes and reads
     from nabla_amd import checkpoint as ck
@@ -50,7 +50,7 @@ def test_cpp_replay_of_reference_tests(gpu, tmp_path):
     import oracle as O
     from tests import helpers as H
 
-    assert sorted(os.listdir(tmp_path)) == ["groups", "meta.txt", "mixed", "optim.nbla", "params.nbla"]
+    assert sorted(os.listdir(tmp_path)) == ["groups", "groups_mixed", "meta.txt", "mixed", "optim.nbla", "params.nbla"]
     shapes = [(1, 1), (1, 1)]
     opt = nb.Sgd.new(0.7, shapes, dtype="f64")
     scaler = nb.GradScaler.new()
@@ -111,3 +111,31 @@ def test_cpp_replay_of_reference_tests(gpu, tmp_path):
     ck.save_checkpoint(str(mixed_again), named, mopt, mscaler, None, mstate)
     for name in ("meta.txt", "params.nbla", "optim.nbla"):
         assert (mixed_again / name).read_bytes() == (mdir / name).read_bytes(), name
+
+    # and the GroupOptimizer whose groups keep master weights: params.nbla is every group's f32
+    # master weights in the module's order; the Python mirror reads it, narrows the 16-bit tensors
+    # from it and writes the same bytes again
+    gm = tmp_path / "groups_mixed"
+    gnames, gsizes = ["layer.w", "layer.bias", "layer.norm"], [8192 + 37, 300, 64]
+    gnamed = [(n, H.dev_list([np.zeros(k, np.uint16)], [(1, k)])[0]) for n, k in zip(gnames, gsizes)]
+    gopt2 = G.GroupOptimizer.adamw_with_decay_exclusions(gnamed, 1.0, 0.5, ["bias", "norm"], master=True)
+    gscaler = nb.GradScaler.new()
+    _, gstate, gsched = ck.load_checkpoint(str(gm), gopt2, gscaler, into=gnamed)
+    assert (gstate.step, gsched) == (3, None) and [o.step_count() for o in gopt2.group_optimizers()] == [3, 3]
+    assert [o.meta().weight_decay for o in gopt2.group_optimizers()] == [0.0, 0.1]
+    saved = dict(ck.load_tensors(str(gm / "params.nbla")))
+    assert list(saved) == gnames
+    for idxs, o in zip(gopt2.group_indices(), gopt2.group_optimizers()):
+        for k, i in enumerate(idxs):
+            master = H.to_host(o.read_state(f"w{k}"))
+            assert np.array_equal(saved[gnames[i]].reshape(-1), master.astype(np.float64))
+            H.assert_bits_equal([H.to_host(gnamed[i][1]).reshape(-1)], [O.bf16_from_f32(master.reshape(-1))],
+                                "group params narrowed from the master weights")
+    gm_again = tmp_path / "groups_mixed_py"
+    ck.save_checkpoint(str(gm_again), gnamed, gopt2, gscaler, None, gstate)
+    for name in ("meta.txt", "params.nbla", "optim.nbla"):
+        assert (gm_again / name).read_bytes() == (gm / name).read_bytes(), name
+    # the whole file is checked before anything is written: an unknown key, a wrong shape
+    bad_named = [("layer.w", gnamed[0][1]), ("layer.bias", gnamed[1][1]), ("other", gnamed[2][1])]
+    with pytest.raises(ck.CheckpointError, match="unknown parameter key: layer.norm"):
+        ck.load_checkpoint(str(gm), gopt2, gscaler, into=bad_named)

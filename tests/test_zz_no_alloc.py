@@ -99,3 +99,51 @@ def test_allocation_free_fused_step_equals_the_ordinary_one_on_two_calls_in_a_ro
     assert not small.step(400, poison=(2, 8000, 0x7FC1))
     r = small.check("small list with a NaN")
     assert r["trace"][-1][0] == 1 and r["trace"][-1][2] == 1
+
+
+def test_allocation_free_fused_step_allocates_nothing_and_times_nothing(gpu):
+    """What the entry point is for: the call makes no device allocation and, even while the
+    library's per-kernel timing is switched on, creates no events -- its three launches are not
+    timed, where the ordinary entry point's are.  Free device memory is the same before and
+    after, and the step still does its work."""
+    import ctypes as C
+
+    import torch
+
+    from nabla_amd import _lib
+
+    L = _lib.load()
+    shapes = SMALL
+    master0 = H.randn_list(shapes, 5, 0.02)
+    opt = nb.AdamW.new(2e-4, shapes, master=True).beta2(0.95).weight_decay(0.1)
+    for i, a in enumerate(master0):
+        opt.write_state(f"w{i}", H.to_dev(a, shapes[i]))
+    p = nb.TensorList(H.dev_list(H.narrow_list(master0, "bf16"), shapes))
+    g = nb.TensorList(H.dev_list(H.narrow_list(H.randn_list(shapes, 6, 1e-3 * 65536.0), "bf16"), shapes))
+    scaler = nb.GradScaler.new()
+    opt.fused_step(p, g, scaler=scaler, max_norm=0.05, no_alloc=True)  # descriptors, handles: all made by now
+    nb.sync()
+    torch.cuda.synchronize()
+
+    def launches():
+        out = {}
+        for k in ("nbo_norm_bf16", "nbo_finalize", "nbo_update_bf16_adamw"):
+            cnt, ms = C.c_uint64(0), C.c_double(0.0)
+            _lib.check(L.nbo_profile_read(k.encode(), C.byref(cnt), C.byref(ms)))
+            out[k] = cnt.value
+        return out
+
+    _lib.check(L.nbo_profile_enable(1))
+    try:
+        free_before = torch.cuda.mem_get_info()[0]
+        for _ in range(3):
+            opt.fused_step(p, g, scaler=scaler, max_norm=0.05, no_alloc=True)
+        nb.sync()
+        assert torch.cuda.mem_get_info()[0] == free_before, "free device memory changed across the calls"
+        assert launches() == {"nbo_norm_bf16": 0, "nbo_finalize": 0, "nbo_update_bf16_adamw": 0}, \
+            "the allocation-free entry point's launches must not be bracketed by (newly created) events"
+        opt.fused_step(p, g, scaler=scaler, max_norm=0.05)  # the ordinary one is timed
+        assert launches() == {"nbo_norm_bf16": 1, "nbo_finalize": 1, "nbo_update_bf16_adamw": 1}
+    finally:
+        _lib.check(L.nbo_profile_enable(0))
+    assert opt.step_count() == 5 and opt.last_step().clipped == 1
