@@ -15,7 +15,7 @@ use std::os::raw::{c_char, c_int, c_void};
     pub growth_interval: u64, pub consecutive_ok: u64 }
 #[repr(C)] pub struct NboStepInfo { pub scale: f64, pub norm: f64, pub step_count: u64,
     pub found_inf: u32, pub clipped: u32 }
-pub enum NboList {} pub enum NboOptim {} pub enum NboScaler {}
+pub enum NboList {} pub enum NboOptim {} pub enum NboScaler {} pub enum NboPlaced {}
 
 pub const NBO_DT_F32: c_int = 0; pub const NBO_DT_BF16: c_int = 1; pub const NBO_DT_F64: c_int = 2;
 pub const NBO_DT_F16: c_int = 3;
@@ -111,6 +111,11 @@ extern "C" {
     pub fn nbo_optim_state_placement_note(opt: *mut NboOptim, buf: *mut c_char, buf_bytes: u64) -> c_int;
     pub fn nbo_status_string(status: c_int) -> *const c_char;
     pub fn nbo_version() -> *const c_char;
+    // (measurement) the caller's tensors in named HBM regions
+    pub fn nbo_alloc_placed(n_buffers: u32, bytes: u64, region: *const c_int, out_ptrs: *mut *mut c_void,
+                            out: *mut *mut NboPlaced) -> c_int;
+    pub fn nbo_free_placed(p: *mut NboPlaced) -> c_int;
+    pub fn nbo_placed_note(p: *mut NboPlaced, buf: *mut c_char, buf_bytes: u64) -> c_int;
     // measurement helpers of nabla_optim_bench.h (no counterpart in the reference)
     pub fn nbo_copy_bytes(src_dev: *const c_void, dst_dev: *mut c_void, bytes: u64) -> c_int;
     pub fn nbo_hbm_ceiling(pattern: c_int, spread: c_int, bytes_per_stream: u64, reps: c_int, settle_ms: u32,

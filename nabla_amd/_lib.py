@@ -148,6 +148,9 @@ BENCH_SYMBOLS = {
     "nbo_hbm_ceiling_compare": (C.c_int, [C.c_int, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_uint32), C.c_int,
                                           C.c_uint64, C.c_int, C.c_int, C.c_uint32, C.POINTER(C.c_double),
                                           C.POINTER(C.c_double), C.POINTER(C.c_int)]),
+    "nbo_alloc_placed": (C.c_int, [C.c_uint32, C.c_uint64, C.POINTER(C.c_int), C.POINTER(_P), C.POINTER(_P)]),
+    "nbo_free_placed": (C.c_int, [_P]),
+    "nbo_placed_note": (C.c_int, [_P, C.c_char_p, C.c_uint64]),
     "nbo_profile_enable": (C.c_int, [C.c_int]),
     "nbo_profile_read": (C.c_int, [C.c_char_p, _U64P, C.POINTER(C.c_double)]),
 }

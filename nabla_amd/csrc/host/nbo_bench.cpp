@@ -231,6 +231,65 @@ int nbo_hbm_ceiling_compare(int pattern, int n_shapes, const int *shapes, const 
     });
 }
 
+// ---- the caller's own tensors in named HBM regions (a measurement, see the header) ------------
+
+int nbo_alloc_placed(uint32_t n_buffers, uint64_t bytes, const int *region, void **out_ptrs, nbo_placed **out)
+{
+    return guarded([&] {
+        require(out != nullptr, NBO_ERR_ARG, "null output pointer");
+        *out = nullptr;
+        require(n_buffers >= 2 && n_buffers <= 3 && region && out_ptrs, NBO_ERR_ARG,
+                "two or three buffers, with a region number each");
+        bool rotate = true; // every region number -1: the rotation the optimizer's own state gets
+        for (uint32_t k = 0; k < n_buffers; k++) rotate = rotate && region[k] == -1;
+        for (uint32_t k = 0; k < n_buffers && !rotate; k++)
+            require(region[k] >= 0 && region[k] < 3, NBO_ERR_ARG, "region numbers are 0, 1 or 2 (or -1 for all buffers)");
+        require(bytes > 0, NBO_ERR_ARG, "zero-sized buffers");
+        Runtime::get(); // the probe kernel lives in the runtime's code object
+        nbo_placed *p = new nbo_placed();
+        void *ptrs[3] = {nullptr, nullptr, nullptr};
+        bool placed = false;
+        try {
+            if (rotate) {
+                p->placement.allocate(n_buffers, (size_t)bytes, ptrs);
+                placed = p->placement.regions_used() >= 2;
+            } else {
+                placed = p->placement.allocate_whole(n_buffers, (size_t)bytes, region, ptrs);
+            }
+        } catch (...) {
+            delete p;
+            throw;
+        }
+        if (!placed) {
+            const std::string why = p->placement.note();
+            delete p;
+            fail(NBO_ERR_TOO_LARGE, "nbo_alloc_placed: " + why);
+        }
+        for (uint32_t k = 0; k < n_buffers; k++) out_ptrs[k] = ptrs[k];
+        *out = p;
+    });
+}
+
+int nbo_free_placed(nbo_placed *p)
+{
+    return guarded([&] {
+        if (!p) return;
+        Runtime::get().sync();
+        delete p; // ~StatePlacement unmaps and releases
+    });
+}
+
+int nbo_placed_note(nbo_placed *p, char *buf, uint64_t buf_bytes)
+{
+    return guarded([&] {
+        require(p && buf && buf_bytes > 0, NBO_ERR_ARG, "null handle or buffer");
+        const std::string &n = p->placement.note();
+        const size_t k = n.size() < buf_bytes - 1 ? n.size() : (size_t)(buf_bytes - 1);
+        std::memcpy(buf, n.data(), k);
+        buf[k] = '\0';
+    });
+}
+
 int nbo_profile_enable(int on)
 {
     return guarded([&] { Runtime::get().profile_enable(on != 0); });

@@ -184,6 +184,11 @@ struct nbo_optim {
     size_t elem_bytes() const { return state_dtype == NBO_DT_F64 ? 8 : nbo::is_half(state_dtype) ? 2 : 4; }
 };
 
+// Buffers handed out by nbo_alloc_placed: whole arrays in named HBM regions.
+struct nbo_placed {
+    nbo::StatePlacement placement;
+};
+
 namespace nbo {
 // NBLA tensor files (nbo_nbla.cpp)
 void nbla_save_list(const char *path, const nbo_list *list, const char *const *names);

@@ -96,7 +96,19 @@ void StatePlacement::allocate(uint32_t nparts, size_t bytes, void **out)
     }
 }
 
-bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
+bool StatePlacement::allocate_whole(uint32_t nparts, size_t bytes, const int *slot_of, void **out)
+{
+    release();
+    note_.clear();
+    for (uint32_t k = 0; k < 3; k++) out[k] = nullptr;
+    if (nparts < 2 || nparts > 3) note_ = "two or three arrays can be placed against each other";
+    else if (bytes < kMinPlacedBytes) note_ = "less than 128 MiB per array: regions are told apart in chunks of 1 GiB";
+    else if (try_placed(nparts, bytes, out, slot_of)) return true;
+    if (std::getenv("NBO_PLACEMENT_DEBUG")) std::fprintf(stderr, "[nbo placement] %s\n", note_.c_str());
+    return false;
+}
+
+bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out, const int *slot_of)
 {
     Runtime &rt = Runtime::get();
     // 1 GiB: large enough for a steady probe, small enough that a chunk the driver pieced
@@ -104,8 +116,9 @@ bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
     const size_t chunk = kGiB;
     // a part smaller than one chunk still gets a whole chunk of its own (regions can
     // only be told apart at this granularity); larger parts are whole chunks plus a tail
-    const size_t full = bytes < chunk ? 1 : bytes / chunk;
-    const size_t tail = bytes < chunk ? 0 : round_up(bytes - full * chunk, kMapGranule);
+    // (whole arrays in named regions are rounded up to whole chunks: a tail would lie anywhere)
+    const size_t full = slot_of ? (bytes + chunk - 1) / chunk : bytes < chunk ? 1 : bytes / chunk;
+    const size_t tail = slot_of || bytes < chunk ? 0 : round_up(bytes - full * chunk, kMapGranule);
     const size_t part_va = full * chunk + tail;
     const size_t total_full = full * nparts;
     auto give_up = [&](const std::string &why) {
@@ -210,7 +223,9 @@ bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
             size_t usable = chunks.size();
             if (usable && !chunks.back().ready) usable--; // the driver refused to map it or to open it for access
             finder.add_chunks(usable, probe, halves);
-            if (plan::enough(counts(), nparts, full)) break;
+            if (slot_of ? !plan::assign_whole(counts(), std::vector<int>(slot_of, slot_of + nparts), full).empty()
+                        : plan::enough(counts(), nparts, full))
+                break;
             if (!created || chunks.size() >= cap) break;
             target = std::min(cap, chunks.size() + std::max<size_t>({2, total_full / 4, chunks.size() / 4}));
         }
@@ -221,10 +236,20 @@ bool StatePlacement::try_placed(uint32_t nparts, size_t bytes, void **out)
             for (const auto &r : region_chunks) std::fprintf(stderr, " %zu", r.size());
             std::fprintf(stderr, "; %zu needed\n", total_full);
         }
-        if (region_chunks.size() < 2)
+        const bool one_region_will_do = slot_of && std::all_of(slot_of, slot_of + nparts, [&](int x) { return x == slot_of[0]; });
+        if (region_chunks.size() < 2 && !one_region_will_do)
             return fail_with(fmt("%.0f chunks created and probed, all read as one region (two halves of a chunk: %.0f GB/s)",
                                  (double)chunks.size(), finder.same_pair()));
-        const std::vector<std::vector<int>> pick_region = plan::assign(counts(), nparts, full);
+        std::vector<std::vector<int>> pick_region;
+        if (slot_of) { // every array wholly in its slot's region
+            const std::vector<int> region_of_slot =
+                plan::assign_whole(counts(), std::vector<int>(slot_of, slot_of + nparts), full);
+            if (!region_of_slot.empty())
+                for (uint32_t j = 0; j < nparts; j++)
+                    pick_region.push_back(std::vector<int>(full, region_of_slot[(size_t)slot_of[j]]));
+        } else {
+            pick_region = plan::assign(counts(), nparts, full);
+        }
         if (pick_region.empty()) return fail_with("ran out of memory before enough chunks were collected");
         std::vector<std::vector<size_t>> pick(nparts);
         for (uint32_t j = 0; j < nparts; j++)

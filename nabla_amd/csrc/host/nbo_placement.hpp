@@ -53,6 +53,12 @@ public:
     // Allocates nparts (<= 3) arrays of `bytes` bytes each; out[k] receives their device
     // addresses.  Contents are unspecified.  Throws nbo::Error on out-of-memory.
     void allocate(uint32_t nparts, size_t bytes, void **out);
+    // The same search, another layout: array j lies wholly in one region, the one numbered
+    // slot_of[j] (0, 1 or 2; equal numbers share a region, different numbers get different ones).
+    // For memory the caller itself reads and writes -- parameters in one region, gradients in
+    // another -- rather than the engine's state.  Returns false, having allocated nothing, where
+    // allocate() would have fallen back to plain hipMalloc (note() says why).
+    bool allocate_whole(uint32_t nparts, size_t bytes, const int *slot_of, void **out);
     void release();
 
     // How the last allocate() went, for logs and tests: 0 = plain hipMalloc,
@@ -62,7 +68,7 @@ public:
     const std::string &note() const { return note_; }
 
 private:
-    bool try_placed(uint32_t nparts, size_t bytes, void **out);
+    bool try_placed(uint32_t nparts, size_t bytes, void **out, const int *slot_of = nullptr);
 
     std::vector<void *> plain_;                               // hipMalloc'ed parts
     std::vector<hipMemGenericAllocationHandle_t> handles_;    // chunks in use

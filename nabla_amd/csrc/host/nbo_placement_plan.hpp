@@ -245,6 +245,33 @@ inline std::vector<std::vector<int>> assign(std::vector<size_t> avail, uint32_t 
     return pick;
 }
 
+// Whole arrays in one region each (the caller's own tensors: parameters here, gradients there).
+// slot_of[j] names the region array j is to lie in -- a number below kMaxRegions; equal numbers
+// share a region, different numbers get different regions.  Returns the region (index into
+// `avail`) of every slot in use, -1 for unused slots; the slot that needs most chunks gets the
+// region that has most.  Empty result: the chunks at hand do not allow it.
+inline std::vector<int> assign_whole(const std::vector<size_t> &avail, const std::vector<int> &slot_of, size_t full)
+{
+    std::vector<size_t> need(kMaxRegions, 0);
+    for (int s : slot_of) {
+        if (s < 0 || (size_t)s >= kMaxRegions) return {};
+        need[(size_t)s] += full;
+    }
+    std::vector<size_t> slots, regions;
+    for (size_t s = 0; s < kMaxRegions; s++)
+        if (need[s]) slots.push_back(s);
+    for (size_t r = 0; r < avail.size(); r++) regions.push_back(r);
+    if (slots.size() > regions.size()) return {};
+    std::stable_sort(slots.begin(), slots.end(), [&](size_t a, size_t b) { return need[a] > need[b]; });
+    std::stable_sort(regions.begin(), regions.end(), [&](size_t a, size_t b) { return avail[a] > avail[b]; });
+    std::vector<int> out(kMaxRegions, -1);
+    for (size_t k = 0; k < slots.size(); k++) {
+        if (avail[regions[k]] < need[slots[k]]) return {};
+        out[slots[k]] = (int)regions[k];
+    }
+    return out;
+}
+
 // How many chunks the search may create (and hold until it is done) before it settles for what
 // it has.  Regions are runs of consecutively created chunks, up to 96 GiB long, so a search that
 // is to find a second region must be allowed to walk that far: twice what the arrays need plus

@@ -148,6 +148,72 @@ def ceilings_main(args) -> None:
     print("\nmean (best) GB/s")
 
 
+def placed_main(args) -> None:
+    """What placing the caller's own tensors buys: parameters and gradients (and a third list)
+    as flat buffers from `nbo_alloc_placed`, all in one region against spread over regions, for
+    the kernels whose streams are the caller's tensors."""
+    import time
+
+    import torch
+
+    from . import _lib
+    from . import backend as B
+    from . import optim as nb
+    from .placed import PlacedBuffers, carved_bytes
+
+    _lib.init()
+    L = _lib.load()
+    big = max(int(args.elements) // (8192 * 8192), 1)
+    shapes = [(8192, 8192)] * big + [(1, 4096)] * 8
+    n = sum(r * c for r, c in shapes)
+    print(f"{n} f32 elements in {len(shapes)} tensors per list, {args.reps} launches each; the lists are flat buffers from "
+          "`nbo_alloc_placed`, region numbers per list as given (equal numbers: the same HBM region)\n")
+    print("| entry point | kernel | regions of the lists | ms | bytes / element | GB/s |")
+    print("|---|---|---|---|---|---|")
+
+    def timeit(name, fn, bytes_per_elem, kname, where):
+        fn()
+        _lib.check(L.nbo_sync())
+        _lib.check(L.nbo_profile_enable(1))
+        for _ in range(args.reps):
+            fn()
+        _lib.check(L.nbo_sync())
+        cnt, ms = C.c_uint64(0), C.c_double(0)
+        _lib.check(L.nbo_profile_read(kname.encode(), C.byref(cnt), C.byref(ms)))
+        _lib.check(L.nbo_profile_enable(0))
+        t = ms.value / max(cnt.value, 1)
+        print(f"| {name} | `{kname}` | {where} | {t:.3f} | {bytes_per_elem} | {n * bytes_per_elem / t / 1e6:.0f} |", flush=True)
+
+    nbytes = carved_bytes(shapes, 4)
+    for regions in ((0, 0, 0), (0, 1, 0), (0, 1, 1), (-1, -1, -1)):
+        time.sleep(3.0)  # the driver is still clearing what the previous search released
+        try:
+            bufs = PlacedBuffers(nbytes, regions)
+        except Exception as e:  # e.g. no third region on this box
+            print(f"| (regions {regions}: {e}) | | | | | |", flush=True)
+            continue
+        time.sleep(4.0)
+        tensors = [bufs.carve(k, shapes, torch.float32) for k in range(3)]
+        for t3, sigma in zip(tensors, (0.02, 1e-3, 1.0)):
+            for t in t3:
+                t.normal_(0.0, sigma)
+        p, g, o = (nb.TensorList(t) for t in tensors)
+        where = f"params {regions[0]}, grads {regions[1]}, third {regions[2]}"
+        sgd = nb.Sgd.new(0.01, shapes)
+        timeit("Sgd::step f32", lambda: sgd.step(p, g), 12, "nbo_update_f32_sgd", where)
+        del sgd
+        adam = nb.Adam.new(1e-3, shapes)
+        timeit("Adam::step f32", lambda: adam.step(p, g), 28, "nbo_update_f32_adam_self",
+               where + f"; m, v: {adam.state_placement_note().split(';')[0]}")
+        del adam
+        timeit("accumulate f32", lambda: nb.accumulate(p, g), 12, "nbo_accum_f32", where)
+        timeit("backend add f32", lambda: B.add(p, g, out=o), 12, "nbo_ew_f32", where)
+        timeit("backend scale f32", lambda: B.scale(p, 0.5, out=o), 8, "nbo_ew_f32", where)
+        timeit("scale_grad f32", lambda: nb.scale_grad(g, 0.5), 8, "nbo_scale_f32", where)
+        del p, g, o, tensors
+        bufs.close()
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--elements", type=float, default=805e6)
@@ -159,6 +225,9 @@ def main() -> None:
                     help="all access shapes over the same buffers, measured in turn (differences of a per cent "
                          "show here; --ceilings allocates anew for every row)")
     ap.add_argument("--rounds", type=int, default=5, help="--compare: rounds over all shapes")
+    ap.add_argument("--placed", action="store_true",
+                    help="the kernels over the caller's tensors with those tensors placed in named HBM regions "
+                         "(nbo_alloc_placed): one region against several")
     ap.add_argument("--summarize", metavar="DIR", help="turn the rocprofv3 output under DIR into profiles/ summaries "
                                                         "(see nabla_amd/profile_summary.py) instead of measuring")
     args = ap.parse_args()
@@ -170,6 +239,10 @@ def main() -> None:
     if args.compare:
         args.reps = args.reps or 5
         compare_main(args)
+        return
+    if args.placed:
+        args.reps = args.reps or 5
+        placed_main(args)
         return
     if args.ceilings:
         args.reps = args.reps or 10

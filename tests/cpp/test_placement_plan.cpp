@@ -254,6 +254,21 @@ int main()
         for (size_t i = 0; i < 3; i++) CHECK(!(pick[0][i] == pick[1][i] && pick[1][i] == pick[2][i]));
     }
 
+    // whole arrays in named regions: equal numbers share a region, different numbers do not; the
+    // slot that needs most gets the region that has most; not enough of anything gives no plan
+    {
+        const auto r = assign_whole({5, 9}, {0, 1}, 4); // two arrays of 4 chunks, apart
+        CHECK(r.size() == kMaxRegions && r[0] != r[1] && r[0] >= 0 && r[1] >= 0 && r[2] == -1);
+        const auto same = assign_whole({5, 9}, {1, 1}, 4); // both in one region: the one with 9
+        CHECK(same.size() == kMaxRegions && same[1] == 1 && same[0] == -1);
+        const auto two_one = assign_whole({4, 9}, {0, 0, 2}, 4); // slot 0 needs 8: region 1; slot 2 the other
+        CHECK(two_one.size() == kMaxRegions && two_one[0] == 1 && two_one[2] == 0);
+        CHECK(assign_whole({3, 9}, {0, 1}, 4).empty());       // the second region is too small
+        CHECK(assign_whole({9}, {0, 1}, 4).empty());          // one region found, two asked for
+        CHECK(assign_whole({9, 9, 9}, {0, 1, 2}, 9).size() == kMaxRegions);
+        CHECK(assign_whole({9, 9}, {0, 3}, 1).empty());       // no such slot
+    }
+
     // the creation limit: twice the need plus eight or far enough to cross a region boundary
     // (within half of what is free), a user's limit instead, never more than is free
     CHECK(chunk_cap(12, 250, 0, 104) == 104);

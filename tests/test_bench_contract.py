@@ -133,3 +133,47 @@ def test_every_probe_shape_touches_each_vector_exactly_once_per_launch(gpu):
                      lambda: L.nbo_hbm_ceiling_shape(9, len(KB.SHAPES), 0, nbytes, 2, 0, C.byref(best), C.byref(mean), None, None),
                      lambda: L.nbo_hbm_ceiling_shape(9, 6, 0, 32768, 2, 0, C.byref(best), C.byref(mean), None, None)):
         assert bad_call() == _lib.ERR_ARG
+
+
+@pytest.mark.gpu
+def test_placed_buffers_are_usable_memory_in_the_regions_asked_for(gpu):
+    """`nbo_alloc_placed` (measurement entry point): two buffers in different regions, then the
+    rotation the optimizer's state gets; the memory is ordinary device memory (torch reads and
+    writes it, the engine steps over tensors carved from it), and the argument checks hold."""
+    import ctypes as C
+
+    import numpy as np
+    import torch
+
+    import oracle as O
+    from nabla_amd import _lib
+    from nabla_amd import optim as nb
+    from nabla_amd.placed import PlacedBuffers, carved_bytes
+    from tests import helpers as H
+
+    shapes = [(4096, 8192), (1, 4097), (3, 5)]
+    nbytes = carved_bytes(shapes, 4)
+    for regions in ((0, 1), (-1, -1)):
+        bufs = PlacedBuffers(nbytes, regions)
+        assert "2 regions" in bufs.note() or "3 regions" in bufs.note(), bufs.note()
+        p_t, g_t = bufs.carve(0, shapes, torch.float32), bufs.carve(1, shapes, torch.float32)
+        p0, g0 = H.randn_list(shapes[1:], 5, 0.02), H.randn_list(shapes[1:], 6, 1e-2)
+        p_t[0].zero_(), g_t[0].fill_(1.0)
+        for t, a in zip(p_t[1:], p0):
+            t.copy_(torch.from_numpy(a).reshape(t.shape))
+        for t, a in zip(g_t[1:], g0):
+            t.copy_(torch.from_numpy(a).reshape(t.shape))
+        opt = nb.Sgd.new(0.5, shapes)
+        opt.step(p_t, g_t)
+        ref, vel = H.copy_list(p0), H.zeros_like_list(p0)
+        O.sgd_step(O.sgd_meta(0.5), ref, g0, vel)
+        H.assert_bits_equal(H.host_list(p_t[1:]), ref, f"SGD step over placed buffers, regions {regions}")
+        assert bool((p_t[0] == -0.5).all())
+        del p_t, g_t, opt
+        bufs.close()
+    L = _lib.load()
+    h, ptrs = C.c_void_p(), (C.c_void_p * 3)()
+    for n, reg in ((1, [0]), (4, [0, 1, 2, 0]), (2, [0, 3]), (2, [0, -1])):
+        assert L.nbo_alloc_placed(n, 1 << 30, (C.c_int * len(reg))(*reg), ptrs, C.byref(h)) == _lib.ERR_ARG
+    assert L.nbo_alloc_placed(2, 1 << 20, (C.c_int * 2)(0, 1), ptrs, C.byref(h)) == _lib.ERR_TOO_LARGE  # below 128 MiB
+    assert L.nbo_free_placed(None) == 0
