@@ -500,8 +500,12 @@ def measure(name, steps, warmup, zero_grads="off", settle_s=2.0):
         traffic = table.get(f"{name}:{dom}")
         det = table.get("_detail", {}).get(name, {})
         if traffic is not None:
+            from nabla_amd.profile_summary import kernel_source_hash
+
+            same = det.get("kernel_source_sha256") == kernel_source_hash()
             traffic_source = (f"profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command at "
-                              f"commit {det.get('commit', '?')} on {det.get('date', '?')}; not measured in this run)")
+                              f"commit {det.get('commit', '?')} on {det.get('date', '?')}; not measured in this run; the "
+                              f"kernel source is {'the one' if same else 'NOT the one'} those counters were collected for)")
 
     out = {
         "metric": "AdamW step HBM GB/s (% of peak) + params/s, bf16-mixed, whole step "

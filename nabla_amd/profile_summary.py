@@ -58,6 +58,21 @@ def _mean(xs):
     return sum(xs) / len(xs)
 
 
+KERNEL_SOURCES = ("nabla_amd/csrc/kernels/nbo_kernels.hip", "nabla_amd/csrc/nbo_device_types.h")
+
+
+def kernel_source_hash() -> str:
+    """sha256 over the files the step's kernels are compiled from: what a set of counters was
+    collected for.  profiles/traffic.json stores it, bench.py and the tests compare it."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
 def _commit():
     try:
         return subprocess.run(["git", "rev-parse", "--short", "HEAD"], cwd=ROOT, capture_output=True,
@@ -161,7 +176,8 @@ def summarize(base: str) -> str:
     table["_detail"][workload] = {
         "per_launch_bytes": traffic,
         "calibration": {"fetch_KiB_per_unit": f_scale, "write_KiB_per_unit": w_scale},
-        "source": md, "commit": _commit(), "date": datetime.date.today().isoformat()}
+        "source": md, "commit": _commit(), "date": datetime.date.today().isoformat(),
+        "kernel_source_sha256": kernel_source_hash()}
     with open(tpath, "w") as f:
         json.dump(table, f, indent=1)
     return text

@@ -43,6 +43,14 @@ def test_traffic_file_is_consistent_with_the_profile_summary():
     det = t["_detail"].get("llama3-8b", t["_detail"])  # per-workload layout; single-workload in older files
     d = det["per_launch_bytes"]["nbo_update_bf16_adamw"]
     assert d["fetch_bytes"] + d["write_bytes"] == total
+    # the counters were collected for the kernels as they are now: the file carries a hash of the
+    # kernel source of its profile run, and a change to the kernels asks for a new run
+    from nabla_amd.profile_summary import kernel_source_hash
+
+    for workload in ("llama3-8b", "llama-1.1b"):
+        assert t["_detail"][workload].get("kernel_source_sha256") == kernel_source_hash(), (
+            f"profiles/traffic.json [{workload}] was collected for other kernel source: run the commands at the top "
+            "of profiles/adamw_fused_step_*.md again and `python -m nabla_amd.kernel_bench --summarize`")
 
 
 @pytest.mark.gpu
