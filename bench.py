@@ -314,18 +314,29 @@ def parity_check(cfg, steps=3):
         finally:
             O.set_pow_mode(O.POW_LIBM)
 
+    # Where a parameter and its update nearly cancel, one ulp of the update (the reference's
+    # powf(x, 0.5) against the correctly rounded sqrt) is many ulps of the tiny result: such an
+    # element is held to |difference| <= steps * 8 * lr * 2^-23 and magnitude < 16 * lr * steps.
+    bound, small = steps * 8 * cfg["lr"] * 2.0 ** -23, 16.0 * cfg["lr"] * steps
+
     def compare(ref):
         out = {}
         for key, arrs in got.items():
             sixteen = arrs[0].dtype in (np.uint16, np.float16)
-            worst = beyond = 0
+            worst = beyond = outside = 0
             for a, b in zip(arrs, ref[key]):
                 if not a.size:
                     continue
                 d = O.ulp_distance_bf16(a.view(np.uint16), b.view(np.uint16)) if sixteen else O.ulp_distance_f32(a, b)
                 worst = max(worst, int(d.max()))
-                beyond += int((d > (1 if sixteen else 2)).sum())
-            out[key] = {"max_ulp": worst, "beyond_bar": beyond}
+                far = d > (1 if sixteen else 2)
+                beyond += int(far.sum())
+                if far.any() and not sixteen:
+                    x, y = a[far].astype(np.float64), b[far].astype(np.float64)
+                    outside += int(((np.abs(x - y) > bound) | (np.maximum(np.abs(x), np.abs(y)) >= small)).sum())
+                elif far.any():
+                    outside += int(far.sum())
+            out[key] = {"max_ulp": worst, "beyond_bar": beyond, "beyond_bar_and_outside_the_cancellation_clause": outside}
         return out
 
     ref_sqrt, dec_sqrt = oracle_run(O.POW_SQRT)
@@ -333,7 +344,9 @@ def parity_check(cfg, steps=3):
     return {
         "sample": f"first {len(sample)} tensors of the workload ({n} params), {steps} steps, inputs from the "
                   "reference's xorshift64 + Box-Muller generator",
-        "bar": "f32 states within 2 ulp, 16-bit params within 1 ulp, decisions bit-exact",
+        "bar": "f32 states within 2 ulp, 16-bit params within 1 ulp, decisions bit-exact; an f32 parameter beyond 2 ulp "
+               f"must differ by at most steps * 8 * lr * 2^-23 = {bound:.3e} and be smaller than 16 * lr * steps = "
+               f"{small:.3e} (near-cancellation of parameter and update)",
         "decisions_bit_exact": (not fused) or (dev_decisions == dec_sqrt == dec_libm),
         "vs_oracle_sqrt": compare(ref_sqrt),
         "vs_oracle_libm_powf": compare(ref_libm),
@@ -607,7 +620,7 @@ def main():
               "workload.\n")
         print("| workload | params | ms/step (min / median / max) | value GB/s | % of 8 TB/s | params/s | dominant kernel "
               "GB/s | HBM regions of state | CPU params/s (cores) | GPU/CPU | parity vs sqrt oracle: max ulp m / v / "
-              "master / params | parity vs libm-powf oracle: max ulp m / v / master / params (elements beyond the bar) | "
+              "master / params | parity vs libm-powf oracle: max ulp m / v / master / params (elements beyond 2 ulp, or 1 ulp of a 16-bit type) | "
               "decisions |")
         print("|---|---|---|---|---|---|---|---|---|---|---|---|---|")
 
@@ -619,13 +632,14 @@ def main():
             c = cpu_baseline(cfg, args.cpu_seconds)
             par = parity_check(cfg)
             beyond = sum(x["beyond_bar"] for x in par["vs_oracle_libm_powf"].values())
+            outside = sum(x["beyond_bar_and_outside_the_cancellation_clause"] for x in par["vs_oracle_libm_powf"].values())
             sp = d["ms_per_step_spread"]
             print(f"| {name} | {d['config']['params']:,} | {d['ms_per_step']} ({sp['min']} / {sp['median']} / {sp['max']}) | "
                   f"{d['value']} | {d['pct_of_peak']} | "
                   f"{d['params_per_s']:.3e} | {d['roofline']['achieved']} ({d['roofline']['kernel']}) | "
                   f"{d['config']['state_hbm_regions']} | {c['params_per_s']:.3e} ({c['cores']}) | "
                   f"{d['params_per_s'] / c['params_per_s']:.0f}x | {ulps(par['vs_oracle_sqrt'])} | "
-                  f"{ulps(par['vs_oracle_libm_powf'])} ({beyond}) | "
+                  f"{ulps(par['vs_oracle_libm_powf'])} ({beyond}; outside the cancellation clause: {outside}) | "
                   f"{'bit-exact' if par['decisions_bit_exact'] else 'DIFFER'} |", flush=True)
         return
     out, cfg = measure(args.workload, args.steps, args.warmup, args.zero_grads, args.settle_seconds)
