@@ -143,8 +143,6 @@ uint32_t norm_grid(const Layout &L)
     return L.nchunks < NBO_NORM_GRID_MAX ? L.nchunks : NBO_NORM_GRID_MAX;
 }
 
-// First stage of the norm / found_inf pass over `grads`; partials land in the
-// runtime's scratch.  Returns the grid used (0 for an empty list).
 // Where a norm pass leaves its per-workgroup partial results for its second stage.
 struct NormScratch {
     double *partial_sumsq;  // [NBO_NORM_GRID_MAX]
