@@ -56,7 +56,11 @@ typedef enum nbo_probe_shape {
     NBO_SHAPE_FRONTS2 = 12,   /* shape 0's eight rows taken from 2 places of every stream at once (a grid apart) */
     NBO_SHAPE_FRONTS4 = 13,   /* ... from 4 places */
     NBO_SHAPE_FRONTS8 = 14,   /* ... from 8 places */
-    NBO_SHAPE_COUNT = 15
+    NBO_SHAPE_ROWS4 = 15,     /* shape 0 with four rows per workgroup (16 KiB windows) */
+    NBO_SHAPE_ROWS2 = 16,     /* ... two rows (8 KiB windows) */
+    NBO_SHAPE_ROWS1 = 17,     /* ... one row: every thread loads one vector of every stream, stores, and is done (4 KiB
+                                 windows, eight times as many workgroups as shape 0) */
+    NBO_SHAPE_COUNT = 18
 } nbo_probe_shape;
 
 /* What the memory system gives an access pattern, measured with the library's probe kernels:

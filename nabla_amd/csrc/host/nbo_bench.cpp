@@ -66,7 +66,10 @@ ShapeGeometry geometry(int pattern, int shape)
     // the front shapes' workgroups cover F windows of 8 / F rows; "iters" = F makes the grid come out right
     case NBO_SHAPE_FRONTS2: return {256, 256 * 4, 2};
     case NBO_SHAPE_FRONTS4: return {256, 256 * 2, 4};
-    default: return {256, 256 * 1, 8}; // NBO_SHAPE_FRONTS8
+    case NBO_SHAPE_FRONTS8: return {256, 256 * 1, 8};
+    case NBO_SHAPE_ROWS4: return {256, 256 * 4, 1};
+    case NBO_SHAPE_ROWS2: return {256, 256 * 2, 1};
+    default: return {256, 256 * 1, 1}; // NBO_SHAPE_ROWS1
     }
 }
 

@@ -158,7 +158,7 @@ int Runtime::bench_kernel(const char *name)
     return K_COUNT + (int)bench_names_.size() - 1;
 }
 
-void Runtime::launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct, bool may_time)
+void Runtime::launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct, bool may_time, uint32_t idle_lds)
 {
     if (grid == 0) return;
     const hipFunction_t fn = function(kernel);
@@ -170,7 +170,7 @@ void Runtime::launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_st
         hip_check(hipEventCreate(&rec.end), "hipEventCreate");
         hip_check(hipEventRecord(rec.begin, stream_), "hipEventRecord");
     }
-    hip_check(hipModuleLaunchKernel(fn, grid, 1, 1, block, 1, 1, 0, stream_, args, nullptr), kernel_name(kernel));
+    hip_check(hipModuleLaunchKernel(fn, grid, 1, 1, block, 1, 1, idle_lds, stream_, args, nullptr), kernel_name(kernel));
     if (timed) {
         hip_check(hipEventRecord(rec.end, stream_), "hipEventRecord");
         prof_.push_back(rec);

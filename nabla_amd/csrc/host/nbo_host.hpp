@@ -73,13 +73,18 @@ public:
     void set_stream(hipStream_t s);
     void sync();
 
-    template <typename Args> void launch(int kernel, uint32_t grid, uint32_t block, const Args &args)
+    // idle_lds: bytes of LDS every workgroup is given and never touches.  It caps the workgroups
+    // a compute unit holds (160 KiB / idle_lds of them): passes that write at least as much as
+    // they read run faster with fewer in flight.
+    template <typename Args>
+    void launch(int kernel, uint32_t grid, uint32_t block, const Args &args, uint32_t idle_lds = 0)
     {
-        launch_raw(kernel, grid, block, const_cast<Args *>(&args));
+        launch_raw(kernel, grid, block, const_cast<Args *>(&args), true, idle_lds);
     }
     // may_time = false: never bracket the launch with timing events, whatever profile_enable
     // says (creating events allocates host memory)
-    void launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct, bool may_time = true);
+    void launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct, bool may_time = true,
+                    uint32_t idle_lds = 0);
     // Id of kernel `name` of the measurement code object (nbo_bench_kernels.hip), which is
     // loaded when the first such id is asked for; the id works with launch, time_launches and
     // the per-kernel timing like the ids above.

@@ -514,3 +514,19 @@ PROBE_KERNEL(nbo_probe_copy_s14, 256, (probe_fronts<1, 0, 1, 8>))
 PROBE_KERNEL(nbo_probe_rmw1_s14, 256, (probe_fronts<0, 1, 0, 8>))
 PROBE_KERNEL(nbo_probe_rmw3_s14, 256, (probe_fronts<0, 3, 0, 8>))
 PROBE_KERNEL(nbo_probe_r1_rmw3_w1_s14, 256, (probe_fronts<1, 3, 1, 8>))
+
+// shapes 15-17: shape 0 with 4, 2 and 1 rows per workgroup -- more, shorter-lived workgroups
+PROBE_KERNEL(nbo_probe_copy_s15, 256, (probe_regs<1, 0, 1, 256, 4>))
+PROBE_KERNEL(nbo_probe_rmw1_s15, 256, (probe_regs<0, 1, 0, 256, 4>))
+PROBE_KERNEL(nbo_probe_rmw3_s15, 256, (probe_regs<0, 3, 0, 256, 4>))
+PROBE_KERNEL(nbo_probe_r1_rmw3_w1_s15, 256, (probe_regs<1, 3, 1, 256, 4>))
+
+PROBE_KERNEL(nbo_probe_copy_s16, 256, (probe_regs<1, 0, 1, 256, 2>))
+PROBE_KERNEL(nbo_probe_rmw1_s16, 256, (probe_regs<0, 1, 0, 256, 2>))
+PROBE_KERNEL(nbo_probe_rmw3_s16, 256, (probe_regs<0, 3, 0, 256, 2>))
+PROBE_KERNEL(nbo_probe_r1_rmw3_w1_s16, 256, (probe_regs<1, 3, 1, 256, 2>))
+
+PROBE_KERNEL(nbo_probe_copy_s17, 256, (probe_regs<1, 0, 1, 256, 1>))
+PROBE_KERNEL(nbo_probe_rmw1_s17, 256, (probe_regs<0, 1, 0, 256, 1>))
+PROBE_KERNEL(nbo_probe_rmw3_s17, 256, (probe_regs<0, 3, 0, 256, 1>))
+PROBE_KERNEL(nbo_probe_r1_rmw3_w1_s17, 256, (probe_regs<1, 3, 1, 256, 1>))

@@ -47,6 +47,7 @@ typedef float f32x4_e __attribute__((ext_vector_type(4), aligned(4)));
 typedef double f64x2_e __attribute__((ext_vector_type(2), aligned(8)));
 
 #define DEV static __device__ __forceinline__
+#define MEMBER __device__ __forceinline__
 
 // Tuning knobs (the defaults are the measured best on MI355X).
 #ifndef NBO_UNROLL
@@ -500,7 +501,13 @@ DEV void make_uniform(NboOptimDev &o)
 // workgroup has read it: each workgroup, once its read has returned, adds one to a counter in
 // device memory, and the workgroup whose addition completes the grid -- nobody waits for
 // anybody -- writes the advanced step_count and the trace entry and clears the counter.
-template <int ST, int KIND> DEV void update_chunk(const NboUpdateArgs &a, const NboOptimDev *o)
+//
+// BY_ROW (the SGD kernels outside a grouped step): one workgroup per row of a chunk -- every
+// thread loads one vector of every stream, computes, stores and is done.  With SGD's two or
+// three streams that measured 15-20 % faster than eight rows per workgroup (as it does for the
+// element-wise passes, see stream_pieces); the Adam kinds' five streams do best at eight rows.
+// A chunk that is ragged, misaligned or skipped is done by the workgroup of its first row.
+template <int ST, int KIND, bool BY_ROW = false> DEV void update_chunk(const NboUpdateArgs &a, const NboOptimDev *o)
 {
     typedef typename Traits<ST>::T T;
     enum {
@@ -508,15 +515,16 @@ template <int ST, int KIND> DEV void update_chunk(const NboUpdateArgs &a, const 
         SB = Traits<ST>::SBYTES,
         ROW = NBO_BLOCK * VEC,
         ROWS = NBO_CHUNK / ROW,
-        UMAX = sizeof(T) == 8 ? NBO_UNROLL / 2 : NBO_UNROLL,
+        UMAX = BY_ROW ? 1 : sizeof(T) == 8 ? NBO_UNROLL / 2 : NBO_UNROLL,
         U = ROWS < UMAX ? ROWS : UMAX,
-        ITERS = ROWS / U
+        ITERS = BY_ROW ? 1 : ROWS / U
     };
     static_assert(ROWS % U == 0 && ROWS * ROW == NBO_CHUNK, "chunk must be a whole number of unrolled rows");
     const bool mixed = ST == NBO_BF16 || ST == NBO_F16; // f32 master lives in the arena
     const bool has_v = KIND != NBO_SGD;
     const uint32_t tid = threadIdx.x;
-    const ChunkRef c = chunk_ref(a.L, blockIdx.x);
+    const uint32_t row0 = BY_ROW ? blockIdx.x % ROWS : 0;
+    const ChunkRef c = chunk_ref(a.L, BY_ROW ? blockIdx.x / ROWS : blockIdx.x);
 
     char *pp = (char *)a.p_ptrs[c.t] + c.base * SB;
     char *pg = (char *)a.g_ptrs[c.t] + c.base * SB;
@@ -528,11 +536,12 @@ template <int ST, int KIND> DEV void update_chunk(const NboUpdateArgs &a, const 
     const bool vec_ok = ((((uintptr_t)pp) | ((uintptr_t)pg)) & (vbytes - 1)) == 0;
 
     const bool direct = KIND == NBO_SGD && a.direct != 0;
+    if (BY_ROW && row0 != 0 && !(c.cnt == NBO_CHUNK && vec_ok)) return;
     if (!direct && o->skip) {
         // found_inf: parameters, moments and step_count stay untouched
         // (trainer.rs:230-236); the gradients become zeros (core.rs:372-375) if the caller
         // asked for zeroing, after every step or after a skipped one only.
-        if (a.zero_grads != 0)
+        if (a.zero_grads != 0 && row0 == 0)
             for (uint32_t i = tid; i < c.cnt; i += NBO_BLOCK) IO<ST>::st1(pg + (uint64_t)i * SB, (T)0);
         return;
     }
@@ -547,7 +556,7 @@ template <int ST, int KIND> DEV void update_chunk(const NboUpdateArgs &a, const 
             // then sees longer runs per stream, which measured 1.3 % faster on the 8B set (35.0
             // against 35.5 ms in alternating launches inside one process; loads or stores alone
             // in this order: next to nothing).
-            const uint32_t e0 = it * (U * ROW) + tid * VEC;
+            const uint32_t e0 = (BY_ROW ? row0 : it * U) * ROW + tid * VEC;
             T g[U][VEC], p[U][VEC], m[U][VEC] = {}, v[U][VEC] = {};
 #pragma unroll
             for (int u = 0; u < U; u++) IO<ST>::ldv(pg + (uint64_t)(e0 + u * ROW) * SB, g[u]);
@@ -641,7 +650,7 @@ template <int ST, int KIND> DEV void update_chunk(const NboUpdateArgs &a, const 
 template <int ST, int KIND, bool SELF = false> DEV void update_body(const NboUpdateArgs &a)
 {
     if (!SELF) {
-        update_chunk<ST, KIND>(a, a.opt);
+        update_chunk<ST, KIND, KIND == NBO_SGD>(a, a.opt);
         return;
     }
     uint32_t sc_lo = (uint32_t)a.opt->step_count, sc_hi = (uint32_t)(a.opt->step_count >> 32);
@@ -1008,47 +1017,212 @@ NBO_NORM_KERNEL(nbo_norm_pbf16, NBO_PBF16)
 NBO_NORM_KERNEL(nbo_norm_f16, NBO_F16)
 NBO_NORM_KERNEL(nbo_norm_pf16, NBO_PF16)
 
+// Vector accesses of the element-wise passes: 128 bits wide for every element type, i.e. 8
+// elements of a 16-bit tensor computed in f32 (the update kernels take those 4 at a time, in
+// step with their 128-bit f32 state vectors).  A vector can be held as the raw bits it was
+// loaded as (a 16-bit tensor's eight values would take twice the registers once widened) and
+// unpacked into EV values of the arithmetic type only where they are used.
+template <typename T> struct Bits128;
+template <> struct Bits128<float> {
+    enum { EV = 4 };
+    DEV void unpack(int, u32x4 v, float (&x)[4])
+    {
+        x[0] = __uint_as_float(v.x); x[1] = __uint_as_float(v.y); x[2] = __uint_as_float(v.z); x[3] = __uint_as_float(v.w);
+    }
+    DEV u32x4 pack(int, const float (&x)[4])
+    {
+        const u32x4 v = {__float_as_uint(x[0]), __float_as_uint(x[1]), __float_as_uint(x[2]), __float_as_uint(x[3])};
+        return v;
+    }
+};
+template <> struct Bits128<double> {
+    enum { EV = 2 };
+    DEV void unpack(int, u32x4 v, double (&x)[2])
+    {
+        x[0] = __hiloint2double((int)v.y, (int)v.x);
+        x[1] = __hiloint2double((int)v.w, (int)v.z);
+    }
+    DEV u32x4 pack(int, const double (&x)[2])
+    {
+        const u32x4 v = {(uint32_t)__double2loint(x[0]), (uint32_t)__double2hiint(x[0]), (uint32_t)__double2loint(x[1]),
+                         (uint32_t)__double2hiint(x[1])};
+        return v;
+    }
+};
+template <int FMT> struct Bits128<Half16<FMT>> {
+    enum { EV = 8 };
+    DEV void unpack(int, u32x4 v, Half16<FMT> (&x)[8])
+    {
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            x[2 * k] = half_from_bits<FMT>(w[k] & 0xFFFFu);
+            x[2 * k + 1] = half_from_bits<FMT>(w[k] >> 16);
+        }
+    }
+    DEV u32x4 pack(int, const Half16<FMT> (&x)[8])
+    {
+        const u32x4 v = {(uint32_t)x[0].bits | ((uint32_t)x[1].bits << 16), (uint32_t)x[2].bits | ((uint32_t)x[3].bits << 16),
+                         (uint32_t)x[4].bits | ((uint32_t)x[5].bits << 16), (uint32_t)x[6].bits | ((uint32_t)x[7].bits << 16)};
+        return v;
+    }
+};
+// 16-bit tensors computed in f32
+struct Bits128HalfWide {
+    enum { EV = 8 };
+    DEV void unpack(int st, u32x4 v, float (&x)[8])
+    {
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            x[2 * k] = st == NBO_BF16 ? bf16_bits_to_f32(w[k] & 0xFFFFu) : f16_bits_to_f32(w[k] & 0xFFFFu);
+            x[2 * k + 1] = st == NBO_BF16 ? bf16_bits_to_f32(w[k] >> 16) : f16_bits_to_f32(w[k] >> 16);
+        }
+    }
+    DEV u32x4 pack(int st, const float (&x)[8])
+    {
+        uint32_t w[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+            w[k] = st == NBO_BF16 ? f32_to_bf16_bits(x[2 * k]) | (f32_to_bf16_bits(x[2 * k + 1]) << 16)
+                                  : f32_to_f16_bits(x[2 * k]) | (f32_to_f16_bits(x[2 * k + 1]) << 16);
+        const u32x4 v = {w[0], w[1], w[2], w[3]};
+        return v;
+    }
+};
+template <int ST> struct EwBits : Bits128<typename Traits<ST>::T> {};
+template <> struct EwBits<NBO_BF16> : Bits128HalfWide {};
+template <> struct EwBits<NBO_F16> : Bits128HalfWide {};
+
+template <int ST> struct EwIO {
+    typedef typename Traits<ST>::T T;
+    enum { EV = EwBits<ST>::EV };
+    DEV u32x4 ld(const char *p) { return NBO_LOAD(GLOBAL_PTR(const u32x4, p)); }
+    DEV void st(char *p, u32x4 v) { NBO_STORE(v, GLOBAL_PTR(u32x4, p)); }
+    DEV void unpack(u32x4 v, T (&x)[EV]) { EwBits<ST>::unpack(ST, v, x); }
+    DEV u32x4 pack(const T (&x)[EV]) { return EwBits<ST>::pack(ST, x); }
+    DEV void ld(const char *p, T (&x)[EV]) { unpack(ld(p), x); }
+    DEV void st(char *p, const T (&x)[EV]) { st(p, pack(x)); }
+};
+
+// ---------------------------------------------------------------------------------
+// Element-wise passes over NS tensor lists of one layout: one workgroup per piece of
+// PIECE_BYTES of every list (a whole number of rows of one 128-bit vector per thread), every
+// row of every list loaded before the first is used.  `op` supplies: loads(s) / stores(s) --
+// whether list s is read / written; apply(x) -- the arithmetic on one vector of every list;
+// ragged(c, p) -- a chunk that is not whole or not vector-aligned, element by element (done by
+// the workgroup of the chunk's first piece).
+template <int ST, int NS, uint32_t PIECE_BYTES, typename Op>
+DEV void stream_pieces(const NboLayoutDev &L, const uint64_t *const (&lists)[NS], const Op &op)
+{
+    typedef typename Traits<ST>::T T;
+    enum {
+        SB = Traits<ST>::SBYTES,
+        VEC = EwIO<ST>::EV,
+        ROWB = NBO_BLOCK * VEC * SB,
+        PIECE = PIECE_BYTES < NBO_CHUNK * SB ? PIECE_BYTES : NBO_CHUNK * SB,
+        R = PIECE / ROWB,
+        PPC = NBO_CHUNK * SB / PIECE
+    };
+    static_assert(R >= 1 && PPC >= 1 && R * PPC * ROWB == NBO_CHUNK * SB, "pieces divide the chunk");
+    const uint32_t piece = blockIdx.x;
+    const ChunkRef c = chunk_ref(L, piece / PPC);
+    char *p[NS];
+    uintptr_t all = 0;
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        p[s] = (char *)lists[s][c.t] + c.base * SB;
+        all |= (uintptr_t)p[s];
+    }
+    if (c.cnt != NBO_CHUNK || (all & (VEC * SB - 1)) != 0) {
+        if (piece % PPC == 0) op.ragged(c, p);
+        return;
+    }
+    const uint64_t off = (uint64_t)(piece % PPC) * (R * ROWB) + threadIdx.x * (VEC * SB);
+    u32x4 x[NS][R] = {};
+#pragma unroll
+    for (int s = 0; s < NS; s++)
+        if (op.loads(s)) {
+#pragma unroll
+            for (int u = 0; u < R; u++) x[s][u] = EwIO<ST>::ld(p[s] + off + u * ROWB);
+        }
+#pragma unroll
+    for (int u = 0; u < R; u++) {
+        T v[NS][VEC];
+#pragma unroll
+        for (int s = 0; s < NS; s++) EwIO<ST>::unpack(x[s][u], v[s]);
+        op.apply(v);
+#pragma unroll
+        for (int s = 0; s < NS; s++) x[s][u] = EwIO<ST>::pack(v[s]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 0; s < NS; s++)
+        if (op.stores(s)) {
+#pragma unroll
+            for (int u = 0; u < R; u++) EwIO<ST>::st(p[s] + off + u * ROWB, x[s][u]);
+        }
+}
+
 // ---------------------------------------------------------------------------------
 // In-place gradient passes of the unfused API: multiply by a factor, or zero.
+template <int ST> struct ScaleOp {
+    typedef typename Traits<ST>::T T;
+    enum { SB = Traits<ST>::SBYTES, VEC = Traits<ST>::VEC };
+    bool zero;
+    T f;
+    MEMBER bool loads(int) const { return !zero; }
+    MEMBER bool stores(int) const { return true; }
+    MEMBER void apply(T (&x)[1][EwIO<ST>::EV]) const
+    {
+#pragma unroll
+        for (int k = 0; k < EwIO<ST>::EV; k++) x[0][k] = zero ? (T)0 : x[0][k] * f;
+    }
+    MEMBER void ragged(const ChunkRef &c, char *const (&ptr)[1]) const
+    {
+        const uint32_t tid = threadIdx.x;
+        char *pg = ptr[0];
+        const Peel pl = peel(c.cnt, VEC, SB, false, (uintptr_t)pg);
+        for (uint32_t q = tid; q < pl.nvec; q += NBO_BLOCK) {
+            T x[VEC] = {};
+            char *p = pg + ((uint64_t)pl.head + (uint64_t)q * VEC) * SB;
+            if (!zero) {
+                IO<ST>::ldv(p, x);
+#pragma unroll
+                for (int k = 0; k < VEC; k++) x[k] = x[k] * f;
+            }
+            IO<ST>::stv(p, x);
+        }
+        const uint32_t n_single = c.cnt - pl.nvec * VEC; // elements [0, head) and [head + nvec * VEC, cnt)
+        for (uint32_t i = tid; i < n_single; i += NBO_BLOCK) {
+            const uint32_t e = i < pl.head ? i : i + pl.nvec * VEC;
+            char *p = pg + (uint64_t)e * SB;
+            const T x = zero ? (T)0 : IO<ST>::ld1(p) * f;
+            IO<ST>::st1(p, x);
+        }
+    }
+};
+
 template <int ST> DEV void scale_body(const NboScaleArgs &a)
 {
     typedef typename Traits<ST>::T T;
-    enum { SB = Traits<ST>::SBYTES, VEC = Traits<ST>::VEC };
-    const uint32_t tid = threadIdx.x;
-    const ChunkRef c = chunk_ref(a.L, blockIdx.x);
-    char *pg = (char *)a.g_ptrs[c.t] + c.base * SB;
-    bool zero = a.mode == 3;
-    T f = (T)a.factor;
+    ScaleOp<ST> op;
+    op.zero = a.mode == 3;
+    op.f = (T)a.factor;
     if (a.gf) {
         if (a.mode == 0) {
-            if (a.gf->found_inf) zero = true;
-            f = sizeof(T) == 4 ? (T)a.gf->inv_scale32 : (T)a.gf->inv_scale64;
+            if (a.gf->found_inf) op.zero = true;
+            op.f = sizeof(T) == 4 ? (T)a.gf->inv_scale32 : (T)a.gf->inv_scale64;
         } else if (a.mode == 1) {
             if (!a.gf->clipped) return; // trainer.rs:515: untouched when norm <= max_norm
-            f = sizeof(T) == 4 ? (T)a.gf->clip32 : (T)a.gf->clip64;
+            op.f = sizeof(T) == 4 ? (T)a.gf->clip32 : (T)a.gf->clip64;
         } else if (a.mode == 4) {
             if (!a.gf->found_inf) return; // core.rs:372-375 alone: zeros on a non-finite gradient
-            zero = true;
+            op.zero = true;
         }
     }
-    const Peel pl = peel(c.cnt, VEC, SB, false, (uintptr_t)pg);
-    for (uint32_t q = tid; q < pl.nvec; q += NBO_BLOCK) {
-        T x[VEC] = {};
-        char *p = pg + ((uint64_t)pl.head + (uint64_t)q * VEC) * SB;
-        if (!zero) {
-            IO<ST>::ldv(p, x);
-#pragma unroll
-            for (int k = 0; k < VEC; k++) x[k] = x[k] * f;
-        }
-        IO<ST>::stv(p, x);
-    }
-    const uint32_t n_single = c.cnt - pl.nvec * VEC; // elements [0, head) and [head + nvec * VEC, cnt)
-    for (uint32_t i = tid; i < n_single; i += NBO_BLOCK) {
-        const uint32_t e = i < pl.head ? i : i + pl.nvec * VEC;
-        char *p = pg + (uint64_t)e * SB;
-        const T x = zero ? (T)0 : IO<ST>::ld1(p) * f;
-        IO<ST>::st1(p, x);
-    }
+    const uint64_t *const lists[1] = {a.g_ptrs};
+    stream_pieces<ST, 1, NBO_EW_PIECE_BYTES>(a.L, lists, op);
 }
 
 #define NBO_SCALE_KERNEL(name, ST)                                                          \
@@ -1066,35 +1240,54 @@ NBO_SCALE_KERNEL(nbo_scale_f64, NBO_F64)
 // Gradient accumulation of the Trainer: buf[i] = &buf[i] + g (trainer.rs:262-266 ->
 // B::add, cpu/mod.rs:181: one rounding in T; for bf16 the f32 sum is rounded to bf16,
 // scalar/mod.rs:253-351), optionally clearing g afterwards.
-template <int ST> DEV void accum_body(const NboAccumArgs &a)
-{
+template <int ST> struct AccumOp {
     typedef typename Traits<ST>::T T;
     enum { SB = Traits<ST>::SBYTES, VEC = Traits<ST>::VEC };
-    const uint32_t tid = threadIdx.x;
-    const ChunkRef c = chunk_ref(a.L, blockIdx.x);
-    char *pa = (char *)a.a_ptrs[c.t] + c.base * SB;
-    char *pb = (char *)a.b_ptrs[c.t] + c.base * SB;
-    const Peel pl = peel(c.cnt, VEC, SB, false, (uintptr_t)pa, (uintptr_t)pb);
-    for (uint32_t q = tid; q < pl.nvec; q += NBO_BLOCK) {
-        const uint64_t off = ((uint64_t)pl.head + (uint64_t)q * VEC) * SB;
-        T x[VEC], y[VEC];
-        IO<ST>::ldv(pa + off, x);
-        IO<ST>::ldv(pb + off, y);
+    bool zero_b;
+    MEMBER bool loads(int) const { return true; }
+    MEMBER bool stores(int s) const { return s == 0 || zero_b; }
+    MEMBER void apply(T (&x)[2][EwIO<ST>::EV]) const
+    {
 #pragma unroll
-        for (int k = 0; k < VEC; k++) x[k] = x[k] + y[k];
-        IO<ST>::stv(pa + off, x);
-        if (a.zero_b) {
-            T z[VEC] = {};
-            IO<ST>::stv(pb + off, z);
+        for (int k = 0; k < EwIO<ST>::EV; k++) {
+            x[0][k] = x[0][k] + x[1][k];
+            x[1][k] = (T)0;
         }
     }
-    const uint32_t n_single = c.cnt - pl.nvec * VEC; // elements [0, head) and [head + nvec * VEC, cnt)
-    for (uint32_t i = tid; i < n_single; i += NBO_BLOCK) {
-        const uint64_t off = (uint64_t)(i < pl.head ? i : i + pl.nvec * VEC) * SB;
-        const T x = IO<ST>::ld1(pa + off) + IO<ST>::ld1(pb + off);
-        IO<ST>::st1(pa + off, x);
-        if (a.zero_b) IO<ST>::st1(pb + off, (T)0);
+    MEMBER void ragged(const ChunkRef &c, char *const (&ptr)[2]) const
+    {
+        const uint32_t tid = threadIdx.x;
+        char *pa = ptr[0], *pb = ptr[1];
+        const Peel pl = peel(c.cnt, VEC, SB, false, (uintptr_t)pa, (uintptr_t)pb);
+        for (uint32_t q = tid; q < pl.nvec; q += NBO_BLOCK) {
+            const uint64_t off = ((uint64_t)pl.head + (uint64_t)q * VEC) * SB;
+            T x[VEC], y[VEC];
+            IO<ST>::ldv(pa + off, x);
+            IO<ST>::ldv(pb + off, y);
+#pragma unroll
+            for (int k = 0; k < VEC; k++) x[k] = x[k] + y[k];
+            IO<ST>::stv(pa + off, x);
+            if (zero_b) {
+                T z[VEC] = {};
+                IO<ST>::stv(pb + off, z);
+            }
+        }
+        const uint32_t n_single = c.cnt - pl.nvec * VEC; // elements [0, head) and [head + nvec * VEC, cnt)
+        for (uint32_t i = tid; i < n_single; i += NBO_BLOCK) {
+            const uint64_t off = (uint64_t)(i < pl.head ? i : i + pl.nvec * VEC) * SB;
+            const T x = IO<ST>::ld1(pa + off) + IO<ST>::ld1(pb + off);
+            IO<ST>::st1(pa + off, x);
+            if (zero_b) IO<ST>::st1(pb + off, (T)0);
+        }
     }
+};
+
+template <int ST> DEV void accum_body(const NboAccumArgs &a)
+{
+    AccumOp<ST> op;
+    op.zero_b = a.zero_b != 0;
+    const uint64_t *const lists[2] = {a.a_ptrs, a.b_ptrs};
+    stream_pieces<ST, 2, NBO_EW_PIECE_BYTES>(a.L, lists, op);
 }
 
 #define NBO_ACCUM_KERNEL(name, ST)                                                          \
@@ -1218,41 +1411,6 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_cast_master(const Nb
 // operation is one IEEE operation in the arithmetic type, rounded to the element type:
 // for bf16 that is the f32 operation followed by bf16::from_f32
 // (common/scalar/mod.rs:253-351), including the product inside axpy.
-// Vector accesses of the element-wise passes: 128 bits wide for every element type, i.e. 8
-// elements of a 16-bit tensor computed in f32 (the update kernels take those 4 at a time, in
-// step with their 128-bit f32 state vectors).
-template <int ST> struct EwIO {
-    typedef typename Traits<ST>::T T;
-    enum { EV = Traits<ST>::VEC };
-    DEV void ld(const char *p, T (&x)[EV]) { IO<ST>::ldv(p, x); }
-    DEV void st(char *p, const T (&x)[EV]) { IO<ST>::stv(p, x); }
-};
-template <int ST> struct EwIOHalfWide {
-    enum { EV = 8 };
-    DEV void ld(const char *p, float (&x)[8])
-    {
-        const u32x4 v = NBO_LOAD(GLOBAL_PTR(const u32x4, p));
-        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            x[2 * k] = from_half_bits<ST>(w[k] & 0xFFFFu);
-            x[2 * k + 1] = from_half_bits<ST>(w[k] >> 16);
-        }
-    }
-    DEV void st(char *p, const float (&x)[8])
-    {
-        uint32_t w[4];
-#pragma unroll
-        for (int k = 0; k < 4; k++)
-            w[k] = ST == NBO_BF16 ? f32_to_bf16_bits(x[2 * k]) | (f32_to_bf16_bits(x[2 * k + 1]) << 16)
-                                  : f32_to_f16_bits(x[2 * k]) | (f32_to_f16_bits(x[2 * k + 1]) << 16);
-        const u32x4 v = {w[0], w[1], w[2], w[3]};
-        NBO_STORE(v, GLOBAL_PTR(u32x4, p));
-    }
-};
-template <> struct EwIO<NBO_BF16> : EwIOHalfWide<NBO_BF16> {};
-template <> struct EwIO<NBO_F16> : EwIOHalfWide<NBO_F16> {};
-
 template <int ST> DEV typename Traits<ST>::T to_storage_precision(typename Traits<ST>::T x) { return x; }
 template <> __device__ __forceinline__ float to_storage_precision<NBO_BF16>(float x)
 {
@@ -1292,39 +1450,58 @@ template <int ST, typename T> DEV T ew_elem(uint32_t op, T o, T a, T b, T s)
     }
 }
 
+template <int ST> struct EwOp {
+    typedef typename Traits<ST>::T T;
+    enum { SB = Traits<ST>::SBYTES, VEC = EwIO<ST>::EV };
+    uint32_t op;
+    bool use_a, use_b, use_o;
+    T s;
+    MEMBER bool loads(int i) const { return i == 0 ? use_o : i == 1 ? use_a : use_b; }
+    MEMBER bool stores(int i) const { return i == 0; }
+    MEMBER void apply(T (&x)[3][VEC]) const
+    {
+#pragma unroll
+        for (int k = 0; k < VEC; k++) x[0][k] = ew_elem<ST, T>(op, x[0][k], x[1][k], x[2][k], s);
+    }
+    MEMBER void ragged(const ChunkRef &c, char *const (&ptr)[3]) const
+    {
+        const uint32_t tid = threadIdx.x;
+        char *po = ptr[0];
+        const char *pa = ptr[1], *pb = ptr[2];
+        const Peel pl = peel(c.cnt, VEC, SB, false, (uintptr_t)po, (uintptr_t)pa, (uintptr_t)pb);
+        for (uint32_t q = tid; q < pl.nvec; q += NBO_BLOCK) {
+            const uint64_t off = ((uint64_t)pl.head + (uint64_t)q * VEC) * SB;
+            T o[VEC] = {}, x[VEC] = {}, y[VEC] = {};
+            if (use_a) EwIO<ST>::ld(pa + off, x);
+            if (use_b) EwIO<ST>::ld(pb + off, y);
+            if (use_o) EwIO<ST>::ld(po + off, o);
+#pragma unroll
+            for (int k = 0; k < VEC; k++) o[k] = ew_elem<ST, T>(op, o[k], x[k], y[k], s);
+            EwIO<ST>::st(po + off, o);
+        }
+        const uint32_t n_single = c.cnt - pl.nvec * VEC; // elements [0, head) and [head + nvec * VEC, cnt)
+        for (uint32_t i = tid; i < n_single; i += NBO_BLOCK) {
+            const uint64_t off = (uint64_t)(i < pl.head ? i : i + pl.nvec * VEC) * SB;
+            const T x = use_a ? IO<ST>::ld1(pa + off) : (T)0;
+            const T y = use_b ? IO<ST>::ld1(pb + off) : (T)0;
+            const T o = use_o ? IO<ST>::ld1(po + off) : (T)0;
+            IO<ST>::st1(po + off, ew_elem<ST, T>(op, o, x, y, s));
+        }
+    }
+};
+
 template <int ST> DEV void ew_body(const NboEwArgs &a)
 {
     typedef typename Traits<ST>::T T;
-    enum { SB = Traits<ST>::SBYTES, VEC = EwIO<ST>::EV };
-    const uint32_t tid = threadIdx.x;
-    const ChunkRef c = chunk_ref(a.L, blockIdx.x);
-    const uint32_t op = a.op;
-    const bool use_a = op != NBO_EW_ZEROS;
-    const bool use_b = op == NBO_EW_ADD || op == NBO_EW_EMUL || op == NBO_EW_EDIV;
-    const bool use_o = op == NBO_EW_AXPY;
-    char *po = (char *)a.out_ptrs[c.t] + c.base * SB;
-    const char *pa = use_a ? (const char *)a.a_ptrs[c.t] + c.base * SB : po;
-    const char *pb = use_b ? (const char *)a.b_ptrs[c.t] + c.base * SB : po;
-    const T s = to_storage_precision<ST>((T)a.s);
-    const Peel pl = peel(c.cnt, VEC, SB, false, (uintptr_t)po, (uintptr_t)pa, (uintptr_t)pb);
-    for (uint32_t q = tid; q < pl.nvec; q += NBO_BLOCK) {
-        const uint64_t off = ((uint64_t)pl.head + (uint64_t)q * VEC) * SB;
-        T o[VEC] = {}, x[VEC] = {}, y[VEC] = {};
-        if (use_a) EwIO<ST>::ld(pa + off, x);
-        if (use_b) EwIO<ST>::ld(pb + off, y);
-        if (use_o) EwIO<ST>::ld(po + off, o);
-#pragma unroll
-        for (int k = 0; k < VEC; k++) o[k] = ew_elem<ST, T>(op, o[k], x[k], y[k], s);
-        EwIO<ST>::st(po + off, o);
-    }
-    const uint32_t n_single = c.cnt - pl.nvec * VEC; // elements [0, head) and [head + nvec * VEC, cnt)
-    for (uint32_t i = tid; i < n_single; i += NBO_BLOCK) {
-        const uint64_t off = (uint64_t)(i < pl.head ? i : i + pl.nvec * VEC) * SB;
-        const T x = use_a ? IO<ST>::ld1(pa + off) : (T)0;
-        const T y = use_b ? IO<ST>::ld1(pb + off) : (T)0;
-        const T o = use_o ? IO<ST>::ld1(po + off) : (T)0;
-        IO<ST>::st1(po + off, ew_elem<ST, T>(op, o, x, y, s));
-    }
+    EwOp<ST> op;
+    op.op = a.op;
+    op.use_a = a.op != NBO_EW_ZEROS;
+    op.use_b = a.op == NBO_EW_ADD || a.op == NBO_EW_EMUL || a.op == NBO_EW_EDIV;
+    op.use_o = a.op == NBO_EW_AXPY;
+    op.s = to_storage_precision<ST>((T)a.s);
+    // an operand the operation does not have stands for the output: never read, same alignment
+    const uint64_t *const lists[3] = {a.out_ptrs, op.use_a ? a.a_ptrs : a.out_ptrs, op.use_b ? a.b_ptrs : a.out_ptrs};
+    stream_pieces<ST, 3, NBO_BACKEND_PIECE_BYTES>(a.L, lists, op);
 }
 
 #define NBO_EW_KERNEL(name, ST)                                                             \
@@ -1379,12 +1556,23 @@ template <int ST> DEV void cast_store4(char *p, uint64_t e, const double (&v)[4]
 template <int SRC, int DST> DEV void cast_body(const NboCastListArgs &a)
 {
     enum { SS = Traits<SRC>::SBYTES, DS = Traits<DST>::SBYTES };
-    const ChunkRef c = chunk_ref(a.L, blockIdx.x);
+    // one workgroup per NBO_CAST_ROW elements of a chunk (four per thread), as the other
+    // element-wise passes run; a ragged or misaligned chunk is done by its first workgroup
+    const uint32_t row = blockIdx.x % (NBO_CHUNK / NBO_CAST_ROW);
+    const ChunkRef c = chunk_ref(a.L, blockIdx.x / (NBO_CHUNK / NBO_CAST_ROW));
     const char *ps = (const char *)a.src_ptrs[c.t] + c.base * SS;
     char *pd = (char *)a.dst_ptrs[c.t] + c.base * DS;
     // groups of four while both addresses allow whole vectors (16 bytes at most per access)
     const uint32_t sa = SS * 4 > 16 ? 16 : SS * 4, da = DS * 4 > 16 ? 16 : DS * 4;
     const bool vec_ok = (((uintptr_t)ps & (sa - 1)) | ((uintptr_t)pd & (da - 1))) == 0;
+    if (vec_ok && c.cnt == NBO_CHUNK) {
+        double v[4];
+        const uint64_t e = (uint64_t)row * NBO_CAST_ROW + threadIdx.x * 4;
+        cast_load4<SRC>(ps, e, v);
+        cast_store4<DST>(pd, e, v);
+        return;
+    }
+    if (row != 0) return;
     const uint32_t nquad = vec_ok ? c.cnt / 4 : 0;
     for (uint32_t q = threadIdx.x; q < nquad; q += NBO_BLOCK) {
         double v[4];

@@ -43,6 +43,9 @@ SHAPES = [  # nbo_probe_shape
     "shape 0's eight rows taken from 2 places of every stream at once (windows of 4 rows, a grid apart)",
     "shape 0's eight rows taken from 4 places of every stream at once (windows of 2 rows)",
     "shape 0's eight rows taken from 8 places of every stream at once (windows of 1 row)",
+    "shape 0 with four rows per workgroup (16 KiB windows, twice the workgroups)",
+    "shape 0 with two rows per workgroup (8 KiB windows)",
+    "shape 0 with one row per workgroup: one vector of every stream per thread (4 KiB windows, eight times the workgroups)",
 ]
 NEIGHBOURS = 0x80000000  # flag on a compare run's window count: the windows of a workgroup are neighbours
 FULL_PATTERNS = (4, 5, 7, 9)  # the 1:1 read/write patterns every shape exists for
