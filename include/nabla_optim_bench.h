@@ -100,8 +100,8 @@ int nbo_hbm_ceiling_compare(int pattern, int n_shapes, const int *shapes, const 
  * rounded up to whole GiB), or, with -1 for every buffer, the buffers rotate over the regions GiB
  * by GiB as the optimizer's state arrays do.  NBO_ERR_TOO_LARGE with the reason in
  * nbo_last_error() when the search finds no second region or memory runs short.  Measured
- * (python -m nabla_amd.kernel_bench --placed): the kernels over the caller's tensors gain 0-3 %,
- * which is why the drop-in header offers no such allocator. */
+ * (python -m nabla_amd.kernel_bench --placed): the kernels over the caller's tensors gain nothing
+ * (-3 to +0 %), which is why the drop-in header offers no such allocator. */
 typedef struct nbo_placed nbo_placed;
 int nbo_alloc_placed(uint32_t n_buffers, uint64_t bytes, const int *region, void **out_ptrs, nbo_placed **out);
 int nbo_free_placed(nbo_placed *p);

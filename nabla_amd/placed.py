@@ -2,7 +2,7 @@
 or three flat device buffers, each wholly inside one of the regions the placement search tells
 apart -- or, with -1 for every buffer, rotating over the regions as the optimizer's state does --
 to measure what such placement of a framework's parameter and gradient storage would buy
-(`python -m nabla_amd.kernel_bench --placed`: 0-3 %).  `regions` gives a region number per
+(`python -m nabla_amd.kernel_bench --placed`: nothing, -3 to +0 %).  `regions` gives a region number per
 buffer: equal numbers share a region, different numbers lie in different regions."""
 from __future__ import annotations
 
