@@ -240,7 +240,9 @@ int nbo_fused_step_noalloc(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params,
 /* The same tail for GroupOptimizer (optim/groups.rs:269-293): one unscale / found-inf /
  * clip decision over `all_grads` (every gradient, in the module's order), then each
  * group's update with its own hyper-parameters.  params[g] / grads[g] are the lists of
- * group g's tensors; together the groups must cover all_grads.  Asynchronous. */
+ * group g's tensors; together the groups must cover all_grads.  Three launches: the norm
+ * pass, its second stage and one update launch for up to sixteen groups of one optimizer kind
+ * and element type (further groups, or groups of another kind, add a launch).  Asynchronous. */
 int nbo_fused_step_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,
                           nbo_list *const *grads, nbo_scaler *scaler, nbo_list *all_grads,
                           double max_norm, uint32_t flags);

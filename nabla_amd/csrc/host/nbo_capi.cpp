@@ -138,15 +138,26 @@ int self_update_kernel(const nbo_optim *opt, const nbo_list *params)
 // skipped) and writes the trace entry.  Not for an empty list: no workgroup would run.
 bool self_update_possible(const nbo_optim *opt) { return opt->layout.nchunks > 0; }
 
-void launch_self_update(nbo_optim *opt, nbo_list *params, nbo_list *grads, const NboGradFactors *gf, uint32_t zero_grads,
-                        NboTraceDev *trace, const NboScalerDev *scaler)
+NboUpdateArgs self_update_args(nbo_optim *opt, nbo_list *params, nbo_list *grads, const NboGradFactors *gf,
+                               uint32_t zero_grads, NboTraceDev *trace, const NboScalerDev *scaler)
 {
     NboUpdateArgs a = update_args(opt, params, grads, false, zero_grads, gf);
     a.hyper = hyper_of(opt);
     a.opt_rw = opt->dev;
     a.trace = trace;
     a.scaler = scaler;
-    Runtime::get().launch(self_update_kernel(opt, params), opt->layout.nchunks, NBO_BLOCK, a);
+    return a;
+}
+
+void launch_self_update(nbo_optim *opt, nbo_list *params, nbo_list *grads, const NboGradFactors *gf, uint32_t zero_grads,
+                        NboTraceDev *trace, const NboScalerDev *scaler)
+{
+    static_assert(sizeof(NboGroupedUpdateArgs) <= 4096, "the argument block of a launch");
+    NboGroupedUpdateArgs ga = {};
+    ga.g[0] = self_update_args(opt, params, grads, gf, zero_grads, trace, scaler);
+    ga.first_wg[1] = opt->layout.nchunks;
+    ga.n_groups = 1;
+    Runtime::get().launch(self_update_kernel(opt, params), opt->layout.nchunks, NBO_BLOCK, ga);
 }
 
 uint32_t norm_grid(const Layout &L)
@@ -915,30 +926,45 @@ static uint64_t check_group_args(uint64_t n_groups, nbo_optim *const *opts, nbo_
     return covered;
 }
 
-// Each group's scalars and update from the one decision in the runtime's scratch: one launch
-// per group (two for an empty group, see self_update_possible).
+// Every group's scalars and update from the one decision in the runtime's scratch, in ONE
+// launch for up to NBO_GROUPS_PER_LAUNCH groups of one optimizer kind and element types (what a
+// GroupOptimizer<O> holds, optim/groups.rs:269-293); groups of another kind or type start a launch
+// of their own, and an empty group, in which no workgroup would run, gets the scalar part alone.
 static void launch_group_updates(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,
                                  nbo_list *const *grads, nbo_scaler *scaler, uint32_t flags)
 {
     Runtime &rt = Runtime::get();
+    NboGroupedUpdateArgs ga = {};
+    int kernel = -1;
+    uint64_t wgs = 0;
+    auto flush = [&] {
+        if (ga.n_groups) rt.launch(kernel, (uint32_t)wgs, NBO_BLOCK, ga);
+        ga.n_groups = 0;
+        wgs = 0;
+    };
     for (uint64_t g = 0; g < n_groups; g++) {
-        if (self_update_possible(opts[g])) {
-            // one launch per group: it derives the group's scalars from the shared decision itself
-            launch_self_update(opts[g], params[g], grads[g], rt.gf_scratch(), zero_mode(flags),
-                               opts[g]->trace, scaler ? scaler->dev : nullptr);
+        if (!self_update_possible(opts[g])) {
+            NboPrepArgs p = {};
+            p.opt = opts[g]->dev;
+            p.gf = rt.gf_scratch();
+            p.scaler = scaler ? scaler->dev : nullptr;
+            p.trace = opts[g]->trace;
+            p.hyper = hyper_of(opts[g]);
+            rt.launch(K_PREP, 1, 64, p);
             continue;
         }
-        NboPrepArgs p = {};
-        p.opt = opts[g]->dev;
-        p.gf = rt.gf_scratch();
-        p.scaler = scaler ? scaler->dev : nullptr;
-        p.trace = opts[g]->trace;
-        p.hyper = hyper_of(opts[g]);
-        rt.launch(K_PREP, 1, 64, p);
-        const NboUpdateArgs a = update_args(opts[g], params[g], grads[g], true,
-                                            zero_mode(flags), rt.gf_scratch());
-        rt.launch(update_kernel(opts[g], params[g]), update_grid(opts[g], params[g]), NBO_BLOCK, a);
+        const int k = self_update_kernel(opts[g], params[g]);
+        if (ga.n_groups == NBO_GROUPS_PER_LAUNCH || (ga.n_groups && k != kernel) ||
+            wgs + opts[g]->layout.nchunks > 0x7FFFFFFFull)
+            flush();
+        kernel = k;
+        ga.g[ga.n_groups] = self_update_args(opts[g], params[g], grads[g], rt.gf_scratch(), zero_mode(flags),
+                                             opts[g]->trace, scaler ? scaler->dev : nullptr);
+        ga.first_wg[ga.n_groups] = (uint32_t)wgs;
+        wgs += opts[g]->layout.nchunks;
+        ga.first_wg[++ga.n_groups] = (uint32_t)wgs;
     }
+    flush();
 }
 
 int nbo_fused_step_groups(uint64_t n_groups, nbo_optim *const *opts, nbo_list *const *params,

@@ -507,7 +507,8 @@ DEV void make_uniform(NboOptimDev &o)
 // three streams that measured 15-20 % faster than eight rows per workgroup (as it does for the
 // element-wise passes, see stream_pieces); the Adam kinds' five streams do best at eight rows.
 // A chunk that is ragged, misaligned or skipped is done by the workgroup of its first row.
-template <int ST, int KIND, bool BY_ROW = false> DEV void update_chunk(const NboUpdateArgs &a, const NboOptimDev *o)
+template <int ST, int KIND, bool BY_ROW = false>
+DEV void update_chunk(const NboUpdateArgs &a, const NboOptimDev *o, uint32_t wg)
 {
     typedef typename Traits<ST>::T T;
     enum {
@@ -523,8 +524,8 @@ template <int ST, int KIND, bool BY_ROW = false> DEV void update_chunk(const Nbo
     const bool mixed = ST == NBO_BF16 || ST == NBO_F16; // f32 master lives in the arena
     const bool has_v = KIND != NBO_SGD;
     const uint32_t tid = threadIdx.x;
-    const uint32_t row0 = BY_ROW ? blockIdx.x % ROWS : 0;
-    const ChunkRef c = chunk_ref(a.L, BY_ROW ? blockIdx.x / ROWS : blockIdx.x);
+    const uint32_t row0 = BY_ROW ? wg % ROWS : 0;
+    const ChunkRef c = chunk_ref(a.L, BY_ROW ? wg / ROWS : wg);
 
     char *pp = (char *)a.p_ptrs[c.t] + c.base * SB;
     char *pg = (char *)a.g_ptrs[c.t] + c.base * SB;
@@ -647,10 +648,12 @@ template <int ST, int KIND, bool BY_ROW = false> DEV void update_chunk(const Nbo
     }
 }
 
-template <int ST, int KIND, bool SELF = false> DEV void update_body(const NboUpdateArgs &a)
+// wg of nwg: the workgroup's number among those that work on a's lists (the whole grid, or
+// one group's share of a grouped launch)
+template <int ST, int KIND, bool SELF = false> DEV void update_body(const NboUpdateArgs &a, uint32_t wg, uint32_t nwg)
 {
     if (!SELF) {
-        update_chunk<ST, KIND, KIND == NBO_SGD>(a, a.opt);
+        update_chunk<ST, KIND, KIND == NBO_SGD>(a, a.opt, wg);
         return;
     }
     uint32_t sc_lo = (uint32_t)a.opt->step_count, sc_hi = (uint32_t)(a.opt->step_count >> 32);
@@ -663,10 +666,10 @@ template <int ST, int KIND, bool SELF = false> DEV void update_body(const NboUpd
     own.step_count = ((uint64_t)sc_hi << 32) | sc_lo;
     prep_step(&own, a.hyper, a.gf);
     make_uniform(own);
-    update_chunk<ST, KIND>(a, &own);
+    update_chunk<ST, KIND>(a, &own, wg);
     // the counter's answer is not looked at before the chunk is done: it has long arrived then
     __builtin_amdgcn_sched_barrier(0);
-    if (threadIdx.x == 0 && readers_before == gridDim.x - 1) {
+    if (threadIdx.x == 0 && readers_before == nwg - 1) {
         a.opt_rw->step_count = own.step_count;
         if (a.trace) trace_step(a.trace, a.gf, &own, a.scaler ? a.scaler->scale : 0.0);
         __hip_atomic_store(&a.opt_rw->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -676,7 +679,7 @@ template <int ST, int KIND, bool SELF = false> DEV void update_body(const NboUpd
 #define NBO_UPDATE_KERNEL(name, ST, KIND)                                                   \
     extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboUpdateArgs a) \
     {                                                                                       \
-        update_body<ST, KIND>(a);                                                           \
+        update_body<ST, KIND>(a, blockIdx.x, gridDim.x);                                    \
     }
 
 NBO_UPDATE_KERNEL(nbo_update_f32_adamw, NBO_F32, NBO_ADAMW)
@@ -698,12 +701,18 @@ NBO_UPDATE_KERNEL(nbo_update_pf16_adamw, NBO_PF16, NBO_ADAMW)
 NBO_UPDATE_KERNEL(nbo_update_pf16_adam, NBO_PF16, NBO_ADAM)
 NBO_UPDATE_KERNEL(nbo_update_pf16_sgd, NBO_PF16, NBO_SGD)
 
-// Adam / AdamW launches that prepare their own scalars: the unfused Optimizer::step (one launch
-// per call, as the reference's one call) and every group of a grouped fused step.
-#define NBO_UPDATE_SELF_KERNEL(name, ST, KIND)                                              \
-    extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboUpdateArgs a)     \
-    {                                                                                       \
-        update_body<ST, KIND, true>(a);                                                     \
+// Launches that prepare their own scalars: the unfused Optimizer::step (one launch per call, as
+// the reference's one call) and a grouped fused step, whose groups -- each with its own lists,
+// state, hyper-parameters and step_count (optim/groups.rs:269-293) -- share ONE launch: the
+// argument block carries up to NBO_GROUPS_PER_LAUNCH groups' arguments, and a workgroup first
+// finds the group whose range of the grid it lies in.
+#define NBO_UPDATE_SELF_KERNEL(name, ST, KIND)                                                    \
+    extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboGroupedUpdateArgs ga)   \
+    {                                                                                             \
+        uint32_t gi = 0;                                                                          \
+        for (uint32_t k = 1; k < ga.n_groups; k++) gi = blockIdx.x >= ga.first_wg[k] ? k : gi;    \
+        update_body<ST, KIND, true>(ga.g[gi], blockIdx.x - ga.first_wg[gi],                       \
+                                    ga.first_wg[gi + 1] - ga.first_wg[gi]);                       \
     }
 NBO_UPDATE_SELF_KERNEL(nbo_update_f32_adamw_self, NBO_F32, NBO_ADAMW)
 NBO_UPDATE_SELF_KERNEL(nbo_update_f32_adam_self, NBO_F32, NBO_ADAM)

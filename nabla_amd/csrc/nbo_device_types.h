@@ -164,6 +164,15 @@ struct NboUpdateArgs {
     const NboScalerDev *scaler;
 };
 
+// Argument block of the "_self" update kernels: one launch over several groups' lists.
+// Workgroups [first_wg[k], first_wg[k + 1]) work on group k; first_wg[n_groups] is the grid.
+#define NBO_GROUPS_PER_LAUNCH 16u
+struct NboGroupedUpdateArgs {
+    NboUpdateArgs g[NBO_GROUPS_PER_LAUNCH];
+    uint32_t first_wg[NBO_GROUPS_PER_LAUNCH + 1];
+    uint32_t n_groups;
+};
+
 struct NboFinalizeArgs {
     const double *partial_sumsq;
     const uint32_t *partial_flag;

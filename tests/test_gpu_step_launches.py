@@ -2,7 +2,8 @@
 
 The reference's `Adam::step` / `AdamW::step` is one call (alg.rs:109-150, 254-291): here it is
 one launch of a kernel that prepares its own per-step scalars and advances step_count exactly
-once; a grouped fused step is the norm pass, its second stage and one launch per group.
+once; a grouped fused step is the norm pass, its second stage and ONE update launch for up to
+sixteen groups of one optimizer kind (each with its own hyper-parameters, optim/groups.rs:269-293).
 `unscale_and_update` leaves zeros in the gradients when it finds inf / NaN (core.rs:372-375):
 the fused step does so with NBO_STEP_ZERO_ON_SKIP."""
 import ctypes as C
@@ -98,8 +99,8 @@ def test_set_lr_load_meta_and_reset_between_one_launch_steps(gpu):
     H.assert_bits_equal(H.host_list(opt.moments()[1]), v, "v")
 
 
-def test_grouped_fused_step_is_one_launch_per_group(gpu):
-    """Two groups: norm pass + second stage + two update launches, no scalar-preparation launch."""
+def test_grouped_fused_step_is_three_launches(gpu):
+    """Two groups: norm pass + second stage + one update launch for both, no scalar-preparation launch."""
     names = ["w", "bias", "w2"]
     shapes = [(16, 600), (1, 600), (40, 300)]
     w0 = H.randn_list(shapes, 60, 0.02)
@@ -116,9 +117,61 @@ def test_grouped_fused_step_is_one_launch_per_group(gpu):
     opt.fused_step(p_dev, g_dev, scaler=scaler, max_norm=1.0)
     n = _launches(["nbo_norm_bf16", "nbo_finalize", "nbo_update_bf16_adamw_self", "nbo_update_bf16_adamw", "nbo_prep"])
     _lib.check(L.nbo_profile_enable(0))
-    assert n == {"nbo_norm_bf16": 1, "nbo_finalize": 1, "nbo_update_bf16_adamw_self": 2, "nbo_update_bf16_adamw": 0,
+    assert n == {"nbo_norm_bf16": 1, "nbo_finalize": 1, "nbo_update_bf16_adamw_self": 1, "nbo_update_bf16_adamw": 0,
                  "nbo_prep": 0}
     assert [o.step_count() for o in opt.group_optimizers()] == [2, 2]
+
+
+def test_nineteen_groups_of_their_own_hyper_parameters_in_two_launches(gpu):
+    """Nineteen f32 AdamW groups, each with its own lr, weight decay and betas, plus tensors of
+    ragged sizes: two update launches per step (sixteen groups, then three), every group's
+    parameters and moments equal to the oracle's bit for bit after four clipped steps -- a group
+    that took another group's scalars, range of workgroups or step_count would differ everywhere."""
+    n_groups = 19
+    names = [f"t{i}" for i in range(n_groups)] + ["rest0", "rest1"]
+    shapes = [(1 + i % 3, 1000 + 977 * i) for i in range(n_groups)] + [(2, 8192), (1, 5)]
+    w0 = H.randn_list(shapes, 300, 0.02)
+    p_dev = H.dev_list(w0, shapes)
+    cfgs = [G.ParamGroupConfig.adamw(f"g{i}", G.ParamSelector.Any([G.Equals(f"t{i}")]), 1e-3 * (1 + i), 0.01 * i)
+            .betas(0.9 - 0.01 * i, 0.999 - 0.002 * i) for i in range(n_groups - 1)]
+    last = G.ParamGroupConfig.adamw("rest", G.ParamSelector.All(), 5e-4, 0.3)
+    opt = G.GroupOptimizer.from_named_params(list(zip(names, p_dev)), cfgs, last)
+    idx = opt.group_indices()
+    assert len(idx) == n_groups and idx[-1] == [18, 19, 20]
+    metas = [O.adamw_meta(c.lr, beta1=c.beta1, beta2=c.beta2, weight_decay=c.weight_decay) for c in cfgs] + \
+            [O.adamw_meta(5e-4, weight_decay=0.3)]
+    ref = dict(w=H.copy_list(w0), m=H.zeros_like_list(w0), v=H.zeros_like_list(w0))
+    L = _lib.load()
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        for step in range(4):
+            g = H.randn_list(shapes, 900 + 7 * step, 1e-2)
+            _lib.check(L.nbo_profile_enable(1))
+            opt.fused_step(p_dev, H.dev_list(g, shapes), max_norm=0.5)
+            n = _launches(["nbo_norm_f32", "nbo_finalize", "nbo_update_f32_adamw_self", "nbo_prep"])
+            _lib.check(L.nbo_profile_enable(0))
+            assert n == {"nbo_norm_f32": 1, "nbo_finalize": 1, "nbo_update_f32_adamw_self": 2, "nbo_prep": 0}
+            gf = H.copy_list(g)
+            info = opt.last_step()
+
+            def oracle_step():
+                norm = O.clip_grad_norm(gf, 0.5)
+                return True, norm
+
+            H.oracle_step_with_device_norm(oracle_step, [gf], [], 0.5, info, f"19 groups, step {step}")
+            assert info.clipped == 1
+            for gi, meta in zip(idx, metas):
+                O.adam_step(meta, [ref["w"][i] for i in gi], [gf[i] for i in gi],
+                            [ref["m"][i] for i in gi], [ref["v"][i] for i in gi])
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+    assert [o.step_count() for o in opt.group_optimizers()] == [4] * n_groups
+    H.assert_bits_equal(H.host_list(p_dev), ref["w"], "params")
+    state = dict(opt.state_tensors())
+    for gno, gi in enumerate(idx):
+        for k, i in enumerate(gi):
+            H.assert_bits_equal([H.to_host(state[f"g{gno}.m{k}"])], [ref["m"][i]], f"g{gno}.m{k}")
+            H.assert_bits_equal([H.to_host(state[f"g{gno}.v{k}"])], [ref["v"][i]], f"g{gno}.v{k}")
 
 
 @pytest.mark.parametrize("grouped", [False, True])
