@@ -1,0 +1,115 @@
+"""The element-wise passes and the SGD step run one workgroup per 4 KiB piece (one row) of a
+work chunk, and leave a chunk that is ragged or not vector-aligned to the workgroup of its first
+piece.  Every combination of whole / ragged chunks and aligned / unaligned addresses must give
+the oracle's bits: a piece done twice, skipped, or done by both paths would show here.
+
+Lists of several tensors as views into one buffer, at an aligned offset and at an odd element
+offset; sizes below one piece, between piece and chunk, exactly one chunk, chunks plus a ragged
+rest, and a few whole chunks."""
+import numpy as np
+import pytest
+
+import oracle as O
+from nabla_amd import optim as nb
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [5, 1024, 4099, 8192, 8200, 3 * 8192, 20011]
+NP = {"f32": np.float32, "f64": np.float64}
+
+
+def _views(arrs, odd, torch_dtype):
+    """The arrays as (1, n) views into one device buffer; with `odd`, each starts one element
+    past a 16-byte boundary."""
+    import torch
+
+    pad = 16
+    total = sum((a.size + pad + 15) // 16 * 16 for a in arrs) + pad
+    buf = torch.zeros(total, dtype=torch_dtype, device="cuda:0")
+    views, off = [], 0
+    for a in arrs:
+        start = off + (1 if odd else 0)
+        v = buf[start:start + a.size].reshape(1, a.size)
+        src = torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16) if a.dtype == np.uint16 else torch.from_numpy(a.copy())
+        v.copy_(src.reshape(1, a.size))
+        views.append(v)
+        off += (a.size + pad + 15) // 16 * 16
+    assert all((v.data_ptr() % 16 != 0) == odd for v in views)
+    return buf, views
+
+
+def _make(dtype, seed, sigma, odd):
+    import torch
+
+    if dtype == "bf16":
+        arrs = [O.bf16_from_f32(O.randn_f32(n, seed + i, sigma)) for i, n in enumerate(SIZES)]
+        return arrs, _views(arrs, odd, torch.bfloat16)
+    arrs = [(O.randn_f64(n, seed + i) * sigma).astype(NP[dtype]) for i, n in enumerate(SIZES)]
+    return arrs, _views(arrs, odd, torch.float32 if dtype == "f32" else torch.float64)
+
+
+def _as_f32(arrs):
+    return [O.bf16_to_f32(a) if a.dtype == np.uint16 else a for a in arrs]
+
+
+def _like(ref_f32, like):
+    return [O.bf16_from_f32(a) if b.dtype == np.uint16 else a for a, b in zip(ref_f32, like)]
+
+
+@pytest.mark.parametrize("odd", [False, True])
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f64"])
+def test_scale_zero_and_accumulate_over_views(gpu, dtype, odd):
+    g0, (gbuf, g) = _make(dtype, 11, 1.0, odd)
+    a0, (abuf, a) = _make(dtype, 31, 1.0, odd)
+    before_g, before_a = gbuf.clone(), abuf.clone()
+
+    # scale_grad: g * T(factor), rounded to the element type
+    nb.scale_grad(g, 0.3)
+    ref = [x.copy() for x in g0]
+    O.scale_grad(ref, 0.3)
+    H.assert_bits_equal(H.host_list(g), ref, f"scale_grad {dtype} odd={odd}")
+
+    # accumulate: a + g in the element type (bf16: the f32 sum rounded)
+    nb.accumulate(a, g)
+    acc = [O.add(x, y) for x, y in zip(a0, ref)]
+    H.assert_bits_equal(H.host_list(a), acc, f"accumulate {dtype} odd={odd}")
+    H.assert_bits_equal(H.host_list(g), ref, "accumulate leaves the gradients")
+
+    # accumulate and clear
+    nb.accumulate(a, g, True)
+    acc = [O.add(x, y) for x, y in zip(acc, ref)]
+    H.assert_bits_equal(H.host_list(a), acc, f"accumulate + zero {dtype} odd={odd}")
+    assert not any(t.any() for t in H.host_list(g))
+
+    # zero_grad
+    nb.zero_grad(a)
+    assert not any(t.any() for t in H.host_list(a))
+
+    # nothing outside the views was touched: the gaps between them still hold zeros
+    import torch
+
+    for buf, before, views in ((gbuf, before_g, g), (abuf, before_a, a)):
+        mask = torch.ones_like(buf, dtype=torch.bool)
+        base = buf.data_ptr()
+        for v in views:
+            s = (v.data_ptr() - base) // buf.element_size()
+            mask[s:s + v.numel()] = False
+        assert bool((buf[mask] == before[mask]).all()) and not bool(buf[mask].any())
+
+
+@pytest.mark.parametrize("odd", [False, True])
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+@pytest.mark.parametrize("momentum,wd", [(0.0, 0.0), (0.9, 0.01)])
+def test_sgd_steps_over_views(gpu, dtype, odd, momentum, wd):
+    p0, (pbuf, p) = _make(dtype, 51, 0.05, odd)
+    g0, (_, g) = _make(dtype, 71, 1e-2, odd)
+    shapes = [(1, n) for n in SIZES]
+    opt = nb.Sgd.new(0.05, shapes, dtype=dtype).momentum(momentum).weight_decay(wd)
+    meta = O.sgd_meta(0.05, momentum=momentum, weight_decay=wd)
+    ref, vel = [x.copy() for x in p0], [np.zeros_like(x) for x in p0]
+    for _ in range(3):
+        opt.step(p, g)
+        O.sgd_step(meta, ref, g0, vel)
+    H.assert_bits_equal(H.host_list(p), ref, f"Sgd {dtype} odd={odd} momentum={momentum}")
+    H.assert_bits_equal(H.host_list(g), g0, "Sgd leaves the gradients")
