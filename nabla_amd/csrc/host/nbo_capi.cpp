@@ -106,32 +106,63 @@ bool pure_half(const nbo_optim *opt) { return is_half(opt->state_dtype); }
 // kernel id for element type `dtype`: f32 / bf16 / f64 are `base + dtype`, f16 has its own
 int kernel_for(int base, int f16_id, int dtype) { return dtype == NBO_DT_F16 ? f16_id : base + dtype; }
 
+// Element-type family of an optimizer's update kernels: f32 0, bf16 over f32 master weights 1,
+// f64 2, f16 over f32 master weights 3, bf16 throughout 4, f16 throughout 5.
+int update_family(const nbo_optim *opt, const nbo_list *params)
+{
+    return opt->state_dtype == NBO_DT_BF16 ? 4 : opt->state_dtype == NBO_DT_F16 ? 5 :
+           params->dtype == NBO_DT_F16 ? 3 : params->dtype; // f32 0, bf16 1, f64 2
+}
+
+// Lists of fewer chunks than this take the Adam kinds' by-row kernels.  Measured in alternating
+// launches inside one process, whole fused step, by chunk against by row: GPT-2-small f32 0.637 /
+// 0.625 ms, 1.1 G mixed 5.177 / 5.135, 1.9 G 9.00 / 8.96, 2.8 G 13.10 / 13.10, 4.1 G 19.22 / 19.13,
+// 8 G 37.42 / 37.51; f64 lists of 0.3 and 0.8 G parameters 2 % faster by row.  Short-lived
+// workgroups fill and drain the chip in an eighth of the time, and below some 4 G parameters the
+// steady state is no slower.
+constexpr uint32_t NBO_ROWS_MAX_CHUNKS = 524288;
+// ... and an unfused Adam / AdamW step over fewer chunks than this stays one launch: below some
+// 20 us of work a second launch costs more than the shape gains.
+constexpr uint32_t NBO_ROWS_MIN_CHUNKS_UNFUSED = 512;
+
+// By row, a chunk is eight (f64: sixteen) workgroups whether it is whole or the ragged end of a
+// tensor, and the workgroups of rows it does not have still look their chunk up before they end:
+// a list of many small tensors is slower by row (the 4096-tensor ragged set: 0.150 against
+// 0.137 ms per step).  So: by row only if nine chunks in ten are whole.  16-bit state and
+// arithmetic has four rows to a chunk as it is and is level or slower by row (1.1 G parameters:
+// 2.86 against 2.80 ms): never.
+bool update_by_row(const nbo_optim *opt)
+{
+    if (opt->meta.kind == NBO_KIND_SGD) return true; // the SGD kernels are by row throughout
+    return !pure_half(opt) && opt->layout.nchunks < NBO_ROWS_MAX_CHUNKS &&
+           (uint64_t)opt->layout.whole_chunks * 10 >= (uint64_t)opt->layout.nchunks * 9;
+}
+
 int update_kernel(const nbo_optim *opt, const nbo_list *params)
 {
     const int kind = opt->meta.kind;
+    if (kind != NBO_KIND_SGD && update_by_row(opt)) return K_UPDATE_ROWS_BASE + update_family(opt, params) * 2 + kind;
     if (opt->state_dtype == NBO_DT_BF16) return K_UPDATE_PBF16_BASE + kind;
     if (opt->state_dtype == NBO_DT_F16) return K_UPDATE_PF16_BASE + kind;
     if (params->dtype == NBO_DT_F16) return K_UPDATE_F16_BASE + kind;
     return K_UPDATE_BASE + params->dtype * 3 + kind;
 }
 
-// Grid of update_kernel(): one workgroup per chunk; the SGD kernels run one per row of a chunk
-// (a row: one vector of 2, 4 or 8 elements per thread; update_chunk's BY_ROW in the kernels).
+// Grid of update_kernel(): one workgroup per chunk, or, by row, one per row of a chunk (a row:
+// one vector of 2, 4 or 8 elements per thread; update_chunk's BY_ROW in the kernels).
 uint32_t update_grid(const nbo_optim *opt, const nbo_list *params)
 {
-    if (opt->meta.kind != NBO_SGD) return opt->layout.nchunks;
+    if (!update_by_row(opt)) return opt->layout.nchunks;
     const uint32_t vec = is_half(opt->state_dtype) ? 8u : params->dtype == NBO_DT_F64 ? 2u : 4u;
     const uint64_t rows = (uint64_t)opt->layout.nchunks * (NBO_CHUNK / (NBO_BLOCK * vec));
-    require(rows <= 0x7FFFFFFFull, NBO_ERR_TOO_LARGE, "list too large for one launch");
+    require(rows <= 0xFFFFFFFFull, NBO_ERR_TOO_LARGE, "list too large for one launch");
     return (uint32_t)rows;
 }
 
 // ... of the kernels that prepare the step's scalars themselves
 int self_update_kernel(const nbo_optim *opt, const nbo_list *params)
 {
-    const int family = opt->state_dtype == NBO_DT_BF16 ? 4 : opt->state_dtype == NBO_DT_F16 ? 5 :
-                       params->dtype == NBO_DT_F16 ? 3 : params->dtype; // f32 0, bf16 1, f64 2
-    return K_UPDATE_SELF_BASE + family * 3 + opt->meta.kind;
+    return K_UPDATE_SELF_BASE + update_family(opt, params) * 3 + opt->meta.kind;
 }
 
 // One launch that prepares its own scalars, advances step_count (unless *gf says the step is
@@ -227,7 +258,7 @@ void fused_step_launches(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, n
     f.hyper = hyper_of(opt);
     launch_norm(grads, scaler ? scaler->dev : nullptr, pure_half(opt), ws, f);
     NboUpdateArgs a = update_args(opt, params, grads, true, zero_mode(flags));
-    rt.launch_raw(update_kernel(opt, params), update_grid(opt, params), NBO_BLOCK, &a, ws.may_time);
+    rt.launch_raw(update_kernel(opt, params), update_grid(opt, params), NBO_BLOCK, &a, ws.may_time, 0, update_by_row(opt));
 }
 
 // LDS per workgroup that leaves a compute unit room for four workgroups (160 KiB / 40 KiB)
@@ -239,7 +270,7 @@ uint32_t ew_grid(uint32_t nchunks, int dtype, uint32_t piece_bytes)
 {
     const uint32_t chunk_bytes = NBO_CHUNK * (dtype == NBO_DT_F64 ? 8u : is_half(dtype) ? 2u : 4u);
     const uint64_t pieces = (uint64_t)nchunks * (chunk_bytes / (piece_bytes < chunk_bytes ? piece_bytes : chunk_bytes));
-    require(pieces <= 0x7FFFFFFFull, NBO_ERR_TOO_LARGE, "list too large for one launch");
+    require(pieces <= 0xFFFFFFFFull, NBO_ERR_TOO_LARGE, "list too large for one launch");
     return (uint32_t)pieces;
 }
 
@@ -253,9 +284,9 @@ void launch_scale(nbo_list *grads, const NboGradFactors *gf, double factor, uint
     a.mode = mode;
     // a pure fill (nothing is read) measured 5-9 % faster with four workgroups per compute unit
     // than with eight: 7.3 against 6.7 TB/s on 738 M f32 elements
-    Runtime::get().launch(kernel_for(K_SCALE_BASE, K_SCALE_F16, grads->dtype),
-                          ew_grid(grads->layout.nchunks, grads->dtype, NBO_EW_PIECE_BYTES), NBO_BLOCK, a,
-                          mode == 3 ? NBO_WRITE_HEAVY_IDLE_LDS : 0u);
+    Runtime::get().launch_folded(kernel_for(K_SCALE_BASE, K_SCALE_F16, grads->dtype),
+                                 ew_grid(grads->layout.nchunks, grads->dtype, NBO_EW_PIECE_BYTES), NBO_BLOCK, a,
+                                 mode == 3 ? NBO_WRITE_HEAVY_IDLE_LDS : 0u);
 }
 
 // "m12" -> ('m', 12) with the reference's parsing rules (alg.rs:491-507): the prefix
@@ -585,17 +616,22 @@ int nbo_optim_step(nbo_optim *opt, nbo_list *params, nbo_list *grads)
             a.sgd_lr = opt->meta.lr;
             a.sgd_momentum = opt->meta.momentum;
             a.sgd_weight_decay = opt->meta.weight_decay;
-        } else if (self_update_possible(opt)) {
+        } else if (self_update_possible(opt) &&
+                   !(update_by_row(opt) && opt->layout.nchunks >= NBO_ROWS_MIN_CHUNKS_UNFUSED)) {
             // Adam::step / AdamW::step is one call (alg.rs:109-150, 254-291): one launch
             launch_self_update(opt, params, grads, nullptr, 0u, nullptr, nullptr);
             return;
         } else {
+            // a list of middle size: the by-row kernel behind the scalar preparation (1.5 us in
+            // front of it) is faster than the one launch, 0.543 against 0.555 ms for GPT-2-small
+            // (the self-preparing kernels cannot run by row: their once-per-workgroup counter
+            // would take eight times the additions to one address)
             NboPrepArgs p = {};
             p.opt = opt->dev;
             p.hyper = hyper_of(opt);
             rt.launch(K_PREP, 1, 64, p);
         }
-        rt.launch(update_kernel(opt, params), update_grid(opt, params), NBO_BLOCK, a);
+        rt.launch_raw(update_kernel(opt, params), update_grid(opt, params), NBO_BLOCK, &a, true, 0, update_by_row(opt));
     });
 }
 
@@ -1031,9 +1067,9 @@ int nbo_accumulate(nbo_list *accum, nbo_list *grads, int zero_grads)
         a.b_ptrs = grads->ptrs_dev;
         a.zero_b = zero_grads ? 1u : 0u;
         // with the gradients cleared the pass writes as much as it reads: fewer workgroups in flight (+6 %)
-        Runtime::get().launch(kernel_for(K_ACCUM_BASE, K_ACCUM_F16, accum->dtype),
-                              ew_grid(accum->layout.nchunks, accum->dtype, NBO_EW_PIECE_BYTES), NBO_BLOCK, a,
-                              zero_grads ? NBO_WRITE_HEAVY_IDLE_LDS : 0u);
+        Runtime::get().launch_folded(kernel_for(K_ACCUM_BASE, K_ACCUM_F16, accum->dtype),
+                                     ew_grid(accum->layout.nchunks, accum->dtype, NBO_EW_PIECE_BYTES), NBO_BLOCK, a,
+                                     zero_grads ? NBO_WRITE_HEAVY_IDLE_LDS : 0u);
     });
 }
 
@@ -1091,7 +1127,7 @@ int nbo_fused_step_norm(nbo_optim *opt, nbo_list *params, nbo_list *grads, doubl
         rt.launch(K_FINALIZE, 1, NBO_BLOCK, f);
         const NboUpdateArgs a =
             update_args(opt, params, grads, true, zero_mode(flags));
-        rt.launch(update_kernel(opt, params), update_grid(opt, params), NBO_BLOCK, a);
+        rt.launch_raw(update_kernel(opt, params), update_grid(opt, params), NBO_BLOCK, const_cast<NboUpdateArgs *>(&a), true, 0, update_by_row(opt));
     });
 }
 
@@ -1145,7 +1181,8 @@ int nbo_backend_apply(int op, nbo_list *out, nbo_list *a, nbo_list *b, double s)
         e.b_ptrs = needs_b ? b->ptrs_dev : nullptr;
         e.s = s;
         e.op = (uint32_t)op;
-        Runtime::get().launch(kernel_for(K_EW_BASE, K_EW_F16, out->dtype), ew_grid(out->layout.nchunks, out->dtype, NBO_BACKEND_PIECE_BYTES), NBO_BLOCK, e);
+        Runtime::get().launch_folded(kernel_for(K_EW_BASE, K_EW_F16, out->dtype),
+                                     ew_grid(out->layout.nchunks, out->dtype, NBO_BACKEND_PIECE_BYTES), NBO_BLOCK, e);
     });
 }
 
@@ -1161,8 +1198,8 @@ int nbo_backend_cast(nbo_list *dst, nbo_list *src)
         c.dst_type = (uint32_t)dst->dtype;
         c.src_type = (uint32_t)src->dtype;
         const uint64_t rows = (uint64_t)dst->layout.nchunks * (NBO_CHUNK / NBO_CAST_ROW);
-        require(rows <= 0x7FFFFFFFull, NBO_ERR_TOO_LARGE, "list too large for one launch");
-        Runtime::get().launch(K_CAST_LIST, (uint32_t)rows, NBO_BLOCK, c);
+        require(rows <= 0xFFFFFFFFull, NBO_ERR_TOO_LARGE, "list too large for one launch");
+        Runtime::get().launch_folded(K_CAST_LIST, (uint32_t)rows, NBO_BLOCK, c);
     });
 }
 

@@ -55,8 +55,12 @@ static const char *const kKernelNames[K_COUNT] = {
     "nbo_update_f16_adamw_self",   "nbo_update_f16_adam_self",   "nbo_update_f16_sgd_self",
     "nbo_update_pbf16_adamw_self", "nbo_update_pbf16_adam_self", "nbo_update_pbf16_sgd_self",
     "nbo_update_pf16_adamw_self",  "nbo_update_pf16_adam_self",  "nbo_update_pf16_sgd_self",
+    "nbo_update_f32_adamw_rows",   "nbo_update_f32_adam_rows",   "nbo_update_bf16_adamw_rows",
+    "nbo_update_bf16_adam_rows",   "nbo_update_f64_adamw_rows",  "nbo_update_f64_adam_rows",
+    "nbo_update_f16_adamw_rows",   "nbo_update_f16_adam_rows",
 };
-static_assert(K_UPDATE_SELF_BASE + 18 == K_COUNT, "six families of three self-preparing update kernels");
+static_assert(K_UPDATE_SELF_BASE + 18 == K_UPDATE_ROWS_BASE, "six families of three self-preparing update kernels");
+static_assert(K_UPDATE_ROWS_BASE + 8 == K_COUNT, "four families of two by-row update kernels");
 
 static std::mutex g_runtime_mu;
 static Runtime *g_runtime = nullptr;
@@ -83,6 +87,10 @@ Runtime::Runtime()
         fail(NBO_ERR_NO_DEVICE, "no HIP device is visible; this library runs on gfx950 only");
     }
     hip_check(hipSetDevice(0), "hipSetDevice(0)");
+    if (const char *gx = std::getenv("NBO_GRID_X_MAX")) { // test hook: fold the grids of small lists as well
+        const long v = std::atol(gx);
+        if (v >= 1 && v <= 0xFFFFFF) grid_x_max_ = (uint32_t)v;
+    }
     hipDeviceProp_t prop;
     hip_check(hipGetDeviceProperties(&prop, 0), "hipGetDeviceProperties");
     if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
@@ -158,9 +166,15 @@ int Runtime::bench_kernel(const char *name)
     return K_COUNT + (int)bench_names_.size() - 1;
 }
 
-void Runtime::launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct, bool may_time, uint32_t idle_lds)
+void Runtime::launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct, bool may_time, uint32_t idle_lds,
+                         bool folded)
 {
     if (grid == 0) return;
+    uint32_t gx = grid, gy = 1;
+    if (folded && grid > grid_x_max_) {
+        gx = grid_x_max_;
+        gy = (uint32_t)(((uint64_t)grid + gx - 1) / gx);
+    }
     const hipFunction_t fn = function(kernel);
     void *args[1] = {arg_struct};
     ProfRec rec = {kernel, nullptr, nullptr};
@@ -170,7 +184,7 @@ void Runtime::launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_st
         hip_check(hipEventCreate(&rec.end), "hipEventCreate");
         hip_check(hipEventRecord(rec.begin, stream_), "hipEventRecord");
     }
-    hip_check(hipModuleLaunchKernel(fn, grid, 1, 1, block, 1, 1, idle_lds, stream_, args, nullptr), kernel_name(kernel));
+    hip_check(hipModuleLaunchKernel(fn, gx, gy, 1, block, 1, 1, idle_lds, stream_, args, nullptr), kernel_name(kernel));
     if (timed) {
         hip_check(hipEventRecord(rec.end, stream_), "hipEventRecord");
         prof_.push_back(rec);
@@ -384,13 +398,14 @@ void Layout::build(uint64_t nt, const uint64_t *r, const uint64_t *c, bool with_
     n.resize(nt);
     soff.assign(nt, 0);
     std::vector<uint32_t> chunk_begin(nt + 1, 0);
-    uint64_t chunks = 0, off = 0;
+    uint64_t chunks = 0, off = 0, whole = 0;
     for (uint64_t t = 0; t < nt; t++) {
         if (cols[t] != 0 && rows[t] > UINT64_MAX / cols[t])
             fail(NBO_ERR_TOO_LARGE, "tensor element count overflows 64 bits");
         n[t] = rows[t] * cols[t];
         chunk_begin[t] = (uint32_t)chunks;
         chunks += (n[t] + NBO_CHUNK - 1) / NBO_CHUNK;
+        whole += n[t] / NBO_CHUNK;
         // one workgroup per chunk: the launch's total thread count has to stay below 2^32
         if (chunks * NBO_BLOCK > 0xFFFFFFFFull)
             fail(NBO_ERR_TOO_LARGE, "tensor list too large for one launch (more than 2^32 threads)");
@@ -401,6 +416,7 @@ void Layout::build(uint64_t nt, const uint64_t *r, const uint64_t *c, bool with_
     }
     chunk_begin[nt] = (uint32_t)chunks;
     nchunks = (uint32_t)chunks;
+    whole_chunks = (uint32_t)whole;
     arena_elems = off;
     std::vector<uint32_t> chunk_tensor(nchunks);
     for (uint64_t t = 0; t < nt; t++)

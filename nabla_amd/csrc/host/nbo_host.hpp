@@ -61,7 +61,10 @@ enum KernelId {
     // update kernels that prepare their own per-step scalars: + family * 3 + kind, family =
     // f32, bf16, f64, f16, pbf16, pf16
     K_UPDATE_SELF_BASE = 47,
-    K_COUNT = 65 // ids from here on are measurement kernels, handed out by Runtime::bench_kernel
+    // Adam / AdamW one workgroup per row of a chunk: + family * 2 + kind (adamw 0, adam 1), family =
+    // f32, bf16, f64, f16 (state of 32 or 64 bits)
+    K_UPDATE_ROWS_BASE = 65,
+    K_COUNT = 73 // ids from here on are measurement kernels, handed out by Runtime::bench_kernel
 };
 
 // Process-wide runtime: device 0, the loaded module, the stream, scratch buffers.
@@ -81,10 +84,21 @@ public:
     {
         launch_raw(kernel, grid, block, const_cast<Args *>(&args), true, idle_lds);
     }
+    // For the kernels that take their workgroup number from folded_workgroup(): a grid of more
+    // than grid_x_max() workgroups is folded into two dimensions (one dimension of a launch holds
+    // fewer than 2^32 threads).
+    template <typename Args>
+    void launch_folded(int kernel, uint32_t grid, uint32_t block, const Args &args, uint32_t idle_lds = 0)
+    {
+        launch_raw(kernel, grid, block, const_cast<Args *>(&args), true, idle_lds, true);
+    }
     // may_time = false: never bracket the launch with timing events, whatever profile_enable
     // says (creating events allocates host memory)
     void launch_raw(int kernel, uint32_t grid, uint32_t block, void *arg_struct, bool may_time = true,
-                    uint32_t idle_lds = 0);
+                    uint32_t idle_lds = 0, bool folded = false);
+    // 2^24 - 1 workgroups of NBO_BLOCK threads; NBO_GRID_X_MAX in the environment lowers it, so that
+    // a test can fold the grids of small lists
+    uint32_t grid_x_max() const { return grid_x_max_; }
     // Id of kernel `name` of the measurement code object (nbo_bench_kernels.hip), which is
     // loaded when the first such id is asked for; the id works with launch, time_launches and
     // the per-kernel timing like the ids above.
@@ -128,6 +142,7 @@ private:
     const char *kernel_name(int kernel) const;
     hipModule_t module_ = nullptr;
     hipFunction_t fn_[K_COUNT] = {};
+    uint32_t grid_x_max_ = 0xFFFFFFu;
     hipModule_t bench_module_ = nullptr; // loaded on first use
     std::vector<std::string> bench_names_;
     std::vector<hipFunction_t> bench_fn_;
@@ -154,6 +169,7 @@ struct Layout {
     std::vector<uint64_t> rows, cols, n, soff;
     uint64_t arena_elems = 0; // elements an arena needs (with per-tensor alignment)
     uint32_t nchunks = 0;
+    uint32_t whole_chunks = 0; // chunks of NBO_CHUNK elements (the others are the ragged ends of tensors)
     void *blob = nullptr; // one device allocation holding all tables
     NboLayoutDev dev = {};
 

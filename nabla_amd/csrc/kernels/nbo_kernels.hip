@@ -74,6 +74,12 @@ typedef double f64x2_e __attribute__((ext_vector_type(2), aligned(8)));
 // global memory turns flat_* accesses into global_* ones.
 #define GLOBAL_PTR(type, p) ((__attribute__((address_space(1))) type *)(uintptr_t)(p))
 
+// Number of the workgroup in a launch whose grid the host may have folded into two dimensions
+// (one dimension holds fewer than 2^32 threads, i.e. 2^24 workgroups; the passes that run one
+// workgroup per row of a chunk can need more).  The last row of the grid may be partly unused:
+// such kernels compare the number with the count of workgroups they have work for.
+DEV uint32_t folded_workgroup() { return blockIdx.y * gridDim.x + blockIdx.x; }
+
 // ---------------------------------------------------------------------------------
 // bf16 <-> f32, bit for bit what half::bf16 does (from_f32: NaN keeps its payload and
 // gets the quiet bit, everything else rounds to nearest even).
@@ -502,11 +508,17 @@ DEV void make_uniform(NboOptimDev &o)
 // device memory, and the workgroup whose addition completes the grid -- nobody waits for
 // anybody -- writes the advanced step_count and the trace entry and clears the counter.
 //
-// BY_ROW (the SGD kernels outside a grouped step): one workgroup per row of a chunk -- every
-// thread loads one vector of every stream, computes, stores and is done.  With SGD's two or
-// three streams that measured 15-20 % faster than eight rows per workgroup (as it does for the
-// element-wise passes, see stream_pieces); the Adam kinds' five streams do best at eight rows.
-// A chunk that is ragged, misaligned or skipped is done by the workgroup of its first row.
+// BY_ROW (the SGD kernels outside a grouped step, and the "_rows" kernels of the Adam kinds):
+// one workgroup per row of a chunk -- every thread loads one vector of every stream, computes,
+// stores and is done; the chunk's single elements (a ragged end, an unaligned start) go with
+// its first row, and a row the chunk does not have ends at once.  With SGD's two or three
+// streams that is 15-20 % faster than eight rows per workgroup (as it is for the element-wise
+// passes, see stream_pieces).  The Adam kinds' five streams move the same bytes per second
+// either way on the largest lists (0.3 % fewer by row on the 8B set) and 0.5-2 % more by row
+// below some 4 G parameters (GPT-2-small f32 0.555 -> 0.543 ms, the 1.1 G mixed set 5.18 -> 5.14
+// ms, f64 lists 2 %; measured in alternating launches inside one process): the host takes the
+// "_rows" kernels for lists below NBO_ROWS_MAX_CHUNKS chunks.  16-bit state and arithmetic
+// (four rows to a chunk as it is) is level or slower by row and has no such kernels.
 template <int ST, int KIND, bool BY_ROW = false>
 DEV void update_chunk(const NboUpdateArgs &a, const NboOptimDev *o, uint32_t wg)
 {
@@ -516,14 +528,15 @@ DEV void update_chunk(const NboUpdateArgs &a, const NboOptimDev *o, uint32_t wg)
         SB = Traits<ST>::SBYTES,
         ROW = NBO_BLOCK * VEC,
         ROWS = NBO_CHUNK / ROW,
-        UMAX = BY_ROW ? 1 : sizeof(T) == 8 ? NBO_UNROLL / 2 : NBO_UNROLL,
+        UMAX = sizeof(T) == 8 ? NBO_UNROLL / 2 : NBO_UNROLL,
         U = ROWS < UMAX ? ROWS : UMAX,
-        ITERS = BY_ROW ? 1 : ROWS / U
+        ITERS = ROWS / U
     };
     static_assert(ROWS % U == 0 && ROWS * ROW == NBO_CHUNK, "chunk must be a whole number of unrolled rows");
     const bool mixed = ST == NBO_BF16 || ST == NBO_F16; // f32 master lives in the arena
     const bool has_v = KIND != NBO_SGD;
     const uint32_t tid = threadIdx.x;
+    if (BY_ROW && wg / ROWS >= a.L.nchunks) return; // the unused end of a folded grid
     const uint32_t row0 = BY_ROW ? wg % ROWS : 0;
     const ChunkRef c = chunk_ref(a.L, BY_ROW ? wg / ROWS : wg);
 
@@ -537,7 +550,9 @@ DEV void update_chunk(const NboUpdateArgs &a, const NboOptimDev *o, uint32_t wg)
     const bool vec_ok = ((((uintptr_t)pp) | ((uintptr_t)pg)) & (vbytes - 1)) == 0;
 
     const bool direct = KIND == NBO_SGD && a.direct != 0;
-    if (BY_ROW && row0 != 0 && !(c.cnt == NBO_CHUNK && vec_ok)) return;
+    // (by row: how the chunk is walked decides first whether this row exists at all)
+    const Peel pl = peel(c.cnt, VEC, SB, sizeof(T) < 4, (uintptr_t)pp, (uintptr_t)pg);
+    if (BY_ROW && row0 != 0 && row0 * NBO_BLOCK >= pl.nvec) return;
     if (!direct && o->skip) {
         // found_inf: parameters, moments and step_count stay untouched
         // (trainer.rs:230-236); the gradients become zeros (core.rs:372-375) if the caller
@@ -549,7 +564,7 @@ DEV void update_chunk(const NboUpdateArgs &a, const NboOptimDev *o, uint32_t wg)
     const Scal<T> s = direct ? Scal<T>(a.sgd_lr, a.sgd_momentum, a.sgd_weight_decay) : Scal<T>(o, a.gf);
     const bool use_m = KIND != NBO_SGD || s.use_mom;
 
-    if (c.cnt == NBO_CHUNK && vec_ok) {
+    if (!BY_ROW && c.cnt == NBO_CHUNK && vec_ok) {
         for (int it = 0; it < ITERS; it++) {
             // U rows of the workgroup at once.  The memory instructions are issued stream by
             // stream -- every row's gradient load, then every row's master load, ... and after
@@ -557,7 +572,7 @@ DEV void update_chunk(const NboUpdateArgs &a, const NboOptimDev *o, uint32_t wg)
             // then sees longer runs per stream, which measured 1.3 % faster on the 8B set (35.0
             // against 35.5 ms in alternating launches inside one process; loads or stores alone
             // in this order: next to nothing).
-            const uint32_t e0 = (BY_ROW ? row0 : it * U) * ROW + tid * VEC;
+            const uint32_t e0 = it * (U * ROW) + tid * VEC;
             T g[U][VEC], p[U][VEC], m[U][VEC] = {}, v[U][VEC] = {};
 #pragma unroll
             for (int u = 0; u < U; u++) IO<ST>::ldv(pg + (uint64_t)(e0 + u * ROW) * SB, g[u]);
@@ -611,8 +626,8 @@ DEV void update_chunk(const NboUpdateArgs &a, const NboOptimDev *o, uint32_t wg)
     // first vector-aligned address of the caller's tensors, whole vectors from there (the state
     // arrays are then read at element alignment, which needs 32- or 64-bit state), single
     // elements for the rest
-    const Peel pl = peel(c.cnt, VEC, SB, sizeof(T) < 4, (uintptr_t)pp, (uintptr_t)pg);
-    for (uint32_t q = tid; q < pl.nvec; q += NBO_BLOCK) {
+    // (by row: the one vector of this row, if the chunk reaches that far)
+    for (uint32_t q = BY_ROW ? row0 * NBO_BLOCK + tid : tid; q < pl.nvec; q += BY_ROW ? NBO_CHUNK : NBO_BLOCK) {
         const uint32_t e = pl.head + q * VEC;
         T g[VEC], p[VEC], m[VEC] = {}, v[VEC] = {};
         IO<ST>::ldv(pg + (uint64_t)e * SB, g);
@@ -632,6 +647,7 @@ DEV void update_chunk(const NboUpdateArgs &a, const NboOptimDev *o, uint32_t wg)
         }
     }
     // elements [0, head) and [head + nvec * VEC, cnt)
+    if (BY_ROW && row0 != 0) return;
     const uint32_t n_single = c.cnt - pl.nvec * VEC;
     for (uint32_t i = tid; i < n_single; i += NBO_BLOCK) {
         const uint32_t e = i < pl.head ? i : i + pl.nvec * VEC;
@@ -679,7 +695,7 @@ template <int ST, int KIND, bool SELF = false> DEV void update_body(const NboUpd
 #define NBO_UPDATE_KERNEL(name, ST, KIND)                                                   \
     extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboUpdateArgs a) \
     {                                                                                       \
-        update_body<ST, KIND>(a, blockIdx.x, gridDim.x);                                    \
+        update_body<ST, KIND>(a, KIND == NBO_SGD ? folded_workgroup() : blockIdx.x, gridDim.x); \
     }
 
 NBO_UPDATE_KERNEL(nbo_update_f32_adamw, NBO_F32, NBO_ADAMW)
@@ -700,6 +716,22 @@ NBO_UPDATE_KERNEL(nbo_update_f16_sgd, NBO_F16, NBO_SGD)
 NBO_UPDATE_KERNEL(nbo_update_pf16_adamw, NBO_PF16, NBO_ADAMW)
 NBO_UPDATE_KERNEL(nbo_update_pf16_adam, NBO_PF16, NBO_ADAM)
 NBO_UPDATE_KERNEL(nbo_update_pf16_sgd, NBO_PF16, NBO_SGD)
+
+// The Adam kinds one workgroup per row (see update_chunk), for 32- and 64-bit state; SGD's kernels
+// above are by row already.
+#define NBO_UPDATE_ROWS_KERNEL(name, ST, KIND)                                              \
+    extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboUpdateArgs a)     \
+    {                                                                                       \
+        update_chunk<ST, KIND, true>(a, a.opt, folded_workgroup());                         \
+    }
+NBO_UPDATE_ROWS_KERNEL(nbo_update_f32_adamw_rows, NBO_F32, NBO_ADAMW)
+NBO_UPDATE_ROWS_KERNEL(nbo_update_f32_adam_rows, NBO_F32, NBO_ADAM)
+NBO_UPDATE_ROWS_KERNEL(nbo_update_bf16_adamw_rows, NBO_BF16, NBO_ADAMW)
+NBO_UPDATE_ROWS_KERNEL(nbo_update_bf16_adam_rows, NBO_BF16, NBO_ADAM)
+NBO_UPDATE_ROWS_KERNEL(nbo_update_f64_adamw_rows, NBO_F64, NBO_ADAMW)
+NBO_UPDATE_ROWS_KERNEL(nbo_update_f64_adam_rows, NBO_F64, NBO_ADAM)
+NBO_UPDATE_ROWS_KERNEL(nbo_update_f16_adamw_rows, NBO_F16, NBO_ADAMW)
+NBO_UPDATE_ROWS_KERNEL(nbo_update_f16_adam_rows, NBO_F16, NBO_ADAM)
 
 // Launches that prepare their own scalars: the unfused Optimizer::step (one launch per call, as
 // the reference's one call) and a grouped fused step, whose groups -- each with its own lists,
@@ -1134,7 +1166,8 @@ DEV void stream_pieces(const NboLayoutDev &L, const uint64_t *const (&lists)[NS]
         PPC = NBO_CHUNK * SB / PIECE
     };
     static_assert(R >= 1 && PPC >= 1 && R * PPC * ROWB == NBO_CHUNK * SB, "pieces divide the chunk");
-    const uint32_t piece = blockIdx.x;
+    const uint32_t piece = folded_workgroup();
+    if (piece / PPC >= L.nchunks) return; // the unused end of a folded grid
     const ChunkRef c = chunk_ref(L, piece / PPC);
     char *p[NS];
     uintptr_t all = 0;
@@ -1562,13 +1595,13 @@ template <int ST> DEV void cast_store4(char *p, uint64_t e, const double (&v)[4]
     }
 }
 
-template <int SRC, int DST> DEV void cast_body(const NboCastListArgs &a)
+template <int SRC, int DST> DEV void cast_body(const NboCastListArgs &a, uint32_t wg)
 {
     enum { SS = Traits<SRC>::SBYTES, DS = Traits<DST>::SBYTES };
     // one workgroup per NBO_CAST_ROW elements of a chunk (four per thread), as the other
     // element-wise passes run; a ragged or misaligned chunk is done by its first workgroup
-    const uint32_t row = blockIdx.x % (NBO_CHUNK / NBO_CAST_ROW);
-    const ChunkRef c = chunk_ref(a.L, blockIdx.x / (NBO_CHUNK / NBO_CAST_ROW));
+    const uint32_t row = wg % (NBO_CHUNK / NBO_CAST_ROW);
+    const ChunkRef c = chunk_ref(a.L, wg / (NBO_CHUNK / NBO_CAST_ROW));
     const char *ps = (const char *)a.src_ptrs[c.t] + c.base * SS;
     char *pd = (char *)a.dst_ptrs[c.t] + c.base * DS;
     // groups of four while both addresses allow whole vectors (16 bytes at most per access)
@@ -1592,20 +1625,22 @@ template <int SRC, int DST> DEV void cast_body(const NboCastListArgs &a)
         cast_store1<DST>(pd, e, cast_load1<SRC>(ps, e));
 }
 
-template <int SRC> DEV void cast_from(const NboCastListArgs &a)
+template <int SRC> DEV void cast_from(const NboCastListArgs &a, uint32_t wg)
 {
-    if (a.dst_type == NBO_F32) cast_body<SRC, NBO_F32>(a);
-    else if (a.dst_type == NBO_BF16) cast_body<SRC, NBO_BF16>(a);
-    else if (a.dst_type == NBO_F16) cast_body<SRC, NBO_F16>(a);
-    else cast_body<SRC, NBO_F64>(a);
+    if (a.dst_type == NBO_F32) cast_body<SRC, NBO_F32>(a, wg);
+    else if (a.dst_type == NBO_BF16) cast_body<SRC, NBO_BF16>(a, wg);
+    else if (a.dst_type == NBO_F16) cast_body<SRC, NBO_F16>(a, wg);
+    else cast_body<SRC, NBO_F64>(a, wg);
 }
 
 extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_cast_list(const NboCastListArgs a)
 {
-    if (a.src_type == NBO_F32) cast_from<NBO_F32>(a);
-    else if (a.src_type == NBO_BF16) cast_from<NBO_BF16>(a);
-    else if (a.src_type == NBO_F16) cast_from<NBO_F16>(a);
-    else cast_from<NBO_F64>(a);
+    const uint32_t wg = folded_workgroup();
+    if (wg / (NBO_CHUNK / NBO_CAST_ROW) >= a.L.nchunks) return; // the unused end of a folded grid
+    if (a.src_type == NBO_F32) cast_from<NBO_F32>(a, wg);
+    else if (a.src_type == NBO_BF16) cast_from<NBO_BF16>(a, wg);
+    else if (a.src_type == NBO_F16) cast_from<NBO_F16>(a, wg);
+    else cast_from<NBO_F64>(a, wg);
 }
 
 // Zero-fill of an arbitrary byte range: single bytes up to the first 16-byte boundary,

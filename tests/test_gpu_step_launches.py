@@ -4,6 +4,9 @@ The reference's `Adam::step` / `AdamW::step` is one call (alg.rs:109-150, 254-29
 one launch of a kernel that prepares its own per-step scalars and advances step_count exactly
 once; a grouped fused step is the norm pass, its second stage and ONE update launch for up to
 sixteen groups of one optimizer kind (each with its own hyper-parameters, optim/groups.rs:269-293).
+Lists of middle size (512 to 131071 work chunks, nine in ten of them whole) take the update
+kernels that run one workgroup per row of a chunk; unfused, those follow the scalar-preparation
+launch.
 `unscale_and_update` leaves zeros in the gradients when it finds inf / NaN (core.rs:372-375):
 the fused step does so with NBO_STEP_ZERO_ON_SKIP."""
 import ctypes as C
@@ -220,3 +223,116 @@ def test_a_skipped_step_leaves_zeros_in_the_gradients_when_asked_to(gpu, grouped
     opt.fused_step(p_dev, g_dev, scaler=scaler, max_norm=1.0, zero_on_skip=True)
     H.assert_bits_equal(H.host_list(g_dev), g_bits, "gradients of a step that ran")
     assert set(counts()) == {1}
+
+
+def test_a_list_of_middle_size_takes_the_by_row_kernels(gpu):
+    """700 work chunks, most of them whole, one tensor ragged and one tiny: the unfused Adam step
+    is the scalar preparation plus the by-row kernel, the fused AdamW step the norm pass, its
+    second stage and the by-row kernel -- and both give the oracle's bits, step after step."""
+    shapes = [(600, 8192), (1, 8192 * 99 + 4099), (3, 5)]
+    p0, g0 = H.randn_list(shapes, 131, 0.02), H.randn_list(shapes, 132, 1e-3)
+    L = _lib.load()
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        # unfused Adam
+        p_dev, g_dev = H.dev_list(p0, shapes), H.dev_list(g0, shapes)
+        opt = nb.Adam.new(1e-3, shapes)
+        meta = O.adam_meta(1e-3)
+        ref, m, v = H.copy_list(p0), H.zeros_like_list(p0), H.zeros_like_list(p0)
+        for step in range(3):
+            _lib.check(L.nbo_profile_enable(1))
+            opt.step(p_dev, g_dev)
+            n = _launches(["nbo_prep", "nbo_update_f32_adam_rows", "nbo_update_f32_adam_self", "nbo_update_f32_adam"])
+            _lib.check(L.nbo_profile_enable(0))
+            assert n == {"nbo_prep": 1, "nbo_update_f32_adam_rows": 1, "nbo_update_f32_adam_self": 0,
+                         "nbo_update_f32_adam": 0}
+            O.adam_step(meta, ref, g0, m, v)
+        assert opt.step_count() == 3
+        H.assert_bits_equal(H.host_list(p_dev), ref, "unfused Adam by row: params")
+        H.assert_bits_equal(H.host_list(opt.moments()[0]), m, "m")
+        H.assert_bits_equal(H.host_list(opt.moments()[1]), v, "v")
+        del opt
+
+        # fused AdamW with clipping and gradient zeroing
+        p_dev = H.dev_list(p0, shapes)
+        opt = nb.AdamW.new(2e-4, shapes).beta2(0.95).weight_decay(0.1)
+        meta = O.adamw_meta(2e-4, beta2=0.95, weight_decay=0.1)
+        ref, m, v = H.copy_list(p0), H.zeros_like_list(p0), H.zeros_like_list(p0)
+        for step in range(3):
+            g = H.randn_list(shapes, 140 + step, 1e-2)
+            g_dev = H.dev_list(g, shapes)
+            _lib.check(L.nbo_profile_enable(1))
+            opt.fused_step(p_dev, g_dev, max_norm=0.5, zero_grads=True)
+            n = _launches(["nbo_norm_f32", "nbo_finalize", "nbo_update_f32_adamw_rows", "nbo_update_f32_adamw", "nbo_prep"])
+            _lib.check(L.nbo_profile_enable(0))
+            assert n == {"nbo_norm_f32": 1, "nbo_finalize": 1, "nbo_update_f32_adamw_rows": 1, "nbo_update_f32_adamw": 0,
+                         "nbo_prep": 0}
+            info = opt.last_step()
+            gf = H.copy_list(g)
+            H.oracle_step_with_device_norm(lambda: (True, O.clip_grad_norm(gf, 0.5)), [gf], [], 0.5, info,
+                                           f"by-row fused step {step}")
+            O.adam_step(meta, ref, gf, m, v)
+            assert info.clipped == 1 and not any(t.any() for t in H.host_list(g_dev))
+        H.assert_bits_equal(H.host_list(p_dev), ref, "fused AdamW by row: params")
+        H.assert_bits_equal(H.host_list(opt.moments()[0]), m, "m")
+        H.assert_bits_equal(H.host_list(opt.moments()[1]), v, "v")
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+
+
+def test_grids_folded_into_two_dimensions_cover_every_row_once(gpu):
+    """One grid dimension holds fewer than 2^32 threads, so the launches that run one workgroup per
+    row of a chunk fold a larger grid into two dimensions.  With NBO_GRID_X_MAX=37 in the
+    environment (a test hook of the runtime) every such launch here is folded, its last grid row
+    partly unused: the element-wise passes, the cast, SGD and the by-row Adam kernels must still
+    do every row exactly once."""
+    import os
+    import subprocess
+    import sys
+
+    code = r"""
+import numpy as np, torch
+import oracle as O
+from nabla_amd import _lib, optim as nb, backend as B
+from tests import helpers as H
+_lib.init()
+shapes = [(520, 8192), (1, 8192 * 3 + 4099), (3, 5)]
+p0, g0 = H.randn_list(shapes, 231, 0.02), H.randn_list(shapes, 232, 1e-3)
+O.set_pow_mode(O.POW_SQRT)
+# element-wise passes
+a, g = H.dev_list(p0, shapes), H.dev_list(g0, shapes)
+nb.scale_grad(g, 0.3)
+sg = H.copy_list(g0); O.scale_grad(sg, 0.3)
+H.assert_bits_equal(H.host_list(g), sg, "scale_grad")
+nb.accumulate(a, g, True)
+H.assert_bits_equal(H.host_list(a), [O.add(x, y) for x, y in zip(p0, sg)], "accumulate")
+assert not any(t.any() for t in H.host_list(g))
+out = [torch.zeros_like(t) for t in a]
+B.add(H.dev_list(p0, shapes), H.dev_list(g0, shapes), out=out)
+H.assert_bits_equal(H.host_list(out), [O.add(x, y) for x, y in zip(p0, g0)], "backend add")
+half = H.dev_list([np.zeros(x.shape, dtype=np.uint16) for x in p0], shapes)
+B.cast(H.dev_list(p0, shapes), half)
+H.assert_bits_equal(H.host_list(half), [O.bf16_from_f32(x) for x in p0], "cast")
+# SGD with momentum, three steps
+p, g = H.dev_list(p0, shapes), H.dev_list(g0, shapes)
+opt = nb.Sgd.new(0.05, shapes).momentum(0.9).weight_decay(0.01)
+meta = O.sgd_meta(0.05, momentum=0.9, weight_decay=0.01)
+ref, vel = H.copy_list(p0), H.zeros_like_list(p0)
+for _ in range(3):
+    opt.step(p, g); O.sgd_step(meta, ref, g0, vel)
+H.assert_bits_equal(H.host_list(p), ref, "Sgd")
+# Adam by row (unfused: preparation + by-row kernel), three steps
+p = H.dev_list(p0, shapes)
+opt = nb.Adam.new(1e-3, shapes)
+meta = O.adam_meta(1e-3)
+ref, m, v = H.copy_list(p0), H.zeros_like_list(p0), H.zeros_like_list(p0)
+for _ in range(3):
+    opt.step(p, g); O.adam_step(meta, ref, g0, m, v)
+H.assert_bits_equal(H.host_list(p), ref, "Adam")
+H.assert_bits_equal(H.host_list(opt.moments()[1]), v, "v")
+print("folded ok")
+"""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, NBO_GRID_X_MAX="37", PYTHONPATH=root)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300, cwd=root, env=env)
+    assert r.returncode == 0 and "folded ok" in r.stdout, r.stdout[-2000:] + r.stderr[-3000:]
