@@ -120,22 +120,22 @@ int update_family(const nbo_optim *opt, const nbo_list *params)
 // 8 G 37.42 / 37.51; f64 lists of 0.3 and 0.8 G parameters 2 % faster by row.  Short-lived
 // workgroups fill and drain the chip in an eighth of the time, and below some 4 G parameters the
 // steady state is no slower.
-constexpr uint32_t NBO_ROWS_MAX_CHUNKS = 524288;
 // ... and an unfused Adam / AdamW step over fewer chunks than this stays one launch: below some
 // 20 us of work a second launch costs more than the shape gains.
 constexpr uint32_t NBO_ROWS_MIN_CHUNKS_UNFUSED = 512;
 
 // By row, a chunk is eight (f64: sixteen) workgroups whether it is whole or the ragged end of a
-// tensor, and the workgroups of rows it does not have still look their chunk up before they end:
-// a list of many small tensors is slower by row (the 4096-tensor ragged set: 0.150 against
-// 0.137 ms per step).  So: by row only if nine chunks in ten are whole.  16-bit state and
-// arithmetic has four rows to a chunk as it is and is level or slower by row (1.1 G parameters:
-// 2.86 against 2.80 ms): never.
+// tensor, and a workgroup of a row the chunk does not have still looks its chunk up before it
+// ends: launched that way, a list of many small tensors is slower by row (the 4096-tensor ragged
+// set: 0.150 against 0.137 ms per step).  Such a list -- fewer than nine chunks in ten whole --
+// carries a map of the rows that exist (Layout::build), and the launch has a workgroup for each
+// of those and no other.  16-bit state and arithmetic has four rows to a chunk as it is and is
+// level or slower by row (1.1 G parameters: 2.86 against 2.80 ms): never.
 bool update_by_row(const nbo_optim *opt)
 {
     if (opt->meta.kind == NBO_KIND_SGD) return true; // the SGD kernels are by row throughout
     return !pure_half(opt) && opt->layout.nchunks < NBO_ROWS_MAX_CHUNKS &&
-           (uint64_t)opt->layout.whole_chunks * 10 >= (uint64_t)opt->layout.nchunks * 9;
+           (opt->layout.mostly_whole() || opt->layout.dev.row_map != nullptr);
 }
 
 int update_kernel(const nbo_optim *opt, const nbo_list *params)
@@ -153,6 +153,7 @@ int update_kernel(const nbo_optim *opt, const nbo_list *params)
 uint32_t update_grid(const nbo_optim *opt, const nbo_list *params)
 {
     if (!update_by_row(opt)) return opt->layout.nchunks;
+    if (opt->layout.dev.row_map) return opt->layout.dev.nrows;
     const uint32_t vec = is_half(opt->state_dtype) ? 8u : params->dtype == NBO_DT_F64 ? 2u : 4u;
     const uint64_t rows = (uint64_t)opt->layout.nchunks * (NBO_CHUNK / (NBO_BLOCK * vec));
     require(rows <= 0xFFFFFFFFull, NBO_ERR_TOO_LARGE, "list too large for one launch");
@@ -265,11 +266,16 @@ void fused_step_launches(nbo_optim *opt, nbo_scaler *scaler, nbo_list *params, n
 constexpr uint32_t NBO_WRITE_HEAVY_IDLE_LDS = 40960;
 
 // Grid of the element-wise passes (stream_pieces in the kernels): one workgroup per piece of
-// `piece_bytes` (a whole chunk if that is smaller) of a list of `nchunks` chunks of `dtype`.
-uint32_t ew_grid(uint32_t nchunks, int dtype, uint32_t piece_bytes)
+// `piece_bytes` (a whole chunk if that is smaller) of a list -- or, for a list of many small
+// tensors (fewer than nine chunks in ten whole), one per chunk: most pieces of such a list do not
+// exist, and a workgroup has to look its chunk up to find that out (the 4096-tensor ragged set:
+// scale_grad 65 us by piece, 38 us by chunk).  *by_chunk tells the kernel which it is.
+uint32_t ew_grid(const Layout &layout, int dtype, uint32_t piece_bytes, uint32_t *by_chunk)
 {
+    *by_chunk = layout.mostly_whole() ? 0u : 1u;
+    if (*by_chunk) return layout.nchunks;
     const uint32_t chunk_bytes = NBO_CHUNK * (dtype == NBO_DT_F64 ? 8u : is_half(dtype) ? 2u : 4u);
-    const uint64_t pieces = (uint64_t)nchunks * (chunk_bytes / (piece_bytes < chunk_bytes ? piece_bytes : chunk_bytes));
+    const uint64_t pieces = (uint64_t)layout.nchunks * (chunk_bytes / (piece_bytes < chunk_bytes ? piece_bytes : chunk_bytes));
     require(pieces <= 0xFFFFFFFFull, NBO_ERR_TOO_LARGE, "list too large for one launch");
     return (uint32_t)pieces;
 }
@@ -284,8 +290,8 @@ void launch_scale(nbo_list *grads, const NboGradFactors *gf, double factor, uint
     a.mode = mode;
     // a pure fill (nothing is read) measured 5-9 % faster with four workgroups per compute unit
     // than with eight: 7.3 against 6.7 TB/s on 738 M f32 elements
-    Runtime::get().launch_folded(kernel_for(K_SCALE_BASE, K_SCALE_F16, grads->dtype),
-                                 ew_grid(grads->layout.nchunks, grads->dtype, NBO_EW_PIECE_BYTES), NBO_BLOCK, a,
+    const uint32_t grid = ew_grid(grads->layout, grads->dtype, NBO_EW_PIECE_BYTES, &a.by_chunk);
+    Runtime::get().launch_folded(kernel_for(K_SCALE_BASE, K_SCALE_F16, grads->dtype), grid, NBO_BLOCK, a,
                                  mode == 3 ? NBO_WRITE_HEAVY_IDLE_LDS : 0u);
 }
 
@@ -555,7 +561,9 @@ int nbo_optim_create(const nbo_meta *meta, uint64_t n_tensors, const uint64_t *r
             o->meta = *meta;
             o->state_dtype = state_dtype;
             o->keep_master = keep_master != 0;
-            o->layout.build(n_tensors, rows, cols, true);
+            // (a by-row update workgroup takes one 128-bit vector of state per thread)
+            o->layout.build(n_tensors, rows, cols, true,
+                            is_half(state_dtype) ? 0u : NBO_BLOCK * (state_dtype == NBO_DT_F64 ? 2u : 4u));
             const bool adam_like = meta->kind != NBO_KIND_SGD;
             o->arena.nparts = 1u + (adam_like ? 1u : 0u) + (o->keep_master ? 1u : 0u);
             o->arena.part_v = 1;
@@ -1067,8 +1075,8 @@ int nbo_accumulate(nbo_list *accum, nbo_list *grads, int zero_grads)
         a.b_ptrs = grads->ptrs_dev;
         a.zero_b = zero_grads ? 1u : 0u;
         // with the gradients cleared the pass writes as much as it reads: fewer workgroups in flight (+6 %)
-        Runtime::get().launch_folded(kernel_for(K_ACCUM_BASE, K_ACCUM_F16, accum->dtype),
-                                     ew_grid(accum->layout.nchunks, accum->dtype, NBO_EW_PIECE_BYTES), NBO_BLOCK, a,
+        const uint32_t grid = ew_grid(accum->layout, accum->dtype, NBO_EW_PIECE_BYTES, &a.by_chunk);
+        Runtime::get().launch_folded(kernel_for(K_ACCUM_BASE, K_ACCUM_F16, accum->dtype), grid, NBO_BLOCK, a,
                                      zero_grads ? NBO_WRITE_HEAVY_IDLE_LDS : 0u);
     });
 }
@@ -1181,8 +1189,8 @@ int nbo_backend_apply(int op, nbo_list *out, nbo_list *a, nbo_list *b, double s)
         e.b_ptrs = needs_b ? b->ptrs_dev : nullptr;
         e.s = s;
         e.op = (uint32_t)op;
-        Runtime::get().launch_folded(kernel_for(K_EW_BASE, K_EW_F16, out->dtype),
-                                     ew_grid(out->layout.nchunks, out->dtype, NBO_BACKEND_PIECE_BYTES), NBO_BLOCK, e);
+        const uint32_t grid = ew_grid(out->layout, out->dtype, NBO_BACKEND_PIECE_BYTES, &e.by_chunk);
+        Runtime::get().launch_folded(kernel_for(K_EW_BASE, K_EW_F16, out->dtype), grid, NBO_BLOCK, e);
     });
 }
 
@@ -1197,7 +1205,8 @@ int nbo_backend_cast(nbo_list *dst, nbo_list *src)
         c.src_ptrs = src->ptrs_dev;
         c.dst_type = (uint32_t)dst->dtype;
         c.src_type = (uint32_t)src->dtype;
-        const uint64_t rows = (uint64_t)dst->layout.nchunks * (NBO_CHUNK / NBO_CAST_ROW);
+        c.by_chunk = dst->layout.mostly_whole() ? 0u : 1u;
+        const uint64_t rows = (uint64_t)dst->layout.nchunks * (c.by_chunk ? 1u : NBO_CHUNK / NBO_CAST_ROW);
         require(rows <= 0xFFFFFFFFull, NBO_ERR_TOO_LARGE, "list too large for one launch");
         Runtime::get().launch_folded(K_CAST_LIST, (uint32_t)rows, NBO_BLOCK, c);
     });

@@ -391,7 +391,7 @@ void Runtime::dzero(void *p, size_t bytes)
 
 static uint64_t align_up(uint64_t x, uint64_t a) { return (x + a - 1) / a * a; }
 
-void Layout::build(uint64_t nt, const uint64_t *r, const uint64_t *c, bool with_arena)
+void Layout::build(uint64_t nt, const uint64_t *r, const uint64_t *c, bool with_arena, uint32_t row_elems)
 {
     rows.assign(r, r + nt);
     cols.assign(c, c + nt);
@@ -422,13 +422,27 @@ void Layout::build(uint64_t nt, const uint64_t *r, const uint64_t *c, bool with_
     for (uint64_t t = 0; t < nt; t++)
         for (uint32_t ch = chunk_begin[t]; ch < chunk_begin[t + 1]; ch++) chunk_tensor[ch] = (uint32_t)t;
 
-    // one blob: n | soff | chunk_begin | chunk_tensor, each 16-byte aligned
+    // the rows that exist, for by-row launches over a list of many small tensors
+    std::vector<uint32_t> row_map;
+    if (row_elems && !mostly_whole() && nchunks < NBO_ROWS_MAX_CHUNKS) {
+        for (uint64_t t = 0; t < nt; t++)
+            for (uint32_t ch = chunk_begin[t]; ch < chunk_begin[t + 1]; ch++) {
+                const uint64_t left = n[t] - (uint64_t)(ch - chunk_begin[t]) * NBO_CHUNK;
+                const uint64_t cnt = left < NBO_CHUNK ? left : NBO_CHUNK;
+                const uint32_t nrow = (uint32_t)((cnt + row_elems - 1) / row_elems); // >= 1: a chunk is never empty
+                for (uint32_t rw = 0; rw < nrow; rw++) row_map.push_back(ch << 4 | rw);
+            }
+    }
+
+    // one blob: n | soff | chunk_begin | chunk_tensor | row_map, each 16-byte aligned
     const size_t o_n = 0;
     const size_t o_soff = align_up(o_n + nt * 8, 16);
     const size_t o_cb = align_up(o_soff + nt * 8, 16);
     const size_t o_ct = align_up(o_cb + (nt + 1) * 4, 16);
-    const size_t total = align_up(o_ct + (size_t)nchunks * 4, 16);
+    const size_t o_rm = align_up(o_ct + (size_t)nchunks * 4, 16);
+    const size_t total = align_up(o_rm + row_map.size() * 4, 16);
     std::vector<unsigned char> host(total, 0);
+    if (!row_map.empty()) std::memcpy(host.data() + o_rm, row_map.data(), row_map.size() * 4);
     std::memcpy(host.data() + o_n, n.data(), nt * 8);
     std::memcpy(host.data() + o_soff, soff.data(), nt * 8);
     std::memcpy(host.data() + o_cb, chunk_begin.data(), (nt + 1) * 4);
@@ -443,6 +457,8 @@ void Layout::build(uint64_t nt, const uint64_t *r, const uint64_t *c, bool with_
     dev.chunk_tensor = (const uint32_t *)(b + o_ct);
     dev.nt = (uint32_t)nt;
     dev.nchunks = nchunks;
+    dev.row_map = row_map.empty() ? nullptr : (const uint32_t *)(b + o_rm);
+    dev.nrows = (uint32_t)row_map.size();
 }
 
 void Layout::release()

@@ -67,6 +67,9 @@ enum KernelId {
     K_COUNT = 73 // ids from here on are measurement kernels, handed out by Runtime::bench_kernel
 };
 
+// Lists of fewer chunks than this take the Adam kinds' by-row kernels (nbo_capi.cpp has the measurements).
+constexpr uint32_t NBO_ROWS_MAX_CHUNKS = 524288;
+
 // Process-wide runtime: device 0, the loaded module, the stream, scratch buffers.
 class Runtime {
 public:
@@ -173,7 +176,11 @@ struct Layout {
     void *blob = nullptr; // one device allocation holding all tables
     NboLayoutDev dev = {};
 
-    void build(uint64_t nt, const uint64_t *rows, const uint64_t *cols, bool with_arena);
+    // row_elems != 0: the elements a by-row update workgroup takes (one vector per thread); a list in
+    // which fewer than nine chunks in ten are whole then gets a map of the rows that exist
+    // (dev.row_map), so that a by-row launch has a workgroup for every row and none besides
+    void build(uint64_t nt, const uint64_t *rows, const uint64_t *cols, bool with_arena, uint32_t row_elems = 0);
+    bool mostly_whole() const { return (uint64_t)whole_chunks * 10 >= (uint64_t)nchunks * 9; }
     void release();
     uint64_t nt() const { return n.size(); }
 };

@@ -536,9 +536,20 @@ DEV void update_chunk(const NboUpdateArgs &a, const NboOptimDev *o, uint32_t wg)
     const bool mixed = ST == NBO_BF16 || ST == NBO_F16; // f32 master lives in the arena
     const bool has_v = KIND != NBO_SGD;
     const uint32_t tid = threadIdx.x;
-    if (BY_ROW && wg / ROWS >= a.L.nchunks) return; // the unused end of a folded grid
-    const uint32_t row0 = BY_ROW ? wg % ROWS : 0;
-    const ChunkRef c = chunk_ref(a.L, BY_ROW ? wg / ROWS : wg);
+    uint32_t ci = wg, row0 = 0;
+    if (BY_ROW) {
+        if (a.L.row_map) { // a list of many small tensors: only the rows that exist were launched
+            if (wg >= a.L.nrows) return; // (the unused end of a folded grid)
+            const uint32_t e = a.L.row_map[wg];
+            ci = e >> 4;
+            row0 = e & 15u;
+        } else {
+            ci = wg / ROWS;
+            row0 = wg % ROWS;
+            if (ci >= a.L.nchunks) return;
+        }
+    }
+    const ChunkRef c = chunk_ref(a.L, ci);
 
     char *pp = (char *)a.p_ptrs[c.t] + c.base * SB;
     char *pg = (char *)a.g_ptrs[c.t] + c.base * SB;
@@ -1154,7 +1165,7 @@ template <int ST> struct EwIO {
 // ragged(c, p) -- a chunk that is not whole or not vector-aligned, element by element (done by
 // the workgroup of the chunk's first piece).
 template <int ST, int NS, uint32_t PIECE_BYTES, typename Op>
-DEV void stream_pieces(const NboLayoutDev &L, const uint64_t *const (&lists)[NS], const Op &op)
+DEV void stream_pieces(const NboLayoutDev &L, const uint64_t *const (&lists)[NS], const Op &op, bool by_chunk)
 {
     typedef typename Traits<ST>::T T;
     enum {
@@ -1166,7 +1177,10 @@ DEV void stream_pieces(const NboLayoutDev &L, const uint64_t *const (&lists)[NS]
         PPC = NBO_CHUNK * SB / PIECE
     };
     static_assert(R >= 1 && PPC >= 1 && R * PPC * ROWB == NBO_CHUNK * SB, "pieces divide the chunk");
-    const uint32_t piece = folded_workgroup();
+    // by_chunk: a list of many small tensors, most of whose chunks are ragged ends of a row or two.
+    // A workgroup per piece would find most pieces missing (after looking the chunk up); such a list
+    // is launched one workgroup per chunk instead, each walking its chunk like a ragged one.
+    const uint32_t piece = by_chunk ? folded_workgroup() * PPC : folded_workgroup();
     if (piece / PPC >= L.nchunks) return; // the unused end of a folded grid
     const ChunkRef c = chunk_ref(L, piece / PPC);
     char *p[NS];
@@ -1176,7 +1190,7 @@ DEV void stream_pieces(const NboLayoutDev &L, const uint64_t *const (&lists)[NS]
         p[s] = (char *)lists[s][c.t] + c.base * SB;
         all |= (uintptr_t)p[s];
     }
-    if (c.cnt != NBO_CHUNK || (all & (VEC * SB - 1)) != 0) {
+    if (by_chunk || c.cnt != NBO_CHUNK || (all & (VEC * SB - 1)) != 0) {
         if (piece % PPC == 0) op.ragged(c, p);
         return;
     }
@@ -1264,7 +1278,7 @@ template <int ST> DEV void scale_body(const NboScaleArgs &a)
         }
     }
     const uint64_t *const lists[1] = {a.g_ptrs};
-    stream_pieces<ST, 1, NBO_EW_PIECE_BYTES>(a.L, lists, op);
+    stream_pieces<ST, 1, NBO_EW_PIECE_BYTES>(a.L, lists, op, a.by_chunk != 0);
 }
 
 #define NBO_SCALE_KERNEL(name, ST)                                                          \
@@ -1329,7 +1343,7 @@ template <int ST> DEV void accum_body(const NboAccumArgs &a)
     AccumOp<ST> op;
     op.zero_b = a.zero_b != 0;
     const uint64_t *const lists[2] = {a.a_ptrs, a.b_ptrs};
-    stream_pieces<ST, 2, NBO_EW_PIECE_BYTES>(a.L, lists, op);
+    stream_pieces<ST, 2, NBO_EW_PIECE_BYTES>(a.L, lists, op, a.by_chunk != 0);
 }
 
 #define NBO_ACCUM_KERNEL(name, ST)                                                          \
@@ -1543,7 +1557,7 @@ template <int ST> DEV void ew_body(const NboEwArgs &a)
     op.s = to_storage_precision<ST>((T)a.s);
     // an operand the operation does not have stands for the output: never read, same alignment
     const uint64_t *const lists[3] = {a.out_ptrs, op.use_a ? a.a_ptrs : a.out_ptrs, op.use_b ? a.b_ptrs : a.out_ptrs};
-    stream_pieces<ST, 3, NBO_BACKEND_PIECE_BYTES>(a.L, lists, op);
+    stream_pieces<ST, 3, NBO_BACKEND_PIECE_BYTES>(a.L, lists, op, a.by_chunk != 0);
 }
 
 #define NBO_EW_KERNEL(name, ST)                                                             \
@@ -1607,7 +1621,7 @@ template <int SRC, int DST> DEV void cast_body(const NboCastListArgs &a, uint32_
     // groups of four while both addresses allow whole vectors (16 bytes at most per access)
     const uint32_t sa = SS * 4 > 16 ? 16 : SS * 4, da = DS * 4 > 16 ? 16 : DS * 4;
     const bool vec_ok = (((uintptr_t)ps & (sa - 1)) | ((uintptr_t)pd & (da - 1))) == 0;
-    if (vec_ok && c.cnt == NBO_CHUNK) {
+    if (!a.by_chunk && vec_ok && c.cnt == NBO_CHUNK) {
         double v[4];
         const uint64_t e = (uint64_t)row * NBO_CAST_ROW + threadIdx.x * 4;
         cast_load4<SRC>(ps, e, v);
@@ -1635,7 +1649,8 @@ template <int SRC> DEV void cast_from(const NboCastListArgs &a, uint32_t wg)
 
 extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_cast_list(const NboCastListArgs a)
 {
-    const uint32_t wg = folded_workgroup();
+    // (by_chunk: a list of many small tensors, one workgroup per chunk -- see stream_pieces)
+    const uint32_t wg = a.by_chunk ? folded_workgroup() * (NBO_CHUNK / NBO_CAST_ROW) : folded_workgroup();
     if (wg / (NBO_CHUNK / NBO_CAST_ROW) >= a.L.nchunks) return; // the unused end of a folded grid
     if (a.src_type == NBO_F32) cast_from<NBO_F32>(a, wg);
     else if (a.src_type == NBO_BF16) cast_from<NBO_BF16>(a, wg);

@@ -58,6 +58,12 @@ struct NboLayoutDev {
     const uint32_t *chunk_tensor;
     uint32_t nt;
     uint32_t nchunks;
+    // Lists of many small tensors, for the kernels that run one workgroup per row of a chunk: the
+    // rows that exist, in order, as chunk * 16 + row (null: every chunk counts as whole and
+    // workgroup w is row w % rows-per-chunk of chunk w / rows-per-chunk).
+    const uint32_t *row_map;
+    uint32_t nrows;
+    uint32_t pad;
 };
 
 // GradScalerState (optim/core.rs:326-332), device resident.
@@ -227,7 +233,7 @@ struct NboAccumArgs {
     const uint64_t *a_ptrs;
     const uint64_t *b_ptrs;
     uint32_t zero_b; // also clear b after it has been added
-    uint32_t pad;
+    uint32_t by_chunk; // one workgroup per chunk, not per piece (a list of many small tensors)
 };
 
 struct NboScaleArgs {
@@ -237,7 +243,7 @@ struct NboScaleArgs {
                               // on found_inf (mode 0) write zeros instead
     double factor;            // used when gf is null
     uint32_t mode;            // 0 unscale, 1 clip, 2 plain factor, 3 zero fill
-    uint32_t pad;
+    uint32_t by_chunk;        // one workgroup per chunk, not per piece (a list of many small tensors)
 };
 
 struct NboCastArgs {
@@ -276,7 +282,7 @@ struct NboEwArgs {
     const uint64_t *b_ptrs; // null unless the operation has two tensor operands
     double s;               // narrowed to the element type on the device
     uint32_t op;
-    uint32_t pad;
+    uint32_t by_chunk; // one workgroup per chunk, not per piece (a list of many small tensors)
 };
 
 // Element-type conversion of a tensor list through f64, as BackendCore::cast's default
@@ -286,6 +292,8 @@ struct NboCastListArgs {
     const uint64_t *dst_ptrs;
     const uint64_t *src_ptrs;
     uint32_t dst_type, src_type; // NBO_F32 / NBO_BF16 / NBO_F64
+    uint32_t by_chunk;           // one workgroup per chunk, not per row (a list of many small tensors)
+    uint32_t pad;
 };
 
 // Memory-system ceiling probe: which streams are read, rewritten in place or only written.

@@ -15,7 +15,12 @@ from tests import helpers as H
 
 pytestmark = pytest.mark.gpu
 
-SIZES = [5, 1024, 4099, 8192, 8200, 3 * 8192, 20011]
+# Two lists: in the first nine chunks in ten are whole, so the passes run one workgroup per piece
+# (and its ragged and unaligned chunks are the exceptions inside such a launch); the second is a
+# list of small tensors, which the library runs one workgroup per chunk (and the optimizers by row
+# over a map of the rows that exist).
+SIZES_OF = {"mostly whole": [5, 1024, 4099, 8192, 8200, 3 * 8192, 20011, 40 * 8192],
+            "small tensors": [5, 1024, 4099, 8192, 8200, 3 * 8192, 20011]}
 NP = {"f32": np.float32, "f64": np.float64}
 
 
@@ -39,13 +44,13 @@ def _views(arrs, odd, torch_dtype):
     return buf, views
 
 
-def _make(dtype, seed, sigma, odd):
+def _make(dtype, seed, sigma, odd, sizes):
     import torch
 
     if dtype == "bf16":
-        arrs = [O.bf16_from_f32(O.randn_f32(n, seed + i, sigma)) for i, n in enumerate(SIZES)]
+        arrs = [O.bf16_from_f32(O.randn_f32(n, seed + i, sigma)) for i, n in enumerate(sizes)]
         return arrs, _views(arrs, odd, torch.bfloat16)
-    arrs = [(O.randn_f64(n, seed + i) * sigma).astype(NP[dtype]) for i, n in enumerate(SIZES)]
+    arrs = [(O.randn_f64(n, seed + i) * sigma).astype(NP[dtype]) for i, n in enumerate(sizes)]
     return arrs, _views(arrs, odd, torch.float32 if dtype == "f32" else torch.float64)
 
 
@@ -57,23 +62,25 @@ def _like(ref_f32, like):
     return [O.bf16_from_f32(a) if b.dtype == np.uint16 else a for a, b in zip(ref_f32, like)]
 
 
+@pytest.mark.parametrize("kind", list(SIZES_OF))
 @pytest.mark.parametrize("odd", [False, True])
 @pytest.mark.parametrize("dtype", ["f32", "bf16", "f64"])
-def test_scale_zero_and_accumulate_over_views(gpu, dtype, odd):
-    g0, (gbuf, g) = _make(dtype, 11, 1.0, odd)
-    a0, (abuf, a) = _make(dtype, 31, 1.0, odd)
+def test_scale_zero_and_accumulate_over_views(gpu, dtype, odd, kind):
+    sizes = SIZES_OF[kind]
+    g0, (gbuf, g) = _make(dtype, 11, 1.0, odd, sizes)
+    a0, (abuf, a) = _make(dtype, 31, 1.0, odd, sizes)
     before_g, before_a = gbuf.clone(), abuf.clone()
 
     # scale_grad: g * T(factor), rounded to the element type
     nb.scale_grad(g, 0.3)
     ref = [x.copy() for x in g0]
     O.scale_grad(ref, 0.3)
-    H.assert_bits_equal(H.host_list(g), ref, f"scale_grad {dtype} odd={odd}")
+    H.assert_bits_equal(H.host_list(g), ref, f"scale_grad {dtype} odd={odd} {kind}")
 
     # accumulate: a + g in the element type (bf16: the f32 sum rounded)
     nb.accumulate(a, g)
     acc = [O.add(x, y) for x, y in zip(a0, ref)]
-    H.assert_bits_equal(H.host_list(a), acc, f"accumulate {dtype} odd={odd}")
+    H.assert_bits_equal(H.host_list(a), acc, f"accumulate {dtype} odd={odd} {kind}")
     H.assert_bits_equal(H.host_list(g), ref, "accumulate leaves the gradients")
 
     # accumulate and clear
@@ -98,13 +105,15 @@ def test_scale_zero_and_accumulate_over_views(gpu, dtype, odd):
         assert bool((buf[mask] == before[mask]).all()) and not bool(buf[mask].any())
 
 
+@pytest.mark.parametrize("kind", list(SIZES_OF))
 @pytest.mark.parametrize("odd", [False, True])
 @pytest.mark.parametrize("dtype", ["f32", "f64"])
 @pytest.mark.parametrize("momentum,wd", [(0.0, 0.0), (0.9, 0.01)])
-def test_sgd_steps_over_views(gpu, dtype, odd, momentum, wd):
-    p0, (pbuf, p) = _make(dtype, 51, 0.05, odd)
-    g0, (_, g) = _make(dtype, 71, 1e-2, odd)
-    shapes = [(1, n) for n in SIZES]
+def test_sgd_steps_over_views(gpu, dtype, odd, momentum, wd, kind):
+    sizes = SIZES_OF[kind]
+    p0, (pbuf, p) = _make(dtype, 51, 0.05, odd, sizes)
+    g0, (_, g) = _make(dtype, 71, 1e-2, odd, sizes)
+    shapes = [(1, n) for n in sizes]
     opt = nb.Sgd.new(0.05, shapes, dtype=dtype).momentum(momentum).weight_decay(wd)
     meta = O.sgd_meta(0.05, momentum=momentum, weight_decay=wd)
     ref, vel = [x.copy() for x in p0], [np.zeros_like(x) for x in p0]
@@ -113,3 +122,53 @@ def test_sgd_steps_over_views(gpu, dtype, odd, momentum, wd):
         O.sgd_step(meta, ref, g0, vel)
     H.assert_bits_equal(H.host_list(p), ref, f"Sgd {dtype} odd={odd} momentum={momentum}")
     H.assert_bits_equal(H.host_list(g), g0, "Sgd leaves the gradients")
+
+
+@pytest.mark.parametrize("kind", list(SIZES_OF))
+@pytest.mark.parametrize("odd", [False, True])
+def test_backend_add_cast_and_adam_over_views(gpu, odd, kind):
+    """The backend primitives (two rows per workgroup), the cast (one workgroup per 1024 elements)
+    and the unfused and fused Adam kinds over the same two lists."""
+    import torch
+
+    from nabla_amd import backend as B
+
+    sizes = SIZES_OF[kind]
+    shapes = [(1, n) for n in sizes]
+    a0, (_, a) = _make("f32", 91, 1.0, odd, sizes)
+    b0, (_, b) = _make("f32", 92, 1.0, odd, sizes)
+    _, (obuf, o) = _make("f32", 93, 1.0, odd, sizes)
+    B.add(a, b, out=o)
+    H.assert_bits_equal(H.host_list(o), [O.add(x, y) for x, y in zip(a0, b0)], f"backend add odd={odd} {kind}")
+    B.axpy_inplace(o, 0.25, a)
+    ref = [O.add(x, y) for x, y in zip(a0, b0)]
+    for r, x in zip(ref, a0):
+        O.axpy_inplace(r, 0.25, x)
+    H.assert_bits_equal(H.host_list(o), ref, f"backend axpy odd={odd} {kind}")
+    h0, (_, h) = _make("bf16", 94, 1.0, odd, sizes)
+    B.cast(a, h)
+    H.assert_bits_equal(H.host_list(h), [O.bf16_from_f32(x) for x in a0], f"cast f32 -> bf16 odd={odd} {kind}")
+    B.cast(h, o)
+    H.assert_bits_equal(H.host_list(o), [O.bf16_to_f32(O.bf16_from_f32(x)) for x in a0], f"cast bf16 -> f32 odd={odd} {kind}")
+
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        p0, (_, p) = _make("f32", 95, 0.02, odd, sizes)
+        g0, (_, g) = _make("f32", 96, 1e-3, odd, sizes)
+        opt = nb.Adam.new(1e-3, shapes)
+        meta = O.adam_meta(1e-3)
+        ref, m, v = [x.copy() for x in p0], [np.zeros_like(x) for x in p0], [np.zeros_like(x) for x in p0]
+        for _ in range(3):
+            opt.step(p, g)
+            O.adam_step(meta, ref, g0, m, v)
+        H.assert_bits_equal(H.host_list(p), ref, f"Adam odd={odd} {kind}")
+        H.assert_bits_equal(H.host_list(opt.moments()[1]), v, "v")
+        fused = nb.AdamW.new(2e-4, shapes).weight_decay(0.1)
+        fmeta = O.adamw_meta(2e-4, weight_decay=0.1)
+        m, v = [np.zeros_like(x) for x in p0], [np.zeros_like(x) for x in p0]
+        for _ in range(2):
+            fused.fused_step(p, g)
+            O.adam_step(fmeta, ref, g0, m, v)
+        H.assert_bits_equal(H.host_list(p), ref, f"fused AdamW odd={odd} {kind}")
+    finally:
+        O.set_pow_mode(O.POW_LIBM)

@@ -280,6 +280,59 @@ def test_a_list_of_middle_size_takes_the_by_row_kernels(gpu):
         O.set_pow_mode(O.POW_LIBM)
 
 
+def test_a_list_of_many_small_tensors_runs_by_row_over_the_rows_that_exist(gpu):
+    """700 tensors of 1 to 30000 elements (hardly a whole chunk among them): the optimizer's layout
+    carries a map of the rows that exist, the by-row kernels are launched with exactly that many
+    workgroups, and mixed-precision AdamW (scaler, clip, one step skipped for an inf) and SGD with
+    momentum give the oracle's bits."""
+    from nabla_amd.workloads import ragged_sizes
+
+    sizes = ragged_sizes(700, 1, 30000, seed=77)
+    shapes = [(1, n) for n in sizes]
+    w0 = H.randn_list(shapes, 500, 0.02)
+    L = _lib.load()
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        p_dev = H.dev_list([O.bf16_from_f32(a) for a in w0], shapes)
+        opt = nb.AdamW.new(2e-4, shapes, master=True).beta2(0.95).weight_decay(0.1)
+        for i, a in enumerate(w0):
+            opt.write_state(f"w{i}", H.to_dev(a, shapes[i]))
+        scaler, s_ref = nb.GradScaler.new(), O.default_scaler()
+        meta = O.adamw_meta(2e-4, beta2=0.95, weight_decay=0.1)
+        p_ref = [O.bf16_from_f32(a) for a in w0]
+        master, m, v = H.copy_list(w0), H.zeros_like_list(w0), H.zeros_like_list(w0)
+        for step in range(4):
+            g_bits = [O.bf16_from_f32(a) for a in H.randn_list(shapes, 600 + 13 * step, 1e-3 * 65536.0)]
+            if step == 1:
+                g_bits[5][0] = 0x7F80
+            _lib.check(L.nbo_profile_enable(1))
+            opt.fused_step(p_dev, H.dev_list(g_bits, shapes), scaler=scaler, max_norm=1.0)
+            n = _launches(["nbo_update_bf16_adamw_rows", "nbo_update_bf16_adamw"])
+            _lib.check(L.nbo_profile_enable(0))
+            assert n == {"nbo_update_bf16_adamw_rows": 1, "nbo_update_bf16_adamw": 0}
+            info = opt.last_step()
+            H.oracle_step_with_device_norm(lambda: O.mixed_step(meta, s_ref, 1.0, p_ref, g_bits, master, m, v),
+                                           [p_ref, master, m, v], [meta, s_ref], 1.0, info, f"ragged by row, step {step}")
+            assert info.found_inf == (1 if step == 1 else 0)
+        assert opt.step_count() == 3 == meta.step_count
+        H.assert_bits_equal(H.host_list(p_dev), p_ref, "bf16 params")
+        for name, ref in (("w", master), ("m", m), ("v", v)):
+            H.assert_bits_equal([H.to_host(opt.read_state(f"{name}{i}")) for i in range(len(shapes))], ref, name)
+        del opt
+
+        p0, g0 = H.randn_list(shapes, 700, 0.05), H.randn_list(shapes, 800, 1e-2)
+        p_dev, g_dev = H.dev_list(p0, shapes), H.dev_list(g0, shapes)
+        sgd = nb.Sgd.new(0.05, shapes).momentum(0.9).weight_decay(0.01)
+        smeta = O.sgd_meta(0.05, momentum=0.9, weight_decay=0.01)
+        ref, vel = H.copy_list(p0), H.zeros_like_list(p0)
+        for _ in range(3):
+            sgd.step(p_dev, g_dev)
+            O.sgd_step(smeta, ref, g0, vel)
+        H.assert_bits_equal(H.host_list(p_dev), ref, "Sgd over the ragged list")
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+
+
 def test_grids_folded_into_two_dimensions_cover_every_row_once(gpu):
     """One grid dimension holds fewer than 2^32 threads, so the launches that run one workgroup per
     row of a chunk fold a larger grid into two dimensions.  With NBO_GRID_X_MAX=37 in the
