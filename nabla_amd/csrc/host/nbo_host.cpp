@@ -58,9 +58,12 @@ static const char *const kKernelNames[K_COUNT] = {
     "nbo_update_f32_adamw_rows",   "nbo_update_f32_adam_rows",   "nbo_update_bf16_adamw_rows",
     "nbo_update_bf16_adam_rows",   "nbo_update_f64_adamw_rows",  "nbo_update_f64_adam_rows",
     "nbo_update_f16_adamw_rows",   "nbo_update_f16_adam_rows",
+    "nbo_accscale_f32",            "nbo_accscale_bf16",          "nbo_accscale_f64",
+    "nbo_accscale_f16",
 };
 static_assert(K_UPDATE_SELF_BASE + 18 == K_UPDATE_ROWS_BASE, "six families of three self-preparing update kernels");
-static_assert(K_UPDATE_ROWS_BASE + 8 == K_COUNT, "four families of two by-row update kernels");
+static_assert(K_UPDATE_ROWS_BASE + 8 == K_ACCSCALE_BASE && K_ACCSCALE_F16 + 1 == K_COUNT,
+              "four families of two by-row update kernels, four micro-batch kernels without the sum");
 
 static std::mutex g_runtime_mu;
 static Runtime *g_runtime = nullptr;
@@ -112,6 +115,8 @@ Runtime::Runtime()
     partial_sumsq_ = (double *)dmalloc(NBO_NORM_GRID_MAX * sizeof(double));
     partial_flag_ = (uint32_t *)dmalloc(NBO_NORM_GRID_MAX * sizeof(uint32_t));
     gf_scratch_ = (NboGradFactors *)dmalloc(sizeof(NboGradFactors));
+    any_bad_ = (uint32_t *)dmalloc(256);
+    dzero(any_bad_, 256);
     // The statically allocated scratch of the allocation-free entry point: its device address
     // is looked up here, once, with the device current.  A failure is kept for that entry point
     // to report; nothing else depends on it.

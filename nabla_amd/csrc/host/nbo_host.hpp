@@ -64,7 +64,9 @@ enum KernelId {
     // Adam / AdamW one workgroup per row of a chunk: + family * 2 + kind (adamw 0, adam 1), family =
     // f32, bf16, f64, f16 (state of 32 or 64 bits)
     K_UPDATE_ROWS_BASE = 65,
-    K_COUNT = 73 // ids from here on are measurement kernels, handed out by Runtime::bench_kernel
+    K_ACCSCALE_BASE = 73, // + st (f32 / bf16 / f64): a micro-batch without the sum of squares
+    K_ACCSCALE_F16 = 76,
+    K_COUNT = 77 // ids from here on are measurement kernels, handed out by Runtime::bench_kernel
 };
 
 // Lists of fewer chunks than this take the Adam kinds' by-row kernels (nbo_capi.cpp has the measurements).
@@ -134,6 +136,8 @@ public:
     double *partial_sumsq() const { return partial_sumsq_; }
     uint32_t *partial_flag() const { return partial_flag_; }
     NboGradFactors *gf_scratch() const { return gf_scratch_; }
+    // one word, zero between uses: passes without partial results OR their non-finite findings into it
+    uint32_t *any_bad() const { return any_bad_; }
     // the device this runtime lives on, and how the look-up of the statically allocated
     // scratch's address went there
     int device() const { return device_; }
@@ -157,6 +161,7 @@ private:
     double *partial_sumsq_ = nullptr;
     uint32_t *partial_flag_ = nullptr;
     NboGradFactors *gf_scratch_ = nullptr;
+    uint32_t *any_bad_ = nullptr;
     int device_ = 0;
     hipError_t static_scratch_status_ = hipSuccess;
     struct ProfRec {

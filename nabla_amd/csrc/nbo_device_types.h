@@ -193,6 +193,7 @@ struct NboFinalizeArgs {
     double sumsq_in;       // with use_sumsq_in: the sum of squares, already known (grid = 0)
     uint32_t use_sumsq_in;
     uint32_t pad;
+    uint32_t *any_bad;     // may be null: a word some pass ORed its non-finite findings into; read, then cleared
 };
 
 struct NboNormArgs {
@@ -225,6 +226,12 @@ struct NboAccNormArgs {
     uint32_t *partial_flag;     // [grid]
     uint32_t grid;
     uint32_t write_grads;       // also store the unscaled gradients in place, as the reference does
+    // The variant without the sum of squares (nbo_accscale_*: every micro-batch but the last) runs
+    // like the element-wise passes and leaves only whether it met a non-finite gradient: ORed into
+    // *any_bad, which the second stage reads and clears.
+    uint32_t *any_bad;
+    uint32_t by_chunk; // see NboAccumArgs
+    uint32_t pad;
 };
 
 // a[i] = a[i] + b[i] over two lists of the same shapes (gradient accumulation).

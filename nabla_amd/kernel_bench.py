@@ -319,6 +319,12 @@ def main() -> None:
             nb.unscale_accumulate(a, b, scaler=scaler)
 
         timeit(f"unscale_accumulate {tag}", micro, 3 * sz, f"nbo_accnorm_{tag}")
+
+        def micro_no_sum():
+            fresh_scale()
+            nb.unscale_accumulate(a, b, scaler=scaler, want_sumsq=False)
+
+        timeit(f"unscale_accumulate {tag}, no sum of squares", micro_no_sum, 3 * sz, f"nbo_accscale_{tag}")
         timeit(f"zero_grad {tag}", lambda: nb.zero_grad(a), sz, f"nbo_scale_{tag}")
         timeit(f"scale_grad {tag}", lambda: nb.scale_grad(b, 0.5), 2 * sz, f"nbo_scale_{tag}")
         timeit(f"clip_grad_norm {tag}, norm pass", lambda: nb.clip_grad_norm(b, 1e30), sz, f"nbo_norm_{tag}")

@@ -136,8 +136,10 @@ class TrainerTail:
         else:
             # steps 1-3 in one pass over the gradients; a non-finite micro-batch leaves garbage
             # in the buffer, which is dropped with it
+            # (the clip needs the buffer's sum of squares once the last micro-batch is in)
+            last = self._accum_count + 1 >= self.state.grad_accum
             ok, sumsq = nb.unscale_accumulate(self._accum, grads, scaler=self.scaler,
-                                              check_finite=self.nan_policy is not None)
+                                              check_finite=self.nan_policy is not None, want_sumsq=last)
             if not ok:
                 self._drop()
                 if self.scaler is None and self.nan_policy is GradNanPolicy.STOP:

@@ -275,14 +275,19 @@ def test_accumulate_matches_add(gpu):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("want_sumsq", [True, False])
+@pytest.mark.parametrize("big", [2, 40])
 @pytest.mark.parametrize("dtype", ["f32", "bf16", "f16", "f64"])
-def test_unscale_accumulate_is_unscale_then_accumulate_in_one_pass(gpu, dtype):
+def test_unscale_accumulate_is_unscale_then_accumulate_in_one_pass(gpu, dtype, big, want_sumsq):
     """nbo_unscale_accumulate against nbo_scaler_unscale_and_update + nbo_accumulate and against
     the oracle's unscale / add: same buffer, same gradients written back, same decision and
-    loss-scale sequence, and a sum of squares that is the clip's norm squared."""
+    loss-scale sequence, and a sum of squares that is the clip's norm squared.  Without the sum
+    of squares (every micro-batch but the last) the pass is another kernel, which runs like the
+    element-wise passes: by chunk over a list of small tensors (big = 2), by piece where nine
+    chunks in ten are whole (big = 40)."""
     from tests import helpers as H
 
-    shapes = [(1, 5), (3, 2741), (1, 8193), (0, 4), (2, 8192), (1, 16391)]
+    shapes = [(1, 5), (3, 2741), (1, 8193), (0, 4), (big, 8192), (1, 16391)]
     np_t = {"f32": np.float32, "f64": np.float64}.get(dtype)
 
     def conv(arrs):
@@ -301,7 +306,9 @@ def test_unscale_accumulate_is_unscale_then_accumulate_in_one_pass(gpu, dtype):
             g[4].reshape(-1).view(np.uint16 if g[4].itemsize == 2 else g[4].dtype)[9000] = \
                 {2: 0x7F80 if dtype == "bf16" else 0x7C00}.get(g[4].itemsize, np.inf)
         fused_g, plain_g = H.dev_list(g, shapes), H.dev_list(g, shapes)
-        ok, sumsq = nb.unscale_accumulate(fused_buf, fused_g, scaler=fused_scaler, write_grads=True)
+        ok, sumsq = nb.unscale_accumulate(fused_buf, fused_g, scaler=fused_scaler, write_grads=True,
+                                          want_sumsq=want_sumsq)
+        assert (sumsq is not None) == want_sumsq
         plain_ok = plain_scaler.unscale_and_update(plain_g)
         ref_g = H.copy_list(g)
         assert ok == plain_ok == O.scaler_unscale_and_update(ref_scaler, ref_g), k
@@ -315,18 +322,22 @@ def test_unscale_accumulate_is_unscale_then_accumulate_in_one_pass(gpu, dtype):
         ref_buf = [O.add(b, x) for b, x in zip(ref_buf, ref_g)]
         H.assert_bits_equal(H.host_list(fused_buf), ref_buf, f"buffer, micro-batch {k}")
         H.assert_bits_equal(H.host_list(plain_buf), ref_buf, f"two-pass buffer, micro-batch {k}")
-        norm = O.clip_grad_norm(H.copy_list(ref_buf), 1e30)  # far above the norm: nothing is scaled
-        assert abs(np.sqrt(sumsq) - norm) <= 1e-13 * norm, k
+        if want_sumsq:
+            norm = O.clip_grad_norm(H.copy_list(ref_buf), 1e30)  # far above the norm: nothing is scaled
+            assert abs(np.sqrt(sumsq) - norm) <= 1e-13 * norm, k
     # without write_grads the gradients stay as they were; without a scaler nothing is unscaled
     g = conv(H.randn_list(shapes, 70, 1e-2))
     g_dev = H.dev_list(g, shapes)
-    ok, _ = nb.unscale_accumulate(fused_buf, g_dev)
+    ok, _ = nb.unscale_accumulate(fused_buf, g_dev, want_sumsq=want_sumsq)
     assert ok
     H.assert_bits_equal(H.host_list(g_dev), g, "gradients untouched")
     H.assert_bits_equal(H.host_list(fused_buf), [O.add(b, x) for b, x in zip(ref_buf, g)], "plain accumulation")
     g[1][5] = np.nan if g[1].itemsize != 2 or dtype == "f16" else 0x7FC0
-    assert nb.unscale_accumulate(fused_buf, H.dev_list(g, shapes))[0]            # nobody asked
-    assert not nb.unscale_accumulate(fused_buf, H.dev_list(g, shapes), check_finite=True)[0]
+    assert nb.unscale_accumulate(fused_buf, H.dev_list(g, shapes), want_sumsq=want_sumsq)[0]  # nobody asked
+    assert not nb.unscale_accumulate(fused_buf, H.dev_list(g, shapes), check_finite=True, want_sumsq=want_sumsq)[0]
+    # what the pass before found does not linger: a clean micro-batch after a non-finite one is clean
+    assert nb.unscale_accumulate(fused_buf, H.dev_list(conv(H.randn_list(shapes, 71, 1e-2)), shapes), check_finite=True,
+                                 want_sumsq=want_sumsq)[0]
     with pytest.raises(nb.NablaPanic):
         nb.unscale_accumulate(fused_buf, g_dev[:2])
 
