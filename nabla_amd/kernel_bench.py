@@ -234,6 +234,76 @@ def placed_main(args) -> None:
         bufs.close()
 
 
+def flow_main(args) -> None:
+    """One training step's tail as the reference's four calls (unscale_and_update, clip_grad_norm,
+    step, zero_grad: trainer.rs:230-290, each reading its decision back to the host) against the
+    one fused call, f32 AdamW over the same list with a GradScaler and a clip that bites."""
+    import time
+
+    import torch
+
+    from . import _lib
+    from . import optim as nb
+
+    _lib.init()
+    L = _lib.load()
+    dev = torch.device("cuda:0")
+    big = max(int(args.elements) // (8192 * 8192), 1)
+    shapes = [(8192, 8192)] * big + [(1, 4096)] * 8
+    n = sum(r * c for r, c in shapes)
+    p = nb.TensorList([torch.randn(s, device=dev) * 0.02 for s in shapes])
+    g0 = [torch.randn(s, device=dev) * (1e-3 * 65536.0) for s in shapes]
+    g = nb.TensorList([t.clone() for t in g0])
+    rows = []
+    for fused in (False, True):
+        opt = nb.AdamW.new(2e-4, shapes).beta2(0.95).weight_decay(0.1)
+        scaler = nb.GradScaler.new()
+        scaler.load_state(nb.GradScalerState(65536.0, 2.0, 0.5, 1 << 40, 0))
+
+        def step():
+            for t, t0 in zip(g.tensors, g0):  # the backward pass's part: fresh scaled gradients (not timed apart)
+                t.copy_(t0)
+            if fused:
+                opt.fused_step(p, g, scaler=scaler, max_norm=1.0, zero_grads=True)
+            else:
+                if scaler.unscale_and_update(g):
+                    nb.clip_grad_norm(g, 1.0)
+                    opt.step(p, g)
+                nb.zero_grad(g)
+
+        def refill():
+            for t, t0 in zip(g.tensors, g0):
+                t.copy_(t0)
+
+        for _ in range(2):
+            step()
+        _lib.check(L.nbo_sync())
+        torch.cuda.synchronize()
+        # the refill alone, to take it out of the figure
+        t0 = time.perf_counter()
+        for _ in range(args.reps):
+            refill()
+        torch.cuda.synchronize()
+        t_refill = (time.perf_counter() - t0) / args.reps
+        t0 = time.perf_counter()
+        for _ in range(args.reps):
+            step()
+        _lib.check(L.nbo_sync())
+        torch.cuda.synchronize()
+        rows.append(((time.perf_counter() - t0) / args.reps - t_refill) * 1e3)
+        del opt
+    # bytes per parameter: unscale 4 (scan) + 8 (scale in place), clip 4 (norm) + 8 (scale), step 28, zero 4;
+    # fused: norm pass 4, update 28 + 4 (the zeros)
+    print(f"{n} f32 elements in {len(shapes)} tensors, {args.reps} steps each; the gradients are refilled before every "
+          "step (a device copy, timed alone and subtracted)\n")
+    print("| the step's tail | calls | HBM bytes / param | ms | GB/s |")
+    print("|---|---|---|---|---|")
+    print(f"| as the reference's four calls | unscale_and_update, clip_grad_norm, AdamW::step, zero_grad | 56 | "
+          f"{rows[0]:.3f} | {n * 56 / rows[0] / 1e6:.0f} |")
+    print(f"| fused | nbo_fused_step with NBO_STEP_ZERO_GRADS | 36 | {rows[1]:.3f} | {n * 36 / rows[1] / 1e6:.0f} |")
+    print(f"\nThe fused call takes {rows[1] / rows[0] * 100:.0f} % of the four calls' time.")
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--elements", type=float, default=805e6)
@@ -248,6 +318,8 @@ def main() -> None:
     ap.add_argument("--placed", action="store_true",
                     help="the kernels over the caller's tensors with those tensors placed in named HBM regions "
                          "(nbo_alloc_placed): one region against several")
+    ap.add_argument("--flow", action="store_true",
+                    help="a training step's tail as the reference's four calls against the one fused call")
     ap.add_argument("--summarize", metavar="DIR", help="turn the rocprofv3 output under DIR into profiles/ summaries "
                                                         "(see nabla_amd/profile_summary.py) instead of measuring")
     args = ap.parse_args()
@@ -255,6 +327,10 @@ def main() -> None:
         from . import profile_summary
 
         profile_summary.main(args.summarize)
+        return
+    if args.flow:
+        args.reps = args.reps or 10
+        flow_main(args)
         return
     if args.compare:
         args.reps = args.reps or 5
