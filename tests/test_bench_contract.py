@@ -86,6 +86,19 @@ def test_kernel_bench_prints_a_row_for_every_measurement(gpu):
 
 
 @pytest.mark.gpu
+def test_kernel_bench_flow_compares_the_four_calls_with_the_fused_one(gpu):
+    """`python -m nabla_amd.kernel_bench --flow` on one tensor: both rows with a positive time."""
+    r = subprocess.run([sys.executable, "-m", "nabla_amd.kernel_bench", "--flow", "--elements", "1e6", "--reps", "2"],
+                       capture_output=True, text=True, timeout=300, cwd=ROOT)
+    assert r.returncode == 0, r.stderr[-2000:]
+    rows = [x for x in r.stdout.splitlines() if x.startswith("| ") and ("four calls" in x or "fused" in x)]
+    assert len(rows) == 2
+    for row in rows:
+        cells = [c.strip() for c in row.strip("|").split("|")]
+        assert float(cells[3]) > 0.0 and float(cells[4]) > 0.0, row
+
+
+@pytest.mark.gpu
 def test_every_ceiling_probe_runs_and_reports_a_rate(gpu):
     """`nbo_hbm_ceiling` for every access pattern, in one plain allocation and across the HBM's
     regions, on streams of 192 MiB: a finite positive rate, best >= mean, and the argument checks
