@@ -261,8 +261,10 @@ int nbo_accumulate(nbo_list *accum, nbo_list *grads, int zero_grads);
  * (unscaled, or zeros when non-finite).  Results are those of
  * nbo_scaler_unscale_and_update followed by nbo_accumulate, bit for bit.  accum_sumsq may be
  * null -- only the last micro-batch of an accumulation needs the sum of squares -- and the
- * pass then has nothing to reduce but one bit and runs like the element-wise passes, some
- * 15 % faster.  Synchronous. */
+ * pass then has nothing to reduce but one bit (one small launch fewer).  The sum is added up in
+ * f64 in a fixed order, the same bits on every run; the order is not the norm pass's, so the
+ * norm nbo_fused_step_norm derives from it can differ from nbo_fused_step's in the last bits of
+ * the f64.  Synchronous. */
 #define NBO_ACC_CHECK_FINITE 1u
 #define NBO_ACC_WRITE_GRADS 2u
 int nbo_unscale_accumulate(nbo_scaler *scaler, nbo_list *accum, nbo_list *grads, uint32_t flags, int *ok,

@@ -428,7 +428,7 @@ inline void accumulate(TensorList &accum, TensorList &grads, bool zero_grads = f
 // scan + loss-scale update, buf[i] = &buf[i] + g / scale, and the new buffer's sum of squares.
 // Returns false on a non-finite gradient (the buffer then holds garbage, the Trainer discards it).
 // sumsq may be null: only the last micro-batch of an accumulation needs the sum of squares, and a
-// pass without it has nothing to reduce but one bit and is some 15 % faster.
+// pass without it has nothing to reduce but one bit (one small launch fewer).
 inline bool unscale_accumulate(TensorList &accum, TensorList &grads, GradScaler *scaler, double *sumsq,
                                bool check_finite = false, bool write_grads = false)
 {

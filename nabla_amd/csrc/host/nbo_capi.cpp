@@ -1104,24 +1104,37 @@ int nbo_unscale_accumulate(nbo_scaler *scaler, nbo_list *accum, nbo_list *grads,
         a.acc_ptrs = accum->ptrs_dev;
         a.g_ptrs = grads->ptrs_dev;
         a.scaler = scaler ? scaler->dev : nullptr;
-        a.partial_sumsq = rt.partial_sumsq();
-        a.partial_flag = rt.partial_flag();
-        a.grid = norm_grid(accum->layout);
         a.write_grads = (flags & NBO_ACC_WRITE_GRADS) ? 1u : 0u;
+        a.any_bad = rt.any_bad();
+        // both forms run like the element-wise passes; whether a gradient was non-finite reaches
+        // the second stage as one bit
+        a.grid = ew_grid(accum->layout, accum->dtype, NBO_EW_PIECE_BYTES, &a.by_chunk);
         NboFinalizeArgs f = {};
         f.partial_sumsq = rt.partial_sumsq();
         f.partial_flag = rt.partial_flag();
-        if (accum_sumsq) {
-            rt.launch(kernel_for(K_ACCNORM_BASE, K_ACCNORM_F16, accum->dtype), a.grid, NBO_BLOCK, a);
+        f.any_bad = rt.any_bad();
+        if (!accum_sumsq) {
+            // nobody asked for the sum of squares (every micro-batch but the last): nothing to reduce
+            rt.launch_folded(kernel_for(K_ACCSCALE_BASE, K_ACCSCALE_F16, accum->dtype), a.grid, NBO_BLOCK, a);
+            f.grid = 0;
+        } else if (a.grid <= NBO_NORM_GRID_MAX) {
+            // one sum per workgroup, few enough for the second stage to add up itself
+            a.partial_sumsq = rt.partial_sumsq();
+            a.partial_flag = rt.partial_flag();
+            rt.launch_folded(kernel_for(K_ACCNORM_BASE, K_ACCNORM_F16, accum->dtype), a.grid, NBO_BLOCK, a);
             f.grid = a.grid;
         } else {
-            // nobody asked for the sum of squares (every micro-batch but the last): no reduction, so
-            // the pass runs like the element-wise ones, and the second stage has one bit to read
-            a.any_bad = rt.any_bad();
-            const uint32_t grid = ew_grid(accum->layout, accum->dtype, NBO_EW_PIECE_BYTES, &a.by_chunk);
-            rt.launch_folded(kernel_for(K_ACCSCALE_BASE, K_ACCSCALE_F16, accum->dtype), grid, NBO_BLOCK, a);
-            f.grid = 0;
-            f.any_bad = rt.any_bad();
+            // ... or too many: a launch in between adds runs of `per` of them
+            a.partial_sumsq = rt.piece_partials(a.grid);
+            rt.launch_folded(kernel_for(K_ACCNORM_BASE, K_ACCNORM_F16, accum->dtype), a.grid, NBO_BLOCK, a);
+            NboSumPartialsArgs r = {};
+            r.in = a.partial_sumsq;
+            r.out = rt.partial_sumsq();
+            r.out_flag = rt.partial_flag();
+            r.n = a.grid;
+            r.per = (a.grid + NBO_NORM_GRID_MAX - 1) / NBO_NORM_GRID_MAX;
+            f.grid = (a.grid + r.per - 1) / r.per;
+            rt.launch(K_SUM_PARTIALS, f.grid, NBO_BLOCK, r);
         }
         f.check_finite = (scaler || (flags & NBO_ACC_CHECK_FINITE)) ? 1u : 0u;
         f.scaler = scaler ? scaler->dev : nullptr;

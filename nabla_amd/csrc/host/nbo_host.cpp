@@ -39,7 +39,7 @@ static const char *const kKernelNames[K_COUNT] = {
     "nbo_norm_f32",          "nbo_norm_bf16",        "nbo_norm_f64",
     "nbo_scale_f32",         "nbo_scale_bf16",       "nbo_scale_f64",
     "nbo_prep",              "nbo_finalize",         "nbo_cast_master",
-    nullptr,                 "nbo_probe_rmw2",       "nbo_accum_f32",
+    "nbo_sum_partials",      "nbo_probe_rmw2",       "nbo_accum_f32",
     "nbo_accum_bf16",        "nbo_accum_f64",        "nbo_fill_zero",
     "nbo_ew_f32",            "nbo_ew_bf16",          "nbo_ew_f64",
     "nbo_cast_list",         "nbo_update_pbf16_adamw", "nbo_update_pbf16_adam",
@@ -125,6 +125,19 @@ Runtime::Runtime()
 }
 
 void Runtime::sync() { hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize"); }
+
+double *Runtime::piece_partials(size_t count)
+{
+    if (count > piece_partials_cap_) {
+        sync(); // a pass still in flight may be writing the old array
+        dfree(piece_partials_);
+        piece_partials_ = nullptr;
+        piece_partials_cap_ = 0;
+        piece_partials_ = (double *)dmalloc(count * sizeof(double));
+        piece_partials_cap_ = count;
+    }
+    return piece_partials_;
+}
 
 void Runtime::set_stream(hipStream_t s)
 {

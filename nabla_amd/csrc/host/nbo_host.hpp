@@ -41,7 +41,7 @@ enum KernelId {
     K_PREP = 15,
     K_FINALIZE = 16,
     K_CAST_MASTER = 17,
-    K_UNUSED_18 = 18, // (was the calibration copy: now in the measurement code object)
+    K_SUM_PARTIALS = 18, // per-piece sums of squares -> at most NBO_NORM_GRID_MAX of them
     K_PROBE = 19,
     K_ACCUM_BASE = 20, // + st
     K_FILL_ZERO = 23,
@@ -138,6 +138,9 @@ public:
     NboGradFactors *gf_scratch() const { return gf_scratch_; }
     // one word, zero between uses: passes without partial results OR their non-finite findings into it
     uint32_t *any_bad() const { return any_bad_; }
+    // room for `count` per-piece sums of squares; grows (after a synchronisation) when a larger
+    // list comes along, never shrinks
+    double *piece_partials(size_t count);
     // the device this runtime lives on, and how the look-up of the statically allocated
     // scratch's address went there
     int device() const { return device_; }
@@ -162,6 +165,8 @@ private:
     uint32_t *partial_flag_ = nullptr;
     NboGradFactors *gf_scratch_ = nullptr;
     uint32_t *any_bad_ = nullptr;
+    double *piece_partials_ = nullptr;
+    size_t piece_partials_cap_ = 0;
     int device_ = 0;
     hipError_t static_scratch_status_ = hipSuccess;
     struct ProfRec {

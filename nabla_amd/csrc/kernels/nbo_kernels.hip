@@ -16,7 +16,9 @@
 //   nbo_ew_*        the Backend primitives as single passes (nabla-core/src/cpu/mod.rs:211-272)
 //   nbo_accum_*     gradient accumulation buf += g (trainer.rs:253-267)
 //   nbo_accnorm_*   a whole micro-batch of the accumulating Trainer in one pass: finite scan,
-//                   unscale, accumulate, first stage of the buffer's sum of squares (trainer.rs:230-267)
+//                   unscale, accumulate, first stage of the buffer's sum of squares (trainer.rs:230-267);
+//                   nbo_accscale_* the same without the sum, nbo_sum_partials between the first
+//                   stage's per-piece sums and the second stage
 //
 // Numerics contract: every arithmetic operation of the reference is one IEEE
 // round-to-nearest operation here, in the same order, never contracted into an
@@ -1362,28 +1364,40 @@ NBO_ACCUM_KERNEL(nbo_accum_f16, NBO_F16)
 
 // One micro-batch of the accumulating Trainer in one pass (trainer.rs:230-267): the finite
 // scan of GradScaler::unscale_and_update over g (core.rs:357-368), u = g * T(1 / scale)
-// (core.rs:376-380), buf = buf + u (trainer.rs:262-266), and the first stage of the sum of
-// squares of the new buf, which clip_grad_norm needs once the last micro-batch is in
-// (trainer.rs:504-513).  Same fixed grid, chunk striding and reduction as the norm pass.  On
-// a non-finite gradient buf receives garbage: the Trainer discards the accumulation then.
-template <int ST> DEV void accnorm_body(const NboAccNormArgs &a)
-{
+// (core.rs:376-380), buf = buf + u (trainer.rs:262-266), and -- SUMSQ -- the first stage of the
+// sum of squares of the new buf, which clip_grad_norm needs once the last micro-batch is in
+// (trainer.rs:504-513).  On a non-finite gradient buf receives garbage: the Trainer discards the
+// accumulation then.  It runs like the element-wise passes, one short-lived workgroup per piece,
+// 6.3-6.5 TB/s (a fixed grid of workgroups that stride over the chunks, as the norm pass has it,
+// reached 5.0-5.6 with these three streams).  Whether a gradient was non-finite is one bit, and
+// an OR needs no order: a workgroup that met one ORs it into *a.any_bad, which the second stage
+// reads and clears.  The sum of squares does need an order: every workgroup leaves the sum over
+// its piece, and nbo_sum_partials and the second stage add those up in a fixed order.
+template <int ST, bool SUMSQ> struct AccScaleOp {
     typedef typename Traits<ST>::T T;
-    enum { SB = Traits<ST>::SBYTES, VEC = Traits<ST>::VEC };
-    __shared__ double lds_d[NBO_BLOCK / 64];
-    __shared__ uint32_t lds_u[NBO_BLOCK / 64];
-    const uint32_t tid = threadIdx.x;
-    const T inv = a.scaler ? (T)(1.0 / a.scaler->scale) : (T)1; // core.rs:355
-    const bool write_g = a.write_grads != 0;
-    double acc = 0.0;
-    uint32_t bad = 0;
-
-    for (uint32_t ci = blockIdx.x; ci < a.L.nchunks; ci += a.grid) {
-        const ChunkRef c = chunk_ref(a.L, ci);
-        char *pa = (char *)a.acc_ptrs[c.t] + c.base * SB;
-        char *pg = (char *)a.g_ptrs[c.t] + c.base * SB;
-        // the norm pass's walk: single elements up to the first 16-byte boundary, whole vectors,
-        // single elements for the rest (buffer and gradients misaligned alike, else all single)
+    enum { SB = Traits<ST>::SBYTES, VEC = Traits<ST>::VEC, EV = EwIO<ST>::EV };
+    T inv;
+    bool write_g;
+    uint32_t bad;
+    double acc;
+    MEMBER bool loads(int) const { return true; }
+    MEMBER bool stores(int s) const { return s == 0 || write_g; }
+    MEMBER void apply(T (&x)[2][EV])
+    {
+#pragma unroll
+        for (int k = 0; k < EV; k++) {
+            bad |= (uint32_t)nonfinite<ST>(x[1][k]);
+            x[1][k] = x[1][k] * inv;
+            x[0][k] = x[0][k] + x[1][k];
+            if (SUMSQ) acc = sq_acc<ST>(acc, x[0][k]);
+        }
+    }
+    // the norm pass's walk: single elements up to the first 16-byte boundary, whole vectors,
+    // single elements for the rest (buffer and gradients misaligned alike, else all single)
+    MEMBER void ragged(const ChunkRef &c, char *const (&ptr)[2])
+    {
+        const uint32_t tid = threadIdx.x;
+        char *pa = ptr[0], *pg = ptr[1];
         const Peel pl = peel(c.cnt, VEC, SB, false, (uintptr_t)pa, (uintptr_t)pg);
         auto single = [&](uint32_t e) {
             const uint64_t off = (uint64_t)e * SB;
@@ -1391,7 +1405,7 @@ template <int ST> DEV void accnorm_body(const NboAccNormArgs &a)
             bad |= (uint32_t)nonfinite<ST>(g);
             const T u = g * inv;
             const T b = IO<ST>::ld1(pa + off) + u;
-            acc = sq_acc<ST>(acc, b);
+            if (SUMSQ) acc = sq_acc<ST>(acc, b);
             IO<ST>::st1(pa + off, b);
             if (write_g) IO<ST>::st1(pg + off, u);
         };
@@ -1406,67 +1420,7 @@ template <int ST> DEV void accnorm_body(const NboAccNormArgs &a)
                 bad |= (uint32_t)nonfinite<ST>(g[k]);
                 g[k] = g[k] * inv;
                 b[k] = b[k] + g[k];
-                acc = sq_acc<ST>(acc, b[k]);
-            }
-            IO<ST>::stv(pa + off, b);
-            if (write_g) IO<ST>::stv(pg + off, g);
-        }
-        for (uint32_t e = pl.head + pl.nvec * VEC + tid; e < c.cnt; e += NBO_BLOCK) single(e);
-    }
-    const double bs = block_sum(acc, lds_d);
-    const uint32_t bo = block_or(bad, lds_u);
-    if (tid == 0) {
-        a.partial_sumsq[blockIdx.x] = bs;
-        a.partial_flag[blockIdx.x] = bo;
-    }
-}
-
-// The same micro-batch without the sum of squares (all micro-batches but the last need none):
-// no reduction, so no fixed grid -- it runs like the element-wise passes, one short-lived
-// workgroup per piece, 6.3-6.5 TB/s against the 5.0-5.6 of the looping form above.  What is left
-// to reduce is one bit, and an OR needs no order: a workgroup that met a non-finite gradient ORs
-// it into *a.any_bad, which the second stage reads and clears.
-template <int ST> struct AccScaleOp {
-    typedef typename Traits<ST>::T T;
-    enum { SB = Traits<ST>::SBYTES, VEC = Traits<ST>::VEC, EV = EwIO<ST>::EV };
-    T inv;
-    bool write_g;
-    uint32_t bad;
-    MEMBER bool loads(int) const { return true; }
-    MEMBER bool stores(int s) const { return s == 0 || write_g; }
-    MEMBER void apply(T (&x)[2][EV])
-    {
-#pragma unroll
-        for (int k = 0; k < EV; k++) {
-            bad |= (uint32_t)nonfinite<ST>(x[1][k]);
-            x[1][k] = x[1][k] * inv;
-            x[0][k] = x[0][k] + x[1][k];
-        }
-    }
-    MEMBER void ragged(const ChunkRef &c, char *const (&ptr)[2])
-    {
-        const uint32_t tid = threadIdx.x;
-        char *pa = ptr[0], *pg = ptr[1];
-        const Peel pl = peel(c.cnt, VEC, SB, false, (uintptr_t)pa, (uintptr_t)pg);
-        auto single = [&](uint32_t e) {
-            const uint64_t off = (uint64_t)e * SB;
-            const T g = IO<ST>::ld1(pg + off);
-            bad |= (uint32_t)nonfinite<ST>(g);
-            const T u = g * inv;
-            IO<ST>::st1(pa + off, IO<ST>::ld1(pa + off) + u);
-            if (write_g) IO<ST>::st1(pg + off, u);
-        };
-        for (uint32_t e = tid; e < pl.head; e += NBO_BLOCK) single(e);
-        for (uint32_t q = tid; q < pl.nvec; q += NBO_BLOCK) {
-            const uint64_t off = ((uint64_t)pl.head + (uint64_t)q * VEC) * SB;
-            T g[VEC], b[VEC];
-            IO<ST>::ldv(pg + off, g);
-            IO<ST>::ldv(pa + off, b);
-#pragma unroll
-            for (int k = 0; k < VEC; k++) {
-                bad |= (uint32_t)nonfinite<ST>(g[k]);
-                g[k] = g[k] * inv;
-                b[k] = b[k] + g[k];
+                if (SUMSQ) acc = sq_acc<ST>(acc, b[k]);
             }
             IO<ST>::stv(pa + off, b);
             if (write_g) IO<ST>::stv(pg + off, g);
@@ -1475,24 +1429,49 @@ template <int ST> struct AccScaleOp {
     }
 };
 
-template <int ST> DEV void accscale_body(const NboAccNormArgs &a)
+template <int ST, bool SUMSQ> DEV void accscale_body(const NboAccNormArgs &a)
 {
     typedef typename Traits<ST>::T T;
-    AccScaleOp<ST> op;
+    __shared__ double lds_d[NBO_BLOCK / 64];
+    AccScaleOp<ST, SUMSQ> op;
     op.inv = a.scaler ? (T)(1.0 / a.scaler->scale) : (T)1; // core.rs:355
     op.write_g = a.write_grads != 0;
     op.bad = 0;
+    op.acc = 0.0;
     const uint64_t *const lists[2] = {a.acc_ptrs, a.g_ptrs};
     stream_pieces<ST, 2, NBO_EW_PIECE_BYTES>(a.L, lists, op, a.by_chunk != 0);
     // one addition per wave that found something: in a healthy step, none at all
     if (__builtin_amdgcn_ballot_w64(op.bad != 0) != 0 && (threadIdx.x & 63u) == 0)
         __hip_atomic_fetch_or(a.any_bad, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (!SUMSQ) return;
+    // (a workgroup whose piece a ragged chunk does not have, or past the end of a folded grid,
+    // has added nothing: its sum is the zero it must leave)
+    const double bs = block_sum(op.acc, lds_d);
+    const uint32_t wg = folded_workgroup();
+    if (threadIdx.x == 0 && wg < a.grid) {
+        a.partial_sumsq[wg] = bs;
+        if (a.partial_flag) a.partial_flag[wg] = 0;
+    }
+}
+
+extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_sum_partials(const NboSumPartialsArgs a)
+{
+    __shared__ double lds_d[NBO_BLOCK / 64];
+    const uint64_t lo = (uint64_t)blockIdx.x * a.per;
+    const uint64_t hi = lo + a.per < a.n ? lo + a.per : a.n;
+    double acc = 0.0;
+    for (uint64_t i = lo + threadIdx.x; i < hi; i += NBO_BLOCK) acc = acc + a.in[i];
+    const double bs = block_sum(acc, lds_d);
+    if (threadIdx.x == 0) {
+        a.out[blockIdx.x] = bs;
+        a.out_flag[blockIdx.x] = 0;
+    }
 }
 
 #define NBO_ACCSCALE_KERNEL(name, ST)                                                       \
     extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboAccNormArgs a)    \
     {                                                                                       \
-        accscale_body<ST>(a);                                                               \
+        accscale_body<ST, false>(a);                                                        \
     }
 NBO_ACCSCALE_KERNEL(nbo_accscale_f32, NBO_F32)
 NBO_ACCSCALE_KERNEL(nbo_accscale_bf16, NBO_PBF16)
@@ -1502,7 +1481,7 @@ NBO_ACCSCALE_KERNEL(nbo_accscale_f16, NBO_PF16)
 #define NBO_ACCNORM_KERNEL(name, ST)                                                        \
     extern "C" __global__ __launch_bounds__(NBO_BLOCK) void name(const NboAccNormArgs a)    \
     {                                                                                       \
-        accnorm_body<ST>(a);                                                                \
+        accscale_body<ST, true>(a);                                                         \
     }
 // 16-bit lists: unscale and add in the lists' own type, as the in-place passes do
 NBO_ACCNORM_KERNEL(nbo_accnorm_f32, NBO_F32)

@@ -216,22 +216,33 @@ struct NboPrepArgs {
 };
 
 // One micro-batch of the accumulating Trainer in a single pass (trainer.rs:230-267): finite
-// scan of g, acc[i] = acc[i] + T(g[i] * inv_scale), and the sum of squares of the new acc.
+// scan of g, acc[i] = acc[i] + T(g[i] * inv_scale), and -- nbo_accnorm_* -- the sum of squares of
+// the new acc.  Both forms run like the element-wise passes, one short-lived workgroup per piece
+// (per chunk of a list of small tensors), and OR whether they met a non-finite gradient into
+// *any_bad, which the second stage reads and clears.
 struct NboAccNormArgs {
     NboLayoutDev L;
     const uint64_t *acc_ptrs;
     const uint64_t *g_ptrs;
     const NboScalerDev *scaler; // null: no unscale, inv_scale = 1
-    double *partial_sumsq;      // [grid]
-    uint32_t *partial_flag;     // [grid]
-    uint32_t grid;
+    double *partial_sumsq;      // [grid]: one sum of squares per workgroup (nbo_accnorm_* only)
+    uint32_t *partial_flag;     // [grid] or null: zeroed, for a second stage that reads flags beside the sums
+    uint32_t grid;              // workgroups that have a piece (a folded launch may have more)
     uint32_t write_grads;       // also store the unscaled gradients in place, as the reference does
-    // The variant without the sum of squares (nbo_accscale_*: every micro-batch but the last) runs
-    // like the element-wise passes and leaves only whether it met a non-finite gradient: ORed into
-    // *any_bad, which the second stage reads and clears.
     uint32_t *any_bad;
     uint32_t by_chunk; // see NboAccumArgs
     uint32_t pad;
+};
+
+// Between a pass that leaves one partial sum per piece and the second stage, which reads at most
+// NBO_NORM_GRID_MAX of them: workgroup j adds in[j * per .. min(n, (j + 1) * per)) in a fixed
+// order into out[j] and clears out_flag[j].
+struct NboSumPartialsArgs {
+    const double *in;
+    double *out;
+    uint32_t *out_flag;
+    uint32_t n;
+    uint32_t per;
 };
 
 // a[i] = a[i] + b[i] over two lists of the same shapes (gradient accumulation).

@@ -709,7 +709,7 @@ def unscale_accumulate(accum, grads, scaler: Optional["GradScaler"] = None, chec
     Trainer discards the accumulation then).  The gradients stay as they were unless
     `write_grads` asks for the reference's in-place result.  Only the last micro-batch of an
     accumulation needs the sum of squares (for the clip): with `want_sumsq=False` the pass has
-    nothing to reduce but one bit and runs some 15 % faster; sumsq is then None."""
+    nothing to reduce but one bit (one small launch fewer); sumsq is then None."""
     a = _free_cache.get("accum_a", accum)
     g = _free_cache.get("accum_g", grads)
     ok, sumsq = C.c_int(0), C.c_double(0.0)

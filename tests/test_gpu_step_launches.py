@@ -337,8 +337,8 @@ def test_grids_folded_into_two_dimensions_cover_every_row_once(gpu):
     """One grid dimension holds fewer than 2^32 threads, so the launches that run one workgroup per
     row of a chunk fold a larger grid into two dimensions.  With NBO_GRID_X_MAX=37 in the
     environment (a test hook of the runtime) every such launch here is folded, its last grid row
-    partly unused: the element-wise passes, the cast, SGD and the by-row Adam kernels must still
-    do every row exactly once."""
+    partly unused: the element-wise passes (the accumulating micro-batch with its per-piece sums
+    among them), the cast, SGD and the by-row Adam kernels must still do every row exactly once."""
     import os
     import subprocess
     import sys
@@ -363,6 +363,15 @@ assert not any(t.any() for t in H.host_list(g))
 out = [torch.zeros_like(t) for t in a]
 B.add(H.dev_list(p0, shapes), H.dev_list(g0, shapes), out=out)
 H.assert_bits_equal(H.host_list(out), [O.add(x, y) for x, y in zip(p0, g0)], "backend add")
+# the accumulating micro-batch with its sum of squares: one partial sum per piece, more pieces
+# than the second stage adds up itself
+a, g = H.dev_list(p0, shapes), H.dev_list(g0, shapes)
+ok, sumsq = nb.unscale_accumulate(a, g)
+acc = [O.add(x, y) for x, y in zip(p0, g0)]
+H.assert_bits_equal(H.host_list(a), acc, "unscale_accumulate")
+import math
+exact = math.fsum(np.concatenate([np.square(x.astype(np.float64)).ravel() for x in acc]).tolist())
+assert ok and abs(sumsq - exact) <= 1e-14 * exact, (sumsq, exact)
 half = H.dev_list([np.zeros(x.shape, dtype=np.uint16) for x in p0], shapes)
 B.cast(H.dev_list(p0, shapes), half)
 H.assert_bits_equal(H.host_list(half), [O.bf16_from_f32(x) for x in p0], "cast")
