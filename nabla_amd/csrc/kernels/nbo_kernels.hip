@@ -1095,16 +1095,18 @@ template <> struct Bits128<float> {
 };
 template <> struct Bits128<double> {
     enum { EV = 2 };
+    // (one cast of the whole vector: assembled from its 32-bit halves, the compiler fetched the
+    // first element a second time with a load of its own, and the f64 passes ran 10 % slower)
     DEV void unpack(int, u32x4 v, double (&x)[2])
     {
-        x[0] = __hiloint2double((int)v.y, (int)v.x);
-        x[1] = __hiloint2double((int)v.w, (int)v.z);
+        const f64x2 d = __builtin_bit_cast(f64x2, v);
+        x[0] = d.x;
+        x[1] = d.y;
     }
     DEV u32x4 pack(int, const double (&x)[2])
     {
-        const u32x4 v = {(uint32_t)__double2loint(x[0]), (uint32_t)__double2hiint(x[0]), (uint32_t)__double2loint(x[1]),
-                         (uint32_t)__double2hiint(x[1])};
-        return v;
+        const f64x2 d = {x[0], x[1]};
+        return __builtin_bit_cast(u32x4, d);
     }
 };
 template <int FMT> struct Bits128<Half16<FMT>> {
