@@ -204,6 +204,31 @@ int nbo_copy_bytes(const void *src_dev, void *dst_dev, uint64_t bytes)
     });
 }
 
+int nbo_selftest_bf16_arith(uint64_t *div_mismatches, uint64_t *sqrt_mismatches, uint64_t *example_pair,
+                            uint64_t *example_arg)
+{
+    return guarded([&] {
+        require(div_mismatches && sqrt_mismatches, NBO_ERR_ARG, "null output");
+        Runtime &rt = Runtime::get();
+        unsigned long long *out = (unsigned long long *)rt.dmalloc(4 * sizeof(unsigned long long));
+        try {
+            rt.dzero(out, 4 * sizeof(unsigned long long));
+            NboSelftestArgs a = {out};
+            rt.launch(K_SELFTEST_BF16, 65536, NBO_BLOCK, a);
+            unsigned long long r[4];
+            rt.read_back(r, out, sizeof(r));
+            *div_mismatches = r[0];
+            *sqrt_mismatches = r[1];
+            if (example_pair) *example_pair = r[2];
+            if (example_arg) *example_arg = r[3];
+        } catch (...) {
+            rt.dfree(out);
+            throw;
+        }
+        rt.dfree(out);
+    });
+}
+
 int nbo_hbm_ceiling(int pattern, int spread, uint64_t bytes_per_stream, int reps, uint32_t settle_ms,
                     double *best_gbps, double *mean_gbps, int *regions)
 {

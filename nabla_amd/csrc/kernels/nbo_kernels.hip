@@ -139,6 +139,40 @@ template <int FMT> DEV Half16<FMT> half_from_bits(uint32_t b)
     return r;
 }
 
+// bf16 / bf16 and sqrt(bf16), rounded to f32 and then to bf16 as above, without the correctly
+// rounded f32 operation (eleven and fourteen instructions; with them the all-bf16 Adam kernels
+// were compute-bound: some 76 vector instructions per element for 12 bytes, 6.27 TB/s at most).
+// Both operands have 8 significant bits, so a quotient is either exactly a bf16 rounding boundary
+// (a 9-bit number) or at least 2^-17 of its size away from every one, and a square root is never
+// on one and at least 2^-18 away: an approximation good to a few units of the f32's last place
+// rounds to the same bf16, once a quotient that close to a boundary is taken to be on it.  The
+// hardware's reciprocal and square root are such approximations unless the reciprocal is not a
+// normal number, the quotient not finite or the square root's argument subnormal (the
+// instructions flush those); then the exact operation is done.  That the results are the exact
+// operations' bits has been checked for all 2^32 pairs and all 2^16 arguments
+// (nbo_selftest_bf16_arith).
+enum { CLS_NAN = 0x003, CLS_INF = 0x204, CLS_DENORMAL = 0x090, CLS_ZERO = 0x060 };
+DEV BF div_exact(BF a, BF b) { return BF(a.f() / b.f()); }
+DEV BF sqrt_exact(BF x) { return BF(__builtin_sqrtf(x.f())); }
+DEV BF operator/(BF a, BF b)
+{
+    const float x = a.f(), y = b.f();
+    const float rc = __builtin_amdgcn_rcpf(y);
+    const float q = x * rc;
+    if (__builtin_expect(__builtin_amdgcn_classf(rc, CLS_NAN | CLS_INF | CLS_DENORMAL | CLS_ZERO) ||
+                             __builtin_amdgcn_classf(q, CLS_NAN | CLS_INF),
+                         0))
+        return div_exact(a, b);
+    // within 4 units of a multiple of 8 units (every rounding boundary is one): onto it
+    return BF(__uint_as_float((__float_as_uint(q) + 4u) & ~7u));
+}
+DEV BF sqrt_fast(BF v)
+{
+    const float x = v.f();
+    if (__builtin_expect(__builtin_amdgcn_classf(x, CLS_DENORMAL), 0)) return sqrt_exact(v);
+    return BF(__builtin_amdgcn_sqrtf(x));
+}
+
 // f64::powi as compiler-rt's __powidf2 (alg.rs:122-123).
 DEV double powi_f64(double a, int n)
 {
@@ -377,6 +411,7 @@ template <int FMT> struct Scal<Half16<FMT>> {
 };
 
 template <int FMT> DEV Half16<FMT> sqrt_rn(Half16<FMT> x) { return Half16<FMT>(__builtin_sqrtf(x.f())); }
+DEV BF sqrt_rn(BF x) { return sqrt_fast(x); }
 DEV float sqrt_rn(float x) { return __builtin_sqrtf(x); }
 DEV double sqrt_rn(double x) { return __builtin_sqrt(x); }
 
@@ -1739,6 +1774,31 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_fill_zero(const NboF
         __builtin_nontemporal_store(z, GLOBAL_PTR(u32x4, p + head) + i);
     if (gid < head) p[gid] = 0;
     if (gid < a.bytes - tail0) p[tail0 + gid] = 0;
+}
+
+// Every one of the 2^32 pairs of bf16 patterns through the kernels' bf16 division, every one of the
+// 2^16 patterns through their bf16 square root, compared bit for bit with the exact operations
+// (the f32 operation correctly rounded, then bf16::from_f32).  Workgroup a, thread t: numerator
+// pattern a, denominators t, t + 256, ...
+extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_selftest_bf16_arith(const NboSelftestArgs a)
+{
+    const BF x = half_from_bits<FMT_BF16>(blockIdx.x);
+    unsigned long long bad = 0, example = 0;
+    for (uint32_t b = threadIdx.x; b < 65536u; b += NBO_BLOCK) {
+        const BF y = half_from_bits<FMT_BF16>(b);
+        if ((x / y).bits != div_exact(x, y).bits) {
+            bad++;
+            example = ((unsigned long long)blockIdx.x << 16) | b;
+        }
+    }
+    if (bad) {
+        atomicAdd(&a.out[0], bad);
+        a.out[2] = example;
+    }
+    if (threadIdx.x == 0 && sqrt_fast(x).bits != sqrt_exact(x).bits) {
+        atomicAdd(&a.out[1], 1ull);
+        a.out[3] = blockIdx.x;
+    }
 }
 
 // Placement probe: every workgroup reads and rewrites the same 8 rows of NBO_BLOCK

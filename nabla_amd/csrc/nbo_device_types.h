@@ -278,6 +278,13 @@ struct NboFillArgs {
     uint64_t bytes;
 };
 
+// nbo_selftest_bf16_arith: out[0] = pairs (a, b) of bf16 patterns whose quotient's bits differ between
+// the kernels' bf16 division and the exact one, out[1] = the same for the square root's arguments,
+// out[2], out[3] = one such pair (a << 16 | b) and one such argument.  The caller zeroes out[].
+struct NboSelftestArgs {
+    unsigned long long *out;
+};
+
 // Backend primitives on tensor lists (nabla-core/src/common/backend/mod.rs:82-216,
 // 275-279): one IEEE operation per element, every result rounded to the element type.
 enum {
