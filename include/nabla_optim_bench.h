@@ -2,10 +2,10 @@
  * nabla_optim_bench.h -- measurement entry points of libnabla_optim.so.
  *
  * None of these has a counterpart in the reference's optimizer interface, and no optimizer
- * step needs them: they time the library's own launches and measure what the MI355X memory
- * system gives an access pattern, for benchmarks and profiles.  The drop-in boundary is
- * nabla_optim.h alone.  The probe kernels live in a code object of their own that is loaded
- * when one of these functions first needs it.
+ * step needs them: they time the library's own launches, measure what the MI355X memory
+ * system gives an access pattern, for benchmarks and profiles, and check the library's own
+ * arithmetic exhaustively.  The drop-in boundary is nabla_optim.h alone.  The probe kernels
+ * live in a code object of their own that is loaded when one of these functions first needs it.
  */
 #ifndef NABLA_OPTIM_BENCH_H
 #define NABLA_OPTIM_BENCH_H
