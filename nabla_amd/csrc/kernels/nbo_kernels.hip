@@ -510,8 +510,8 @@ DEV Peel peel(uint32_t cnt, uint32_t vec, uint32_t sb, bool wvo, uintptr_t a0, u
     return peel(cnt, vec, sb, wvo, a0, a1, a0);
 }
 
-DEV void prep_step(NboOptimDev *o, const NboHyper &h, const NboGradFactors *f);
-DEV void trace_step(NboTraceDev *t, const NboGradFactors *f, const NboOptimDev *o, double scale);
+DEV uint64_t prep_step(NboOptimDev *o, const NboHyper &h, const NboGradFactors *f, uint64_t step_count);
+DEV void trace_step(NboTraceDev *t, uint64_t entries, const NboGradFactors *f, uint64_t step_count, double scale);
 
 // A per-step scalar that every lane has computed alike, moved to a scalar register (the
 // vector units do all f64 arithmetic; without this the scalars would occupy a vector register each).
@@ -728,14 +728,14 @@ template <int ST, int KIND, bool SELF = false> DEV void update_body(const NboUpd
         readers_before = __hip_atomic_fetch_add(&a.opt_rw->ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     NboOptimDev own = {};
     own.step_count = ((uint64_t)sc_hi << 32) | sc_lo;
-    prep_step(&own, a.hyper, a.gf);
+    prep_step(&own, a.hyper, a.gf, own.step_count);
     make_uniform(own);
     update_chunk<ST, KIND>(a, &own, wg);
     // the counter's answer is not looked at before the chunk is done: it has long arrived then
     __builtin_amdgcn_sched_barrier(0);
     if (threadIdx.x == 0 && readers_before == nwg - 1) {
         a.opt_rw->step_count = own.step_count;
-        if (a.trace) trace_step(a.trace, a.gf, &own, a.scaler ? a.scaler->scale : 0.0);
+        if (a.trace) trace_step(a.trace, a.trace->count, a.gf, own.step_count, a.scaler ? a.scaler->scale : 0.0);
         __hip_atomic_store(&a.opt_rw->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
@@ -848,8 +848,10 @@ DEV uint32_t block_or(uint32_t x, uint32_t *lds)
 }
 
 // Per-step scalars (alg.rs:120-135 AdamW, 265-277 Adam, 393-395 Sgd).  A skipped
-// step leaves step_count alone, because the reference never calls step() then.
-DEV void prep_step(NboOptimDev *o, const NboHyper &h, const NboGradFactors *f)
+// step leaves step_count alone, because the reference never calls step() then.  step_count is
+// o->step_count, which the caller has read (early, where it waits for other loads anyway);
+// returns its value after the step.
+DEV uint64_t prep_step(NboOptimDev *o, const NboHyper &h, const NboGradFactors *f, uint64_t step_count)
 {
     o->lr = h.lr;
     o->beta1 = h.beta1;
@@ -860,7 +862,7 @@ DEV void prep_step(NboOptimDev *o, const NboHyper &h, const NboGradFactors *f)
     o->kind = h.kind;
     if (f && f->found_inf) {
         o->skip = 1;
-        return;
+        return step_count;
     }
     o->skip = 0;
     if (o->kind == NBO_SGD) {
@@ -871,10 +873,11 @@ DEV void prep_step(NboOptimDev *o, const NboHyper &h, const NboGradFactors *f)
         o->d_neg_lr = -o->lr;
         o->d_momentum = o->momentum;
         o->d_wd = o->weight_decay;
-        return;
+        return step_count;
     }
-    o->step_count += 1;
-    const int step = (int)o->step_count;
+    step_count += 1;
+    o->step_count = step_count;
+    const int step = (int)step_count;
     const double bc1 = 1.0 - powi_f64(o->beta1, step);
     const double bc2 = 1.0 - powi_f64(o->beta2, step);
     const double step_size = o->lr / bc1;
@@ -900,15 +903,17 @@ DEV void prep_step(NboOptimDev *o, const NboHyper &h, const NboGradFactors *f)
     o->d_ss = step_size;
     o->d_ibc2 = ibc2;
     o->d_omw = 1.0 - wd_lr;
+    return step_count;
 }
 
-DEV void trace_step(NboTraceDev *t, const NboGradFactors *f, const NboOptimDev *o, double scale)
+// entries = t->count, read by the caller
+DEV void trace_step(NboTraceDev *t, uint64_t entries, const NboGradFactors *f, uint64_t step_count, double scale)
 {
-    const uint64_t i = t->count;
+    const uint64_t i = entries;
     NboTraceEntry e;
     e.scale = scale;
     e.norm = f ? f->norm : 0.0;
-    e.step_count = o ? o->step_count : 0;
+    e.step_count = step_count;
     e.found_inf = f ? f->found_inf : 0u;
     e.clipped = f ? f->clipped : 0u;
     t->e[i % NBO_TRACE_LEN] = e;
@@ -918,8 +923,9 @@ DEV void trace_step(NboTraceDev *t, const NboGradFactors *f, const NboOptimDev *
 extern "C" __global__ __launch_bounds__(64) void nbo_prep(const NboPrepArgs a)
 {
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    prep_step(a.opt, a.hyper, a.gf);
-    if (a.trace) trace_step(a.trace, a.gf, a.opt, a.scaler ? a.scaler->scale : 0.0);
+    const uint64_t entries = a.trace ? a.trace->count : 0;
+    const uint64_t step_count = prep_step(a.opt, a.hyper, a.gf, a.opt->step_count);
+    if (a.trace) trace_step(a.trace, entries, a.gf, step_count, a.scaler ? a.scaler->scale : 0.0);
 }
 
 // Second stage: reduce the per-block partials in a fixed order, then the scalar
@@ -930,17 +936,41 @@ extern "C" __global__ __launch_bounds__(64) void nbo_prep(const NboPrepArgs a)
 DEV void finalize_body(const NboFinalizeArgs &a, double *lds_d, uint32_t *lds_u)
 {
     const uint32_t tid = threadIdx.x;
+    // Everything this kernel reads is asked for here, at once: a read takes about a microsecond
+    // to come back, and one after the other -- partial sums, the word of a pass without them, the
+    // scaler, the step count, the trace's length -- they were most of the kernel's five.
+    enum { PER = NBO_NORM_GRID_MAX / NBO_BLOCK };
+    static_assert(PER * NBO_BLOCK == NBO_NORM_GRID_MAX, "whole rounds of the workgroup");
+    double part[PER];
+    uint32_t flag[PER];
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const uint32_t i = tid + j * NBO_BLOCK;
+        part[j] = i < a.grid ? a.partial_sumsq[i] : 0.0;
+        flag[j] = i < a.grid ? a.partial_flag[i] : 0u;
+    }
+    uint32_t word = 0;
+    uint64_t step_count = 0, entries = 0;
+    NboScalerDev s = {};
+    if (tid == 0) {
+        if (a.any_bad) word = *a.any_bad;
+        if (a.scaler) s = *a.scaler;
+        if (a.opt) step_count = a.opt->step_count;
+        if (a.trace) entries = a.trace->count;
+    }
+    // (the sums are squares, never -0.0: adding the 0.0 of a slot that does not exist changes nothing)
     double acc = 0.0;
     uint32_t bad = 0;
-    for (uint32_t i = tid; i < a.grid; i += NBO_BLOCK) {
-        acc = acc + a.partial_sumsq[i];
-        bad |= a.partial_flag[i];
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        acc = acc + part[j];
+        bad |= flag[j];
     }
     const double reduced = block_sum(acc, lds_d);
     uint32_t any_bad = block_or(bad, lds_u);
     if (tid != 0) return;
     if (a.any_bad) { // what a pass without partial results found, and the word clean again for the next one
-        any_bad |= *a.any_bad;
+        any_bad |= word;
         *a.any_bad = 0;
     }
 
@@ -951,7 +981,6 @@ DEV void finalize_body(const NboFinalizeArgs &a, double *lds_d, uint32_t *lds_u)
     double inv = 1.0;
     double scale_after = 0.0;
     if (a.scaler) {
-        NboScalerDev s = *a.scaler;
         inv = 1.0 / s.scale; // core.rs:355, from the scale before its update
         if (found) {
             s.scale = s.scale * s.backoff_factor;
@@ -984,8 +1013,8 @@ DEV void finalize_body(const NboFinalizeArgs &a, double *lds_d, uint32_t *lds_u)
         }
     }
     *a.gf = f;
-    if (a.opt) prep_step(a.opt, a.hyper, &f);
-    if (a.trace) trace_step(a.trace, &f, a.opt, scale_after);
+    if (a.opt) step_count = prep_step(a.opt, a.hyper, &f, step_count);
+    if (a.trace) trace_step(a.trace, entries, &f, step_count, scale_after);
 }
 
 extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_finalize(const NboFinalizeArgs a)
