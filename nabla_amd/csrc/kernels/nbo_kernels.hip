@@ -47,6 +47,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // accesses in one instruction; the type keeps the compiler from assuming more)
 typedef float f32x4_e __attribute__((ext_vector_type(4), aligned(4)));
 typedef double f64x2_e __attribute__((ext_vector_type(2), aligned(8)));
+typedef uint32_t u32x2_e __attribute__((ext_vector_type(2), aligned(2)));
 
 #define DEV static __device__ __forceinline__
 #define MEMBER __device__ __forceinline__
@@ -294,23 +295,31 @@ template <int ST> struct IO;
 template <> struct IO<NBO_F32> {
     DEV void ldv(const char *p, float (&x)[4]) { ld_state((const float *)p, x); }
     DEV void stv(char *p, const float (&x)[4]) { st_state((float *)p, x); }
+    DEV void ldv_e(const char *p, float (&x)[4]) { ld_state_e((const float *)p, x); }
+    DEV void stv_e(char *p, const float (&x)[4]) { st_state_e((float *)p, x); }
     DEV float ld1(const char *p) { return *GLOBAL_PTR(const float, p); }
     DEV void st1(char *p, float x) { *GLOBAL_PTR(float, p) = x; }
 };
 template <> struct IO<NBO_F64> {
     DEV void ldv(const char *p, double (&x)[2]) { ld_state((const double *)p, x); }
     DEV void stv(char *p, const double (&x)[2]) { st_state((double *)p, x); }
+    DEV void ldv_e(const char *p, double (&x)[2]) { ld_state_e((const double *)p, x); }
+    DEV void stv_e(char *p, const double (&x)[2]) { st_state_e((double *)p, x); }
     DEV double ld1(const char *p) { return *GLOBAL_PTR(const double, p); }
     DEV void st1(char *p, double x) { *GLOBAL_PTR(double, p) = x; }
 };
 template <> struct IO<NBO_BF16> {
+    DEV void widen(uint32_t lo, uint32_t hi, float (&x)[4])
+    {
+        x[0] = __uint_as_float(lo << 16);
+        x[1] = __uint_as_float(lo & 0xFFFF0000u);
+        x[2] = __uint_as_float(hi << 16);
+        x[3] = __uint_as_float(hi & 0xFFFF0000u);
+    }
     DEV void ldv(const char *p, float (&x)[4])
     {
         u32x2 v = NBO_LOAD(GLOBAL_PTR(const u32x2, p));
-        x[0] = __uint_as_float(v.x << 16);
-        x[1] = __uint_as_float(v.x & 0xFFFF0000u);
-        x[2] = __uint_as_float(v.y << 16);
-        x[3] = __uint_as_float(v.y & 0xFFFF0000u);
+        widen(v.x, v.y, x);
     }
     DEV void stv(char *p, const float (&x)[4])
     {
@@ -318,6 +327,19 @@ template <> struct IO<NBO_BF16> {
         v.x = f32_to_bf16_bits(x[0]) | (f32_to_bf16_bits(x[1]) << 16);
         v.y = f32_to_bf16_bits(x[2]) | (f32_to_bf16_bits(x[3]) << 16);
         NBO_STORE(v, GLOBAL_PTR(u32x2, p));
+    }
+    // ... at an address that is a whole number of elements, but not of vectors
+    DEV void ldv_e(const char *p, float (&x)[4])
+    {
+        u32x2_e v = NBO_LOAD(GLOBAL_PTR(const u32x2_e, p));
+        widen(v.x, v.y, x);
+    }
+    DEV void stv_e(char *p, const float (&x)[4])
+    {
+        u32x2_e v;
+        v.x = f32_to_bf16_bits(x[0]) | (f32_to_bf16_bits(x[1]) << 16);
+        v.y = f32_to_bf16_bits(x[2]) | (f32_to_bf16_bits(x[3]) << 16);
+        NBO_STORE(v, GLOBAL_PTR(u32x2_e, p));
     }
     DEV float ld1(const char *p) { return bf16_bits_to_f32(*GLOBAL_PTR(const uint16_t, p)); }
     DEV void st1(char *p, float x) { *GLOBAL_PTR(uint16_t, p) = (uint16_t)f32_to_bf16_bits(x); }
@@ -327,19 +349,25 @@ template <int FMT> struct IOHalf16 {
     typedef Half16<FMT> H;
     DEV void ldv(const char *p, H (&x)[8]) { ld_state((const H *)p, x); }
     DEV void stv(char *p, const H (&x)[8]) { st_state((H *)p, x); }
+    DEV void ldv_e(const char *p, H (&x)[8]) { ld_state((const H *)p, x); } // (only ever at vector alignment)
+    DEV void stv_e(char *p, const H (&x)[8]) { st_state((H *)p, x); }
     DEV H ld1(const char *p) { return half_from_bits<FMT>(*GLOBAL_PTR(const uint16_t, p)); }
     DEV void st1(char *p, H x) { *GLOBAL_PTR(uint16_t, p) = x.bits; }
 };
 template <> struct IO<NBO_PBF16> : IOHalf16<FMT_BF16> {};
 template <> struct IO<NBO_PF16> : IOHalf16<FMT_F16> {};
 template <> struct IO<NBO_F16> {
+    DEV void widen(uint32_t lo, uint32_t hi, float (&x)[4])
+    {
+        x[0] = f16_bits_to_f32(lo & 0xFFFFu);
+        x[1] = f16_bits_to_f32(lo >> 16);
+        x[2] = f16_bits_to_f32(hi & 0xFFFFu);
+        x[3] = f16_bits_to_f32(hi >> 16);
+    }
     DEV void ldv(const char *p, float (&x)[4])
     {
         u32x2 v = NBO_LOAD(GLOBAL_PTR(const u32x2, p));
-        x[0] = f16_bits_to_f32(v.x & 0xFFFFu);
-        x[1] = f16_bits_to_f32(v.x >> 16);
-        x[2] = f16_bits_to_f32(v.y & 0xFFFFu);
-        x[3] = f16_bits_to_f32(v.y >> 16);
+        widen(v.x, v.y, x);
     }
     DEV void stv(char *p, const float (&x)[4])
     {
@@ -347,6 +375,18 @@ template <> struct IO<NBO_F16> {
         v.x = f32_to_f16_bits(x[0]) | (f32_to_f16_bits(x[1]) << 16);
         v.y = f32_to_f16_bits(x[2]) | (f32_to_f16_bits(x[3]) << 16);
         NBO_STORE(v, GLOBAL_PTR(u32x2, p));
+    }
+    DEV void ldv_e(const char *p, float (&x)[4])
+    {
+        u32x2_e v = NBO_LOAD(GLOBAL_PTR(const u32x2_e, p));
+        widen(v.x, v.y, x);
+    }
+    DEV void stv_e(char *p, const float (&x)[4])
+    {
+        u32x2_e v;
+        v.x = f32_to_f16_bits(x[0]) | (f32_to_f16_bits(x[1]) << 16);
+        v.y = f32_to_f16_bits(x[2]) | (f32_to_f16_bits(x[3]) << 16);
+        NBO_STORE(v, GLOBAL_PTR(u32x2_e, p));
     }
     DEV float ld1(const char *p) { return f16_bits_to_f32(*GLOBAL_PTR(const uint16_t, p)); }
     DEV void st1(char *p, float x) { *GLOBAL_PTR(uint16_t, p) = (uint16_t)f32_to_f16_bits(x); }
@@ -599,7 +639,13 @@ DEV void update_chunk(const NboUpdateArgs &a, const NboOptimDev *o, uint32_t wg)
 
     const bool direct = KIND == NBO_SGD && a.direct != 0;
     // (by row: how the chunk is walked decides first whether this row exists at all)
-    const Peel pl = peel(c.cnt, VEC, SB, sizeof(T) < 4, (uintptr_t)pp, (uintptr_t)pg);
+    // 16-bit tensors over f32 state: the state moves six times the tensors' bytes, and the arena is
+    // vector-aligned at every chunk's start -- so the state is accessed in whole aligned vectors
+    // from the chunk's first element on, and it is the tensors that are read and written at element
+    // alignment where they are not vector-aligned (packed back to back, or each misaligned
+    // differently).  The 4096-tensor packed set: 0.123 -> 0.115 ms.
+    const Peel whole = {0, c.cnt / VEC};
+    const Peel pl = mixed ? whole : peel(c.cnt, VEC, SB, sizeof(T) < 4, (uintptr_t)pp, (uintptr_t)pg);
     if (BY_ROW && row0 != 0 && row0 * NBO_BLOCK >= pl.nvec) return;
     if (!direct && o->skip) {
         // found_inf: parameters, moments and step_count stay untouched
@@ -673,25 +719,38 @@ DEV void update_chunk(const NboUpdateArgs &a, const NboOptimDev *o, uint32_t wg)
     // ragged chunk, or caller tensors that are not vector-aligned: single elements up to the
     // first vector-aligned address of the caller's tensors, whole vectors from there (the state
     // arrays are then read at element alignment, which needs 32- or 64-bit state), single
-    // elements for the rest
+    // elements for the rest -- or, 16-bit tensors over f32 state, whole vectors from the start
     // (by row: the one vector of this row, if the chunk reaches that far)
     for (uint32_t q = BY_ROW ? row0 * NBO_BLOCK + tid : tid; q < pl.nvec; q += BY_ROW ? NBO_CHUNK : NBO_BLOCK) {
         const uint32_t e = pl.head + q * VEC;
         T g[VEC], p[VEC], m[VEC] = {}, v[VEC] = {};
-        IO<ST>::ldv(pg + (uint64_t)e * SB, g);
-        if (mixed) ld_state_e(aw + e, p);
-        else IO<ST>::ldv(pp + (uint64_t)e * SB, p);
-        if (use_m) ld_state_e(am + e, m);
-        if (has_v) ld_state_e(av + e, v);
+        if (mixed) {
+            IO<ST>::ldv_e(pg + (uint64_t)e * SB, g);
+            ld_state(aw + e, p);
+            if (use_m) ld_state(am + e, m);
+            if (has_v) ld_state(av + e, v);
+        } else {
+            IO<ST>::ldv(pg + (uint64_t)e * SB, g);
+            IO<ST>::ldv(pp + (uint64_t)e * SB, p);
+            if (use_m) ld_state_e(am + e, m);
+            if (has_v) ld_state_e(av + e, v);
+        }
 #pragma unroll
         for (int k = 0; k < VEC; k++) step_elem<T, KIND>(p[k], g[k], m[k], v[k], s);
-        if (mixed) st_state_e(aw + e, p);
-        IO<ST>::stv(pp + (uint64_t)e * SB, p);
-        if (use_m) st_state_e(am + e, m);
-        if (has_v) st_state_e(av + e, v);
+        if (mixed) {
+            st_state(aw + e, p);
+            IO<ST>::stv_e(pp + (uint64_t)e * SB, p);
+            if (use_m) st_state(am + e, m);
+            if (has_v) st_state(av + e, v);
+        } else {
+            IO<ST>::stv(pp + (uint64_t)e * SB, p);
+            if (use_m) st_state_e(am + e, m);
+            if (has_v) st_state_e(av + e, v);
+        }
         if (zero_g) {
             T z[VEC] = {};
-            IO<ST>::stv(pg + (uint64_t)e * SB, z);
+            if (mixed) IO<ST>::stv_e(pg + (uint64_t)e * SB, z);
+            else IO<ST>::stv(pg + (uint64_t)e * SB, z);
         }
     }
     // elements [0, head) and [head + nvec * VEC, cnt)

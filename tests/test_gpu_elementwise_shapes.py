@@ -172,3 +172,67 @@ def test_backend_add_cast_and_adam_over_views(gpu, odd, kind):
         H.assert_bits_equal(H.host_list(p), ref, f"fused AdamW odd={odd} {kind}")
     finally:
         O.set_pow_mode(O.POW_LIBM)
+
+
+@pytest.mark.parametrize("kind", list(SIZES_OF))
+@pytest.mark.parametrize("p_off,g_off", [(0, 0), (1, 1), (1, 3), (0, 5), (2, 0)])
+def test_mixed_adamw_over_views_misaligned_each_in_its_own_way(gpu, kind, p_off, g_off):
+    """bf16 parameters and gradients over f32 master weights, the parameter views starting p_off
+    elements and the gradient views g_off elements past a 16-byte boundary: the update reads the
+    state in whole aligned vectors and the tensors at element alignment, whatever the two offsets
+    are, with and without zeroing of the gradients; neighbours of every view stay untouched."""
+    import torch
+
+    sizes = SIZES_OF[kind]
+    shapes = [(1, n) for n in sizes]
+
+    def views(arrs, off_elems):
+        pad = 16
+        total = sum((a.size + pad + 15) // 16 * 16 for a in arrs) + pad
+        buf = torch.full((total,), 7.0, dtype=torch.bfloat16, device="cuda:0")
+        out, off = [], 0
+        for a in arrs:
+            v = buf[off + off_elems:off + off_elems + a.size].reshape(1, a.size)
+            v.copy_(torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16).reshape(1, a.size))
+            out.append(v)
+            off += (a.size + pad + 15) // 16 * 16
+        return buf, out
+
+    master0 = [O.randn_f32(n, 300 + i, 0.02) for i, n in enumerate(sizes)]
+    p_bits = [O.bf16_from_f32(x) for x in master0]
+    pbuf, p = views(p_bits, p_off)
+    opt = nb.AdamW.new(1e-3, shapes, master=True).beta2(0.95).weight_decay(0.1)
+    for i, a in enumerate(master0):
+        opt.write_state(f"w{i}", H.to_dev(a.reshape(1, -1), shapes[i]))
+    meta = O.adamw_meta(1e-3, beta2=0.95, weight_decay=0.1)
+    ref = dict(p=[x.copy() for x in p_bits], w=[x.copy() for x in master0],
+               m=[np.zeros_like(x) for x in master0], v=[np.zeros_like(x) for x in master0])
+    O.set_pow_mode(O.POW_SQRT)
+    try:
+        for step in range(3):
+            g_bits = [O.bf16_from_f32(O.randn_f32(n, 400 + 31 * step + i, 1e-2)) for i, n in enumerate(sizes)]
+            gbuf, g = views(g_bits, g_off)
+            opt.fused_step(p, g, zero_grads=step == 1)
+            O.mixed_step(meta, None, 0.0, ref["p"], g_bits, ref["w"], ref["m"], ref["v"])
+            got_g = H.host_list(g)
+            if step == 1:
+                assert not any(x.any() for x in got_g), "gradients zeroed"
+            else:
+                H.assert_bits_equal(got_g, g_bits, "gradients untouched")
+            # what lies between the views keeps its fill
+            mask = torch.ones_like(gbuf, dtype=torch.bool)
+            for v in g:
+                start = (v.data_ptr() - gbuf.data_ptr()) // 2
+                mask[start:start + v.numel()] = False
+            assert bool((gbuf[mask] == 7.0).all()), "gaps between the gradient views"
+    finally:
+        O.set_pow_mode(O.POW_LIBM)
+    H.assert_bits_equal(H.host_list(p), ref["p"], f"params p_off={p_off} g_off={g_off} {kind}")
+    H.assert_bits_equal(H.host_list([opt.read_state(f"w{i}") for i in range(len(shapes))]),
+                        ref["w"], "master")
+    H.assert_bits_equal(H.host_list(opt.moments()[1]), ref["v"], "v")
+    mask = torch.ones_like(pbuf, dtype=torch.bool)
+    for v in p:
+        start = (v.data_ptr() - pbuf.data_ptr()) // 2
+        mask[start:start + v.numel()] = False
+    assert bool((pbuf[mask] == 7.0).all()), "gaps between the parameter views"
