@@ -1798,8 +1798,9 @@ template <int ST> DEV void cast_store4(char *p, uint64_t e, const double (&v)[4]
 template <int SRC, int DST> DEV void cast_body(const NboCastListArgs &a, uint32_t wg)
 {
     enum { SS = Traits<SRC>::SBYTES, DS = Traits<DST>::SBYTES };
-    // one workgroup per NBO_CAST_ROW elements of a chunk (four per thread), as the other
-    // element-wise passes run; a ragged or misaligned chunk is done by its first workgroup
+    // one workgroup per NBO_CAST_ROW elements of a chunk (NBO_CAST_QUADS groups of four per thread,
+    // all loaded before the first is stored), as the other element-wise passes run; a ragged or
+    // misaligned chunk is done by its first workgroup
     const uint32_t row = wg % (NBO_CHUNK / NBO_CAST_ROW);
     const ChunkRef c = chunk_ref(a.L, wg / (NBO_CHUNK / NBO_CAST_ROW));
     const char *ps = (const char *)a.src_ptrs[c.t] + c.base * SS;
@@ -1808,10 +1809,12 @@ template <int SRC, int DST> DEV void cast_body(const NboCastListArgs &a, uint32_
     const uint32_t sa = SS * 4 > 16 ? 16 : SS * 4, da = DS * 4 > 16 ? 16 : DS * 4;
     const bool vec_ok = (((uintptr_t)ps & (sa - 1)) | ((uintptr_t)pd & (da - 1))) == 0;
     if (!a.by_chunk && vec_ok && c.cnt == NBO_CHUNK) {
-        double v[4];
+        double v[NBO_CAST_QUADS][4];
         const uint64_t e = (uint64_t)row * NBO_CAST_ROW + threadIdx.x * 4;
-        cast_load4<SRC>(ps, e, v);
-        cast_store4<DST>(pd, e, v);
+#pragma unroll
+        for (uint32_t j = 0; j < NBO_CAST_QUADS; j++) cast_load4<SRC>(ps, e + j * (4 * NBO_BLOCK), v[j]);
+#pragma unroll
+        for (uint32_t j = 0; j < NBO_CAST_QUADS; j++) cast_store4<DST>(pd, e + j * (4 * NBO_BLOCK), v[j]);
         return;
     }
     if (row != 0) return;

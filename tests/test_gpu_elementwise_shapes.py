@@ -127,7 +127,7 @@ def test_sgd_steps_over_views(gpu, dtype, odd, momentum, wd, kind):
 @pytest.mark.parametrize("kind", list(SIZES_OF))
 @pytest.mark.parametrize("odd", [False, True])
 def test_backend_add_cast_and_adam_over_views(gpu, odd, kind):
-    """The backend primitives (two rows per workgroup), the cast (one workgroup per 1024 elements)
+    """The backend primitives (two rows per workgroup), the cast (one workgroup per 2048 elements)
     and the unfused and fused Adam kinds over the same two lists."""
     import torch
 
