@@ -108,15 +108,18 @@ int nbo_free_placed(nbo_placed *p);
 /* One sentence on what the search found (as nbo_optim_state_placement_note). */
 int nbo_placed_note(nbo_placed *p, char *buf, uint64_t buf_bytes);
 
-/* Self-test of the all-bf16 optimizers' arithmetic.  Their division and square root (bf16 operands,
- * the f32 result rounded to bf16) take the hardware's approximate reciprocal and square root where
- * that provably rounds to the same bf16, and the correctly rounded operation elsewhere; this runs
- * all 2^32 pairs of bf16 patterns through the division and all 2^16 patterns through the square
- * root and counts the results whose bits differ from the correctly rounded operation's.  Anything
- * but 0 and 0 is a bug; *example_pair (numerator << 16 | denominator) and *example_arg (may be
- * null) then name one case each.  A few milliseconds.  Synchronous. */
-int nbo_selftest_bf16_arith(uint64_t *div_mismatches, uint64_t *sqrt_mismatches, uint64_t *example_pair,
-                            uint64_t *example_arg);
+/* Self-test of the all-16-bit optimizers' arithmetic (half_type NBO_DT_BF16 or NBO_DT_F16).  Their
+ * division and square root -- 16-bit operands, the f32 result rounded to the type -- do not run the
+ * correctly rounded f32 operation where something cheaper provably rounds to the same 16 bits (bf16:
+ * the hardware's approximate reciprocal and square root, by this library; f16: the compiler's
+ * lowering of a division whose result is narrowed to f16).  This runs all 2^32 pairs of patterns
+ * through the division and all 2^16 patterns through the square root and counts the results that
+ * differ from the exact operation's: the f64 operation narrowed to f32 and then to the type (any NaN
+ * equals any NaN) and, for bf16, also bit for bit the correctly rounded f32 operation followed by
+ * bf16::from_f32.  Anything but 0 and 0 is a bug; *example_pair (numerator << 16 | denominator) and
+ * *example_arg (may be null) then name one case each.  A few milliseconds.  Synchronous. */
+int nbo_selftest_half_arith(int half_type, uint64_t *div_mismatches, uint64_t *sqrt_mismatches,
+                            uint64_t *example_pair, uint64_t *example_arg);
 
 /* Per-kernel timing: while enabled, every kernel launch is bracketed by HIP events on
  * the launch stream.  nbo_profile_read synchronises and returns the number of

@@ -126,8 +126,8 @@ extern "C" {
     pub fn nbo_hbm_ceiling_compare(pattern: c_int, n_shapes: c_int, shapes: *const c_int, iters: *const u32,
                                    spread: c_int, bytes_per_stream: u64, rounds: c_int, reps: c_int, settle_ms: u32,
                                    best_gbps: *mut f64, mean_gbps: *mut f64, regions: *mut c_int) -> c_int;
-    pub fn nbo_selftest_bf16_arith(div_mismatches: *mut u64, sqrt_mismatches: *mut u64, example_pair: *mut u64,
-                                   example_arg: *mut u64) -> c_int;
+    pub fn nbo_selftest_half_arith(half_type: c_int, div_mismatches: *mut u64, sqrt_mismatches: *mut u64,
+                                   example_pair: *mut u64, example_arg: *mut u64) -> c_int;
     pub fn nbo_profile_enable(on: c_int) -> c_int;
     pub fn nbo_profile_read(kernel_name: *const c_char, launches: *mut u64, total_ms: *mut f64) -> c_int;
 }

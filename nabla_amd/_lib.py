@@ -153,7 +153,7 @@ BENCH_SYMBOLS = {
     "nbo_placed_note": (C.c_int, [_P, C.c_char_p, C.c_uint64]),
     "nbo_profile_enable": (C.c_int, [C.c_int]),
     "nbo_profile_read": (C.c_int, [C.c_char_p, _U64P, C.POINTER(C.c_double)]),
-    "nbo_selftest_bf16_arith": (C.c_int, [_U64P, _U64P, _U64P, _U64P]),
+    "nbo_selftest_half_arith": (C.c_int, [C.c_int, _U64P, _U64P, _U64P, _U64P]),
 }
 
 

@@ -204,17 +204,18 @@ int nbo_copy_bytes(const void *src_dev, void *dst_dev, uint64_t bytes)
     });
 }
 
-int nbo_selftest_bf16_arith(uint64_t *div_mismatches, uint64_t *sqrt_mismatches, uint64_t *example_pair,
+int nbo_selftest_half_arith(int half_type, uint64_t *div_mismatches, uint64_t *sqrt_mismatches, uint64_t *example_pair,
                             uint64_t *example_arg)
 {
     return guarded([&] {
         require(div_mismatches && sqrt_mismatches, NBO_ERR_ARG, "null output");
+        require(half_type == NBO_DT_BF16 || half_type == NBO_DT_F16, NBO_ERR_DTYPE, "bf16 or f16");
         Runtime &rt = Runtime::get();
         unsigned long long *out = (unsigned long long *)rt.dmalloc(4 * sizeof(unsigned long long));
         try {
             rt.dzero(out, 4 * sizeof(unsigned long long));
             NboSelftestArgs a = {out};
-            rt.launch(K_SELFTEST_BF16, 65536, NBO_BLOCK, a);
+            rt.launch(half_type == NBO_DT_BF16 ? K_SELFTEST_BF16 : K_SELFTEST_F16, 65536, NBO_BLOCK, a);
             unsigned long long r[4];
             rt.read_back(r, out, sizeof(r));
             *div_mismatches = r[0];

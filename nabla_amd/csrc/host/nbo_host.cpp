@@ -59,10 +59,10 @@ static const char *const kKernelNames[K_COUNT] = {
     "nbo_update_bf16_adam_rows",   "nbo_update_f64_adamw_rows",  "nbo_update_f64_adam_rows",
     "nbo_update_f16_adamw_rows",   "nbo_update_f16_adam_rows",
     "nbo_accscale_f32",            "nbo_accscale_bf16",          "nbo_accscale_f64",
-    "nbo_accscale_f16",            "nbo_selftest_bf16_arith",
+    "nbo_accscale_f16",            "nbo_selftest_bf16_arith",    "nbo_selftest_f16_arith",
 };
 static_assert(K_UPDATE_SELF_BASE + 18 == K_UPDATE_ROWS_BASE, "six families of three self-preparing update kernels");
-static_assert(K_UPDATE_ROWS_BASE + 8 == K_ACCSCALE_BASE && K_ACCSCALE_F16 + 2 == K_COUNT,
+static_assert(K_UPDATE_ROWS_BASE + 8 == K_ACCSCALE_BASE && K_ACCSCALE_F16 + 3 == K_COUNT,
               "four families of two by-row update kernels, four micro-batch kernels without the sum");
 
 static std::mutex g_runtime_mu;

@@ -67,7 +67,8 @@ enum KernelId {
     K_ACCSCALE_BASE = 73, // + st (f32 / bf16 / f64): a micro-batch without the sum of squares
     K_ACCSCALE_F16 = 76,
     K_SELFTEST_BF16 = 77,
-    K_COUNT = 78 // ids from here on are measurement kernels, handed out by Runtime::bench_kernel
+    K_SELFTEST_F16 = 78,
+    K_COUNT = 79 // ids from here on are measurement kernels, handed out by Runtime::bench_kernel
 };
 
 // Lists of fewer chunks than this take the Adam kinds' by-row kernels (nbo_capi.cpp has the measurements).

@@ -151,7 +151,7 @@ template <int FMT> DEV Half16<FMT> half_from_bits(uint32_t b)
 // normal number, the quotient not finite or the square root's argument subnormal (the
 // instructions flush those); then the exact operation is done.  That the results are the exact
 // operations' bits has been checked for all 2^32 pairs and all 2^16 arguments
-// (nbo_selftest_bf16_arith).
+// (the kernel nbo_selftest_bf16_arith below).
 enum { CLS_NAN = 0x003, CLS_INF = 0x204, CLS_DENORMAL = 0x090, CLS_ZERO = 0x060 };
 DEV BF div_exact(BF a, BF b) { return BF(a.f() / b.f()); }
 DEV BF sqrt_exact(BF x) { return BF(__builtin_sqrtf(x.f())); }
@@ -1867,17 +1867,32 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_fill_zero(const NboF
     if (gid < a.bytes - tail0) p[tail0 + gid] = 0;
 }
 
-// Every one of the 2^32 pairs of bf16 patterns through the kernels' bf16 division, every one of the
-// 2^16 patterns through their bf16 square root, compared bit for bit with the exact operations
-// (the f32 operation correctly rounded, then bf16::from_f32).  Workgroup a, thread t: numerator
-// pattern a, denominators t, t + 256, ...
-extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_selftest_bf16_arith(const NboSelftestArgs a)
+// Every one of the 2^32 pairs of 16-bit patterns through the kernels' 16-bit division, every one of
+// the 2^16 patterns through their 16-bit square root, compared with the exact operations.  bf16:
+// bit for bit with the correctly rounded f32 operation followed by bf16::from_f32 (what the
+// kernels computed before they took the hardware's approximations).  Both types: with the f64
+// operation narrowed to f32 and then to the type -- for operands of 8 or 11 significant bits that
+// is the correctly rounded f32 result (a quotient or root that is not exact in 25 bits lies far
+// from every 25-bit number), and it owes nothing to how the compiler lowers an f32 division;
+// any NaN equals any NaN there.  Workgroup a, thread t: numerator pattern a, denominators t,
+// t + 256, ...
+template <int FMT> DEV bool same_or_both_nan(Half16<FMT> x, Half16<FMT> y)
 {
-    const BF x = half_from_bits<FMT_BF16>(blockIdx.x);
+    const uint32_t exp = FMT == FMT_BF16 ? 0x7F80u : 0x7C00u, man = FMT == FMT_BF16 ? 0x007Fu : 0x03FFu;
+    const bool xn = (x.bits & exp) == exp && (x.bits & man) != 0, yn = (y.bits & exp) == exp && (y.bits & man) != 0;
+    return x.bits == y.bits || (xn && yn);
+}
+template <int FMT> DEV void selftest_half_arith(const NboSelftestArgs &a)
+{
+    typedef Half16<FMT> H;
+    const H x = half_from_bits<FMT>(blockIdx.x);
     unsigned long long bad = 0, example = 0;
     for (uint32_t b = threadIdx.x; b < 65536u; b += NBO_BLOCK) {
-        const BF y = half_from_bits<FMT_BF16>(b);
-        if ((x / y).bits != div_exact(x, y).bits) {
+        const H y = half_from_bits<FMT>(b);
+        const H got = x / y;
+        bool ok = same_or_both_nan(got, H((float)((double)x.f() / (double)y.f())));
+        if (FMT == FMT_BF16) ok = ok && got.bits == div_exact(half_from_bits<FMT_BF16>(blockIdx.x), half_from_bits<FMT_BF16>(b)).bits;
+        if (!ok) {
             bad++;
             example = ((unsigned long long)blockIdx.x << 16) | b;
         }
@@ -1886,10 +1901,23 @@ extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_selftest_bf16_arith(
         atomicAdd(&a.out[0], bad);
         a.out[2] = example;
     }
-    if (threadIdx.x == 0 && sqrt_fast(x).bits != sqrt_exact(x).bits) {
-        atomicAdd(&a.out[1], 1ull);
-        a.out[3] = blockIdx.x;
+    if (threadIdx.x == 0) {
+        const H got = sqrt_rn(x);
+        bool ok = same_or_both_nan(got, H((float)__builtin_sqrt((double)x.f())));
+        if (FMT == FMT_BF16) ok = ok && got.bits == sqrt_exact(half_from_bits<FMT_BF16>(blockIdx.x)).bits;
+        if (!ok) {
+            atomicAdd(&a.out[1], 1ull);
+            a.out[3] = blockIdx.x;
+        }
     }
+}
+extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_selftest_bf16_arith(const NboSelftestArgs a)
+{
+    selftest_half_arith<FMT_BF16>(a);
+}
+extern "C" __global__ __launch_bounds__(NBO_BLOCK) void nbo_selftest_f16_arith(const NboSelftestArgs a)
+{
+    selftest_half_arith<FMT_F16>(a);
 }
 
 // Placement probe: every workgroup reads and rewrites the same 8 rows of NBO_BLOCK

@@ -283,8 +283,8 @@ struct NboFillArgs {
     uint64_t bytes;
 };
 
-// nbo_selftest_bf16_arith: out[0] = pairs (a, b) of bf16 patterns whose quotient's bits differ between
-// the kernels' bf16 division and the exact one, out[1] = the same for the square root's arguments,
+// nbo_selftest_{bf16,f16}_arith: out[0] = pairs (a, b) of 16-bit patterns whose quotient differs between
+// the kernels' division and the exact one, out[1] = the same for the square root's arguments,
 // out[2], out[3] = one such pair (a << 16 | b) and one such argument.  The caller zeroes out[].
 struct NboSelftestArgs {
     unsigned long long *out;

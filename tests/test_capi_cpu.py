@@ -254,7 +254,7 @@ def test_null_arguments_are_errors_not_crashes():
         lambda: lib.nbo_optim_load_state(null, b"/nonexistent/x"),
         lambda: lib.nbo_copy_bytes(null, null, 16),
         lambda: lib.nbo_profile_read(null, null, null),
-        lambda: lib.nbo_selftest_bf16_arith(null, null, null, null),
+        lambda: lib.nbo_selftest_half_arith(1, null, null, null, null),
         lambda: lib.nbo_fused_step_noalloc(null, null, null, null, 1.0, 0),
         lambda: lib.nbo_fused_step_norm(null, null, null, 1.0, 1.0, 0),
         lambda: lib.nbo_unscale_accumulate(null, null, null, 0, null, null),

@@ -1,5 +1,5 @@
-"""The all-bf16 optimizers' division and square root against the correctly rounded operations,
-exhaustively: every pair of bf16 patterns, every bf16 pattern."""
+"""The all-16-bit optimizers' division and square root against the exact operations, exhaustively:
+every pair of 16-bit patterns, every 16-bit pattern."""
 import ctypes as C
 
 import pytest
@@ -8,16 +8,20 @@ from nabla_amd import _lib
 
 
 @pytest.mark.gpu
-def test_bf16_division_and_square_root_equal_the_exact_operations_for_every_operand(gpu):
-    """Optimizer<bf16> divides and takes square roots of bf16 numbers (the f32 operation, rounded to
-    bf16: common/scalar/mod.rs:253-351).  The kernels use the hardware's approximate reciprocal and
-    square root where the operands' 8 significant bits guarantee the same bf16, and the exact
-    operation elsewhere; the library compares both forms on the device for all 2^32 quotients and
-    all 2^16 square roots, NaN payloads and signed zeros included."""
+@pytest.mark.parametrize("half", ["bf16", "f16"])
+def test_16_bit_division_and_square_root_equal_the_exact_operations_for_every_operand(gpu, half):
+    """Optimizer<bf16> / Optimizer<f16> divide and take square roots of 16-bit numbers (the f32
+    operation, rounded to the type: common/scalar/mod.rs:253-351).  The bf16 kernels use the
+    hardware's approximate reciprocal and square root where the operands' 8 significant bits
+    guarantee the same bf16, and the exact operation elsewhere; for f16 the compiler lowers the
+    division whose result is narrowed to f16 more cheaply than a correctly rounded f32 division.
+    The library compares what the kernels compute with the exact operation (through f64; bf16 also
+    bit for bit with the correctly rounded f32 operation) on the device for all 2^32 quotients and
+    all 2^16 square roots, signed zeros, subnormals and infinities included."""
     _lib.init()
     lib = _lib.load()
     div, sq, pair, arg = C.c_uint64(1), C.c_uint64(1), C.c_uint64(0), C.c_uint64(0)
-    _lib.check(lib.nbo_selftest_bf16_arith(C.byref(div), C.byref(sq), C.byref(pair), C.byref(arg)))
+    _lib.check(lib.nbo_selftest_half_arith({"bf16": _lib.DT_BF16, "f16": _lib.DT_F16}[half], C.byref(div), C.byref(sq), C.byref(pair), C.byref(arg)))
     assert (div.value, sq.value) == (0, 0), (
         f"{div.value} quotients differ (e.g. {pair.value >> 16:#06x} / {pair.value & 0xFFFF:#06x}), "
         f"{sq.value} square roots (e.g. of {arg.value:#06x})")
