@@ -114,7 +114,10 @@ const char *nbo_version(void);
  * what the HIP runtime knows about it -- device-accessible memory, the tensor ending
  * inside its allocation -- and return NBO_ERR_ARG otherwise (a host pointer or an
  * oversized shape would fault the GPU); NBO_CHECK_POINTERS=0 in the environment skips
- * that.  The same holds for the device buffers of nbo_optim_state_read / _write. */
+ * that.  The same holds for the device buffers of nbo_optim_state_read / _write.  A tensor
+ * may start at any address that is a multiple of its element size (views into flat buffers,
+ * tensors packed back to back): whole 16-byte vectors are used wherever the addresses allow,
+ * and 16-bit tensors over f32 state are accessed in whole vectors at any even address. */
 int nbo_list_create(uint64_t n_tensors, const uint64_t *rows, const uint64_t *cols, int dtype,
                     const void *const *dev_ptrs, nbo_list **out);
 int nbo_list_set_ptrs(nbo_list *list, const void *const *dev_ptrs);
